@@ -1,0 +1,151 @@
+/*
+ * ace_eval.h -- C ABI of the MI355X batched plan evaluator (libace_eval.so).
+ *
+ * The reference (microsoft/SuperScaler, Aceso artifact) has no FFI on this path: the
+ * boundary is the Python module search/aceso_cost_model.py, imported by
+ * search/aceso_search.py:4, search/aceso_prims.py:7 and search/gen_megatron_plan.py:8.
+ * Each entry point below names the reference function(s) it replaces.
+ *
+ * Conventions: plain pointers and sizes only; every "d_" pointer is DEVICE memory owned by
+ * the caller (a torch tensor's data_ptr(), a hipMalloc'ed block ...); nothing allocated by
+ * the library crosses the boundary except the opaque handle.  All calls return 0 or a
+ * negative ACE_E* code; ace_strerror() names it.  Work is enqueued on the hipStream_t the
+ * caller passes (as void*, NULL = the default stream); results are valid once that stream
+ * has been synchronised.  One handle belongs to one device and must be created after any
+ * fork() (the reference's search forks one process per pipeline depth).
+ */
+#ifndef ACE_EVAL_H
+#define ACE_EVAL_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ACE_ABI_VERSION 1
+#define ACE_MAX_STAGES 16      /* aceso_utils.py:502: end_num_stages = min(num_gpus, 16) */
+#define ACE_STAGE_REC 18       /* doubles per stage record, see ACE_R_* */
+
+enum {
+    ACE_OK = 0,
+    ACE_EINVAL = -1,      /* null pointer / bad size / bad table geometry */
+    ACE_ETOOBIG = -2,     /* a single op type's table row exceeds LDS */
+    ACE_EHIP = -3,        /* a HIP runtime call failed (ace_last_hip_error() says which) */
+    ACE_ENOMEM = -4,
+    ACE_EVERSION = -5,
+};
+
+/* per-plan status bytes written by ace_score_batch */
+enum {
+    ACE_PLAN_OK = 0,
+    ACE_PLAN_BAD_MBS = 1,      /* micro_bs // dp not a profiled micro-batch size: the reference raises
+                                  KeyError (aceso_cost_model.py:22-25) */
+    ACE_PLAN_BAD_RESHARD = 2,  /* inconsistent specs inside a stage (TypeError at aceso_cost_model.py:344)
+                                  or a collective never profiled for that group size (KeyError, :251) */
+};
+
+/* indices into a stage record (doubles); units as in the reference: us, MB */
+enum {
+    ACE_R_FWD = 0, ACE_R_BWD, ACE_R_IN_COMM, ACE_R_OUT_COMM, ACE_R_RECOMP,   /* get_time_v3 / get_recompute_time_v3 */
+    ACE_R_WEIGHTS, ACE_R_INPUTS, ACE_R_ACT, ACE_R_SAVED, ACE_R_PEAK, ACE_R_RESERVED, /* get_memory_v3 ... get_reserved_memory */
+    ACE_R_IDEAL_FWD, ACE_R_IDEAL_BWD, ACE_R_IDEAL_IN, ACE_R_IDEAL_OUT,       /* the tp=dp=1 pass, aceso_cost_model.py:588-592 */
+    ACE_R_STAGE_MS, ACE_R_STAGE_MB, ACE_R_SPARE
+};
+
+/*
+ * Compiled tables of one (model, profile database, settings) triple; built on the host by
+ * superscaler_amd.tables.compile_tables().  All pointers are HOST memory, copied during
+ * ace_create().  Replaces the module state read_profiled_time() fills
+ * (aceso_cost_model.py:27-183) plus the per-call lookups get_op_spec / get_reshard_primitives
+ * / get_reshard_time / intra_node_band / inter_node_band (:185-299), which are resolved into
+ * these tables ahead of time.
+ */
+typedef struct ace_tables {
+    int32_t abi_version;
+    int32_t num_ops;        /* N: positions in the op sequence */
+    int32_t num_types;      /* distinct op names (table rows) */
+    int32_t n_mbs, n_tp, n_algo;
+    int32_t n_diag;         /* distinct (micro_bs, stage gpus) -> per-tp micro-batch index maps */
+    int32_t n_glog;         /* stage device counts 2^0 .. 2^(n_glog-1) */
+    int32_t n_z;            /* resharding cost tables (one per (collective, group size) in use) */
+    int32_t n_pair_kinds;   /* distinct adjacent-op spec pairings */
+    int32_t row_doubles;    /* doubles per type row (even) */
+    int32_t hot_off, start_off, out_off, z_off;   /* sub-table offsets inside a row, in doubles */
+    int32_t n_windows;      /* >= 1; > 1 when the rows do not all fit in LDS */
+    int32_t lds_row_bytes;  /* bytes of LDS reserved for resident rows */
+    int32_t flags;          /* ACE_F_* */
+    double main_params, optimizer;   /* aceso_utils.py:48-52 */
+    const double *rows;            /* [num_types][row_doubles] */
+    const uint32_t *pos_info;      /* [num_ops + 1][4]: row byte offset, previous op's row byte offset,
+                                      pair kind | flags << 8, spare */
+    const uint8_t *pair_kinds;     /* [n_pair_kinds][n_glog][C][C], C = n_tp * n_algo */
+    const uint32_t *stage_lut;     /* [n_mbs][16]: diag | per-tp mbs-index nibbles << 8 */
+    const double *nb_minus_1;      /* [n_mbs]: global_bs // micro_bs - 1 */
+    const int32_t *win_pos;        /* [n_windows + 1] first position of each window */
+    const int32_t *win_row_begin;  /* [n_windows + 1] into win_rows */
+    const uint32_t *win_rows;      /* [..][2]: type id, LDS byte offset */
+} ace_tables_t;
+
+#define ACE_F_RESHARDING 1      /* args.resharding (aceso_utils.py:523-526) */
+#define ACE_F_RESERVED_MIN 2    /* memory_pred_type == "MIN" (aceso_cost_model.py:482) */
+#define ACE_F_NO_RESERVED 4     /* not consider_reserved_space (aceso_cost_model.py:525-528) */
+
+typedef struct ace_handle ace_handle_t;
+
+/* A batch of plans, structure-of-arrays, resident in device memory.
+ *  d_codes: uint8, one byte per (op, plan): bits 0-2 = tp_log2 * n_algo + algo, bit 3 = recompute,
+ *           bit 4 = this op starts a pipeline stage.  Laid out [ceil(N/16)][n_plans][16]: sixteen
+ *           consecutive ops of one plan are contiguous, consecutive plans follow each other, so a
+ *           wavefront (one plan per lane) reads 1 KiB contiguous per load.
+ *  d_hdr:   uint32[n_plans][4]: num_stages | micro-batch index << 8;  log2(stage gpus), 4 bits per
+ *           stage (two words);  in-cross-node bit per stage | out-cross-node bits << 16
+ *           (aceso_cost_model.py:572-574).
+ * Replaces AcesoConfig / AcesoStageInfo (aceso_utils.py:58-89) as the scoring input. */
+typedef struct ace_batch {
+    const uint8_t *d_codes;
+    const uint32_t *d_hdr;
+    size_t n_plans;
+} ace_batch_t;
+
+int ace_abi_version(void);
+const char *ace_strerror(int code);
+const char *ace_last_hip_error(void);
+
+/* Upload tables to the current device.  Replaces read_profiled_time (aceso_cost_model.py:27). */
+int ace_create(const ace_tables_t *tables, ace_handle_t **out);
+void ace_destroy(ace_handle_t *h);
+
+/* Score every plan of the batch: predict_time_breakdown (aceso_cost_model.py:541-672) followed by
+ * the callers' reductions max(time_list), max(memory_list) and the feasibility test
+ * max(memory_list) <= memory_limit (aceso_search.py:66; strict != 0 selects `<`,
+ * gen_megatron_plan.py:111).
+ *  d_iter_ms, d_peak_mb: double[n_plans];  d_feasible, d_status: uint8[n_plans] (d_status may be NULL)
+ *  d_stage_out: NULL, or double[n_plans][ACE_MAX_STAGES][ACE_STAGE_REC] receiving the per-stage
+ *  quantities predict_time_breakdown / predict_stage_time / predict_stage_memory are made of. */
+int ace_score_batch(ace_handle_t *h, const ace_batch_t *batch, double memory_limit, int strict,
+                    double *d_iter_ms, double *d_peak_mb, uint8_t *d_feasible, uint8_t *d_status,
+                    double *d_stage_out, void *stream);
+
+/* The k feasible plans with the smallest iteration time, ascending, ties broken by the lower plan
+ * index: the order sort_configs (aceso_utils.py:723-740) / gen_megatron_plan.py:131-135 produce.
+ *  d_idx: int64[k], d_val: double[k]; entries past the number of feasible plans are -1 / +inf.
+ *  d_workspace: device scratch of at least ace_topk_workspace_bytes(n, k) bytes.
+ *  *d_count (int32, device, may be NULL) receives min(k, number of feasible plans). */
+size_t ace_topk_workspace_bytes(size_t n, int k);
+int ace_topk(ace_handle_t *h, const double *d_iter_ms, const uint8_t *d_feasible, size_t n, int k,
+             int64_t *d_idx, double *d_val, int32_t *d_count, void *d_workspace, size_t workspace_bytes,
+             void *stream);
+
+/* Average duration in milliseconds of the `reps` scoring-kernel launches of one
+ * ace_score_batch-equivalent call sequence, measured with hipEvents on `stream`
+ * (for bench.py's roofline figure; not part of the reference). */
+int ace_time_score_kernel(ace_handle_t *h, const ace_batch_t *batch, double memory_limit, int strict,
+                          double *d_iter_ms, double *d_peak_mb, uint8_t *d_feasible, int reps,
+                          void *stream, double *avg_ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ACE_EVAL_H */

@@ -1,0 +1,555 @@
+// MI355X (gfx950) batched plan evaluator: kernels and C ABI (see include/ace_eval.h).
+//
+// Scoring kernel: one plan per lane.  All lanes of a workgroup walk the op sequence in
+// lockstep, so the op type at each step is wave-uniform: the row of profiled values for
+// that type sits in LDS at a scalar base address and each lane only adds its own
+// (micro-batch, tp, algo) offset -- at most n_tp*n_algo distinct, consecutive entries per
+// sub-table, i.e. LDS reads without bank conflicts.  Plan bytes are stored plan-minor
+// ([16-op group][plan][16 bytes]) so a wavefront's load covers 1 KiB of consecutive HBM.
+// Every plan's sums run sequentially in op order in fp64, which reproduces the reference's
+// Python floats bit for bit.  When the rows of all op types do not fit in LDS the op
+// sequence is cut into windows and the workgroup restages the rows at each window boundary.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+#include <new>
+
+#include "ace_plan_state.h"
+
+namespace {
+
+constexpr int kBlock = 1024;             // lanes (= plans) per workgroup: 16 wavefronts, 4 per SIMD
+constexpr uint32_t kMaxLds = 160 * 1024;  // CDNA4 LDS per workgroup
+
+thread_local char g_hip_err[256] = "";
+
+#define ACE_HIP(call)                                                                          \
+    do {                                                                                       \
+        hipError_t e_ = (call);                                                                \
+        if (e_ != hipSuccess) {                                                                \
+            snprintf(g_hip_err, sizeof(g_hip_err), "%s failed: %s", #call, hipGetErrorString(e_)); \
+            return ACE_EHIP;                                                                   \
+        }                                                                                      \
+    } while (0)
+
+struct AceKernelArgs {
+    AceGeom g;
+    const ace_u4 *codes;        // [G][P] 16 op bytes each
+    const ace_u4 *hdr;          // [P]
+    const double *rows;         // [n_types][row_doubles]
+    const ace_u4 *pos_info;     // [N + 1]
+    const uint8_t *pair_kinds;  // -> LDS
+    const uint32_t *stage_lut;  // -> LDS
+    const double *nbm1;         // [n_mbs]
+    const int32_t *win_pos;     // [n_windows + 1]
+    const int32_t *win_row_begin;
+    const uint32_t *win_rows;   // pairs (type, lds byte offset)
+    int32_t n_windows, row_doubles, rk_bytes, stg_words;
+    double *iter_ms, *peak_mb;
+    uint8_t *feasible, *status;
+    double *stage_out;
+};
+
+template <bool BD>
+__global__ __launch_bounds__(kBlock) void ace_score_kernel(const AceKernelArgs a) {
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    const AceGeom &g = a.g;
+    const int tid = threadIdx.x;
+    const long long plan = (long long)blockIdx.x * kBlock + tid;
+    const bool active = plan < g.P;
+    const long long pl = active ? plan : (long long)g.P - 1;
+
+    // small tables: pair kinds and the (micro-batch, stage gpus) LUT
+    for (int j = tid; j < a.rk_bytes; j += kBlock) lds_raw[g.rk_lds_off + j] = a.pair_kinds[j];
+    for (int j = tid; j < a.stg_words; j += kBlock)
+        reinterpret_cast<uint32_t *>(lds_raw + g.stg_lds_off)[j] = a.stage_lut[j];
+    __syncthreads();
+
+    AceLds lds{lds_raw};
+    PlanState<BD> st;
+    const ace_u4 h = a.hdr[pl];
+    st.init(g, lds, h);
+    const double nbm1 = a.nbm1[st.bidx];
+    double *rec = (BD && a.stage_out && active) ? a.stage_out + (size_t)plan * (ACE_MAX_STAGES * ACE_STAGE_REC) : nullptr;
+
+    int w = 0;
+    int next_win = a.win_pos[0];
+    ace_u4 cw = a.codes[pl];
+    for (int grp = 0; grp < g.G; ++grp) {
+        ace_u4 nxt = cw;
+        if (grp + 1 < g.G) nxt = a.codes[(size_t)(grp + 1) * g.P + pl];
+        const uint32_t words[4] = {cw.x, cw.y, cw.z, cw.w};
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            const int i = grp * 16 + k;
+            if (i >= g.N) break;
+            if (i == next_win) {
+                // restage the rows this window needs; every lane of the workgroup gets here together
+                __syncthreads();
+                const int rb = a.win_row_begin[w], re = a.win_row_begin[w + 1];
+                const int n16 = a.row_doubles / 2;
+                for (int r = rb; r < re; ++r) {
+                    const uint32_t type = a.win_rows[2 * r], off = a.win_rows[2 * r + 1];
+                    const ace_d2 *src = reinterpret_cast<const ace_d2 *>(a.rows + (size_t)type * a.row_doubles);
+                    ace_d2 *dst = reinterpret_cast<ace_d2 *>(lds_raw + off);
+                    for (int j = tid; j < n16; j += kBlock) dst[j] = src[j];
+                }
+                __syncthreads();
+                ++w;
+                next_win = a.win_pos[w];
+            }
+            const uint32_t byte = (words[k >> 2] >> ((k & 3) * 8)) & 0xffu;
+            const ace_u4 info = a.pos_info[i];
+            st.step(g, lds, byte, info, rec);
+        }
+        cw = nxt;
+    }
+    const ace_u4 last = a.pos_info[g.N];
+    st.finish(g, lds, last.y, rec);
+    double iter, peak;
+    uint8_t feas, stat;
+    st.result(g, nbm1, iter, peak, feas, stat);
+    if (active) {
+        a.iter_ms[plan] = iter;
+        a.peak_mb[plan] = peak;
+        a.feasible[plan] = feas;
+        if (a.status) a.status[plan] = stat;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// top-k: radix select on the order-preserving 64-bit image of the iteration time, then a
+// gather of everything below the k-th key plus the lowest-indexed ties, then a small sort.
+// ------------------------------------------------------------------------------------------
+constexpr int kTopBlock = 256;
+constexpr int kRadixBits = 11;
+constexpr int kRadix = 1 << kRadixBits;
+constexpr int kPasses = 6;               // 6 * 11 = 66 >= 64 key bits
+constexpr unsigned long long kInfKey = 0xffffffffffffffffull;
+
+struct TopkState {                     // lives in the caller's workspace
+    unsigned long long prefix;         // key bits fixed so far (from the top)
+    unsigned long long thr;            // final k-th smallest key
+    unsigned int k_rem;                // how many still to pick inside the current bucket
+    unsigned int n_feasible;
+    unsigned int n_less;               // entries with key < thr
+    unsigned int n_out_less;           // atomic cursor for the gather of "< thr"
+    unsigned int n_ties;               // atomic cursor for tie candidates
+    unsigned int pad;
+};
+
+__device__ __forceinline__ unsigned long long time_key(double t, uint8_t feasible) {
+    // positive doubles order like their bit patterns; infeasible or NaN plans sort last
+    if (!feasible || !(t == t)) return kInfKey;
+    unsigned long long b = (unsigned long long)__double_as_longlong(t);
+    return (b >> 63) ? ~b : (b | 0x8000000000000000ull);
+}
+
+__device__ __forceinline__ int pass_shift(int pass) {
+    int s = 64 - kRadixBits * (pass + 1);
+    return s < 0 ? 0 : s;
+}
+__device__ __forceinline__ int pass_bits(int pass) {
+    int hi = 64 - kRadixBits * pass;
+    int lo = pass_shift(pass);
+    return hi - lo;
+}
+
+__global__ void topk_init(TopkState *st, unsigned int *hist, int k) {
+    for (int j = threadIdx.x; j < kRadix; j += blockDim.x) hist[j] = 0;
+    if (threadIdx.x == 0) {
+        st->prefix = 0; st->thr = 0; st->k_rem = (unsigned)k; st->n_feasible = 0;
+        st->n_less = 0; st->n_out_less = 0; st->n_ties = 0; st->pad = 0;
+    }
+}
+
+__global__ __launch_bounds__(kTopBlock) void topk_hist(const double *t, const uint8_t *f, size_t n, int pass,
+                                                       const TopkState *st, unsigned int *hist) {
+    __shared__ unsigned int lh[kRadix];
+    for (int j = threadIdx.x; j < kRadix; j += kTopBlock) lh[j] = 0;
+    __syncthreads();
+    const int shift = pass_shift(pass);
+    const int bits = pass_bits(pass);
+    const unsigned long long prefix = st->prefix;
+    const int hi_shift = shift + bits;   // bits above this are already fixed
+    for (size_t i = (size_t)blockIdx.x * kTopBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kTopBlock) {
+        unsigned long long key = time_key(t[i], f[i]);
+        bool match = hi_shift >= 64 ? true : ((key >> hi_shift) == (prefix >> hi_shift));
+        if (match) atomicAdd(&lh[(unsigned)((key >> shift) & ((1ull << bits) - 1))], 1u);
+    }
+    __syncthreads();
+    for (int j = threadIdx.x; j < kRadix; j += kTopBlock)
+        if (lh[j]) atomicAdd(&hist[j], lh[j]);
+}
+
+__global__ void topk_pick(TopkState *st, unsigned int *hist, int pass) {
+    // single workgroup: find the bucket holding the k_rem-th entry, descend into it
+    __shared__ unsigned int sh[kRadix];
+    for (int j = threadIdx.x; j < kRadix; j += blockDim.x) sh[j] = hist[j];
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const int bits = pass_bits(pass);
+        const int shift = pass_shift(pass);
+        unsigned int rem = st->k_rem, acc = 0;
+        int b = 0;
+        const int nb = 1 << bits;
+        for (; b < nb; ++b) {
+            if (acc + sh[b] >= rem) break;
+            acc += sh[b];
+        }
+        if (b >= nb) b = nb - 1;         // fewer than k entries overall: everything qualifies
+        st->prefix |= ((unsigned long long)b) << shift;
+        st->k_rem = rem - acc;
+        st->n_less += acc;
+        if (pass == kPasses - 1) st->thr = st->prefix;
+    }
+    __syncthreads();
+    for (int j = threadIdx.x; j < kRadix; j += blockDim.x) hist[j] = 0;
+}
+
+struct Cand { unsigned long long key; long long idx; };
+
+__global__ __launch_bounds__(kTopBlock) void topk_gather(const double *t, const uint8_t *f, size_t n, TopkState *st,
+                                                         Cand *less, Cand *ties, unsigned int cap_less, unsigned int cap_ties) {
+    const unsigned long long thr = st->thr;
+    for (size_t i = (size_t)blockIdx.x * kTopBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kTopBlock) {
+        unsigned long long key = time_key(t[i], f[i]);
+        if (key == kInfKey) continue;
+        if (key < thr) {
+            unsigned int p = atomicAdd(&st->n_out_less, 1u);
+            if (p < cap_less) less[p] = Cand{key, (long long)i};
+        } else if (key == thr) {
+            unsigned int p = atomicAdd(&st->n_ties, 1u);
+            if (p < cap_ties) ties[p] = Cand{key, (long long)i};
+        }
+    }
+}
+
+// When more ties than fit were seen, pick the lowest-indexed ones with a second select on the
+// index (done by a single workgroup scanning the input: ties beyond capacity are rare --
+// duplicated plans -- and this keeps the result exact).
+__global__ __launch_bounds__(kTopBlock) void topk_ties_exact(const double *t, const uint8_t *f, size_t n, TopkState *st,
+                                                             Cand *ties, unsigned int want) {
+    // sequential-by-chunks scan in index order; each chunk's matches are compacted in order
+    __shared__ unsigned int cnt[kTopBlock];
+    __shared__ unsigned int base;
+    const unsigned long long thr = st->thr;
+    if (threadIdx.x == 0) base = 0;
+    __syncthreads();
+    for (size_t start = 0; start < n; start += kTopBlock) {
+        size_t i = start + threadIdx.x;
+        bool m = i < n && time_key(t[i], f[i]) == thr;
+        cnt[threadIdx.x] = m ? 1u : 0u;
+        __syncthreads();
+        // inclusive scan (Hillis-Steele)
+        for (int off = 1; off < kTopBlock; off <<= 1) {
+            unsigned int v = threadIdx.x >= off ? cnt[threadIdx.x - off] : 0u;
+            __syncthreads();
+            cnt[threadIdx.x] += v;
+            __syncthreads();
+        }
+        unsigned int pos = base + cnt[threadIdx.x] - 1u;
+        if (m && pos < want) ties[pos] = Cand{thr, (long long)i};
+        __syncthreads();
+        if (threadIdx.x == 0) base += cnt[kTopBlock - 1];
+        __syncthreads();
+        if (base >= want) break;
+    }
+    if (threadIdx.x == 0) st->n_ties = base < want ? base : want;
+}
+
+// Sort the candidates (key asc, index asc) in one workgroup (bitonic, in global memory for
+// sizes beyond LDS) and write the first k.
+__global__ __launch_bounds__(1024) void topk_finish(TopkState *st, Cand *less, Cand *ties, unsigned int cap_ties, int k,
+                                                    Cand *buf, unsigned int buf_pow2, long long *out_idx, double *out_val,
+                                                    int *out_count) {
+    const unsigned int n_less = st->n_less;
+    unsigned int n_ties = st->n_ties < cap_ties ? st->n_ties : cap_ties;
+    const unsigned int total = n_less + n_ties;
+    for (unsigned int j = threadIdx.x; j < buf_pow2; j += blockDim.x) {
+        Cand c{kInfKey, 0x7fffffffffffffffll};
+        if (j < n_less) c = less[j];
+        else if (j < total) c = ties[j - n_less];
+        buf[j] = c;
+    }
+    __syncthreads();
+    for (unsigned int size = 2; size <= buf_pow2; size <<= 1) {
+        for (unsigned int stride = size >> 1; stride > 0; stride >>= 1) {
+            for (unsigned int j = threadIdx.x; j < buf_pow2; j += blockDim.x) {
+                unsigned int partner = j ^ stride;
+                if (partner > j) {
+                    Cand x = buf[j], y = buf[partner];
+                    bool up = (j & size) == 0;
+                    bool gt = x.key > y.key || (x.key == y.key && x.idx > y.idx);
+                    if (gt == up) { buf[j] = y; buf[partner] = x; }
+                }
+            }
+            __syncthreads();
+        }
+    }
+    unsigned int cnt = total < (unsigned)k ? total : (unsigned)k;
+    for (unsigned int j = threadIdx.x; j < (unsigned)k; j += blockDim.x) {
+        if (j < cnt) {
+            Cand c = buf[j];
+            unsigned long long b = c.key;
+            b = (b >> 63) ? (b & 0x7fffffffffffffffull) : ~b;
+            out_idx[j] = c.idx;
+            out_val[j] = __longlong_as_double((long long)b);
+        } else {
+            out_idx[j] = -1;
+            out_val[j] = __longlong_as_double(0x7ff0000000000000ll);
+        }
+    }
+    if (threadIdx.x == 0 && out_count) *out_count = (int)cnt;
+}
+
+unsigned int next_pow2(unsigned int v) {
+    unsigned int p = 1;
+    while (p < v) p <<= 1;
+    return p;
+}
+
+}  // namespace
+
+struct ace_handle {
+    int device;
+    AceGeom geom;
+    int32_t n_windows, row_doubles, rk_bytes, stg_words, num_types;
+    uint32_t lds_bytes;
+    // device copies
+    double *d_rows;
+    ace_u4 *d_pos_info;
+    uint8_t *d_pair_kinds;
+    uint32_t *d_stage_lut;
+    double *d_nbm1;
+    int32_t *d_win_pos, *d_win_row_begin;
+    uint32_t *d_win_rows;
+};
+
+extern "C" {
+
+int ace_abi_version(void) { return ACE_ABI_VERSION; }
+
+const char *ace_strerror(int code) {
+    switch (code) {
+        case ACE_OK: return "ok";
+        case ACE_EINVAL: return "invalid argument";
+        case ACE_ETOOBIG: return "table row larger than LDS";
+        case ACE_EHIP: return "HIP runtime error";
+        case ACE_ENOMEM: return "out of memory";
+        case ACE_EVERSION: return "ABI version mismatch";
+        default: return "unknown error";
+    }
+}
+
+const char *ace_last_hip_error(void) { return g_hip_err; }
+
+static int upload(void **dst, const void *src, size_t bytes) {
+    *dst = nullptr;
+    if (bytes == 0) bytes = 16;
+    ACE_HIP(hipMalloc(dst, bytes));
+    if (src) ACE_HIP(hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice));
+    return ACE_OK;
+}
+
+int ace_create(const ace_tables_t *t, ace_handle_t **out) {
+    if (!t || !out) return ACE_EINVAL;
+    *out = nullptr;
+    if (t->abi_version != ACE_ABI_VERSION) return ACE_EVERSION;
+    if (t->num_ops <= 0 || t->num_types <= 0 || t->n_mbs <= 0 || t->n_mbs > 15 || t->n_tp <= 0 || t->n_tp > 4 ||
+        (t->n_algo != 1 && t->n_algo != 2) || t->n_diag <= 0 || t->n_diag > 254 || t->n_glog <= 0 || t->n_glog > 16 ||
+        t->n_z < 0 || t->n_z > 14 || t->n_pair_kinds <= 0 || t->n_pair_kinds > 255 || t->row_doubles <= 0 ||
+        (t->row_doubles & 1) || t->n_windows <= 0 || t->lds_row_bytes <= 0 || (t->lds_row_bytes & 15) ||
+        !t->rows || !t->pos_info || !t->pair_kinds || !t->stage_lut || !t->nb_minus_1 || !t->win_pos ||
+        !t->win_row_begin || !t->win_rows)
+        return ACE_EINVAL;
+    const int C = t->n_tp * t->n_algo;
+    // sub-tables must lie inside a row and be 16-byte aligned
+    const int64_t hot_end = (int64_t)t->hot_off + (int64_t)t->n_diag * C * 6;
+    const int64_t start_end = (int64_t)t->start_off + (int64_t)t->n_diag * C * 4;
+    const int64_t out_end = (int64_t)t->out_off + (int64_t)t->n_mbs * t->n_tp * t->n_algo * 2;
+    const int64_t z_end = (int64_t)t->z_off + (int64_t)t->n_z * t->n_diag * C;
+    if ((t->hot_off & 1) || (t->start_off & 1) || (t->out_off & 1) || (t->z_off & 1) || t->hot_off < 0 ||
+        hot_end > t->row_doubles || start_end > t->row_doubles || out_end > t->row_doubles || z_end > t->row_doubles)
+        return ACE_EINVAL;
+    const int64_t row_bytes = (int64_t)t->row_doubles * 8;
+    if (row_bytes > t->lds_row_bytes) return ACE_ETOOBIG;
+    const int32_t rk_bytes = t->n_pair_kinds * t->n_glog * C * C;
+    const int32_t stg_words = t->n_mbs * 16;
+    const uint32_t rk_off = (uint32_t)t->lds_row_bytes;
+    const uint32_t stg_off = (rk_off + (uint32_t)rk_bytes + 15u) & ~15u;
+    const uint32_t lds_bytes = stg_off + (uint32_t)stg_words * 4u;
+    if (lds_bytes > kMaxLds) return ACE_ETOOBIG;
+    // window tables: every referenced row must fit the resident region; every position's row
+    // offsets must point at a row start inside it
+    const int32_t n_win_rows = t->win_row_begin[t->n_windows];
+    if (t->win_pos[0] != 0 || t->win_row_begin[0] != 0 || n_win_rows <= 0) return ACE_EINVAL;
+    for (int w = 0; w < t->n_windows; ++w) {
+        if (t->win_pos[w + 1] <= t->win_pos[w] || t->win_row_begin[w + 1] < t->win_row_begin[w]) return ACE_EINVAL;
+    }
+    if (t->win_pos[t->n_windows] < t->num_ops) return ACE_EINVAL;
+    for (int r = 0; r < n_win_rows; ++r) {
+        if (t->win_rows[2 * r] >= (uint32_t)t->num_types) return ACE_EINVAL;
+        if ((int64_t)t->win_rows[2 * r + 1] + row_bytes > t->lds_row_bytes || (t->win_rows[2 * r + 1] & 15u)) return ACE_EINVAL;
+    }
+    for (int i = 0; i <= t->num_ops; ++i) {
+        const uint32_t *pi = t->pos_info + 4 * (size_t)i;
+        if ((int64_t)pi[0] + row_bytes > t->lds_row_bytes || (int64_t)pi[1] + row_bytes > t->lds_row_bytes ||
+            (pi[0] & 15u) || (pi[1] & 15u) || (pi[2] & 0xffu) >= (uint32_t)t->n_pair_kinds)
+            return ACE_EINVAL;
+    }
+    for (int j = 0; j < stg_words; ++j) {
+        const uint32_t d = t->stage_lut[j] & 0xffu;
+        if (d != 0xffu && d >= (uint32_t)t->n_diag) return ACE_EINVAL;
+    }
+    for (int j = 0; j < rk_bytes; ++j) {
+        const uint32_t pf = t->pair_kinds[j] & 15u, pb = t->pair_kinds[j] >> 4;
+        if ((pf != 15u && pf > (uint32_t)t->n_z) || (pb != 15u && pb > (uint32_t)t->n_z)) return ACE_EINVAL;
+    }
+
+    ace_handle *h = new (std::nothrow) ace_handle();
+    if (!h) return ACE_ENOMEM;
+    memset(h, 0, sizeof(*h));
+    ACE_HIP(hipGetDevice(&h->device));
+    AceGeom &g = h->geom;
+    g.N = t->num_ops; g.P = 0; g.G = (t->num_ops + 15) / 16;
+    g.C = C; g.A_shift = t->n_algo == 2 ? 1 : 0;
+    g.n_mbs = t->n_mbs; g.n_tp = t->n_tp; g.n_algo = t->n_algo; g.n_glog = t->n_glog; g.n_pair_kinds = t->n_pair_kinds;
+    g.hot_off = (uint32_t)t->hot_off * 8u; g.start_off = (uint32_t)t->start_off * 8u;
+    g.out_off = (uint32_t)t->out_off * 8u; g.z_off = (uint32_t)t->z_off * 8u;
+    g.z_stride = (uint32_t)(t->n_diag * C) * 8u;
+    g.rk_lds_off = rk_off; g.stg_lds_off = stg_off;
+    g.flags = t->flags; g.main_params = t->main_params; g.optimizer = t->optimizer;
+    g.mem_limit = 0.0; g.strict = 0;
+    h->n_windows = t->n_windows; h->row_doubles = t->row_doubles; h->rk_bytes = rk_bytes; h->stg_words = stg_words;
+    h->num_types = t->num_types; h->lds_bytes = lds_bytes;
+    int rc;
+    if ((rc = upload((void **)&h->d_rows, t->rows, (size_t)t->num_types * row_bytes)) ||
+        (rc = upload((void **)&h->d_pos_info, t->pos_info, (size_t)(t->num_ops + 1) * 16)) ||
+        (rc = upload((void **)&h->d_pair_kinds, t->pair_kinds, (size_t)rk_bytes)) ||
+        (rc = upload((void **)&h->d_stage_lut, t->stage_lut, (size_t)stg_words * 4)) ||
+        (rc = upload((void **)&h->d_nbm1, t->nb_minus_1, (size_t)t->n_mbs * 8)) ||
+        (rc = upload((void **)&h->d_win_pos, t->win_pos, (size_t)(t->n_windows + 1) * 4)) ||
+        (rc = upload((void **)&h->d_win_row_begin, t->win_row_begin, (size_t)(t->n_windows + 1) * 4)) ||
+        (rc = upload((void **)&h->d_win_rows, t->win_rows, (size_t)n_win_rows * 8))) {
+        ace_destroy(h);
+        return rc;
+    }
+    ACE_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&ace_score_kernel<false>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
+    ACE_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&ace_score_kernel<true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
+    *out = h;
+    return ACE_OK;
+}
+
+void ace_destroy(ace_handle_t *h) {
+    if (!h) return;
+    (void)hipFree(h->d_rows); (void)hipFree(h->d_pos_info); (void)hipFree(h->d_pair_kinds);
+    (void)hipFree(h->d_stage_lut); (void)hipFree(h->d_nbm1); (void)hipFree(h->d_win_pos);
+    (void)hipFree(h->d_win_row_begin); (void)hipFree(h->d_win_rows);
+    delete h;
+}
+
+static int fill_args(ace_handle_t *h, const ace_batch_t *b, double memory_limit, int strict, double *d_iter_ms,
+                     double *d_peak_mb, uint8_t *d_feasible, uint8_t *d_status, double *d_stage_out, AceKernelArgs *a) {
+    if (!h || !b || !b->d_codes || !b->d_hdr || !d_iter_ms || !d_peak_mb || !d_feasible) return ACE_EINVAL;
+    if (b->n_plans == 0 || b->n_plans > 0x7fffffffull) return ACE_EINVAL;
+    if (((uintptr_t)b->d_codes & 15u) || ((uintptr_t)b->d_hdr & 15u)) return ACE_EINVAL;
+    a->g = h->geom;
+    a->g.P = (int32_t)b->n_plans;
+    a->g.mem_limit = memory_limit;
+    a->g.strict = strict ? 1 : 0;
+    a->codes = reinterpret_cast<const ace_u4 *>(b->d_codes);
+    a->hdr = reinterpret_cast<const ace_u4 *>(b->d_hdr);
+    a->rows = h->d_rows; a->pos_info = h->d_pos_info; a->pair_kinds = h->d_pair_kinds; a->stage_lut = h->d_stage_lut;
+    a->nbm1 = h->d_nbm1; a->win_pos = h->d_win_pos; a->win_row_begin = h->d_win_row_begin; a->win_rows = h->d_win_rows;
+    a->n_windows = h->n_windows; a->row_doubles = h->row_doubles; a->rk_bytes = h->rk_bytes; a->stg_words = h->stg_words;
+    a->iter_ms = d_iter_ms; a->peak_mb = d_peak_mb; a->feasible = d_feasible; a->status = d_status; a->stage_out = d_stage_out;
+    return ACE_OK;
+}
+
+static void launch_score(const ace_handle_t *h, const AceKernelArgs &a, hipStream_t s) {
+    const unsigned blocks = (unsigned)(((size_t)a.g.P + kBlock - 1) / kBlock);
+    if (a.stage_out)
+        hipLaunchKernelGGL(ace_score_kernel<true>, dim3(blocks), dim3(kBlock), h->lds_bytes, s, a);
+    else
+        hipLaunchKernelGGL(ace_score_kernel<false>, dim3(blocks), dim3(kBlock), h->lds_bytes, s, a);
+}
+
+int ace_score_batch(ace_handle_t *h, const ace_batch_t *batch, double memory_limit, int strict, double *d_iter_ms,
+                    double *d_peak_mb, uint8_t *d_feasible, uint8_t *d_status, double *d_stage_out, void *stream) {
+    AceKernelArgs a;
+    int rc = fill_args(h, batch, memory_limit, strict, d_iter_ms, d_peak_mb, d_feasible, d_status, d_stage_out, &a);
+    if (rc) return rc;
+    launch_score(h, a, (hipStream_t)stream);
+    ACE_HIP(hipGetLastError());
+    return ACE_OK;
+}
+
+int ace_time_score_kernel(ace_handle_t *h, const ace_batch_t *batch, double memory_limit, int strict, double *d_iter_ms,
+                          double *d_peak_mb, uint8_t *d_feasible, int reps, void *stream, double *avg_ms) {
+    if (reps <= 0 || !avg_ms) return ACE_EINVAL;
+    AceKernelArgs a;
+    int rc = fill_args(h, batch, memory_limit, strict, d_iter_ms, d_peak_mb, d_feasible, nullptr, nullptr, &a);
+    if (rc) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    hipEvent_t e0, e1;
+    ACE_HIP(hipEventCreate(&e0));
+    ACE_HIP(hipEventCreate(&e1));
+    ACE_HIP(hipEventRecord(e0, s));
+    for (int r = 0; r < reps; ++r) launch_score(h, a, s);
+    ACE_HIP(hipEventRecord(e1, s));
+    ACE_HIP(hipEventSynchronize(e1));
+    float ms = 0.f;
+    ACE_HIP(hipEventElapsedTime(&ms, e0, e1));
+    ACE_HIP(hipEventDestroy(e0));
+    ACE_HIP(hipEventDestroy(e1));
+    ACE_HIP(hipGetLastError());
+    *avg_ms = (double)ms / reps;
+    return ACE_OK;
+}
+
+// workspace layout: TopkState | hist[kRadix] | less[cap] | ties[cap] | buf[pow2(2*cap)]
+static unsigned int topk_cap(int k) { return (unsigned)k; }
+
+size_t ace_topk_workspace_bytes(size_t n, int k) {
+    (void)n;
+    if (k <= 0) return 0;
+    const unsigned cap = topk_cap(k);
+    const unsigned p2 = next_pow2(2 * cap);
+    return 256 + sizeof(unsigned int) * kRadix + sizeof(Cand) * ((size_t)cap * 2 + p2);
+}
+
+int ace_topk(ace_handle_t *h, const double *d_iter_ms, const uint8_t *d_feasible, size_t n, int k, int64_t *d_idx,
+             double *d_val, int32_t *d_count, void *d_workspace, size_t workspace_bytes, void *stream) {
+    if (!h || !d_iter_ms || !d_feasible || !d_idx || !d_val || !d_workspace || n == 0 || k <= 0 || k > (1 << 20)) return ACE_EINVAL;
+    if (workspace_bytes < ace_topk_workspace_bytes(n, k) || ((uintptr_t)d_workspace & 15u)) return ACE_EINVAL;
+    hipStream_t s = (hipStream_t)stream;
+    unsigned char *ws = (unsigned char *)d_workspace;
+    TopkState *st = (TopkState *)ws;
+    unsigned int *hist = (unsigned int *)(ws + 256);
+    const unsigned cap = topk_cap(k);
+    const unsigned p2 = next_pow2(2 * cap);
+    Cand *less = (Cand *)(ws + 256 + sizeof(unsigned int) * kRadix);
+    Cand *ties = less + cap;
+    Cand *buf = ties + cap;
+    unsigned blocks = (unsigned)((n + kTopBlock * 8 - 1) / (kTopBlock * 8));
+    if (blocks < 1) blocks = 1;
+    if (blocks > 2048) blocks = 2048;
+    hipLaunchKernelGGL(topk_init, dim3(1), dim3(256), 0, s, st, hist, k);
+    for (int pass = 0; pass < kPasses; ++pass) {
+        hipLaunchKernelGGL(topk_hist, dim3(blocks), dim3(kTopBlock), 0, s, d_iter_ms, d_feasible, n, pass, st, hist);
+        hipLaunchKernelGGL(topk_pick, dim3(1), dim3(256), 0, s, st, hist, pass);
+    }
+    hipLaunchKernelGGL(topk_gather, dim3(blocks), dim3(kTopBlock), 0, s, d_iter_ms, d_feasible, n, st, less, ties, cap, cap);
+    // ties: the gather keeps an arbitrary subset when more than `cap` plans share the k-th time;
+    // redo them exactly (lowest indices first).  Cheap single-workgroup scan that stops early.
+    hipLaunchKernelGGL(topk_ties_exact, dim3(1), dim3(kTopBlock), 0, s, d_iter_ms, d_feasible, n, st, ties, cap);
+    hipLaunchKernelGGL(topk_finish, dim3(1), dim3(1024), 0, s, st, less, ties, cap, k, buf, p2, (long long *)d_idx, d_val, d_count);
+    ACE_HIP(hipGetLastError());
+    return ACE_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,274 @@
+// Per-plan scoring state machine of the batched Aceso plan evaluator.
+//
+// One instance scores one plan, op by op, in op order, with exactly the floating-point
+// operations (and their association) of the reference's search/aceso_cost_model.py, so the
+// results are bit-identical to the reference's Python floats:
+//   step()    one op: get_time_v3 sums (:307-313), resharding of the (previous, this) op pair
+//             (:340-350), get_recompute_time_v3 (:365-371), get_memory_v3 (:382-392),
+//             get_activations_v3 (:403-415), get_peak_activations (:428-445),
+//             get_reserved_memory maxima (:453-460)
+//   start()   stage head: boundary input size / p2p time (:319-331), per-stage lookup offsets
+//   finish()  stage tail: output p2p (:321-336), stage time (:352-353, :579), stage memory
+//             (predict_stage_memory :514-539, get_reserved_memory :480-483), running
+//             sum / max for the 1F1B composition (:613-619)
+//   result()  iteration time max_s(t_s*(nb-1) + sum t) and peak memory
+//
+// The same source is compiled by hipcc for gfx950 (one plan per lane, tables in LDS) and by
+// g++ with ACE_HOST_EMU for a bounds-checked CPU build used only by tests.
+#pragma once
+#include <stdint.h>
+
+#include "ace_eval.h"
+
+#ifdef ACE_HOST_EMU
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#define ACE_HD inline
+struct AceLds {
+    const unsigned char *base;
+    uint32_t size;
+    template <class T> T ld(uint32_t off) const {
+        if ((uint64_t)off + sizeof(T) > size || (off % (sizeof(T) > 16 ? 16 : sizeof(T))) != 0) {
+            fprintf(stderr, "ace emu: LDS access out of bounds/misaligned: off=%u size=%zu lds=%u\n", off, sizeof(T), size);
+            abort();
+        }
+        T v;
+        memcpy(&v, base + off, sizeof(T));
+        return v;
+    }
+};
+static inline double ace_max(double a, double b) { return a > b ? a : b; }
+static inline bool ace_isnan(double a) { return a != a; }
+#else
+#define ACE_HD __device__ __forceinline__
+struct AceLds {
+    const unsigned char *base;
+    template <class T> ACE_HD T ld(uint32_t off) const { return *reinterpret_cast<const T *>(base + off); }
+};
+ACE_HD double ace_max(double a, double b) { return fmax(a, b); }
+ACE_HD bool ace_isnan(double a) { return a != a; }
+#endif
+
+struct alignas(16) ace_d2 { double x, y; };
+struct alignas(16) ace_u4 { uint32_t x, y, z, w; };
+
+#define ACE_PLAN_MALFORMED 3
+
+// Geometry and constants every lane reads (kernel arguments -> scalar registers).
+struct AceGeom {
+    int32_t N, P, G;            // ops, plans, 16-op groups
+    int32_t C, A_shift;         // codes per diag (n_tp * n_algo), log2(n_algo)
+    int32_t n_mbs, n_tp, n_algo, n_glog, n_pair_kinds;
+    uint32_t hot_off, start_off, out_off, z_off;   // bytes inside a row
+    uint32_t z_stride;          // bytes of one resharding-cost table inside a row (n_diag * C * 8)
+    uint32_t rk_lds_off, stg_lds_off;              // LDS byte offsets of the pair-kind and stage LUT regions
+    int32_t flags;
+    double main_params, optimizer, mem_limit;
+    int32_t strict;
+};
+
+template <bool BD> struct PlanState {
+    // plan constants
+    int S;
+    uint32_t bidx;
+    uint64_t glogs;
+    uint32_t cross;
+    uint32_t ideal_hot_v, ideal_start_v;
+    // stage state
+    int s;
+    uint32_t hot_v, z_v, rk_v, mrow;
+    uint32_t t_first;
+    bool out_cross;
+    double in_comm, inputs, id_in;
+    // per-op accumulators (reset at every stage head)
+    double fwd, bwd, rcs, W, A, saved, run, peak, rfm, rbm, pend_rf, pend_rb, rs_f, rs_b, prev_act;
+    double id_fwd, id_bwd;
+    uint32_t prev_byte;
+    bool lastclose;
+    // plan accumulators
+    double sum_t, max_t, max_mem;
+    uint32_t status;
+
+    ACE_HD void init(const AceGeom &g, const AceLds &lds, ace_u4 h) {
+        S = (int)(h.x & 0xff);
+        bidx = (h.x >> 8) & 0xff;
+        glogs = (uint64_t)h.y | ((uint64_t)h.z << 32);
+        cross = h.w;
+        s = -1;
+        sum_t = 0.0; max_t = 0.0; max_mem = 0.0;
+        status = 0;
+        prev_byte = 0; prev_act = 0.0; lastclose = false;
+        fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = pend_rf = pend_rb = rs_f = rs_b = 0.0;
+        id_fwd = id_bwd = id_in = 0.0;
+        in_comm = inputs = 0.0;
+        hot_v = z_v = rk_v = mrow = t_first = 0;
+        out_cross = false;
+        ideal_hot_v = ideal_start_v = 0;
+        if (bidx >= (uint32_t)g.n_mbs) { status = ACE_PLAN_MALFORMED; bidx = 0; }
+        if (BD) {
+            // the "ideal" pass uses tp = dp = 1 and micro-batch = micro_bs (aceso_cost_model.py:588-590):
+            // the diag of (micro_bs, 1 gpu)
+            uint32_t w = lds.ld<uint32_t>(g.stg_lds_off + (bidx * 16u + 0u) * 4u);
+            uint32_t d = w & 0xff;
+            if (d == 0xff) d = 0;
+            ideal_hot_v = d * (uint32_t)g.C * 48u;
+            ideal_start_v = d * (uint32_t)g.C * 32u;
+        }
+    }
+
+    // Stage head at an op with code `c` whose type row lives at LDS offset `row`.
+    ACE_HD void start(const AceGeom &g, const AceLds &lds, uint32_t row, uint32_t c) {
+        ++s;
+        uint32_t sidx = (uint32_t)(s < ACE_MAX_STAGES ? s : ACE_MAX_STAGES - 1);
+        if (s >= ACE_MAX_STAGES) status = ACE_PLAN_MALFORMED;
+        uint32_t glog = (uint32_t)(glogs >> (4u * sidx)) & 15u;
+        uint32_t w = lds.ld<uint32_t>(g.stg_lds_off + (bidx * 16u + glog) * 4u);
+        uint32_t d = w & 0xff;
+        mrow = w >> 8;
+        if (d == 0xff) { status |= ACE_PLAN_BAD_MBS; d = 0; }
+        if (glog >= (uint32_t)g.n_glog) { status |= ACE_PLAN_BAD_MBS; glog = 0; }
+        hot_v = d * (uint32_t)g.C * 48u;
+        z_v = d * (uint32_t)g.C * 8u;
+        rk_v = glog * (uint32_t)(g.C * g.C);
+        bool in_cross = (cross >> sidx) & 1u;
+        out_cross = (cross >> (16u + sidx)) & 1u;
+        t_first = c >> g.A_shift;
+        uint32_t a = row + g.start_off + d * (uint32_t)g.C * 32u + c * 32u;
+        ace_d2 e0 = lds.ld<ace_d2>(a);          // input size, size / intra-node bandwidth
+        ace_d2 e1 = lds.ld<ace_d2>(a + 16);     // size / inter-node bandwidth, pad
+        inputs = e0.x;
+        in_comm = in_cross ? e1.x : e0.y;
+        if (BD) {
+            uint32_t ai = row + g.start_off + ideal_start_v + (c & (uint32_t)(g.n_algo - 1)) * 32u;
+            ace_d2 i0 = lds.ld<ace_d2>(ai);
+            ace_d2 i1 = lds.ld<ace_d2>(ai + 16);
+            id_in = in_cross ? i1.x : i0.y;
+            id_fwd = 0.0; id_bwd = 0.0;
+        }
+        fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = pend_rf = pend_rb = rs_f = rs_b = 0.0;
+        lastclose = false;
+    }
+
+    // Stage tail; `prevrow` is the LDS offset of the row of the stage's last op, whose code byte
+    // is still in prev_byte.
+    ACE_HD void finish(const AceGeom &g, const AceLds &lds, uint32_t prevrow, double *rec) {
+        uint32_t c_last = prev_byte & 7u;
+        uint32_t t_last = c_last >> g.A_shift;
+        uint32_t a_last = c_last & (uint32_t)(g.n_algo - 1);
+        uint32_t m_last = (mrow >> (4u * t_last)) & 15u;
+        if (m_last >= (uint32_t)g.n_mbs) m_last = 0;   // only for plans already marked BAD_MBS (their sums are NaN)
+        // output_size[ops[-1]][mbs[-1]][tp[0]][algo[-1]]  (sic, aceso_cost_model.py:321-326)
+        uint32_t oidx = ((m_last * (uint32_t)g.n_tp + t_first) << g.A_shift) + a_last;
+        ace_d2 oe = lds.ld<ace_d2>(prevrow + g.out_off + oidx * 16u);
+        double out_comm = out_cross ? oe.y : oe.x;
+        double in_c = in_comm + rs_f * 1000.0;      // :352
+        double out_c = out_comm + rs_b * 1000.0;    // :353
+        double t = ((((fwd + bwd) + in_c) + out_c) + rcs) / 1000.0;   // :579
+        sum_t += t;
+        max_t = ace_max(max_t, t);
+        if (lastclose) peak = ace_max(peak, run);   // :439 "i + 1 == len(ops) - 1" closes the last segment
+        double reserved;
+        if (g.flags & ACE_F_NO_RESERVED) reserved = 0.0;
+        else if (g.flags & ACE_F_RESERVED_MIN) reserved = ace_max(ace_max(rfm, rbm), ace_max(W, 0.0));
+        else reserved = ace_max(rfm + rbm, W) + 0.0;                  // :481 (max_collective = 0)
+        double mp = W * g.main_params;
+        double opt = W * g.optimizer;
+        double x = (inputs + A) - saved;
+        double nsb = (double)(S - 1 - s);
+        double mem_act = x * nsb;                   // :530
+        double mem_peak = x + peak;                 // :531
+        double wts = W + mp;                        // :533
+        double mem = ((((wts + W) + opt) + mem_act) + mem_peak) + reserved;   // :534
+        max_mem = ace_max(max_mem, mem);
+        if (BD && rec != nullptr && s >= 0 && s < ACE_MAX_STAGES) {
+            double *r = rec + (size_t)s * ACE_STAGE_REC;
+            r[ACE_R_FWD] = fwd; r[ACE_R_BWD] = bwd; r[ACE_R_IN_COMM] = in_c; r[ACE_R_OUT_COMM] = out_c;
+            r[ACE_R_RECOMP] = rcs; r[ACE_R_WEIGHTS] = W; r[ACE_R_INPUTS] = inputs; r[ACE_R_ACT] = A;
+            r[ACE_R_SAVED] = saved; r[ACE_R_PEAK] = peak; r[ACE_R_RESERVED] = reserved;
+            // ideal pass: output_size[ops[-1]][mbs index of micro_bs][tp index 0][algo[-1]]
+            uint32_t iidx = ((bidx * (uint32_t)g.n_tp + 0u) << g.A_shift) + a_last;
+            ace_d2 ie = lds.ld<ace_d2>(prevrow + g.out_off + iidx * 16u);
+            r[ACE_R_IDEAL_FWD] = id_fwd; r[ACE_R_IDEAL_BWD] = id_bwd; r[ACE_R_IDEAL_IN] = id_in;
+            r[ACE_R_IDEAL_OUT] = out_cross ? ie.y : ie.x;
+            r[ACE_R_STAGE_MS] = t; r[ACE_R_STAGE_MB] = mem; r[ACE_R_SPARE] = 0.0;
+        }
+    }
+
+    // One op.  `info` is the position's (wave-uniform) descriptor.
+    ACE_HD void step(const AceGeom &g, const AceLds &lds, uint32_t byte, ace_u4 info, double *rec) {
+        const uint32_t c = byte & 7u;
+        const bool rc = (byte >> 3) & 1u;
+        const bool ns = (byte >> 4) & 1u;
+        const uint32_t row = info.x;
+        if (ns) {
+            if (s >= 0) finish(g, lds, info.y, rec);
+            start(g, lds, row, c);
+        }
+        const uint32_t fl = info.z >> 8;
+        uint32_t a = row + g.hot_off + hot_v + c * 48u;
+        ace_d2 e0 = lds.ld<ace_d2>(a);         // fwd us, bwd us
+        ace_d2 e1 = lds.ld<ace_d2>(a + 16);    // weights MB, activations MB (shared-buffer rule applied)
+        ace_d2 e2 = lds.ld<ace_d2>(a + 32);    // fwd / bwd reserved MB
+        // reserved maxima run over every op but the stage's last: fold the previous op now
+        rfm = ace_max(rfm, pend_rf);
+        rbm = ace_max(rbm, pend_rb);
+        pend_rf = e2.x;
+        pend_rb = e2.y;
+        fwd += e0.x;
+        bwd += e0.y;
+        rcs += rc ? e0.x : 0.0;
+        W += e1.x;
+        A += e1.y;
+        if (BD) {
+            ace_d2 ie = lds.ld<ace_d2>(row + g.hot_off + ideal_hot_v + (c & (uint32_t)(g.n_algo - 1)) * 48u);
+            id_fwd += ie.x;
+            id_bwd += ie.y;
+        }
+        // (previous op, this op) both recomputed and in one stage
+        const bool pair = rc && ((prev_byte >> 3) & 1u) && !ns;
+        const bool savez = fl & 1u;     // previous op is an ordinary op followed by a layer start
+        run += pair ? prev_act : 0.0;
+        saved += (pair && !savez) ? prev_act : 0.0;
+        if (!pair || savez) {
+            peak = ace_max(peak, run);
+            run = 0.0;
+        }
+        lastclose = pair && (fl & 2u);
+        prev_act = e1.y;
+        if ((g.flags & ACE_F_RESHARDING) && !ns) {
+            uint32_t pk = info.z & 0xffu;
+            uint32_t pc = prev_byte & 7u;
+            uint32_t r = lds.ld<uint8_t>(g.rk_lds_off + pk * (uint32_t)(g.n_glog * g.C * g.C) + rk_v + pc * (uint32_t)g.C + c);
+            if (r != 0) {
+                uint32_t pf = r & 15u, pb = r >> 4;
+                uint32_t za = row + g.z_off + z_v + c * 8u;
+                if (pf == 15u || pb == 15u) {
+                    status |= ACE_PLAN_BAD_RESHARD;
+                } else {
+                    if (pf) rs_f += lds.ld<double>(za + (pf - 1u) * g.z_stride);
+                    if (pb) rs_b += lds.ld<double>(za + (pb - 1u) * g.z_stride);
+                }
+            }
+        }
+        prev_byte = byte;
+    }
+
+    ACE_HD void result(const AceGeom &g, double nbm1, double &iter_ms, double &peak_mb, uint8_t &feasible, uint8_t &st) {
+        if (s + 1 != S) status = ACE_PLAN_MALFORMED;
+        // max over stages of t_s*(nb-1) + sum(t): rounding is monotonic, so the maximum is attained
+        // at the largest t_s and equals this expression bit for bit
+        iter_ms = max_t * nbm1 + sum_t;
+        peak_mb = max_mem;
+        bool ok = status == 0 && !ace_isnan(iter_ms) && !ace_isnan(max_mem);
+        if (!ok && status == 0) status = ACE_PLAN_BAD_MBS;   // a table entry outside the profiled grid
+        bool feas = g.strict ? (max_mem < g.mem_limit) : (max_mem <= g.mem_limit);
+        feasible = (uint8_t)(ok && feas);
+        st = (uint8_t)status;
+        if (!ok) {
+            iter_ms = __builtin_nan("");
+            peak_mb = __builtin_nan("");
+        }
+    }
+};

@@ -1,0 +1,192 @@
+"""ctypes binding of libace_eval.so and the torch-side plumbing (device buffers, streams).
+
+`PlanEvaluator` owns one ace_handle_t (tables resident on the device).  It never computes a
+score itself: if the HIP library is missing or no GPU is present it raises.
+"""
+import ctypes
+import os
+from typing import Optional, Sequence, Tuple
+
+import numpy as np
+
+from .plan import PlanBatch, validate_batch
+from .tables import MAX_STAGES, STAGE_REC, AceTablesStruct, CompiledTables
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libace_eval.so")
+_lib = None
+
+EXPORTS = ["ace_abi_version", "ace_strerror", "ace_last_hip_error", "ace_create", "ace_destroy",
+           "ace_score_batch", "ace_topk_workspace_bytes", "ace_topk", "ace_time_score_kernel"]
+
+
+class AceBatchStruct(ctypes.Structure):
+    _fields_ = [("d_codes", ctypes.c_void_p), ("d_hdr", ctypes.c_void_p), ("n_plans", ctypes.c_size_t)]
+
+
+class AceError(RuntimeError):
+    pass
+
+
+def load_library():
+    """dlopen the in-tree HIP library; no fallback of any kind."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        raise AceError(f"{_LIB_PATH} is missing: build it with `python -m superscaler_amd.build` "
+                       "(there is no CPU fallback for plan scoring)")
+    lib = ctypes.CDLL(_LIB_PATH)
+    lib.ace_abi_version.restype = ctypes.c_int
+    lib.ace_strerror.restype = ctypes.c_char_p
+    lib.ace_strerror.argtypes = [ctypes.c_int]
+    lib.ace_last_hip_error.restype = ctypes.c_char_p
+    lib.ace_create.restype = ctypes.c_int
+    lib.ace_create.argtypes = [ctypes.POINTER(AceTablesStruct), ctypes.POINTER(ctypes.c_void_p)]
+    lib.ace_destroy.restype = None
+    lib.ace_destroy.argtypes = [ctypes.c_void_p]
+    lib.ace_score_batch.restype = ctypes.c_int
+    lib.ace_score_batch.argtypes = [ctypes.c_void_p, ctypes.POINTER(AceBatchStruct), ctypes.c_double, ctypes.c_int,
+                                    ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                    ctypes.c_void_p, ctypes.c_void_p]
+    lib.ace_topk_workspace_bytes.restype = ctypes.c_size_t
+    lib.ace_topk_workspace_bytes.argtypes = [ctypes.c_size_t, ctypes.c_int]
+    lib.ace_topk.restype = ctypes.c_int
+    lib.ace_topk.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int,
+                             ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+                             ctypes.c_void_p]
+    lib.ace_time_score_kernel.restype = ctypes.c_int
+    lib.ace_time_score_kernel.argtypes = [ctypes.c_void_p, ctypes.POINTER(AceBatchStruct), ctypes.c_double,
+                                          ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                          ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(ctypes.c_double)]
+    if lib.ace_abi_version() != 1:
+        raise AceError("libace_eval.so has a different ABI version")
+    _lib = lib
+    return lib
+
+
+def _check(lib, rc, what):
+    if rc != 0:
+        msg = lib.ace_strerror(rc).decode()
+        hip = lib.ace_last_hip_error().decode()
+        raise AceError(f"{what}: {msg}" + (f" ({hip})" if hip and rc == -3 else ""))
+
+
+class DeviceBatch:
+    """A PlanBatch resident in HBM in the layout the kernel streams."""
+
+    def __init__(self, batch: PlanBatch, device="cuda:0"):
+        import torch
+        self.n_plans = batch.n_plans
+        self.num_ops = batch.num_ops
+        P, N = batch.codes.shape
+        G = (N + 15) // 16
+        codes = torch.from_numpy(np.ascontiguousarray(batch.codes)).to(device)
+        if G * 16 != N:
+            codes = torch.nn.functional.pad(codes, (0, G * 16 - N))
+        # [P, G, 16] -> [G, P, 16]: plan-minor, sixteen ops per 16-byte word
+        self.codes = codes.view(P, G, 16).permute(1, 0, 2).contiguous()
+        self.hdr = torch.from_numpy(np.ascontiguousarray(batch.hdr).view(np.int32)).to(device)
+        self.struct = AceBatchStruct(self.codes.data_ptr(), self.hdr.data_ptr(), P)
+
+    @property
+    def bytes_moved_per_plan(self):
+        return self.codes.shape[0] * 16 + 16
+
+
+class PlanEvaluator:
+    def __init__(self, tables: CompiledTables, device="cuda:0"):
+        import torch
+        if not torch.cuda.is_available():
+            raise AceError("no GPU visible: plan scoring runs on the HIP kernels only")
+        self.lib = load_library()
+        self.tables = tables
+        self.device = torch.device(device)
+        self._torch = torch
+        with torch.cuda.device(self.device):
+            ts = tables.as_struct()
+            h = ctypes.c_void_p()
+            _check(self.lib, self.lib.ace_create(ctypes.byref(ts), ctypes.byref(h)), "ace_create")
+        self.handle = h
+        self._topk_ws = None
+
+    def close(self):
+        if getattr(self, "handle", None):
+            self.lib.ace_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def upload(self, batch: PlanBatch, validate: bool = True) -> DeviceBatch:
+        if validate:
+            msg = validate_batch(batch, self.tables)
+            if msg:
+                raise ValueError(msg)
+        return DeviceBatch(batch, self.device)
+
+    def _stream(self):
+        return ctypes.c_void_p(self._torch.cuda.current_stream(self.device).cuda_stream)
+
+    def score(self, dbatch: DeviceBatch, memory_limit: Optional[float] = None, strict: bool = False,
+              breakdown: bool = False, out=None):
+        """Launch the scoring kernel; returns device tensors (iter_ms, peak_mb, feasible, status[, stage records])."""
+        torch = self._torch
+        P = dbatch.n_plans
+        limit = float(self.tables.settings.memory_limit if memory_limit is None else memory_limit)
+        if out is None:
+            it = torch.empty(P, dtype=torch.float64, device=self.device)
+            pk = torch.empty(P, dtype=torch.float64, device=self.device)
+            fe = torch.empty(P, dtype=torch.uint8, device=self.device)
+            st = torch.empty(P, dtype=torch.uint8, device=self.device)
+        else:
+            it, pk, fe, st = out
+        rec = torch.zeros((P, MAX_STAGES, STAGE_REC), dtype=torch.float64, device=self.device) if breakdown else None
+        with torch.cuda.device(self.device):
+            rc = self.lib.ace_score_batch(self.handle, ctypes.byref(dbatch.struct), limit, int(strict),
+                                          it.data_ptr(), pk.data_ptr(), fe.data_ptr(), st.data_ptr(),
+                                          rec.data_ptr() if breakdown else None, self._stream())
+        _check(self.lib, rc, "ace_score_batch")
+        return (it, pk, fe, st, rec) if breakdown else (it, pk, fe, st)
+
+    def topk(self, iter_ms, feasible, k: int):
+        """Device-wide top-k: (indices int64[k], times f64[k], count)."""
+        torch = self._torch
+        n = iter_ms.numel()
+        need = self.lib.ace_topk_workspace_bytes(n, k)
+        if self._topk_ws is None or self._topk_ws.numel() < need:
+            self._topk_ws = torch.empty(need, dtype=torch.uint8, device=self.device)
+        idx = torch.empty(k, dtype=torch.int64, device=self.device)
+        val = torch.empty(k, dtype=torch.float64, device=self.device)
+        cnt = torch.empty(1, dtype=torch.int32, device=self.device)
+        with torch.cuda.device(self.device):
+            rc = self.lib.ace_topk(self.handle, iter_ms.data_ptr(), feasible.data_ptr(), n, k, idx.data_ptr(),
+                                   val.data_ptr(), cnt.data_ptr(), self._topk_ws.data_ptr(), self._topk_ws.numel(),
+                                   self._stream())
+        _check(self.lib, rc, "ace_topk")
+        return idx, val, cnt
+
+    def time_score_kernel(self, dbatch: DeviceBatch, reps: int, memory_limit: Optional[float] = None) -> float:
+        """Average scoring-kernel duration in ms over `reps` back-to-back launches (hipEvents on the
+        launch stream)."""
+        torch = self._torch
+        P = dbatch.n_plans
+        limit = float(self.tables.settings.memory_limit if memory_limit is None else memory_limit)
+        it = torch.empty(P, dtype=torch.float64, device=self.device)
+        pk = torch.empty(P, dtype=torch.float64, device=self.device)
+        fe = torch.empty(P, dtype=torch.uint8, device=self.device)
+        ms = ctypes.c_double()
+        with torch.cuda.device(self.device):
+            rc = self.lib.ace_time_score_kernel(self.handle, ctypes.byref(dbatch.struct), limit, 0, it.data_ptr(),
+                                                pk.data_ptr(), fe.data_ptr(), reps, self._stream(), ctypes.byref(ms))
+        _check(self.lib, rc, "ace_time_score_kernel")
+        return ms.value
+
+    # convenience: host in, host out
+    def score_host(self, batch: PlanBatch, memory_limit=None, strict=False, breakdown=False):
+        d = self.upload(batch)
+        out = self.score(d, memory_limit, strict, breakdown)
+        self._torch.cuda.synchronize(self.device)
+        return tuple(None if t is None else t.cpu().numpy() for t in out)

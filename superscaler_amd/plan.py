@@ -1,0 +1,224 @@
+"""Plans: the reference's object form and the structure-of-arrays form the GPU scores.
+
+Object form mirrors search/aceso_utils.py:58-115 (AcesoStageInfo / AcesoConfig / get_config)
+and its JSON layout (:137-242) so the reference's search code can hand its own objects in:
+only attributes are read, any object with the same fields works.
+
+Array form (`PlanBatch`): one byte per (plan, op) --
+    bits 0-2  tp_log2 * n_algo + algo        bit 3  recompute        bit 4  first op of a stage
+plus four 32-bit words per plan --
+    [0] num_stages | micro-batch index << 8
+    [1..2] log2(stage gpus), 4 bits per stage
+    [3] in-cross-node bit per stage | out-cross-node bits << 16   (aceso_cost_model.py:572-574)
+"""
+import json
+from dataclasses import dataclass, field
+from typing import List, Optional, Sequence
+
+import numpy as np
+
+from .tables import MAX_STAGES, CompiledTables
+
+
+@dataclass
+class AcesoStageInfo:
+    index: int
+    num_stages_behind: int
+    num_gpus: int
+    ops: List[str]
+    recompute_ops: List[int]
+    tp_size: List[int]
+    dp_size: List[int]
+    algo: List[int]
+
+
+@dataclass
+class AcesoConfig:
+    global_bs: int
+    micro_bs: int
+    stages: List[AcesoStageInfo]
+    num_stages: int
+    history: str = ""
+    time_list: List[float] = field(default_factory=list)
+    memory_list: List[float] = field(default_factory=list)
+    compute_time_list: List[float] = field(default_factory=list)
+    total_gpu_time: float = 0
+    breakdown_ideal_time_per_gpu: List[float] = field(default_factory=list)
+    breakdown_eff_loss_time_per_gpu: List[float] = field(default_factory=list)
+    breakdown_recomp_time_per_gpu: List[float] = field(default_factory=list)
+    efficient_time_list: List[float] = field(default_factory=list)
+    adaptive_times: int = 0
+
+
+def get_config(num_ops_list, tp_size_list, dp_size_list, recompute_ops, aggregate_mbs, global_batch_size,
+               full_op_list, algo_list) -> AcesoConfig:
+    """Flat per-op lists + ops per stage -> AcesoConfig (aceso_utils.py:96-115): a stage's
+    device count is tp*dp of its first op."""
+    stages, start = [], 0
+    num_stages = len(num_ops_list)
+    for i, n in enumerate(num_ops_list):
+        end = start + n
+        stages.append(AcesoStageInfo(
+            index=i, num_stages_behind=num_stages - 1 - i,
+            num_gpus=tp_size_list[start] * dp_size_list[start],
+            ops=list(full_op_list[start:end]), recompute_ops=list(recompute_ops[start:end]),
+            tp_size=list(tp_size_list[start:end]), dp_size=list(dp_size_list[start:end]),
+            algo=list(algo_list[start:end])))
+        start = end
+    return AcesoConfig(global_bs=global_batch_size, micro_bs=aggregate_mbs, stages=stages, num_stages=num_stages)
+
+
+def config_from_json(path_or_dict, full_op_list) -> AcesoConfig:
+    """Plan JSON as the reference writes it (aceso_utils.py:137-211) -> AcesoConfig (:213-242)."""
+    d = path_or_dict
+    if not isinstance(d, dict):
+        with open(d) as f:
+            d = json.load(f)
+    flat = lambda ll: [x for l in ll for x in l]
+    return get_config(d["num_ops_in_each_stage"], flat(d["model_parallel_size_of_each_op"]),
+                      flat(d["data_parallel_size_of_each_op"]), flat(d["recompute_ops"]),
+                      d["micro_batch_size"], d["global_batch_size"], full_op_list, flat(d["algo_of_each_op"]))
+
+
+def cross_node_bits(stage_gpus: Sequence[int], gpus_per_node: int) -> int:
+    """in/out cross-node flags of every stage (aceso_cost_model.py:572-574)."""
+    bits, till_now = 0, 0
+    for s, g in enumerate(stage_gpus):
+        if till_now % gpus_per_node == 0 and till_now > 0:
+            bits |= 1 << s
+        till_now += g
+        if till_now % gpus_per_node == 0:
+            bits |= 1 << (16 + s)
+    return bits
+
+
+@dataclass
+class PlanBatch:
+    codes: np.ndarray        # uint8 [P, N]
+    hdr: np.ndarray          # uint32 [P, 4]
+
+    @property
+    def n_plans(self):
+        return self.codes.shape[0]
+
+    @property
+    def num_ops(self):
+        return self.codes.shape[1]
+
+    def slice(self, lo, hi):
+        return PlanBatch(self.codes[lo:hi], self.hdr[lo:hi])
+
+    @staticmethod
+    def concat(batches):
+        return PlanBatch(np.concatenate([b.codes for b in batches]), np.concatenate([b.hdr for b in batches]))
+
+    # ---- object form -> array form -----------------------------------------------------------
+    @classmethod
+    def from_configs(cls, configs: Sequence, tables: CompiledTables, single_stage_intra_node: bool = False):
+        """Encode AcesoConfig-like objects.  Raises KeyError for a micro-batch size that is not
+        profiled (as aceso_cost_model.py:22-25 does) and ValueError for plans the encoding cannot
+        hold.  `single_stage_intra_node` forces both cross-node flags off, which is what the
+        single-stage queries do (aceso_cost_model.py:494-495)."""
+        db = tables.db
+        N = tables.graph.num_ops
+        A = db.n_algo
+        mbs_index = {m: k for k, m in enumerate(db.mbs_list)}
+        tp_index = {t: k for k, t in enumerate(db.tp_list)}
+        P = len(configs)
+        codes = np.zeros((P, N), dtype=np.uint8)
+        hdr = np.zeros((P, 4), dtype=np.uint32)
+        gpn = tables.settings.num_gpus_per_node
+        for p, cfg in enumerate(configs):
+            S = cfg.num_stages
+            if S < 1 or S > MAX_STAGES:
+                raise ValueError(f"plan {p}: {S} stages (1..{MAX_STAGES} supported)")
+            bidx = mbs_index[cfg.micro_bs]
+            pos = 0
+            glogs = 0
+            gl = []
+            for s, st in enumerate(cfg.stages):
+                n = len(st.ops)
+                if n == 0:
+                    raise ValueError(f"plan {p}: stage {s} is empty")
+                g = st.tp_size[0] * st.dp_size[0]
+                if g & (g - 1) or g.bit_length() - 1 > 15:
+                    raise ValueError(f"plan {p}: stage {s} has {g} devices (power of two expected)")
+                gl.append(g)
+                glogs |= (g.bit_length() - 1) << (4 * s)
+                tp = np.asarray(st.tp_size, dtype=np.int64)
+                dp = np.asarray(st.dp_size, dtype=np.int64)
+                if np.any(tp * dp != g):
+                    raise ValueError(f"plan {p}: stage {s} mixes tp*dp products")
+                for d in set(st.dp_size):
+                    if cfg.micro_bs // d not in mbs_index:
+                        raise KeyError(cfg.micro_bs // d)
+                try:
+                    t = np.array([tp_index[x] for x in st.tp_size], dtype=np.uint8)
+                except KeyError as e:
+                    raise ValueError(f"plan {p}: tp size {e} is not in the profile database") from None
+                al = np.asarray(st.algo, dtype=np.uint8)
+                if np.any(al >= A):
+                    raise ValueError(f"plan {p}: algo index outside the profile database")
+                rc = (np.asarray(st.recompute_ops) == 1).astype(np.uint8)
+                codes[p, pos:pos + n] = (t * A + al) | (rc << 3)
+                codes[p, pos] |= 1 << 4
+                pos += n
+            if pos != N:
+                raise ValueError(f"plan {p} has {pos} ops, the op graph {N}")
+            hdr[p, 0] = S | (bidx << 8)
+            hdr[p, 1] = glogs & 0xFFFFFFFF
+            hdr[p, 2] = glogs >> 32
+            hdr[p, 3] = 0 if single_stage_intra_node else cross_node_bits(gl, gpn)
+        return cls(codes, hdr)
+
+    # ---- array form -> object form -------------------------------------------------------------
+    def to_config(self, p: int, tables: CompiledTables, cls_config=AcesoConfig, cls_stage=AcesoStageInfo):
+        db = tables.db
+        A = db.n_algo
+        row = self.codes[p]
+        S = int(self.hdr[p, 0] & 0xff)
+        micro_bs = db.mbs_list[int(self.hdr[p, 0] >> 8) & 0xff]
+        glogs = int(self.hdr[p, 1]) | (int(self.hdr[p, 2]) << 32)
+        starts = np.flatnonzero(row & 16).tolist() + [len(row)]
+        assert len(starts) - 1 == S and starts[0] == 0
+        ops = tables.graph.ops
+        stages = []
+        for s in range(S):
+            lo, hi = starts[s], starts[s + 1]
+            g = 1 << ((glogs >> (4 * s)) & 15)
+            c = row[lo:hi] & 7
+            tp = [db.tp_list[int(x) // A] for x in c]
+            stages.append(cls_stage(index=s, num_stages_behind=S - 1 - s, num_gpus=g, ops=list(ops[lo:hi]),
+                                    recompute_ops=[int(x) for x in (row[lo:hi] >> 3) & 1], tp_size=tp,
+                                    dp_size=[g // t for t in tp], algo=[int(x) % A for x in c]))
+        return cls_config(global_bs=tables.settings.global_batch_size, micro_bs=micro_bs, stages=stages, num_stages=S)
+
+    # ---- device layout -------------------------------------------------------------------------
+    def device_codes_host(self) -> np.ndarray:
+        """[ceil(N/16)][P][16] uint8, the layout ace_batch_t.d_codes expects (built on the host)."""
+        P, N = self.codes.shape
+        G = (N + 15) // 16
+        padded = np.zeros((P, G * 16), dtype=np.uint8)
+        padded[:, :N] = self.codes
+        return np.ascontiguousarray(padded.reshape(P, G, 16).transpose(1, 0, 2))
+
+
+def validate_batch(batch: PlanBatch, tables: CompiledTables) -> Optional[str]:
+    """Cheap structural check of an array-form batch; returns a message or None."""
+    P, N = batch.codes.shape
+    if N != tables.graph.num_ops:
+        return f"batch has {N} ops per plan, op graph {tables.graph.num_ops}"
+    if P == 0:
+        return "empty batch"
+    S = batch.hdr[:, 0] & 0xff
+    if np.any(S < 1) or np.any(S > MAX_STAGES):
+        return "num_stages outside 1..16"
+    if np.any(((batch.codes >> 4) & 1).sum(axis=1) != S):
+        return "stage-start bits disagree with num_stages"
+    if np.any((batch.codes[:, 0] & 16) == 0):
+        return "op 0 must start a stage"
+    if np.any((batch.hdr[:, 0] >> 8) & 0xff >= len(tables.db.mbs_list)):
+        return "micro-batch index outside the profile database"
+    if np.any((batch.codes & 7) >= tables.C):
+        return "tp/algo code outside the profile database"
+    return None

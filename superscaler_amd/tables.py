@@ -1,0 +1,365 @@
+"""Table compiler: profile database + op graph + settings -> the dense tables the HIP kernel
+gathers from.
+
+Everything in search/aceso_cost_model.py that involves a string, a dict probe, a logarithm or
+an op name is evaluated here, once, on the host, with the reference's own arithmetic
+(Python floats, math.log), so the device only ever adds, multiplies, divides and takes
+maxima of table entries:
+
+  row[type]  per op type, contiguous (staged in LDS as a unit):
+     hot   [diag][code][6]   fwd us, bwd us, weights MB, activations MB (x1.5 / 0 rule of
+                             :386-391 applied), fwd_reserved MB, bwd_reserved MB
+     start [diag][code][4]   input MB, input/intra-node-bandwidth, input/inter-node-bandwidth, 0
+                             (:319-336 for the stage's first op, with the index quirks of :275-299)
+     out   [mbs][tp][algo][2] output/intra-bandwidth, output/inter-bandwidth (indexed the way
+                             :321-326 mixes the first op's tp with the last op's mbs and algo)
+     z     [k][diag][code]   ms of collective k (one per (primitive, group size) in use) on this
+                             op's input (:247-260, string keys resolved here)
+  code = tp_log2 * n_algo + algo.  A "diag" is one way of turning an op's tp into its micro-batch
+  index: micro_bs // dp with dp = stage_gpus / tp (:496) depends only on (micro_bs, stage_gpus,
+  tp), so each (micro_bs, stage_gpus) pair maps to a tuple (mbs index for tp=1,2,4,8); equal
+  tuples share a diag.  Entries whose micro-batch is not profiled are NaN (the reference
+  raises KeyError there).
+  pair_kinds[kind][glog][code_prev][code_cur]  byte: forward | backward << 4 collective table
+     ids (1-based, 0 = nothing to do, 15 = the reference would raise) for an adjacent op
+     pair, from get_op_spec / get_reshard_primitives (model_ops_info.py:92-150, cost_model:185-245)
+  stage_lut[mbs index][glog]  diag | per-tp mbs-index nibbles << 8 (0xF = not profiled)
+  pos_info[i]  LDS byte offset of op i's row, of op i-1's row, pair kind | flags << 8
+"""
+import ctypes
+import math
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Tuple
+
+import numpy as np
+
+from . import opgraph as og
+from .profile_db import CostModelSettings, ProfileDB
+
+ABI_VERSION = 1
+MAX_STAGES = 16
+STAGE_REC = 18
+LDS_BYTES = 160 * 1024
+F_RESHARDING, F_RESERVED_MIN, F_NO_RESERVED = 1, 2, 4
+
+(R_FWD, R_BWD, R_IN_COMM, R_OUT_COMM, R_RECOMP, R_WEIGHTS, R_INPUTS, R_ACT, R_SAVED, R_PEAK,
+ R_RESERVED, R_IDEAL_FWD, R_IDEAL_BWD, R_IDEAL_IN, R_IDEAL_OUT, R_STAGE_MS, R_STAGE_MB, R_SPARE) = range(18)
+
+
+class AceTablesStruct(ctypes.Structure):
+    """ace_tables_t of include/ace_eval.h."""
+    _fields_ = [
+        ("abi_version", ctypes.c_int32), ("num_ops", ctypes.c_int32), ("num_types", ctypes.c_int32),
+        ("n_mbs", ctypes.c_int32), ("n_tp", ctypes.c_int32), ("n_algo", ctypes.c_int32),
+        ("n_diag", ctypes.c_int32), ("n_glog", ctypes.c_int32), ("n_z", ctypes.c_int32),
+        ("n_pair_kinds", ctypes.c_int32), ("row_doubles", ctypes.c_int32),
+        ("hot_off", ctypes.c_int32), ("start_off", ctypes.c_int32), ("out_off", ctypes.c_int32),
+        ("z_off", ctypes.c_int32), ("n_windows", ctypes.c_int32), ("lds_row_bytes", ctypes.c_int32),
+        ("flags", ctypes.c_int32), ("main_params", ctypes.c_double), ("optimizer", ctypes.c_double),
+        ("rows", ctypes.c_void_p), ("pos_info", ctypes.c_void_p), ("pair_kinds", ctypes.c_void_p),
+        ("stage_lut", ctypes.c_void_p), ("nb_minus_1", ctypes.c_void_p), ("win_pos", ctypes.c_void_p),
+        ("win_row_begin", ctypes.c_void_p), ("win_rows", ctypes.c_void_p),
+    ]
+
+
+@dataclass
+class CompiledTables:
+    graph: og.OpGraph
+    db: ProfileDB
+    settings: CostModelSettings
+    n_diag: int
+    n_glog: int
+    n_z: int
+    n_pair_kinds: int
+    row_doubles: int
+    hot_off: int
+    start_off: int
+    out_off: int
+    z_off: int
+    lds_row_bytes: int
+    flags: int
+    rows: np.ndarray            # float64 [n_types, row_doubles]
+    pos_info: np.ndarray        # uint32 [N + 1, 4]
+    pair_kinds: np.ndarray      # uint8 [n_pk, n_glog, C, C]
+    stage_lut: np.ndarray       # uint32 [n_mbs, 16]
+    nb_minus_1: np.ndarray      # float64 [n_mbs]
+    win_pos: np.ndarray         # int32 [n_win + 1]
+    win_row_begin: np.ndarray   # int32 [n_win + 1]
+    win_rows: np.ndarray        # uint32 [n_rows_total, 2]
+    diag_tuples: List[Tuple[int, ...]]
+    z_keys: List[Tuple[int, int]]   # (prim id, group size) per collective table
+
+    @property
+    def n_windows(self):
+        return len(self.win_pos) - 1
+
+    @property
+    def C(self):
+        return len(self.db.tp_list) * self.db.n_algo
+
+    def as_struct(self) -> AceTablesStruct:
+        db = self.db
+        s = AceTablesStruct()
+        s.abi_version = ABI_VERSION
+        s.num_ops = self.graph.num_ops
+        s.num_types = len(db.op_names)
+        s.n_mbs, s.n_tp, s.n_algo = len(db.mbs_list), len(db.tp_list), db.n_algo
+        s.n_diag, s.n_glog, s.n_z, s.n_pair_kinds = self.n_diag, self.n_glog, self.n_z, self.n_pair_kinds
+        s.row_doubles = self.row_doubles
+        s.hot_off, s.start_off, s.out_off, s.z_off = self.hot_off, self.start_off, self.out_off, self.z_off
+        s.n_windows = self.n_windows
+        s.lds_row_bytes = self.lds_row_bytes
+        s.flags = self.flags
+        s.main_params = float(self.settings.memory_main_params)
+        s.optimizer = float(self.settings.memory_optimizer)
+        for name in ("rows", "pos_info", "pair_kinds", "stage_lut", "nb_minus_1", "win_pos",
+                     "win_row_begin", "win_rows"):
+            arr = getattr(self, name)
+            assert arr.flags["C_CONTIGUOUS"]
+            setattr(s, name, arr.ctypes.data)
+        return s
+
+    # what a (micro_bs index, log2 stage gpus) pair allows
+    def allowed_tp_logs(self, bidx: int, glog: int) -> List[int]:
+        w = int(self.stage_lut[bidx, glog])
+        if (w & 0xff) == 0xff:
+            return []
+        return [t for t in range(len(self.db.tp_list)) if ((w >> (8 + 4 * t)) & 15) != 15]
+
+
+def _mbs_tuple(db: ProfileDB, micro_bs: int, gpus: int) -> Tuple[Optional[int], ...]:
+    """mbs index per tp for a stage of `gpus` devices: 15 = micro_bs // dp is not a profiled size
+    (the reference raises KeyError), None = tp does not divide into the stage (never encoded)."""
+    idx = {m: k for k, m in enumerate(db.mbs_list)}
+    out = []
+    for tp in db.tp_list:
+        if tp > gpus or gpus % tp:
+            out.append(None)
+            continue
+        dp = gpus // tp
+        out.append(idx.get(micro_bs // dp, 15))   # aceso_cost_model.py:496, :22-25
+    return tuple(out)
+
+
+def _merge_diag(diags: List[List[Optional[int]]], tup) -> int:
+    """Index of a diag compatible with `tup` (equal wherever both are defined), extended by
+    tup's entries; a new diag if there is none."""
+    for d, cur in enumerate(diags):
+        if all(a is None or b is None or a == b for a, b in zip(cur, tup)):
+            diags[d] = [b if a is None else a for a, b in zip(cur, tup)]
+            return d
+    diags.append(list(tup))
+    return len(diags) - 1
+
+
+def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings,
+                   lds_budget: int = LDS_BYTES, max_glog: int = 16) -> CompiledTables:
+    if list(db.op_names) != list(graph.type_names):
+        raise ValueError("op graph and profile database list different op types")
+    n_types, M, T, A = len(db.op_names), len(db.mbs_list), len(db.tp_list), db.n_algo
+    if M > 15 or T > 4 or A not in (1, 2):
+        raise ValueError("table geometry outside what the evaluator encodes (<=15 mbs, <=4 tp, 1-2 algos)")
+    C = T * A
+    tb = db.tables
+    shared = settings.consider_shared_space
+
+    # ---- diags and the stage LUT -----------------------------------------------------------
+    diags: List[List[Optional[int]]] = []
+    stage_lut = np.full((M, 16), 0xFF, dtype=np.uint32)
+    n_glog = 1
+    for bi, mb in enumerate(db.mbs_list):
+        for glog in range(min(16, max_glog)):
+            tup = _mbs_tuple(db, mb, 1 << glog)
+            if all(x is None or x == 15 for x in tup):
+                continue
+            d = _merge_diag(diags, tup)
+            word = d
+            for t in range(4):
+                x = tup[t] if t < T else None
+                word |= (15 if x is None else x) << (8 + 4 * t)
+            stage_lut[bi, glog] = word
+            n_glog = max(n_glog, glog + 1)
+    diag_tuples = [tuple(15 if x is None else x for x in d) for d in diags]
+    ND = len(diag_tuples)
+    if ND == 0 or ND > 254:
+        raise ValueError("no scorable (micro-batch, stage size) combination")
+
+    # ---- adjacent-pair kinds and the collectives in use ----------------------------------------
+    z_keys: List[Tuple[int, int]] = []
+
+    def z_id(prim, n):
+        if prim in (og.P_NONE, og.P_SPLIT):
+            return 0          # nothing to pay: split is free (aceso_cost_model.py:257-258)
+        name = og.PRIM_NAMES[prim]
+        if name not in db.collectives or n not in db.collectives[name]:
+            return 15         # KeyError in the reference (:251)
+        if (prim, n) not in z_keys:
+            if len(z_keys) >= 14:
+                raise ValueError("more than 14 distinct (collective, group size) pairs")
+            z_keys.append((prim, n))
+        return z_keys.index((prim, n)) + 1
+
+    pk_blocks: List[bytes] = []
+    pk_arrays: List[np.ndarray] = []
+    pk_of_pos = np.zeros(graph.num_ops + 1, dtype=np.int64)
+    kinds = [og.spec_kinds(n) for n in db.op_names]
+    pair_cache: Dict[Tuple[int, int], int] = {}
+    zero_block = np.zeros((n_glog, C, C), dtype=np.uint8)
+
+    def pair_block(tprev: int, tcur: int) -> np.ndarray:
+        blk = np.zeros((n_glog, C, C), dtype=np.uint8)
+        if not settings.resharding:
+            return blk
+        for glog in range(n_glog):
+            g = 1 << glog
+            for cp in range(C):
+                tp0, a0 = db.tp_list[cp // A], cp % A
+                if tp0 > g:
+                    continue
+                for cc in range(C):
+                    tp1, a1 = db.tp_list[cc // A], cc % A
+                    if tp1 > g:
+                        continue
+                    src = og.kind_layout(kinds[tprev][a0][1], tp0, g // tp0)
+                    dst = og.kind_layout(kinds[tcur][a1][0], tp1, g // tp1)
+                    try:
+                        pf, pb, n = og.reshard_prims(src, dst)
+                        blk[glog, cp, cc] = z_id(pf, n) | (z_id(pb, n) << 4)
+                    except og.InconsistentSpecs:
+                        blk[glog, cp, cc] = 0xFF
+        return blk
+
+    def intern(blk: np.ndarray) -> int:
+        key = blk.tobytes()
+        if key in pk_blocks:
+            return pk_blocks.index(key)
+        pk_blocks.append(key)
+        pk_arrays.append(blk)
+        return len(pk_blocks) - 1
+
+    intern(zero_block)     # kind 0: no resharding (also used for position 0)
+    for i in range(1, graph.num_ops):
+        key = (int(graph.type_of_pos[i - 1]), int(graph.type_of_pos[i]))
+        if key not in pair_cache:
+            pair_cache[key] = intern(pair_block(*key))
+        pk_of_pos[i] = pair_cache[key]
+    if len(pk_arrays) > 255:
+        raise ValueError("more than 255 distinct adjacent-op spec pairings")
+    pair_kinds = np.ascontiguousarray(np.stack(pk_arrays))
+    NZ = len(z_keys)
+
+    # ---- rows ------------------------------------------------------------------------------
+    hot_off = 0
+    start_off = hot_off + ND * C * 6
+    out_off = start_off + ND * C * 4
+    z_off = out_off + M * T * A * 2
+    row_doubles = z_off + NZ * ND * C
+    row_doubles += row_doubles & 1
+    rows = np.zeros((n_types, row_doubles), dtype=np.float64)
+    nan = math.nan
+    reserved_on = settings.consider_reserved_space
+    for ty, name in enumerate(db.op_names):
+        fl = int(graph.flags[ty])
+        hot = np.full((ND, C, 6), nan)
+        start = np.full((ND, C, 4), nan)
+        z = np.full((max(NZ, 1), ND, C), nan)
+        for d, tup in enumerate(diag_tuples):
+            for t in range(T):
+                m = tup[t]
+                if m == 15:
+                    continue
+                for a in range(A):
+                    c = t * A + a
+                    act = float(tb["activations"][ty, m, t, a])
+                    if shared and (fl & og.F_ACT_X1_5):
+                        act = act * 1.5
+                    elif shared and (fl & og.F_ACT_ZERO):
+                        act = 0.0
+                    rf = float(tb["reserved_fwd"][ty, m, t, a]) if reserved_on else 0.0
+                    rb = float(tb["reserved_bwd"][ty, m, t, a]) if reserved_on else 0.0
+                    hot[d, c] = (float(tb["fwd"][ty, m, t, a]), float(tb["bwd"][ty, m, t, a]),
+                                 float(tb["weights"][ty, m, t, a]), act, rf, rb)
+                    insz = float(tb["input_size"][ty, m, t, a])
+                    start[d, c] = (insz, db.p2p_time(insz, db.intra_band), db.p2p_time(insz, db.inter_band), 0.0)
+                    for k, (prim, n) in enumerate(z_keys):
+                        z[k, d, c] = db.reshard_time(og.PRIM_NAMES[prim], n, insz)
+        out = np.zeros((M, T, A, 2))
+        for m in range(M):
+            for t in range(T):
+                for a in range(A):
+                    osz = float(tb["output_size"][ty, m, t, a])
+                    out[m, t, a] = (db.p2p_time(osz, db.intra_band), db.p2p_time(osz, db.inter_band))
+        rows[ty, hot_off:hot_off + hot.size] = hot.ravel()
+        rows[ty, start_off:start_off + start.size] = start.ravel()
+        rows[ty, out_off:out_off + out.size] = out.ravel()
+        if NZ:
+            rows[ty, z_off:z_off + NZ * ND * C] = z[:NZ].ravel()
+
+    # ---- LDS residency: one window if every row fits, else windows over op positions ----------
+    row_bytes = row_doubles * 8
+    rk_bytes = pair_kinds.size
+    small = ((rk_bytes + 15) & ~15) + M * 16 * 4
+    avail = (lds_budget - small) & ~15
+    if avail < 2 * row_bytes:
+        raise ValueError(f"one op type's row ({row_bytes} B) does not fit LDS twice ({avail} B available)")
+    slots = avail // row_bytes
+    pos_info = np.zeros((graph.num_ops + 1, 4), dtype=np.uint32)
+    win_pos, win_row_begin, win_rows = [0], [0], []
+    tp = graph.type_of_pos
+    i = 0
+    N = graph.num_ops
+    while i < N:
+        # a window holds the row of the op just before it (stage tails look back one op)
+        slot_of: Dict[int, int] = {}
+        if i > 0:
+            slot_of[int(tp[i - 1])] = 0
+        j = i
+        while j < N:
+            ty = int(tp[j])
+            if ty not in slot_of:
+                if len(slot_of) >= slots:
+                    break
+                slot_of[ty] = len(slot_of)
+            j += 1
+        for k in range(i, j):
+            pos_info[k, 0] = slot_of[int(tp[k])] * row_bytes
+            pos_info[k, 1] = slot_of[int(tp[k - 1])] * row_bytes if k > 0 else 0
+        if j == N:
+            pos_info[N, 0] = 0
+            pos_info[N, 1] = slot_of[int(tp[N - 1])] * row_bytes
+        for ty, sl in slot_of.items():
+            win_rows.append((ty, sl * row_bytes))
+        win_row_begin.append(len(win_rows))
+        win_pos.append(j)
+        i = j
+    win_pos[-1] = max(win_pos[-1], N + 1)      # never reached: no restaging after the last window
+    lds_row_bytes = max(off for _, off in win_rows) + row_bytes
+
+    # flags about the previous op, seen from position i
+    normal = [not (shared and (int(graph.flags[t]) & (og.F_ACT_X1_5 | og.F_ACT_ZERO))) for t in range(n_types)]
+    for k in range(1, N):
+        prev_t, cur_t = int(tp[k - 1]), int(tp[k])
+        fl = 0
+        if normal[prev_t] and (int(graph.flags[cur_t]) & og.F_LAYER_START):
+            fl |= 1      # ordinary op right before a layer start: saved += 0, peak segment closes
+        if normal[prev_t]:
+            fl |= 2      # ordinary op: closes the last segment when the pair ends the stage
+        pos_info[k, 2] = int(pk_of_pos[k]) | (fl << 8)
+
+    flags = 0
+    if settings.resharding and (pair_kinds != 0).any():
+        flags |= F_RESHARDING
+    if not settings.consider_reserved_space:
+        flags |= F_NO_RESERVED
+    elif settings.memory_pred_type == "MIN":
+        flags |= F_RESERVED_MIN
+    nbm1 = np.array([float(settings.global_batch_size // mb - 1) for mb in db.mbs_list], dtype=np.float64)
+    return CompiledTables(
+        graph=graph, db=db, settings=settings, n_diag=ND, n_glog=n_glog, n_z=NZ,
+        n_pair_kinds=len(pk_arrays), row_doubles=row_doubles, hot_off=hot_off, start_off=start_off,
+        out_off=out_off, z_off=z_off, lds_row_bytes=int(lds_row_bytes), flags=flags,
+        rows=np.ascontiguousarray(rows), pos_info=np.ascontiguousarray(pos_info),
+        pair_kinds=pair_kinds, stage_lut=np.ascontiguousarray(stage_lut), nb_minus_1=nbm1,
+        win_pos=np.array(win_pos, dtype=np.int32), win_row_begin=np.array(win_row_begin, dtype=np.int32),
+        win_rows=np.ascontiguousarray(np.array(win_rows, dtype=np.uint32).reshape(-1, 2)),
+        diag_tuples=diag_tuples, z_keys=z_keys)

@@ -1,0 +1,67 @@
+"""The kernel's per-plan state machine (compiled for the CPU with bounds checks) and the table
+compiler, against the oracle: every value bit-identical."""
+import numpy as np
+import pytest
+
+from superscaler_amd import synth
+from superscaler_amd.tables import (R_ACT, R_BWD, R_FWD, R_IDEAL_BWD, R_IDEAL_FWD, R_IDEAL_IN, R_IDEAL_OUT,
+                                    R_IN_COMM, R_INPUTS, R_OUT_COMM, R_PEAK, R_RECOMP, R_RESERVED, R_SAVED,
+                                    R_STAGE_MB, R_STAGE_MS, R_WEIGHTS)
+from tests.helpers import emu_score, oracle_for, oracle_scores
+
+CASES = [("gpt3_1_3b", 96), ("t5_770m", 48), ("wresnet_1b", 128), ("gpt3_13b", 96), ("gpt3_175b", 16)]
+
+
+@pytest.fixture(scope="module", params=CASES, ids=[c[0] for c in CASES])
+def case(request):
+    name, n = request.param
+    w = synth.WORKLOADS[name]
+    tables = synth.make_tables(w)
+    batch = synth.make_plans(w, tables, n_plans=n)
+    return w, tables, batch, oracle_for(tables)
+
+
+def test_scores_bit_exact(case):
+    w, tables, batch, orc = case
+    it, pk, fe, st, _ = emu_score(tables, batch)
+    oit, opk, ofe, _ = oracle_scores(orc, batch, tables)
+    assert (st == 0).all()
+    assert np.array_equal(it, oit)
+    assert np.array_equal(pk, opk)
+    assert np.array_equal(fe, ofe)
+    # strict comparison flips only plans that sit exactly on the limit
+    it2, pk2, fe2, _, _ = emu_score(tables, batch, memory_limit=float(np.median(opk)), strict=True)
+    assert np.array_equal(fe2, (opk < float(np.median(opk))).astype(np.uint8))
+
+
+def test_stage_records_bit_exact(case):
+    w, tables, batch, orc = case
+    it, pk, fe, st, rec = emu_score(tables, batch, breakdown=True)
+    it0, pk0, _, _, _ = emu_score(tables, batch)
+    assert np.array_equal(it, it0) and np.array_equal(pk, pk0)
+    for p in range(min(batch.n_plans, 24)):
+        cfg = batch.to_config(p, tables)
+        from tests.helpers import oracle_config
+        oc = oracle_config(batch, p, tables)
+        gpn = tables.settings.num_gpus_per_node
+        till = 0
+        for s, stg in enumerate(oc.stages):
+            mbs = [oc.micro_bs // d for d in stg.dp_size]
+            in_cross = (till % gpn == 0) and till > 0
+            till += stg.num_gpus
+            out_cross = till % gpn == 0
+            f, b, ic, ocm, _ = orc.get_time_v3(stg.ops, mbs, stg.tp_size, stg.algo, stg.dp_size, in_cross, out_cross)
+            r = rec[p, s]
+            assert (r[R_FWD], r[R_BWD], r[R_IN_COMM], r[R_OUT_COMM]) == (f, b, ic, ocm)
+            assert r[R_RECOMP] == orc.get_recompute_time_v3(stg.ops, stg.recompute_ops, mbs, stg.tp_size, stg.algo)
+            wts, inputs, acts = orc.get_memory_v3(stg.ops, mbs, stg.tp_size, stg.algo)
+            assert (r[R_WEIGHTS], r[R_INPUTS], r[R_ACT]) == (wts, inputs, acts)
+            assert r[R_SAVED] == orc.get_activations_v3(stg.ops, stg.recompute_ops, mbs, stg.tp_size, stg.algo)
+            assert r[R_PEAK] == orc.get_peak_activations(stg.ops, stg.recompute_ops, mbs, stg.tp_size, stg.algo)
+            assert r[R_RESERVED] == orc.get_reserved_memory(stg.ops, mbs, stg.tp_size, stg.dp_size, stg.algo, wts)
+            n = len(stg.ops)
+            f1, b1, i1, o1, _ = orc.get_time_v3(stg.ops, [oc.micro_bs] * n, [1] * n, stg.algo, [1] * n, in_cross, out_cross)
+            assert (r[R_IDEAL_FWD], r[R_IDEAL_BWD], r[R_IDEAL_IN], r[R_IDEAL_OUT]) == (f1, b1, i1, o1)
+            assert r[R_STAGE_MB] == orc.predict_stage_memory(stg.ops, stg.recompute_ops, stg.tp_size, stg.dp_size,
+                                                             oc.micro_bs, stg.num_stages_behind, stg.algo)
+            assert r[R_STAGE_MS] == (f + b + ic + ocm + r[R_RECOMP]) / 1000

@@ -183,29 +183,51 @@ __global__ __launch_bounds__(kTopBlock) void topk_hist(const double *t, const ui
         if (lh[j]) atomicAdd(&hist[j], lh[j]);
 }
 
-__global__ void topk_pick(TopkState *st, unsigned int *hist, int pass) {
-    // single workgroup: find the bucket holding the k_rem-th entry, descend into it
-    __shared__ unsigned int sh[kRadix];
-    for (int j = threadIdx.x; j < kRadix; j += blockDim.x) sh[j] = hist[j];
+__global__ __launch_bounds__(kTopBlock) void topk_pick(TopkState *st, unsigned int *hist, int pass) {
+    // single workgroup: find the bucket holding the k_rem-th entry of the current prefix, descend into it
+    constexpr int kPer = kRadix / kTopBlock;          // buckets per lane
+    __shared__ unsigned int part[kTopBlock];
+    const int tid = threadIdx.x;
+    unsigned int loc[kPer];
+    unsigned int sum = 0;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) { loc[j] = hist[tid * kPer + j]; sum += loc[j]; }
+    part[tid] = sum;
     __syncthreads();
-    if (threadIdx.x == 0) {
-        const int bits = pass_bits(pass);
-        const int shift = pass_shift(pass);
-        unsigned int rem = st->k_rem, acc = 0;
-        int b = 0;
-        const int nb = 1 << bits;
-        for (; b < nb; ++b) {
-            if (acc + sh[b] >= rem) break;
-            acc += sh[b];
+    for (int off = 1; off < kTopBlock; off <<= 1) {   // inclusive scan of the per-lane sums
+        unsigned int v = tid >= off ? part[tid - off] : 0u;
+        __syncthreads();
+        part[tid] += v;
+        __syncthreads();
+    }
+    const unsigned int rem = st->k_rem;
+    const unsigned int incl = part[tid], excl = incl - sum;
+    const unsigned int total = part[kTopBlock - 1];
+    const int shift = pass_shift(pass);
+    __syncthreads();
+    bool mine = excl < rem && rem <= incl;            // exactly one lane when total >= rem
+    if (total < rem) mine = (tid == kTopBlock - 1);   // fewer entries than asked for: take the last bucket
+    if (mine) {
+        unsigned int acc = excl;
+        int b = tid * kPer;
+        if (total >= rem) {
+            for (int j = 0; j < kPer; ++j) {
+                if (acc + loc[j] >= rem) { b = tid * kPer + j; break; }
+                acc += loc[j];
+            }
+        } else {
+            const int nb = 1 << pass_bits(pass);
+            b = nb - 1;
+            acc = total - hist[b];
         }
-        if (b >= nb) b = nb - 1;         // fewer than k entries overall: everything qualifies
         st->prefix |= ((unsigned long long)b) << shift;
         st->k_rem = rem - acc;
         st->n_less += acc;
         if (pass == kPasses - 1) st->thr = st->prefix;
     }
     __syncthreads();
-    for (int j = threadIdx.x; j < kRadix; j += blockDim.x) hist[j] = 0;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) hist[tid * kPer + j] = 0;
 }
 
 struct Cand { unsigned long long key; long long idx; };
@@ -235,6 +257,9 @@ __global__ __launch_bounds__(kTopBlock) void topk_ties_exact(const double *t, co
     __shared__ unsigned int cnt[kTopBlock];
     __shared__ unsigned int base;
     const unsigned long long thr = st->thr;
+    // nothing to redo unless the gather overflowed its tie buffer (every lane reads the same value;
+    // it is only rewritten after the last barrier below)
+    if (st->n_ties <= want || thr == kInfKey) return;
     if (threadIdx.x == 0) base = 0;
     __syncthreads();
     for (size_t start = 0; start < n; start += kTopBlock) {
@@ -541,7 +566,7 @@ int ace_topk(ace_handle_t *h, const double *d_iter_ms, const uint8_t *d_feasible
     hipLaunchKernelGGL(topk_init, dim3(1), dim3(256), 0, s, st, hist, k);
     for (int pass = 0; pass < kPasses; ++pass) {
         hipLaunchKernelGGL(topk_hist, dim3(blocks), dim3(kTopBlock), 0, s, d_iter_ms, d_feasible, n, pass, st, hist);
-        hipLaunchKernelGGL(topk_pick, dim3(1), dim3(256), 0, s, st, hist, pass);
+        hipLaunchKernelGGL(topk_pick, dim3(1), dim3(kTopBlock), 0, s, st, hist, pass);
     }
     hipLaunchKernelGGL(topk_gather, dim3(blocks), dim3(kTopBlock), 0, s, d_iter_ms, d_feasible, n, st, less, ties, cap, cap);
     // ties: the gather keeps an arbitrary subset when more than `cap` plans share the k-th time;

@@ -151,10 +151,16 @@ def test_full_size_properties(torch_mod):
     it2, pk2, fe2, st2 = ev.score_host(PlanBatch(batch.codes[perm], batch.hdr[perm]))
     assert np.array_equal(it[perm], it2) and np.array_equal(pk[perm], pk2) and np.array_equal(fe[perm], fe2)
     assert (st == 0).all() and np.isfinite(it).all()
-    # clearing every recompute bit can only remove recompute time and raise memory
+    # clearing every recompute bit can only remove recompute time (memory may move either way:
+    # the peak segment can outweigh what recomputation saves)
     nb = PlanBatch(batch.codes & np.uint8(0xF7), batch.hdr)
     it3, pk3, fe3, _ = ev.score_host(nb)
-    assert (it3 <= it).all() and (pk3 >= pk).all()
+    assert (it3 <= it).all() and (it3 < it).any()
+    # a single-stage plan's iteration time is (number of micro-batches) x (stage time)
+    one = np.flatnonzero((batch.hdr[:, 0] & 0xff) == 1)[:2048]
+    _, _, _, _, rec = ev.score_host(PlanBatch(batch.codes[one], batch.hdr[one]), breakdown=True)
+    nbm1 = tables.nb_minus_1[(batch.hdr[one, 0] >> 8) & 0xff]
+    assert np.array_equal(it[one], rec[:, 0, 15] * nbm1 + rec[:, 0, 15])
     # feasibility is monotone in the limit
     _, _, fe_lo, _ = ev.score_host(batch, memory_limit=40000.0)
     _, _, fe_hi, _ = ev.score_host(batch, memory_limit=160000.0)

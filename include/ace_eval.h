@@ -40,10 +40,11 @@ enum {
 /* per-plan status bytes written by ace_score_batch */
 enum {
     ACE_PLAN_OK = 0,
-    ACE_PLAN_BAD_MBS = 1,      /* micro_bs // dp not a profiled micro-batch size: the reference raises
-                                  KeyError (aceso_cost_model.py:22-25) */
-    ACE_PLAN_BAD_RESHARD = 2,  /* inconsistent specs inside a stage (TypeError at aceso_cost_model.py:344)
-                                  or a collective never profiled for that group size (KeyError, :251) */
+    ACE_PLAN_UNSCORABLE = 1,   /* the reference raises for this plan: micro_bs // dp is not a profiled
+                                  micro-batch size (KeyError, aceso_cost_model.py:22-25), the specs of two
+                                  adjacent ops of a stage are inconsistent (TypeError, :344) or a collective
+                                  was never profiled for the group size (KeyError, :251).  Scores are NaN. */
+    ACE_PLAN_MALFORMED = 3,    /* the encoding itself is inconsistent (stage bits vs num_stages ...) */
 };
 
 /* indices into a stage record (doubles); units as in the reference: us, MB */
@@ -69,7 +70,8 @@ typedef struct ace_tables {
     int32_t n_mbs, n_tp, n_algo;
     int32_t n_diag;         /* distinct (micro_bs, stage gpus) -> per-tp micro-batch index maps */
     int32_t n_glog;         /* stage device counts 2^0 .. 2^(n_glog-1) */
-    int32_t n_z;            /* resharding cost tables (one per (collective, group size) in use) */
+    int32_t n_z;            /* resharding cost tables: table 0 is all zeros (nothing to pay), then one per
+                               (collective, group size) in use, the last one all NaN (the reference raises) */
     int32_t n_pair_kinds;   /* distinct adjacent-op spec pairings */
     int32_t row_doubles;    /* doubles per type row (even) */
     int32_t hot_off, start_off, out_off, z_off;   /* sub-table offsets inside a row, in doubles */
@@ -78,12 +80,12 @@ typedef struct ace_tables {
     int32_t flags;          /* ACE_F_* */
     double main_params, optimizer;   /* aceso_utils.py:48-52 */
     const double *rows;            /* [num_types][row_doubles] */
-    const uint32_t *pos_info;      /* [num_ops + 1][4]: row byte offset, previous op's row byte offset,
-                                      pair kind | flags << 8, spare */
+    const uint32_t *pos_info;      /* [num_ops + 1][2]: row LDS offset / 16 | previous op's row offset / 16 << 16;
+                                      pair kind | flags << 8 */
     const uint8_t *pair_kinds;     /* [n_pair_kinds][n_glog][C][C], C = n_tp * n_algo */
     const uint32_t *stage_lut;     /* [n_mbs][16]: diag | per-tp mbs-index nibbles << 8 */
     const double *nb_minus_1;      /* [n_mbs]: global_bs // micro_bs - 1 */
-    const int32_t *win_pos;        /* [n_windows + 1] first position of each window */
+    const int32_t *win_pos;        /* [n_windows + 1] first position of each window (multiples of 16) */
     const int32_t *win_row_begin;  /* [n_windows + 1] into win_rows */
     const uint32_t *win_rows;      /* [..][2]: type id, LDS byte offset */
 } ace_tables_t;
@@ -106,6 +108,11 @@ typedef struct ace_handle ace_handle_t;
 typedef struct ace_batch {
     const uint8_t *d_codes;
     const uint32_t *d_hdr;
+    const uint32_t *d_range;   /* NULL, or uint32[n_plans][2] = (first op, one past the last op): each plan is ONE
+                                  stage over that slice of the op sequence (bit 4 set on its first op only,
+                                  num_stages field = num_stages_behind + 1).  The form of the single-stage queries
+                                  predict_stage_time / predict_stage_memory (aceso_cost_model.py:493-539);
+                                  results are read from stage record 0, so d_stage_out is required. */
     size_t n_plans;
 } ace_batch_t;
 

@@ -37,12 +37,13 @@ struct AceKernelArgs {
     AceGeom g;
     const ace_u4 *codes;        // [G][P] 16 op bytes each
     const ace_u4 *hdr;          // [P]
+    const ace_u2 *range;        // [P] (first op, one past the last op) or null
     const double *rows;         // [n_types][row_doubles]
-    const ace_u4 *pos_info;     // [N + 1]
+    const ace_u2 *pos_info;     // [N + 1], padded to a multiple of 4 entries
     const uint8_t *pair_kinds;  // -> LDS
     const uint32_t *stage_lut;  // -> LDS
     const double *nbm1;         // [n_mbs]
-    const int32_t *win_pos;     // [n_windows + 1]
+    const int32_t *win_pos;     // [n_windows + 1], multiples of 16
     const int32_t *win_row_begin;
     const uint32_t *win_rows;   // pairs (type, lds byte offset)
     int32_t n_windows, row_doubles, rk_bytes, stg_words;
@@ -51,7 +52,21 @@ struct AceKernelArgs {
     double *stage_out;
 };
 
-template <bool BD>
+// Copy the rows window `w` needs from global memory into LDS (whole workgroup).
+__device__ __forceinline__ void stage_window(const AceKernelArgs &a, unsigned char *lds_raw, int w, int tid) {
+    const int rb = a.win_row_begin[w], re = a.win_row_begin[w + 1];
+    const int n16 = a.row_doubles / 2;
+    for (int r = rb; r < re; ++r) {
+        const uint32_t type = a.win_rows[2 * r], off = a.win_rows[2 * r + 1];
+        const ace_d2 *src = reinterpret_cast<const ace_d2 *>(a.rows + (size_t)type * a.row_doubles);
+        ace_d2 *dst = reinterpret_cast<ace_d2 *>(lds_raw + off);
+        for (int j = tid; j < n16; j += kBlock) dst[j] = src[j];
+    }
+}
+
+// BD: also write per-stage records.  RANGED: each plan is one stage over an op sub-range.
+// WIN: the rows of all op types do not fit in LDS together; restage at window boundaries.
+template <bool BD, bool RANGED, bool WIN>
 __global__ __launch_bounds__(kBlock) void ace_score_kernel(const AceKernelArgs a) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
     const AceGeom &g = a.g;
@@ -60,53 +75,56 @@ __global__ __launch_bounds__(kBlock) void ace_score_kernel(const AceKernelArgs a
     const bool active = plan < g.P;
     const long long pl = active ? plan : (long long)g.P - 1;
 
-    // small tables: pair kinds and the (micro-batch, stage gpus) LUT
+    // small tables: pair kinds and the (micro-batch, stage gpus) LUT; without windows, every row
     for (int j = tid; j < a.rk_bytes; j += kBlock) lds_raw[g.rk_lds_off + j] = a.pair_kinds[j];
     for (int j = tid; j < a.stg_words; j += kBlock)
         reinterpret_cast<uint32_t *>(lds_raw + g.stg_lds_off)[j] = a.stage_lut[j];
+    if (!WIN) stage_window(a, lds_raw, 0, tid);
     __syncthreads();
 
     AceLds lds{lds_raw};
-    PlanState<BD> st;
+    PlanState<BD, RANGED> st;
     const ace_u4 h = a.hdr[pl];
-    st.init(g, lds, h);
+    ace_u2 range{0u, 0u};
+    if (RANGED) range = a.range[pl];
+    st.init(g, lds, h, range);
     const double nbm1 = a.nbm1[st.bidx];
     double *rec = (BD && a.stage_out && active) ? a.stage_out + (size_t)plan * (ACE_MAX_STAGES * ACE_STAGE_REC) : nullptr;
 
     int w = 0;
-    int next_win = a.win_pos[0];
-    ace_u4 cw = a.codes[pl];
-    for (int grp = 0; grp < g.G; ++grp) {
-        ace_u4 nxt = cw;
-        if (grp + 1 < g.G) nxt = a.codes[(size_t)(grp + 1) * g.P + pl];
-        const uint32_t words[4] = {cw.x, cw.y, cw.z, cw.w};
-#pragma unroll
-        for (int k = 0; k < 16; ++k) {
-            const int i = grp * 16 + k;
-            if (i >= g.N) break;
-            if (i == next_win) {
-                // restage the rows this window needs; every lane of the workgroup gets here together
+    int next_win = WIN ? a.win_pos[0] : 0x7fffffff;
+    ace_u4 cw = a.codes[pl];                 // sixteen op bytes; consumed one 32-bit word (4 ops) at a time
+    ace_u4 nxt = cw;
+    uint32_t pbyte = 0;                      // code byte of the previous op
+    const int quads = (g.N + 3) >> 2;
+    for (int q = 0; q < quads; ++q) {
+        const int base = q << 2;
+        if ((q & 3) == 0) {
+            if (q) cw = nxt;
+            const int grp = (q >> 2) + 1;
+            if (grp < g.G) nxt = a.codes[(size_t)grp * g.P + pl];
+            if (WIN && base == next_win) {
+                // every lane of the workgroup reaches this point together
                 __syncthreads();
-                const int rb = a.win_row_begin[w], re = a.win_row_begin[w + 1];
-                const int n16 = a.row_doubles / 2;
-                for (int r = rb; r < re; ++r) {
-                    const uint32_t type = a.win_rows[2 * r], off = a.win_rows[2 * r + 1];
-                    const ace_d2 *src = reinterpret_cast<const ace_d2 *>(a.rows + (size_t)type * a.row_doubles);
-                    ace_d2 *dst = reinterpret_cast<ace_d2 *>(lds_raw + off);
-                    for (int j = tid; j < n16; j += kBlock) dst[j] = src[j];
-                }
+                stage_window(a, lds_raw, w, tid);
                 __syncthreads();
                 ++w;
                 next_win = a.win_pos[w];
             }
-            const uint32_t byte = (words[k >> 2] >> ((k & 3) * 8)) & 0xffu;
-            const ace_u4 info = a.pos_info[i];
-            st.step(g, lds, byte, info, rec);
         }
-        cw = nxt;
+        const uint32_t word = cw.x;
+        cw.x = cw.y; cw.y = cw.z; cw.z = cw.w;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int i = base + k;
+            if (i < g.N) {
+                const uint32_t byte = (word >> (8 * k)) & 0xffu;
+                st.step(g, lds, i, byte, pbyte, a.pos_info[i], rec);
+                pbyte = byte;
+            }
+        }
     }
-    const ace_u4 last = a.pos_info[g.N];
-    st.finish(g, lds, last.y, rec);
+    if (!RANGED || !st.done) st.finish(g, lds, info_prevrow(a.pos_info[g.N]), pbyte & 7u, rec);
     double iter, peak;
     uint8_t feas, stat;
     st.result(g, nbm1, iter, peak, feas, stat);
@@ -344,7 +362,7 @@ struct ace_handle {
     uint32_t lds_bytes;
     // device copies
     double *d_rows;
-    ace_u4 *d_pos_info;
+    ace_u2 *d_pos_info;
     uint8_t *d_pair_kinds;
     uint32_t *d_stage_lut;
     double *d_nbm1;
@@ -370,13 +388,25 @@ const char *ace_strerror(int code) {
 
 const char *ace_last_hip_error(void) { return g_hip_err; }
 
-static int upload(void **dst, const void *src, size_t bytes) {
+static int upload(void **dst, const void *src, size_t bytes, size_t alloc_bytes = 0) {
     *dst = nullptr;
-    if (bytes == 0) bytes = 16;
-    ACE_HIP(hipMalloc(dst, bytes));
-    if (src) ACE_HIP(hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice));
+    if (alloc_bytes < bytes) alloc_bytes = bytes;
+    if (alloc_bytes == 0) alloc_bytes = 16;
+    ACE_HIP(hipMalloc(dst, alloc_bytes));
+    if (alloc_bytes > bytes) ACE_HIP(hipMemset(*dst, 0, alloc_bytes));
+    if (src && bytes) ACE_HIP(hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice));
     return ACE_OK;
 }
+
+}  // extern "C"
+
+template <bool BD, bool RANGED, bool WIN> static int allow_big_lds() {
+    ACE_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&ace_score_kernel<BD, RANGED, WIN>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
+    return ACE_OK;
+}
+
+extern "C" {
 
 int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     if (!t || !out) return ACE_EINVAL;
@@ -384,7 +414,7 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     if (t->abi_version != ACE_ABI_VERSION) return ACE_EVERSION;
     if (t->num_ops <= 0 || t->num_types <= 0 || t->n_mbs <= 0 || t->n_mbs > 15 || t->n_tp <= 0 || t->n_tp > 4 ||
         (t->n_algo != 1 && t->n_algo != 2) || t->n_diag <= 0 || t->n_diag > 254 || t->n_glog <= 0 || t->n_glog > 16 ||
-        t->n_z < 0 || t->n_z > 14 || t->n_pair_kinds <= 0 || t->n_pair_kinds > 255 || t->row_doubles <= 0 ||
+        t->n_z < 2 || t->n_z > 15 || t->n_pair_kinds <= 0 || t->n_pair_kinds > 255 || t->row_doubles <= 0 ||
         (t->row_doubles & 1) || t->n_windows <= 0 || t->lds_row_bytes <= 0 || (t->lds_row_bytes & 15) ||
         !t->rows || !t->pos_info || !t->pair_kinds || !t->stage_lut || !t->nb_minus_1 || !t->win_pos ||
         !t->win_row_begin || !t->win_rows)
@@ -396,22 +426,24 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     const int64_t out_end = (int64_t)t->out_off + (int64_t)t->n_mbs * t->n_tp * t->n_algo * 2;
     const int64_t z_end = (int64_t)t->z_off + (int64_t)t->n_z * t->n_diag * C;
     if ((t->hot_off & 1) || (t->start_off & 1) || (t->out_off & 1) || (t->z_off & 1) || t->hot_off < 0 ||
+        t->start_off < 0 || t->out_off < 0 || t->z_off < 0 ||
         hot_end > t->row_doubles || start_end > t->row_doubles || out_end > t->row_doubles || z_end > t->row_doubles)
         return ACE_EINVAL;
     const int64_t row_bytes = (int64_t)t->row_doubles * 8;
-    if (row_bytes > t->lds_row_bytes) return ACE_ETOOBIG;
+    if (row_bytes > t->lds_row_bytes || t->lds_row_bytes > (int32_t)kMaxLds) return ACE_ETOOBIG;
     const int32_t rk_bytes = t->n_pair_kinds * t->n_glog * C * C;
     const int32_t stg_words = t->n_mbs * 16;
     const uint32_t rk_off = (uint32_t)t->lds_row_bytes;
     const uint32_t stg_off = (rk_off + (uint32_t)rk_bytes + 15u) & ~15u;
     const uint32_t lds_bytes = stg_off + (uint32_t)stg_words * 4u;
     if (lds_bytes > kMaxLds) return ACE_ETOOBIG;
-    // window tables: every referenced row must fit the resident region; every position's row
-    // offsets must point at a row start inside it
+    // window tables: window starts are multiples of 16 ops; every referenced row must fit the
+    // resident region; every position's row offsets must point at a row start inside it
     const int32_t n_win_rows = t->win_row_begin[t->n_windows];
     if (t->win_pos[0] != 0 || t->win_row_begin[0] != 0 || n_win_rows <= 0) return ACE_EINVAL;
     for (int w = 0; w < t->n_windows; ++w) {
-        if (t->win_pos[w + 1] <= t->win_pos[w] || t->win_row_begin[w + 1] < t->win_row_begin[w]) return ACE_EINVAL;
+        if (t->win_pos[w + 1] <= t->win_pos[w] || t->win_row_begin[w + 1] < t->win_row_begin[w] || (t->win_pos[w] & 15))
+            return ACE_EINVAL;
     }
     if (t->win_pos[t->n_windows] < t->num_ops) return ACE_EINVAL;
     for (int r = 0; r < n_win_rows; ++r) {
@@ -419,9 +451,10 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
         if ((int64_t)t->win_rows[2 * r + 1] + row_bytes > t->lds_row_bytes || (t->win_rows[2 * r + 1] & 15u)) return ACE_EINVAL;
     }
     for (int i = 0; i <= t->num_ops; ++i) {
-        const uint32_t *pi = t->pos_info + 4 * (size_t)i;
-        if ((int64_t)pi[0] + row_bytes > t->lds_row_bytes || (int64_t)pi[1] + row_bytes > t->lds_row_bytes ||
-            (pi[0] & 15u) || (pi[1] & 15u) || (pi[2] & 0xffu) >= (uint32_t)t->n_pair_kinds)
+        const uint32_t *pi = t->pos_info + 2 * (size_t)i;
+        const int64_t row = (int64_t)(pi[0] & 0xffffu) * 16, prow = (int64_t)(pi[0] >> 16) * 16;
+        if (row + row_bytes > t->lds_row_bytes || prow + row_bytes > t->lds_row_bytes ||
+            (pi[1] & 0xffu) >= (uint32_t)t->n_pair_kinds)
             return ACE_EINVAL;
     }
     for (int j = 0; j < stg_words; ++j) {
@@ -429,14 +462,12 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
         if (d != 0xffu && d >= (uint32_t)t->n_diag) return ACE_EINVAL;
     }
     for (int j = 0; j < rk_bytes; ++j) {
-        const uint32_t pf = t->pair_kinds[j] & 15u, pb = t->pair_kinds[j] >> 4;
-        if ((pf != 15u && pf > (uint32_t)t->n_z) || (pb != 15u && pb > (uint32_t)t->n_z)) return ACE_EINVAL;
+        if ((t->pair_kinds[j] & 15u) >= (uint32_t)t->n_z || (uint32_t)(t->pair_kinds[j] >> 4) >= (uint32_t)t->n_z) return ACE_EINVAL;
     }
 
     ace_handle *h = new (std::nothrow) ace_handle();
     if (!h) return ACE_ENOMEM;
     memset(h, 0, sizeof(*h));
-    ACE_HIP(hipGetDevice(&h->device));
     AceGeom &g = h->geom;
     g.N = t->num_ops; g.P = 0; g.G = (t->num_ops + 15) / 16;
     g.C = C; g.A_shift = t->n_algo == 2 ? 1 : 0;
@@ -445,26 +476,28 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     g.out_off = (uint32_t)t->out_off * 8u; g.z_off = (uint32_t)t->z_off * 8u;
     g.z_stride = (uint32_t)(t->n_diag * C) * 8u;
     g.rk_lds_off = rk_off; g.stg_lds_off = stg_off;
+    g.rk_kind_stride = (uint32_t)(t->n_glog * C * C);
     g.flags = t->flags; g.main_params = t->main_params; g.optimizer = t->optimizer;
     g.mem_limit = 0.0; g.strict = 0;
     h->n_windows = t->n_windows; h->row_doubles = t->row_doubles; h->rk_bytes = rk_bytes; h->stg_words = stg_words;
     h->num_types = t->num_types; h->lds_bytes = lds_bytes;
+    const size_t pos_entries = ((size_t)t->num_ops + 1 + 3) & ~(size_t)3;
     int rc;
-    if ((rc = upload((void **)&h->d_rows, t->rows, (size_t)t->num_types * row_bytes)) ||
-        (rc = upload((void **)&h->d_pos_info, t->pos_info, (size_t)(t->num_ops + 1) * 16)) ||
+    if ((rc = hipGetDevice(&h->device) == hipSuccess ? ACE_OK : ACE_EHIP) ||
+        (rc = upload((void **)&h->d_rows, t->rows, (size_t)t->num_types * row_bytes)) ||
+        (rc = upload((void **)&h->d_pos_info, t->pos_info, (size_t)(t->num_ops + 1) * 8, pos_entries * 8)) ||
         (rc = upload((void **)&h->d_pair_kinds, t->pair_kinds, (size_t)rk_bytes)) ||
         (rc = upload((void **)&h->d_stage_lut, t->stage_lut, (size_t)stg_words * 4)) ||
         (rc = upload((void **)&h->d_nbm1, t->nb_minus_1, (size_t)t->n_mbs * 8)) ||
         (rc = upload((void **)&h->d_win_pos, t->win_pos, (size_t)(t->n_windows + 1) * 4)) ||
         (rc = upload((void **)&h->d_win_row_begin, t->win_row_begin, (size_t)(t->n_windows + 1) * 4)) ||
-        (rc = upload((void **)&h->d_win_rows, t->win_rows, (size_t)n_win_rows * 8))) {
+        (rc = upload((void **)&h->d_win_rows, t->win_rows, (size_t)n_win_rows * 8)) ||
+        (rc = allow_big_lds<false, false, false>()) || (rc = allow_big_lds<false, false, true>()) ||
+        (rc = allow_big_lds<true, false, false>()) || (rc = allow_big_lds<true, false, true>()) ||
+        (rc = allow_big_lds<true, true, false>()) || (rc = allow_big_lds<true, true, true>())) {
         ace_destroy(h);
         return rc;
     }
-    ACE_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&ace_score_kernel<false>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
-    ACE_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&ace_score_kernel<true>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
     *out = h;
     return ACE_OK;
 }
@@ -481,13 +514,15 @@ static int fill_args(ace_handle_t *h, const ace_batch_t *b, double memory_limit,
                      double *d_peak_mb, uint8_t *d_feasible, uint8_t *d_status, double *d_stage_out, AceKernelArgs *a) {
     if (!h || !b || !b->d_codes || !b->d_hdr || !d_iter_ms || !d_peak_mb || !d_feasible) return ACE_EINVAL;
     if (b->n_plans == 0 || b->n_plans > 0x7fffffffull) return ACE_EINVAL;
-    if (((uintptr_t)b->d_codes & 15u) || ((uintptr_t)b->d_hdr & 15u)) return ACE_EINVAL;
+    if (((uintptr_t)b->d_codes & 15u) || ((uintptr_t)b->d_hdr & 15u) || ((uintptr_t)b->d_range & 7u)) return ACE_EINVAL;
+    if (b->d_range && !d_stage_out) return ACE_EINVAL;   // single-stage queries are read from their stage record
     a->g = h->geom;
     a->g.P = (int32_t)b->n_plans;
     a->g.mem_limit = memory_limit;
     a->g.strict = strict ? 1 : 0;
     a->codes = reinterpret_cast<const ace_u4 *>(b->d_codes);
     a->hdr = reinterpret_cast<const ace_u4 *>(b->d_hdr);
+    a->range = reinterpret_cast<const ace_u2 *>(b->d_range);
     a->rows = h->d_rows; a->pos_info = h->d_pos_info; a->pair_kinds = h->d_pair_kinds; a->stage_lut = h->d_stage_lut;
     a->nbm1 = h->d_nbm1; a->win_pos = h->d_win_pos; a->win_row_begin = h->d_win_row_begin; a->win_rows = h->d_win_rows;
     a->n_windows = h->n_windows; a->row_doubles = h->row_doubles; a->rk_bytes = h->rk_bytes; a->stg_words = h->stg_words;
@@ -495,13 +530,24 @@ static int fill_args(ace_handle_t *h, const ace_batch_t *b, double memory_limit,
     return ACE_OK;
 }
 
+}  // extern "C"
+
+template <bool BD, bool RANGED>
+static void launch_score_w(const ace_handle_t *h, const AceKernelArgs &a, hipStream_t s, unsigned blocks) {
+    if (h->n_windows > 1)
+        hipLaunchKernelGGL((ace_score_kernel<BD, RANGED, true>), dim3(blocks), dim3(kBlock), h->lds_bytes, s, a);
+    else
+        hipLaunchKernelGGL((ace_score_kernel<BD, RANGED, false>), dim3(blocks), dim3(kBlock), h->lds_bytes, s, a);
+}
+
 static void launch_score(const ace_handle_t *h, const AceKernelArgs &a, hipStream_t s) {
     const unsigned blocks = (unsigned)(((size_t)a.g.P + kBlock - 1) / kBlock);
-    if (a.stage_out)
-        hipLaunchKernelGGL(ace_score_kernel<true>, dim3(blocks), dim3(kBlock), h->lds_bytes, s, a);
-    else
-        hipLaunchKernelGGL(ace_score_kernel<false>, dim3(blocks), dim3(kBlock), h->lds_bytes, s, a);
+    if (a.range) launch_score_w<true, true>(h, a, s, blocks);
+    else if (a.stage_out) launch_score_w<true, false>(h, a, s, blocks);
+    else launch_score_w<false, false>(h, a, s, blocks);
 }
+
+extern "C" {
 
 int ace_score_batch(ace_handle_t *h, const ace_batch_t *batch, double memory_limit, int strict, double *d_iter_ms,
                     double *d_peak_mb, uint8_t *d_feasible, uint8_t *d_status, double *d_stage_out, void *stream) {

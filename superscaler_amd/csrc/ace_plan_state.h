@@ -40,21 +40,29 @@ struct AceLds {
     }
 };
 static inline double ace_max(double a, double b) { return a > b ? a : b; }
-static inline bool ace_isnan(double a) { return a != a; }
 #else
 #define ACE_HD __device__ __forceinline__
 struct AceLds {
     const unsigned char *base;
     template <class T> ACE_HD T ld(uint32_t off) const { return *reinterpret_cast<const T *>(base + off); }
 };
-ACE_HD double ace_max(double a, double b) { return fmax(a, b); }
-ACE_HD bool ace_isnan(double a) { return a != a; }
+// One v_max_f64.  fmax() makes the compiler quiet both operands first (two more instructions);
+// table values are never signalling NaNs, and a NaN operand only occurs in plans that are
+// reported as unscorable anyway.
+ACE_HD double ace_max(double a, double b) {
+    double r;
+    asm("v_max_f64 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
 #endif
+ACE_HD bool ace_isnan(double a) { return a != a; }
 
 struct alignas(16) ace_d2 { double x, y; };
 struct alignas(16) ace_u4 { uint32_t x, y, z, w; };
+struct alignas(8) ace_u2 { uint32_t x, y; };
 
-#define ACE_PLAN_MALFORMED 3
+#define ACE_HOT_STRIDE 48u     // bytes per (diag, code) entry of the hot sub-table
+#define ACE_START_STRIDE 32u
 
 // Geometry and constants every lane reads (kernel arguments -> scalar registers).
 struct AceGeom {
@@ -64,18 +72,26 @@ struct AceGeom {
     uint32_t hot_off, start_off, out_off, z_off;   // bytes inside a row
     uint32_t z_stride;          // bytes of one resharding-cost table inside a row (n_diag * C * 8)
     uint32_t rk_lds_off, stg_lds_off;              // LDS byte offsets of the pair-kind and stage LUT regions
+    uint32_t rk_kind_stride;    // bytes of one pair kind (n_glog * C * C)
     int32_t flags;
     double main_params, optimizer, mem_limit;
     int32_t strict;
 };
 
-template <bool BD> struct PlanState {
+// position descriptor (wave-uniform): x = row offset / 16 | previous op's row offset / 16 << 16,
+// y = pair kind | flags << 8 (bit 0: previous op is an ordinary op followed by a layer start;
+// bit 1: previous op is an ordinary op)
+ACE_HD uint32_t info_row(ace_u2 i) { return (i.x & 0xffffu) << 4; }
+ACE_HD uint32_t info_prevrow(ace_u2 i) { return (i.x >> 16) << 4; }
+
+template <bool BD, bool RANGED> struct PlanState {
     // plan constants
     int S;
     uint32_t bidx;
     uint64_t glogs;
     uint32_t cross;
     uint32_t ideal_hot_v, ideal_start_v;
+    int lo, hi;                 // RANGED: only ops lo <= i < hi belong to the plan (one stage)
     // stage state
     int s;
     uint32_t hot_v, z_v, rk_v, mrow;
@@ -85,21 +101,23 @@ template <bool BD> struct PlanState {
     // per-op accumulators (reset at every stage head)
     double fwd, bwd, rcs, W, A, saved, run, peak, rfm, rbm, pend_rf, pend_rb, rs_f, rs_b, prev_act;
     double id_fwd, id_bwd;
-    uint32_t prev_byte;
     bool lastclose;
+    bool done;                  // RANGED: the stage was finished inside the op loop
     // plan accumulators
     double sum_t, max_t, max_mem;
     uint32_t status;
 
-    ACE_HD void init(const AceGeom &g, const AceLds &lds, ace_u4 h) {
+    ACE_HD void init(const AceGeom &g, const AceLds &lds, ace_u4 h, ace_u2 range) {
         S = (int)(h.x & 0xff);
         bidx = (h.x >> 8) & 0xff;
         glogs = (uint64_t)h.y | ((uint64_t)h.z << 32);
         cross = h.w;
+        lo = RANGED ? (int)range.x : 0;
+        hi = RANGED ? (int)range.y : g.N;
         s = -1;
         sum_t = 0.0; max_t = 0.0; max_mem = 0.0;
         status = 0;
-        prev_byte = 0; prev_act = 0.0; lastclose = false;
+        prev_act = 0.0; lastclose = false; done = false;
         fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = pend_rf = pend_rb = rs_f = rs_b = 0.0;
         id_fwd = id_bwd = id_in = 0.0;
         in_comm = inputs = 0.0;
@@ -107,14 +125,15 @@ template <bool BD> struct PlanState {
         out_cross = false;
         ideal_hot_v = ideal_start_v = 0;
         if (bidx >= (uint32_t)g.n_mbs) { status = ACE_PLAN_MALFORMED; bidx = 0; }
+        if (RANGED && (lo < 0 || hi > g.N || lo >= hi)) { status = ACE_PLAN_MALFORMED; lo = 0; hi = 1; }
         if (BD) {
             // the "ideal" pass uses tp = dp = 1 and micro-batch = micro_bs (aceso_cost_model.py:588-590):
             // the diag of (micro_bs, 1 gpu)
             uint32_t w = lds.ld<uint32_t>(g.stg_lds_off + (bidx * 16u + 0u) * 4u);
             uint32_t d = w & 0xff;
             if (d == 0xff) d = 0;
-            ideal_hot_v = d * (uint32_t)g.C * 48u;
-            ideal_start_v = d * (uint32_t)g.C * 32u;
+            ideal_hot_v = d * (uint32_t)g.C * ACE_HOT_STRIDE;
+            ideal_start_v = d * (uint32_t)g.C * ACE_START_STRIDE;
         }
     }
 
@@ -124,24 +143,25 @@ template <bool BD> struct PlanState {
         uint32_t sidx = (uint32_t)(s < ACE_MAX_STAGES ? s : ACE_MAX_STAGES - 1);
         if (s >= ACE_MAX_STAGES) status = ACE_PLAN_MALFORMED;
         uint32_t glog = (uint32_t)(glogs >> (4u * sidx)) & 15u;
+        if (glog >= (uint32_t)g.n_glog) { status |= ACE_PLAN_UNSCORABLE; glog = 0; }
         uint32_t w = lds.ld<uint32_t>(g.stg_lds_off + (bidx * 16u + glog) * 4u);
         uint32_t d = w & 0xff;
         mrow = w >> 8;
-        if (d == 0xff) { status |= ACE_PLAN_BAD_MBS; d = 0; }
-        if (glog >= (uint32_t)g.n_glog) { status |= ACE_PLAN_BAD_MBS; glog = 0; }
-        hot_v = d * (uint32_t)g.C * 48u;
-        z_v = d * (uint32_t)g.C * 8u;
+        if (d == 0xff) { status |= ACE_PLAN_UNSCORABLE; d = 0; }
+        uint32_t dc = d * (uint32_t)g.C;
+        hot_v = dc * ACE_HOT_STRIDE;
+        z_v = dc * 8u;
         rk_v = glog * (uint32_t)(g.C * g.C);
         bool in_cross = (cross >> sidx) & 1u;
         out_cross = (cross >> (16u + sidx)) & 1u;
         t_first = c >> g.A_shift;
-        uint32_t a = row + g.start_off + d * (uint32_t)g.C * 32u + c * 32u;
+        uint32_t a = row + g.start_off + (dc + c) * ACE_START_STRIDE;
         ace_d2 e0 = lds.ld<ace_d2>(a);          // input size, size / intra-node bandwidth
         ace_d2 e1 = lds.ld<ace_d2>(a + 16);     // size / inter-node bandwidth, pad
         inputs = e0.x;
         in_comm = in_cross ? e1.x : e0.y;
         if (BD) {
-            uint32_t ai = row + g.start_off + ideal_start_v + (c & (uint32_t)(g.n_algo - 1)) * 32u;
+            uint32_t ai = row + g.start_off + ideal_start_v + (c & (uint32_t)(g.n_algo - 1)) * ACE_START_STRIDE;
             ace_d2 i0 = lds.ld<ace_d2>(ai);
             ace_d2 i1 = lds.ld<ace_d2>(ai + 16);
             id_in = in_cross ? i1.x : i0.y;
@@ -151,14 +171,12 @@ template <bool BD> struct PlanState {
         lastclose = false;
     }
 
-    // Stage tail; `prevrow` is the LDS offset of the row of the stage's last op, whose code byte
-    // is still in prev_byte.
-    ACE_HD void finish(const AceGeom &g, const AceLds &lds, uint32_t prevrow, double *rec) {
-        uint32_t c_last = prev_byte & 7u;
+    // Stage tail; `prevrow` is the LDS offset of the row of the stage's last op, `c_last` its code.
+    ACE_HD void finish(const AceGeom &g, const AceLds &lds, uint32_t prevrow, uint32_t c_last, double *rec) {
         uint32_t t_last = c_last >> g.A_shift;
         uint32_t a_last = c_last & (uint32_t)(g.n_algo - 1);
         uint32_t m_last = (mrow >> (4u * t_last)) & 15u;
-        if (m_last >= (uint32_t)g.n_mbs) m_last = 0;   // only for plans already marked BAD_MBS (their sums are NaN)
+        if (m_last >= (uint32_t)g.n_mbs) m_last = 0;   // only for plans whose sums are NaN already
         // output_size[ops[-1]][mbs[-1]][tp[0]][algo[-1]]  (sic, aceso_cost_model.py:321-326)
         uint32_t oidx = ((m_last * (uint32_t)g.n_tp + t_first) << g.A_shift) + a_last;
         ace_d2 oe = lds.ld<ace_d2>(prevrow + g.out_off + oidx * 16u);
@@ -196,18 +214,23 @@ template <bool BD> struct PlanState {
         }
     }
 
-    // One op.  `info` is the position's (wave-uniform) descriptor.
-    ACE_HD void step(const AceGeom &g, const AceLds &lds, uint32_t byte, ace_u4 info, double *rec) {
+    // One op at position i.  `byte` is its code byte, `pbyte` the previous op's, `info` the
+    // position's (wave-uniform) descriptor.
+    ACE_HD void step(const AceGeom &g, const AceLds &lds, int i, uint32_t byte, uint32_t pbyte, ace_u2 info, double *rec) {
+        if (RANGED) {
+            if (i == hi) { finish(g, lds, info_prevrow(info), pbyte & 7u, rec); done = true; }
+            if (i < lo || i >= hi) return;
+        }
         const uint32_t c = byte & 7u;
         const bool rc = (byte >> 3) & 1u;
         const bool ns = (byte >> 4) & 1u;
-        const uint32_t row = info.x;
+        const uint32_t row = info_row(info);
         if (ns) {
-            if (s >= 0) finish(g, lds, info.y, rec);
+            if (s >= 0) finish(g, lds, info_prevrow(info), pbyte & 7u, rec);
             start(g, lds, row, c);
         }
-        const uint32_t fl = info.z >> 8;
-        uint32_t a = row + g.hot_off + hot_v + c * 48u;
+        const uint32_t fl = info.y >> 8;
+        uint32_t a = row + g.hot_off + hot_v + c * ACE_HOT_STRIDE;
         ace_d2 e0 = lds.ld<ace_d2>(a);         // fwd us, bwd us
         ace_d2 e1 = lds.ld<ace_d2>(a + 16);    // weights MB, activations MB (shared-buffer rule applied)
         ace_d2 e2 = lds.ld<ace_d2>(a + 32);    // fwd / bwd reserved MB
@@ -218,51 +241,48 @@ template <bool BD> struct PlanState {
         pend_rb = e2.y;
         fwd += e0.x;
         bwd += e0.y;
-        rcs += rc ? e0.x : 0.0;
+        if (rc) rcs += e0.x;
         W += e1.x;
         A += e1.y;
         if (BD) {
-            ace_d2 ie = lds.ld<ace_d2>(row + g.hot_off + ideal_hot_v + (c & (uint32_t)(g.n_algo - 1)) * 48u);
+            ace_d2 ie = lds.ld<ace_d2>(row + g.hot_off + ideal_hot_v + (c & (uint32_t)(g.n_algo - 1)) * ACE_HOT_STRIDE);
             id_fwd += ie.x;
             id_bwd += ie.y;
         }
         // (previous op, this op) both recomputed and in one stage
-        const bool pair = rc && ((prev_byte >> 3) & 1u) && !ns;
+        const bool pair = ((byte & pbyte) >> 3) & ~(byte >> 4) & 1u;
         const bool savez = fl & 1u;     // previous op is an ordinary op followed by a layer start
-        run += pair ? prev_act : 0.0;
-        saved += (pair && !savez) ? prev_act : 0.0;
+        if (pair) {
+            run += prev_act;
+            if (!savez) saved += prev_act;
+        }
         if (!pair || savez) {
             peak = ace_max(peak, run);
             run = 0.0;
         }
         lastclose = pair && (fl & 2u);
         prev_act = e1.y;
-        if ((g.flags & ACE_F_RESHARDING) && !ns) {
-            uint32_t pk = info.z & 0xffu;
-            uint32_t pc = prev_byte & 7u;
-            uint32_t r = lds.ld<uint8_t>(g.rk_lds_off + pk * (uint32_t)(g.n_glog * g.C * g.C) + rk_v + pc * (uint32_t)g.C + c);
-            if (r != 0) {
-                uint32_t pf = r & 15u, pb = r >> 4;
-                uint32_t za = row + g.z_off + z_v + c * 8u;
-                if (pf == 15u || pb == 15u) {
-                    status |= ACE_PLAN_BAD_RESHARD;
-                } else {
-                    if (pf) rs_f += lds.ld<double>(za + (pf - 1u) * g.z_stride);
-                    if (pb) rs_b += lds.ld<double>(za + (pb - 1u) * g.z_stride);
-                }
-            }
+        if (g.flags & ACE_F_RESHARDING) {
+            // collective ids of the (previous, this) op pair; id 0 is an all-zero cost table, so a
+            // pair that needs nothing adds 0.0, and the id past the last real table is all NaN
+            // (the reference raises there)
+            uint32_t pk = info.y & 0xffu;
+            uint32_t pc = pbyte & 7u;
+            uint32_t r = ns ? 0u : (uint32_t)lds.ld<uint8_t>(g.rk_lds_off + pk * g.rk_kind_stride + rk_v + pc * (uint32_t)g.C + c);
+            uint32_t za = row + g.z_off + z_v + c * 8u;
+            rs_f += lds.ld<double>(za + (r & 15u) * g.z_stride);
+            rs_b += lds.ld<double>(za + (r >> 4) * g.z_stride);
         }
-        prev_byte = byte;
     }
 
     ACE_HD void result(const AceGeom &g, double nbm1, double &iter_ms, double &peak_mb, uint8_t &feasible, uint8_t &st) {
-        if (s + 1 != S) status = ACE_PLAN_MALFORMED;
+        if (!RANGED && s + 1 != S) status = ACE_PLAN_MALFORMED;
         // max over stages of t_s*(nb-1) + sum(t): rounding is monotonic, so the maximum is attained
         // at the largest t_s and equals this expression bit for bit
         iter_ms = max_t * nbm1 + sum_t;
         peak_mb = max_mem;
         bool ok = status == 0 && !ace_isnan(iter_ms) && !ace_isnan(max_mem);
-        if (!ok && status == 0) status = ACE_PLAN_BAD_MBS;   // a table entry outside the profiled grid
+        if (!ok && status == 0) status = ACE_PLAN_UNSCORABLE;   // a table entry outside the profiled grid
         bool feas = g.strict ? (max_mem < g.mem_limit) : (max_mem <= g.mem_limit);
         feasible = (uint8_t)(ok && feas);
         st = (uint8_t)status;
@@ -272,3 +292,6 @@ template <bool BD> struct PlanState {
         }
     }
 };
+
+// byte k (0..15) of a 16-op group held in four 32-bit words
+ACE_HD uint32_t group_byte(const uint32_t w[4], int k) { return (w[k >> 2] >> ((k & 3) * 8)) & 0xffu; }

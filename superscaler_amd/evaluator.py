@@ -20,7 +20,8 @@ EXPORTS = ["ace_abi_version", "ace_strerror", "ace_last_hip_error", "ace_create"
 
 
 class AceBatchStruct(ctypes.Structure):
-    _fields_ = [("d_codes", ctypes.c_void_p), ("d_hdr", ctypes.c_void_p), ("n_plans", ctypes.c_size_t)]
+    _fields_ = [("d_codes", ctypes.c_void_p), ("d_hdr", ctypes.c_void_p), ("d_range", ctypes.c_void_p),
+                ("n_plans", ctypes.c_size_t)]
 
 
 class AceError(RuntimeError):
@@ -74,7 +75,7 @@ def _check(lib, rc, what):
 class DeviceBatch:
     """A PlanBatch resident in HBM in the layout the kernel streams."""
 
-    def __init__(self, batch: PlanBatch, device="cuda:0"):
+    def __init__(self, batch: PlanBatch, device="cuda:0", ranges: Optional[np.ndarray] = None):
         import torch
         self.n_plans = batch.n_plans
         self.num_ops = batch.num_ops
@@ -86,7 +87,13 @@ class DeviceBatch:
         # [P, G, 16] -> [G, P, 16]: plan-minor, sixteen ops per 16-byte word
         self.codes = codes.view(P, G, 16).permute(1, 0, 2).contiguous()
         self.hdr = torch.from_numpy(np.ascontiguousarray(batch.hdr).view(np.int32)).to(device)
-        self.struct = AceBatchStruct(self.codes.data_ptr(), self.hdr.data_ptr(), P)
+        self.ranges = None
+        if ranges is not None:
+            r = np.ascontiguousarray(ranges, dtype=np.uint32)
+            assert r.shape == (P, 2)
+            self.ranges = torch.from_numpy(r.view(np.int32)).to(device)
+        self.struct = AceBatchStruct(self.codes.data_ptr(), self.hdr.data_ptr(),
+                                     self.ranges.data_ptr() if self.ranges is not None else None, P)
 
     @property
     def bytes_moved_per_plan(self):
@@ -120,12 +127,12 @@ class PlanEvaluator:
         except Exception:
             pass
 
-    def upload(self, batch: PlanBatch, validate: bool = True) -> DeviceBatch:
-        if validate:
+    def upload(self, batch: PlanBatch, validate: bool = True, ranges: Optional[np.ndarray] = None) -> DeviceBatch:
+        if validate and ranges is None:
             msg = validate_batch(batch, self.tables)
             if msg:
                 raise ValueError(msg)
-        return DeviceBatch(batch, self.device)
+        return DeviceBatch(batch, self.device, ranges)
 
     def _stream(self):
         return ctypes.c_void_p(self._torch.cuda.current_stream(self.device).cuda_stream)
@@ -143,6 +150,7 @@ class PlanEvaluator:
             st = torch.empty(P, dtype=torch.uint8, device=self.device)
         else:
             it, pk, fe, st = out
+        breakdown = breakdown or dbatch.ranges is not None
         rec = torch.zeros((P, MAX_STAGES, STAGE_REC), dtype=torch.float64, device=self.device) if breakdown else None
         with torch.cuda.device(self.device):
             rc = self.lib.ace_score_batch(self.handle, ctypes.byref(dbatch.struct), limit, int(strict),
@@ -185,8 +193,8 @@ class PlanEvaluator:
         return ms.value
 
     # convenience: host in, host out
-    def score_host(self, batch: PlanBatch, memory_limit=None, strict=False, breakdown=False):
-        d = self.upload(batch)
+    def score_host(self, batch: PlanBatch, memory_limit=None, strict=False, breakdown=False, ranges=None):
+        d = self.upload(batch, ranges=ranges)
         out = self.score(d, memory_limit, strict, breakdown)
         self._torch.cuda.synchronize(self.device)
         return tuple(None if t is None else t.cpu().numpy() for t in out)

@@ -21,10 +21,11 @@ maxima of table entries:
   tuples share a diag.  Entries whose micro-batch is not profiled are NaN (the reference
   raises KeyError there).
   pair_kinds[kind][glog][code_prev][code_cur]  byte: forward | backward << 4 collective table
-     ids (1-based, 0 = nothing to do, 15 = the reference would raise) for an adjacent op
+     ids (0 = the all-zero table: nothing to do, last id = the all-NaN table: the reference would
+     raise) for an adjacent op
      pair, from get_op_spec / get_reshard_primitives (model_ops_info.py:92-150, cost_model:185-245)
   stage_lut[mbs index][glog]  diag | per-tp mbs-index nibbles << 8 (0xF = not profiled)
-  pos_info[i]  LDS byte offset of op i's row, of op i-1's row, pair kind | flags << 8
+  pos_info[i]  LDS offset / 16 of op i's row | of op i-1's row << 16;  pair kind | flags << 8
 """
 import ctypes
 import math
@@ -79,7 +80,7 @@ class CompiledTables:
     lds_row_bytes: int
     flags: int
     rows: np.ndarray            # float64 [n_types, row_doubles]
-    pos_info: np.ndarray        # uint32 [N + 1, 4]
+    pos_info: np.ndarray        # uint32 [N + 1, 2]
     pair_kinds: np.ndarray      # uint8 [n_pk, n_glog, C, C]
     stage_lut: np.ndarray       # uint32 [n_mbs, 16]
     nb_minus_1: np.ndarray      # float64 [n_mbs]
@@ -187,15 +188,17 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
     # ---- adjacent-pair kinds and the collectives in use ----------------------------------------
     z_keys: List[Tuple[int, int]] = []
 
+    ERR = 15   # placeholder while the number of real tables is still growing
+
     def z_id(prim, n):
         if prim in (og.P_NONE, og.P_SPLIT):
             return 0          # nothing to pay: split is free (aceso_cost_model.py:257-258)
         name = og.PRIM_NAMES[prim]
         if name not in db.collectives or n not in db.collectives[name]:
-            return 15         # KeyError in the reference (:251)
+            return ERR        # KeyError in the reference (:251)
         if (prim, n) not in z_keys:
-            if len(z_keys) >= 14:
-                raise ValueError("more than 14 distinct (collective, group size) pairs")
+            if len(z_keys) >= 13:
+                raise ValueError("more than 13 distinct (collective, group size) pairs")
             z_keys.append((prim, n))
         return z_keys.index((prim, n)) + 1
 
@@ -226,7 +229,7 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
                         pf, pb, n = og.reshard_prims(src, dst)
                         blk[glog, cp, cc] = z_id(pf, n) | (z_id(pb, n) << 4)
                     except og.InconsistentSpecs:
-                        blk[glog, cp, cc] = 0xFF
+                        blk[glog, cp, cc] = ERR | (ERR << 4)
         return blk
 
     def intern(blk: np.ndarray) -> int:
@@ -246,7 +249,12 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
     if len(pk_arrays) > 255:
         raise ValueError("more than 255 distinct adjacent-op spec pairings")
     pair_kinds = np.ascontiguousarray(np.stack(pk_arrays))
-    NZ = len(z_keys)
+    # cost-table ids: 0 = all zeros, 1..len(z_keys) = real collectives, last = all NaN (errors)
+    NZ = len(z_keys) + 2
+    lo, hi = pair_kinds & 15, pair_kinds >> 4
+    lo = np.where(lo == ERR, NZ - 1, lo)
+    hi = np.where(hi == ERR, NZ - 1, hi)
+    pair_kinds = np.ascontiguousarray((lo | (hi << 4)).astype(np.uint8))
 
     # ---- rows ------------------------------------------------------------------------------
     hot_off = 0
@@ -262,7 +270,8 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
         fl = int(graph.flags[ty])
         hot = np.full((ND, C, 6), nan)
         start = np.full((ND, C, 4), nan)
-        z = np.full((max(NZ, 1), ND, C), nan)
+        z = np.full((NZ, ND, C), nan)
+        z[0] = 0.0
         for d, tup in enumerate(diag_tuples):
             for t in range(T):
                 m = tup[t]
@@ -282,7 +291,7 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
                     insz = float(tb["input_size"][ty, m, t, a])
                     start[d, c] = (insz, db.p2p_time(insz, db.intra_band), db.p2p_time(insz, db.inter_band), 0.0)
                     for k, (prim, n) in enumerate(z_keys):
-                        z[k, d, c] = db.reshard_time(og.PRIM_NAMES[prim], n, insz)
+                        z[k + 1, d, c] = db.reshard_time(og.PRIM_NAMES[prim], n, insz)
         out = np.zeros((M, T, A, 2))
         for m in range(M):
             for t in range(T):
@@ -292,8 +301,7 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
         rows[ty, hot_off:hot_off + hot.size] = hot.ravel()
         rows[ty, start_off:start_off + start.size] = start.ravel()
         rows[ty, out_off:out_off + out.size] = out.ravel()
-        if NZ:
-            rows[ty, z_off:z_off + NZ * ND * C] = z[:NZ].ravel()
+        rows[ty, z_off:z_off + NZ * ND * C] = z.ravel()
 
     # ---- LDS residency: one window if every row fits, else windows over op positions ----------
     row_bytes = row_doubles * 8
@@ -303,17 +311,19 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
     if avail < 2 * row_bytes:
         raise ValueError(f"one op type's row ({row_bytes} B) does not fit LDS twice ({avail} B available)")
     slots = avail // row_bytes
-    pos_info = np.zeros((graph.num_ops + 1, 4), dtype=np.uint32)
+    pos_info = np.zeros((graph.num_ops + 1, 2), dtype=np.uint32)
     win_pos, win_row_begin, win_rows = [0], [0], []
     tp = graph.type_of_pos
     i = 0
     N = graph.num_ops
     while i < N:
-        # a window holds the row of the op just before it (stage tails look back one op)
+        # a window holds the row of the op just before it (stage tails look back one op) and ends
+        # at a multiple of 16 ops (the kernel restages between 16-op groups) or at the last op
         slot_of: Dict[int, int] = {}
         if i > 0:
             slot_of[int(tp[i - 1])] = 0
         j = i
+        good = None
         while j < N:
             ty = int(tp[j])
             if ty not in slot_of:
@@ -321,18 +331,22 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
                     break
                 slot_of[ty] = len(slot_of)
             j += 1
+            if j % 16 == 0 or j == N:
+                good = (j, dict(slot_of))
+        if good is None:
+            raise ValueError("LDS too small for a 16-op window of this op graph")
+        j, slot_of = good
         for k in range(i, j):
-            pos_info[k, 0] = slot_of[int(tp[k])] * row_bytes
-            pos_info[k, 1] = slot_of[int(tp[k - 1])] * row_bytes if k > 0 else 0
+            prev = slot_of[int(tp[k - 1])] if k > 0 else 0
+            pos_info[k, 0] = (slot_of[int(tp[k])] * row_bytes // 16) | ((prev * row_bytes // 16) << 16)
         if j == N:
-            pos_info[N, 0] = 0
-            pos_info[N, 1] = slot_of[int(tp[N - 1])] * row_bytes
+            pos_info[N, 0] = (slot_of[int(tp[N - 1])] * row_bytes // 16) << 16
         for ty, sl in slot_of.items():
             win_rows.append((ty, sl * row_bytes))
         win_row_begin.append(len(win_rows))
         win_pos.append(j)
         i = j
-    win_pos[-1] = max(win_pos[-1], N + 1)      # never reached: no restaging after the last window
+    win_pos[-1] = max((win_pos[-1] + 15) // 16 * 16, N + 1)      # never reached: no restaging after the last window
     lds_row_bytes = max(off for _, off in win_rows) + row_bytes
 
     # flags about the previous op, seen from position i
@@ -344,7 +358,7 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
             fl |= 1      # ordinary op right before a layer start: saved += 0, peak segment closes
         if normal[prev_t]:
             fl |= 2      # ordinary op: closes the last segment when the pair ends the stage
-        pos_info[k, 2] = int(pk_of_pos[k]) | (fl << 8)
+        pos_info[k, 1] = int(pk_of_pos[k]) | (fl << 8)
 
     flags = 0
     if settings.resharding and (pair_kinds != 0).any():

@@ -8,10 +8,40 @@
 
 #include <vector>
 
+namespace {
+
+template <bool BD, bool RANGED>
+void score_one(const ace_tables_t *t, const AceGeom &g, std::vector<unsigned char> &lds, uint32_t lds_bytes,
+               const uint8_t *codes, ace_u4 h, ace_u2 range, double *rec, double &iter, double &peak, uint8_t &feas,
+               uint8_t &st) {
+    const size_t row_bytes = (size_t)t->row_doubles * 8;
+    const ace_u2 *pos = reinterpret_cast<const ace_u2 *>(t->pos_info);
+    AceLds view{lds.data(), lds_bytes};
+    PlanState<BD, RANGED> s;
+    s.init(g, view, h, range);
+    int w = 0, next_win = t->win_pos[0];
+    uint32_t pbyte = 0;
+    for (int i = 0; i < g.N; ++i) {
+        if (i == next_win) {
+            // poison, then stage exactly the rows the window lists: a read of any other row yields NaN
+            memset(lds.data(), 0xff, t->lds_row_bytes);
+            for (int r = t->win_row_begin[w]; r < t->win_row_begin[w + 1]; ++r)
+                memcpy(lds.data() + t->win_rows[2 * r + 1], t->rows + (size_t)t->win_rows[2 * r] * t->row_doubles, row_bytes);
+            next_win = t->win_pos[++w];
+        }
+        s.step(g, view, i, codes[i], pbyte, pos[i], rec);
+        pbyte = codes[i];
+    }
+    if (!RANGED || !s.done) s.finish(g, view, info_prevrow(pos[g.N]), pbyte & 7u, rec);
+    s.result(g, t->nb_minus_1[s.bidx], iter, peak, feas, st);
+}
+
+}  // namespace
+
 extern "C" int ace_emu_score(const ace_tables_t *t, const uint8_t *codes /* [P][N] plan-major */,
-                             const uint32_t *hdr /* [P][4] */, long long P, double memory_limit, int strict,
-                             double *iter_ms, double *peak_mb, uint8_t *feasible, uint8_t *status,
-                             double *stage_out /* nullable [P][16][18] */) {
+                             const uint32_t *hdr /* [P][4] */, const uint32_t *range /* nullable [P][2] */,
+                             long long P, double memory_limit, int strict, double *iter_ms, double *peak_mb,
+                             uint8_t *feasible, uint8_t *status, double *stage_out /* nullable [P][16][18] */) {
     const int C = t->n_tp * t->n_algo;
     AceGeom g;
     memset(&g, 0, sizeof(g));
@@ -23,55 +53,30 @@ extern "C" int ace_emu_score(const ace_tables_t *t, const uint8_t *codes /* [P][
     const int32_t rk_bytes = t->n_pair_kinds * t->n_glog * C * C;
     g.rk_lds_off = (uint32_t)t->lds_row_bytes;
     g.stg_lds_off = (g.rk_lds_off + (uint32_t)rk_bytes + 15u) & ~15u;
+    g.rk_kind_stride = (uint32_t)(t->n_glog * C * C);
     const uint32_t lds_bytes = g.stg_lds_off + (uint32_t)t->n_mbs * 16u * 4u;
     g.flags = t->flags; g.main_params = t->main_params; g.optimizer = t->optimizer;
     g.mem_limit = memory_limit; g.strict = strict ? 1 : 0;
-    const size_t row_bytes = (size_t)t->row_doubles * 8;
+    if (range && !stage_out) return -1;
 
     std::vector<unsigned char> lds(lds_bytes);
-    const ace_u4 *pos = reinterpret_cast<const ace_u4 *>(t->pos_info);
     for (long long p = 0; p < P; ++p) {
-        // poison the row region so that a read of a row the window did not stage is caught as NaN
         memset(lds.data(), 0xff, lds.size());
         memcpy(lds.data() + g.rk_lds_off, t->pair_kinds, rk_bytes);
         memcpy(lds.data() + g.stg_lds_off, t->stage_lut, (size_t)t->n_mbs * 16 * 4);
-        AceLds view{lds.data(), lds_bytes};
         ace_u4 h;
         memcpy(&h, hdr + 4 * p, 16);
+        ace_u2 rg{0u, 0u};
+        if (range) memcpy(&rg, range + 2 * p, 8);
         double *rec = stage_out ? stage_out + (size_t)p * ACE_MAX_STAGES * ACE_STAGE_REC : nullptr;
-        int w = 0, next_win = t->win_pos[0];
+        const uint8_t *c = codes + (size_t)p * g.N;
         double iter, peak;
         uint8_t feas, st;
-        if (stage_out) {
-            PlanState<true> s;
-            s.init(g, view, h);
-            for (int i = 0; i < g.N; ++i) {
-                if (i == next_win) {
-                    memset(lds.data(), 0xff, t->lds_row_bytes);
-                    for (int r = t->win_row_begin[w]; r < t->win_row_begin[w + 1]; ++r)
-                        memcpy(lds.data() + t->win_rows[2 * r + 1], t->rows + (size_t)t->win_rows[2 * r] * t->row_doubles, row_bytes);
-                    next_win = t->win_pos[++w];
-                }
-                s.step(g, view, codes[p * g.N + i], pos[i], rec);
-            }
-            s.finish(g, view, pos[g.N].y, rec);
-            s.result(g, t->nb_minus_1[s.bidx], iter, peak, feas, st);
-        } else {
-            PlanState<false> s;
-            s.init(g, view, h);
-            for (int i = 0; i < g.N; ++i) {
-                if (i == next_win) {
-                    memset(lds.data(), 0xff, t->lds_row_bytes);
-                    for (int r = t->win_row_begin[w]; r < t->win_row_begin[w + 1]; ++r)
-                        memcpy(lds.data() + t->win_rows[2 * r + 1], t->rows + (size_t)t->win_rows[2 * r] * t->row_doubles, row_bytes);
-                    next_win = t->win_pos[++w];
-                }
-                s.step(g, view, codes[p * g.N + i], pos[i], nullptr);
-            }
-            s.finish(g, view, pos[g.N].y, nullptr);
-            s.result(g, t->nb_minus_1[s.bidx], iter, peak, feas, st);
-        }
-        iter_ms[p] = iter; peak_mb[p] = peak; feasible[p] = feas; if (status) status[p] = st;
+        if (range) score_one<true, true>(t, g, lds, lds_bytes, c, h, rg, rec, iter, peak, feas, st);
+        else if (stage_out) score_one<true, false>(t, g, lds, lds_bytes, c, h, rg, rec, iter, peak, feas, st);
+        else score_one<false, false>(t, g, lds, lds_bytes, c, h, rg, rec, iter, peak, feas, st);
+        iter_ms[p] = iter; peak_mb[p] = peak; feasible[p] = feas;
+        if (status) status[p] = st;
     }
     return 0;
 }

@@ -64,7 +64,7 @@ def emu_lib():
     return _emu
 
 
-def emu_score(tables, batch, memory_limit=None, strict=False, breakdown=False):
+def emu_score(tables, batch, memory_limit=None, strict=False, breakdown=False, ranges=None):
     lib = emu_lib()
     ts = tables.as_struct()
     P = batch.n_plans
@@ -72,10 +72,13 @@ def emu_score(tables, batch, memory_limit=None, strict=False, breakdown=False):
     hdr = np.ascontiguousarray(batch.hdr)
     it = np.zeros(P); pk = np.zeros(P)
     fe = np.zeros(P, dtype=np.uint8); st = np.zeros(P, dtype=np.uint8)
-    rec = np.zeros((P, 16, 18)) if breakdown else None
+    rec = np.zeros((P, 16, 18)) if (breakdown or ranges is not None) else None
     limit = tables.settings.memory_limit if memory_limit is None else memory_limit
+    if ranges is not None:
+        ranges = np.ascontiguousarray(ranges, dtype=np.uint32)
+        breakdown = True
     rc = lib.ace_emu_score(ctypes.byref(ts), codes.ctypes.data_as(ctypes.c_void_p), hdr.ctypes.data_as(ctypes.c_void_p),
-                           ctypes.c_longlong(P), ctypes.c_double(limit), ctypes.c_int(int(strict)),
+                           ranges.ctypes.data_as(ctypes.c_void_p) if ranges is not None else None, ctypes.c_longlong(P), ctypes.c_double(limit), ctypes.c_int(int(strict)),
                            it.ctypes.data_as(ctypes.c_void_p), pk.ctypes.data_as(ctypes.c_void_p),
                            fe.ctypes.data_as(ctypes.c_void_p), st.ctypes.data_as(ctypes.c_void_p),
                            rec.ctypes.data_as(ctypes.c_void_p) if breakdown else None)

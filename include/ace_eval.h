@@ -52,7 +52,8 @@ enum {
     ACE_R_FWD = 0, ACE_R_BWD, ACE_R_IN_COMM, ACE_R_OUT_COMM, ACE_R_RECOMP,   /* get_time_v3 / get_recompute_time_v3 */
     ACE_R_WEIGHTS, ACE_R_INPUTS, ACE_R_ACT, ACE_R_SAVED, ACE_R_PEAK, ACE_R_RESERVED, /* get_memory_v3 ... get_reserved_memory */
     ACE_R_IDEAL_FWD, ACE_R_IDEAL_BWD, ACE_R_IDEAL_IN, ACE_R_IDEAL_OUT,       /* the tp=dp=1 pass, aceso_cost_model.py:588-592 */
-    ACE_R_STAGE_MS, ACE_R_STAGE_MB, ACE_R_SPARE
+    ACE_R_STAGE_MS, ACE_R_STAGE_MB,                                          /* stage time ms (:579), stage memory MB (:534) */
+    ACE_R_RESHARD                                                            /* (fwd + bwd resharding) us, the print-only column of :355 */
 };
 
 /*

@@ -1,0 +1,550 @@
+"""GPU-backed stand-in for the reference's search/aceso_cost_model.py.
+
+Same function names, argument meaning and error behaviour as the module that
+search/aceso_search.py:4, search/aceso_prims.py:7 and search/gen_megatron_plan.py:8 import,
+so the search loop, the policy and the move primitives keep running unchanged on the host
+while every number comes from the HIP kernels (libace_eval.so through `PlanEvaluator`).
+There is no CPU scoring path in this module: without the library or a GPU it raises.
+
+What stays on the host, on purpose:
+  * control flow of the greedy recompute pass (check_recompute, aceso_cost_model.py:794-872),
+    which asks the GPU for the stage's memory / saved / peak activations at every step;
+  * the float compositions the reference performs on per-stage values (time breakdown lists,
+    delta-time sign variants, memory breakdown tuple): they are evaluated here with Python
+    floats from the per-stage records the kernel writes, i.e. the same IEEE operations in
+    the same order as the reference.
+
+New, batched entry points (no reference counterpart): predict_time_breakdown_batch(),
+score_batch(), top_k().
+
+Module-level use mirrors the reference: `configure(args)` once (the reference evaluates its
+argparse singleton at import, aceso_cost_model.py:10), `read_profiled_time(...)`, then the
+functions below.
+"""
+import math
+from typing import List, Optional, Sequence
+
+import numpy as np
+
+from . import opgraph as og
+from .plan import AcesoConfig, AcesoStageInfo, PlanBatch, get_config  # noqa: F401 (re-exported)
+from .profile_db import CostModelSettings, ProfileDB
+from .tables import (MAX_STAGES, R_ACT, R_BWD, R_FWD, R_IDEAL_BWD, R_IDEAL_FWD, R_IDEAL_IN, R_IDEAL_OUT, R_IN_COMM,
+                     R_INPUTS, R_OUT_COMM, R_PEAK, R_RECOMP, R_RESERVED, R_SAVED, R_RESHARD, R_STAGE_MB, R_STAGE_MS,
+                     R_WEIGHTS, CompiledTables, compile_tables)
+
+
+def settings_from_args(args) -> CostModelSettings:
+    """The reference's argparse namespace (aceso_utils.py:455-531) -> CostModelSettings."""
+    if getattr(args, "consider_collective_memory", False):
+        raise NotImplementedError("--consider-collective-memory (aceso_cost_model.py:463-478) is not supported")
+    gpn = args.num_gpus_per_node
+    return CostModelSettings(
+        model_name=args.model_name, micro_batch_size=list(args.micro_batch_size), num_gpus_per_node=gpn,
+        global_batch_size=args.global_batch_size if getattr(args, "global_batch_size", None) else 1024,
+        memory_limit=float(getattr(args, "memory_limit", 28000)), max_tp=getattr(args, "max_tp", None) or gpn,
+        consider_shared_space=getattr(args, "consider_shared_space", True),
+        consider_reserved_space=getattr(args, "consider_reserved_space", True),
+        flex_recompute=getattr(args, "flex_recompute", True),
+        peak_mem_in_backward=getattr(args, "peak_mem_in_backward", 0),
+        memory_pred_type=getattr(args, "memory_pred_type", "MAX"),
+        resharding=getattr(args, "resharding", None))
+
+
+class CostModel:
+    """One profile database + op graph + settings, scored on one GPU."""
+
+    def __init__(self, settings: CostModelSettings, db: ProfileDB, graph: og.OpGraph, device="cuda:0"):
+        self.settings = settings
+        self.db = db
+        self.graph = graph
+        self.tables: CompiledTables = compile_tables(graph, db, settings)
+        self.device = device
+        self._evaluator = None        # created on first use: HIP must be initialised after any fork()
+        self._mbs_index = {m: k for k, m in enumerate(db.mbs_list)}
+        self._type_index = {n: k for k, n in enumerate(db.op_names)}
+        self._first_pos = {}
+        for i, name in enumerate(graph.ops):
+            self._first_pos.setdefault(name, []).append(i)
+        self._slice_cache = {}
+        # memo caches with the reference's keys and hit counters (aceso_cost_model.py:743-791)
+        self.stage_memory_set, self.stage_memory_visit, self.stage_memory_hit = {}, 0, 0
+        self.stage_time_set, self.stage_time_visit, self.stage_time_hit = {}, 0, 0
+
+    @classmethod
+    def from_directory(cls, args_or_settings, model_name, model_size, time_path, num_layers=None, device="cuda:0"):
+        st = args_or_settings if isinstance(args_or_settings, CostModelSettings) else settings_from_args(args_or_settings)
+        db = ProfileDB.from_directory(model_name, model_size, time_path, st, verbose=True)
+        if num_layers is None:
+            num_layers = getattr(args_or_settings, "num_layers", None)
+        graph = og.OpGraph.build("gpt" if model_name == "scale-layer" else model_name, db.op_names, num_layers)
+        return cls(st, db, graph, device)
+
+    @property
+    def evaluator(self):
+        if self._evaluator is None:
+            from .evaluator import PlanEvaluator
+            self._evaluator = PlanEvaluator(self.tables, self.device)
+        return self._evaluator
+
+    def close(self):
+        if self._evaluator is not None:
+            self._evaluator.close()
+            self._evaluator = None
+
+    # ---- batched scoring ------------------------------------------------------------------------
+    def encode(self, configs: Sequence) -> PlanBatch:
+        return PlanBatch.from_configs(configs, self.tables)
+
+    def score_batch(self, plans, memory_limit: Optional[float] = None, strict: bool = False):
+        """(iter_ms, peak_mb, feasible) numpy arrays for a PlanBatch or a list of configs."""
+        batch = plans if isinstance(plans, PlanBatch) else self.encode(plans)
+        it, pk, fe, st = self.evaluator.score_host(batch, memory_limit, strict)
+        self._raise_for_status(st)
+        return it, pk, fe
+
+    def top_k(self, plans, k: int, memory_limit: Optional[float] = None, strict: bool = False):
+        """Indices and times of the k fastest feasible plans (ascending, ties -> lower index)."""
+        batch = plans if isinstance(plans, PlanBatch) else self.encode(plans)
+        ev = self.evaluator
+        d = ev.upload(batch)
+        it, pk, fe, st = ev.score(d, memory_limit, strict)
+        idx, val, cnt = ev.topk(it, fe, k)
+        n = int(cnt.item())
+        return idx[:n].cpu().numpy(), val[:n].cpu().numpy()
+
+    @staticmethod
+    def _raise_for_status(status):
+        bad = np.flatnonzero(status)
+        if len(bad):
+            p = int(bad[0])
+            if int(status[p]) == 1:
+                raise KeyError(f"plan {p}: a micro-batch size, collective or spec pairing is outside the profile "
+                               "database (the reference raises KeyError / TypeError here)")
+            raise ValueError(f"plan {p}: malformed encoding")
+
+    def predict_time_breakdown_batch(self, configs: Sequence) -> None:
+        """predict_time_breakdown for many plans with one kernel launch; fills the same attributes."""
+        if not configs:
+            return
+        batch = self.encode(configs)
+        it, pk, fe, st, rec = self.evaluator.score_host(batch, breakdown=True)
+        self._raise_for_status(st)
+        for p, cfg in enumerate(configs):
+            self._fill_breakdown(cfg, rec[p])
+
+    def _fill_breakdown(self, config, rec, print_time=False, print_memory=False):
+        """aceso_cost_model.py:541-672 from the kernel's per-stage records."""
+        args = self.settings
+        num_batches = config.global_bs // config.micro_bs
+        _time_list, memory_list, compute_time_list, efficiency_list, gpu_time_list = [], [], [], [], []
+        ideal_per_gpu, eff_loss_list, recomp_list = [], [], []
+        time_strings, memory_strings = [], []
+        for i in range(config.num_stages):
+            r = [float(x) for x in rec[i]]
+            num_gpus = config.stages[i].num_gpus
+            fwd, bwd, in_comm, out_comm, recomp = r[R_FWD], r[R_BWD], r[R_IN_COMM], r[R_OUT_COMM], r[R_RECOMP]
+            sum_time = (fwd + bwd + in_comm + out_comm + recomp) / 1000
+            _time_list.append(sum_time)
+            compute_time_list.append((fwd + bwd + recomp) / 1000)
+            gpu_time_list.append(sum_time * num_gpus)
+            _fwd, _bwd, _in, _out = r[R_IDEAL_FWD], r[R_IDEAL_BWD], r[R_IDEAL_IN], r[R_IDEAL_OUT]
+            ideal_time = (_fwd + _bwd + _in + _out) / 1000
+            eff_loss_time = (fwd + bwd) - (_fwd + _bwd) / num_gpus
+            ideal_per_gpu.append(((_fwd + _bwd) / num_gpus) / 1000)
+            eff_loss_list.append(eff_loss_time / 1000)
+            recomp_list.append(recomp / 1000)
+            mw, mg, mo, ma, mp, mr = self._memory_breakdown(r, config.stages[i].num_stages_behind)
+            memory_sum = mw + mg + mo + ma + mp + mr
+            memory_list.append(memory_sum)
+            efficiency_list.append(ideal_time / (sum_time * num_gpus))
+            if print_time:
+                time_strings.append("[stage {}], {:.2f}, {:.2f}, {:.2f}, {:.2f}, {:.2f}, {:.2f}, ".format(
+                    i, fwd / 1000 * num_batches, (bwd + recomp) / 1000 * num_batches, recomp / 1000 * num_batches,
+                    in_comm / 1000 * num_batches, out_comm / 1000 * num_batches, r[R_RESHARD] / 1000 * num_batches))
+            if print_memory:
+                memory_strings.append(f"[stage {i}] memory = {memory_sum:.2f} MB. weights = {mw:.0f}, gradients = {mg:.0f}, "
+                                      f"optimizer = {mo:.0f}, activations = {ma:.0f}, peak += {mp:.0f}, "
+                                      f"memory_reserved = {mr:.0f}")
+        sum_stage_time = sum(_time_list)
+        time_list = [(_time_list[i] * (num_batches - 1) + sum_stage_time) for i in range(config.num_stages)]
+        config.time_list = time_list
+        config.memory_list = memory_list
+        config.compute_time_list = compute_time_list
+        config.total_gpu_time = sum(gpu_time_list) * (num_batches - 1)
+        config.breakdown_ideal_time_per_gpu = ideal_per_gpu
+        config.breakdown_eff_loss_time_per_gpu = eff_loss_list
+        config.breakdown_recomp_time_per_gpu = recomp_list
+        max_time = max(time_list)
+        max_mem = args.memory_limit
+        efficient_time_list = []
+        for i in range(config.num_stages):
+            used_time, used_memory = time_list[i], memory_list[i]
+            if sum(config.stages[i].recompute_ops) > 0:
+                idle_time = (max_time - used_time) / 2
+            else:
+                under_time = max_time - used_time
+                under_memory = ((max_mem - used_memory) / used_memory) * used_time
+                idle_time = under_time if under_memory > under_time else under_memory + (under_time - under_memory) / 2
+            efficient_time_list.append(idle_time * config.stages[i].num_gpus * efficiency_list[i])
+        config.efficient_time_list = efficient_time_list
+        if print_time:
+            b = max(range(config.num_stages), key=lambda k: (time_list[k], -k))
+            print("overall time = {:.2f} ms".format(max_time))
+            print("stage, fwd_comp, bwd_comp+recomp, recomp, in_comm(+reshard), out_comm(+reshard), reshard, sum(us)")
+            for i in range(config.num_stages):
+                print((" * " if i == b else "") + time_strings[i] + f"{time_list[i]:.2f}")
+        if print_memory:
+            b = max(range(config.num_stages), key=lambda k: (memory_list[k], -k))
+            print("\nmax allocated memory = {:.2f} MB".format(max(memory_list)))
+            for i in range(config.num_stages):
+                print((" * " if i == b else "") + memory_strings[i])
+            print(" ")
+
+    def _memory_breakdown(self, r, num_stages_behind):
+        """The 6-tuple of predict_stage_memory(breakdown=True) (aceso_cost_model.py:517-537)."""
+        args = self.settings
+        memory_weights = r[R_WEIGHTS]
+        memory_gradients = memory_weights
+        memory_main_params = memory_weights * args.memory_main_params
+        memory_optimizer = memory_weights * args.memory_optimizer
+        inputs, activations, saved, peak = r[R_INPUTS], r[R_ACT], r[R_SAVED], r[R_PEAK]
+        memory_reserved = r[R_RESERVED] if args.consider_reserved_space else 0
+        memory_activations = (inputs + activations - saved) * (num_stages_behind)
+        memory_peak = inputs + activations - saved + peak
+        memory_weights += memory_main_params
+        return memory_weights, memory_gradients, memory_optimizer, memory_activations, memory_peak, memory_reserved
+
+    # ---- the reference's function set --------------------------------------------------------------
+    def predict_time_breakdown(self, config, print_time=False, print_memory=False):
+        """aceso_cost_model.py:541: writes time_list, memory_list, ... onto `config`."""
+        batch = self.encode([config])
+        it, pk, fe, st, rec = self.evaluator.score_host(batch, breakdown=True)
+        self._raise_for_status(st)
+        self._fill_breakdown(config, rec[0], print_time, print_memory)
+
+    def _locate(self, ops: Sequence[str]) -> int:
+        """First position at which `ops` occurs as a contiguous slice of the model's op sequence."""
+        n = len(ops)
+        key = (ops[0], n, ops[-1])
+        lo = self._slice_cache.get(key)
+        full = self.graph.ops
+        if lo is not None and full[lo:lo + n] == list(ops):
+            return lo
+        for lo in self._first_pos.get(ops[0], ()):
+            if lo + n <= len(full) and full[lo:lo + n] == list(ops):
+                self._slice_cache[key] = lo
+                return lo
+        raise ValueError("the op list is not a contiguous slice of the model's op sequence")
+
+    def _stage_records(self, queries) -> np.ndarray:
+        """One GPU launch for single-stage queries [(ops, recompute_ops, tp, dp, micro_bs, num_stages_behind, algo)];
+        returns the stage records [len(queries), STAGE_REC].  Cross-node flags are off, as in
+        predict_stage_time (aceso_cost_model.py:494-495)."""
+        tb = self.tables
+        N, A = self.graph.num_ops, self.db.n_algo
+        tp_index = {t: k for k, t in enumerate(self.db.tp_list)}
+        P = len(queries)
+        codes = np.zeros((P, N), dtype=np.uint8)
+        hdr = np.zeros((P, 4), dtype=np.uint32)
+        ranges = np.zeros((P, 2), dtype=np.uint32)
+        for p, (ops, rc, tp, dp, micro_bs, nsb, algo) in enumerate(queries):
+            n = len(ops)
+            if n == 0:
+                raise ValueError("empty stage")
+            lo = self._locate(ops)
+            for d in set(dp):
+                self._mbs_index[micro_bs // d]          # KeyError like aceso_cost_model.py:22-25
+            bidx = self._mbs_index[micro_bs]
+            g = tp[0] * dp[0]
+            if g & (g - 1) or any(t * d != g for t, d in zip(tp, dp)):
+                raise ValueError("a stage's tp*dp must be one power of two")
+            if not 0 <= nsb < MAX_STAGES:
+                raise ValueError("num_stages_behind outside 0..15")
+            t = np.array([tp_index[x] for x in tp], dtype=np.uint8)
+            al = np.asarray(algo, dtype=np.uint8)
+            r = (np.asarray(rc) == 1).astype(np.uint8)
+            codes[p, lo:lo + n] = (t * A + al) | (r << 3)
+            codes[p, lo] |= 1 << 4
+            hdr[p, 0] = (nsb + 1) | (bidx << 8)
+            hdr[p, 1] = g.bit_length() - 1
+            ranges[p] = (lo, lo + n)
+        it, pk, fe, st, rec = self.evaluator.score_host(PlanBatch(codes, hdr), breakdown=True, ranges=ranges)
+        self._raise_for_status(st)
+        return rec[:, 0, :]
+
+    def predict_stage_time(self, ops, recompute_ops, tp_size, dp_size, base_batch_size, algo_list,
+                           delta=False, on_the_right=False, decrease=True):
+        """aceso_cost_model.py:493-512 (ms; cross-node bandwidth never used here)."""
+        if len(ops) == 0:
+            return 0 / 1000
+        r = [float(x) for x in self._stage_records([(ops, recompute_ops, tp_size, dp_size, base_batch_size, 0, algo_list)])[0]]
+        fwd_comp, bwd_comp, in_comm, out_comm, recomp_time = r[R_FWD], r[R_BWD], r[R_IN_COMM], r[R_OUT_COMM], r[R_RECOMP]
+        if not delta:
+            sum_time = fwd_comp + bwd_comp + in_comm + out_comm + recomp_time
+        elif on_the_right == decrease:
+            sum_time = fwd_comp + bwd_comp - in_comm + out_comm + recomp_time
+        else:
+            sum_time = fwd_comp + bwd_comp + in_comm - out_comm + recomp_time
+        return sum_time / 1000
+
+    def predict_stage_memory(self, ops, recompute_ops, tp_size, dp_size, base_batch_size, num_stages_behind,
+                             algo_list, breakdown=False):
+        """aceso_cost_model.py:514-539 (MB)."""
+        r = [float(x) for x in self._stage_records([(ops, recompute_ops, tp_size, dp_size, base_batch_size,
+                                                      num_stages_behind, algo_list)])[0]]
+        mw, mg, mo, ma, mp, mr = self._memory_breakdown(r, num_stages_behind)
+        if breakdown:
+            return mw, mg, mo, ma, mp, mr
+        return mw + mg + mo + ma + mp + mr
+
+    def get_reserved_memory_list(self, config):
+        """aceso_cost_model.py:674-691."""
+        if config is None:
+            return []
+        qs = [(st.ops, st.recompute_ops, st.tp_size, st.dp_size, config.micro_bs, st.num_stages_behind, st.algo)
+              for st in config.stages]
+        rec = self._stage_records(qs)
+        return [float(rec[i, R_RESERVED]) if self.settings.consider_reserved_space else 0 for i in range(len(qs))]
+
+    def get_activation_size(self, op_name, mbs, tp, algo_index=0):
+        """aceso_cost_model.py:487-491: one raw table entry."""
+        return float(self.db.tables["activations"][self._type_index[op_name], self._mbs_index[mbs],
+                                                    int(math.log(tp, 2)), algo_index])
+
+    def predict_stage_memory_helper(self, config, stage_index, ops=None, recompute_ops=None, tp_size=None,
+                                    dp_size=None, base_batch_size=None, num_stages_behind=None, algo_list=None):
+        """aceso_cost_model.py:747-767 (memo with the reference's key)."""
+        if ops is None:
+            st = config.stages[stage_index]
+            ops, recompute_ops, tp_size, dp_size = st.ops, st.recompute_ops, st.tp_size, st.dp_size
+            base_batch_size = getattr(st, "base_bs", config.micro_bs)
+            algo_list, num_stages_behind = st.algo, st.num_stages_behind
+        key = f"ops{ops[0]}{len(ops)}tp{tp_size}dp{dp_size}rc{recompute_ops}algo{algo_list}bs{base_batch_size}stage{num_stages_behind}"
+        self.stage_memory_visit += 1
+        if self.stage_memory_set.get(key) is not None:
+            self.stage_memory_hit += 1
+            return self.stage_memory_set[key]
+        v = self.predict_stage_memory(ops, recompute_ops, tp_size, dp_size, base_batch_size, num_stages_behind, algo_list)
+        self.stage_memory_set[key] = v
+        return v
+
+    def predict_stage_time_helper(self, config, stage_index):
+        """aceso_cost_model.py:773-791."""
+        st = config.stages[stage_index]
+        key = f"ops{st.ops[0]}{len(st.ops)}tp{st.tp_size}dp{st.dp_size}rc{st.recompute_ops}algo{st.algo}bs{config.micro_bs}"
+        self.stage_time_visit += 1
+        if self.stage_time_set.get(key) is not None:
+            self.stage_time_hit += 1
+            return self.stage_time_set[key]
+        v = self.predict_stage_time(st.ops, st.recompute_ops, st.tp_size, st.dp_size, config.micro_bs, st.algo)
+        self.stage_time_set[key] = v
+        return v
+
+    def _next_recompute_op_group(self, ops, op_groups, exceed_memory):
+        """aceso_cost_model.py:794-820."""
+        best_size, best_name = 0, None
+        flags = self.graph.flags
+        for name, g in op_groups.items():
+            if (not g["recomputed"] and g["sum_size"] > best_size and
+                    not (int(flags[self._type_index[name]]) & og.F_NO_RECOMPUTE)):
+                best_size, best_name = g["sum_size"], name
+        if best_size == 0:
+            return None, None
+        g = op_groups[best_name]
+        g["recomputed"] = True
+        nxt = g["index"][0] + 1
+        if nxt >= len(ops):
+            return None, None
+        op_groups[ops[nxt]]["recomputed"] = True
+        if best_size < exceed_memory:
+            return g["index"], g["activation_size"]
+        saved_size, index = 0, 0
+        while saved_size <= exceed_memory and index < len(g["activation_size"]):
+            saved_size += g["activation_size"][index]
+            index += 1
+        return list(g["index"][:index]), list(g["activation_size"][:index])
+
+    def check_recompute(self, ops, base_batch_size, tp_size, dp_size, num_stages_behind, algo_list):
+        """Greedy choice of recomputed ops until the stage fits the memory limit
+        (aceso_cost_model.py:822-872).  The loop runs here; stage memory and the saved / peak
+        activations of each trial come from the GPU."""
+        args = self.settings
+        num_ops = len(ops)
+        if not args.flex_recompute:
+            return [1 for _ in range(num_ops)]
+        recompute_ops = [0 for _ in range(num_ops)]
+        stage_memory = self.predict_stage_memory_helper(None, None, ops, recompute_ops, tp_size, dp_size,
+                                                        base_batch_size, num_stages_behind, algo_list)
+        stage_memory += args.peak_mem_in_backward
+        if stage_memory - args.memory_limit <= 0:
+            return recompute_ops
+        op_groups = {}
+        for index in range(num_ops):
+            g = op_groups.setdefault(ops[index], {"index": [], "activation_size": [], "recomputed": False, "sum_size": 0})
+            g["index"].append(index)
+            sz = self.get_activation_size(ops[index], base_batch_size // dp_size[index], tp_size[index],
+                                          algo_list[index]) * (num_stages_behind + 1)
+            g["activation_size"].append(sz)
+            g["sum_size"] += sz
+        initial_saved = 0
+        current_peak = 0        # get_peak_activations of an all-zero recompute list is 0 (:421)
+        while stage_memory - args.memory_limit > 0:
+            idx_group, _ = self._next_recompute_op_group(ops, op_groups, stage_memory - args.memory_limit)
+            if idx_group is None:
+                break
+            for si in idx_group:
+                if si < 0:
+                    break
+                recompute_ops[si] = 1
+                if si < num_ops - 1:
+                    recompute_ops[si + 1] = 1
+            r = self._stage_records([(ops, recompute_ops, tp_size, dp_size, base_batch_size, num_stages_behind, algo_list)])[0]
+            new_saved, new_peak = float(r[R_SAVED]), float(r[R_PEAK])
+            stage_memory -= (new_saved - initial_saved) * (num_stages_behind + 1)
+            initial_saved = new_saved
+            stage_memory += (new_peak - current_peak)
+            current_peak = new_peak
+        return recompute_ops
+
+    def update_recompute(self, config, stage_idx=None):
+        """aceso_cost_model.py:874-883."""
+        for k in ([stage_idx] if stage_idx is not None else range(config.num_stages)):
+            st = config.stages[k]
+            st.recompute_ops = self.check_recompute(st.ops, config.micro_bs, st.tp_size, st.dp_size,
+                                                    st.num_stages_behind, st.algo)
+
+    def predict_value_after_move(self, config, bottleneck, partner, num_ops_moved, metric, inc_gpus=False,
+                                 dec_gpus=False, dim=None):
+        """aceso_cost_model.py:693-739."""
+        st = config.stages[bottleneck]
+        ops, tp_size, dp_size = list(st.ops), list(st.tp_size), list(st.dp_size)
+        algo_list, recompute_ops = list(st.algo), list(st.recompute_ops)
+        if num_ops_moved > 0:
+            sl = slice(None, -num_ops_moved) if bottleneck < partner else slice(num_ops_moved, None)
+            ops, tp_size, dp_size, algo_list = ops[sl], tp_size[sl], dp_size[sl], algo_list[sl]
+        if inc_gpus:
+            if dim == "tp":
+                tp_size = [t * 2 for t in tp_size]
+            elif dim == "dp":
+                dp_size = [d * 2 for d in dp_size]
+        if dec_gpus:
+            if dim == "tp":
+                tp_size = [t // 2 for t in tp_size]
+            elif dim == "dp":
+                dp_size = [d // 2 for d in dp_size]
+        if num_ops_moved > 0 or inc_gpus or dec_gpus:
+            recompute_ops = self.check_recompute(ops, config.micro_bs, tp_size, dp_size, st.num_stages_behind, algo_list)
+        if metric in ["time", "time_with_efficiency"]:
+            value = self.predict_stage_time(ops, recompute_ops, tp_size, dp_size, config.micro_bs, algo_list)
+        elif metric == "memory":
+            value = self.predict_stage_memory(ops, recompute_ops, tp_size, dp_size, config.micro_bs,
+                                              st.num_stages_behind, algo_list)
+        else:
+            raise RuntimeError(f"metric {metric} not implemented.")
+        return value, recompute_ops
+
+    def wrap_predict_delta_time(self, config, longest_stage, shortest_stage, num_ops_moved, decrease=True):
+        """aceso_cost_model.py:885-922."""
+        st = config.stages[longest_stage]
+        num_ops = len(st.ops)
+        if longest_stage == shortest_stage:
+            raise RuntimeError("")
+        right = longest_stage < shortest_stage
+        sl = slice(num_ops - num_ops_moved, None) if right else slice(0, num_ops_moved)
+        ops, algo_list = st.ops[sl], st.algo[sl]
+        if decrease:
+            recompute_ops, tp_size, dp_size = list(st.recompute_ops[sl]), st.tp_size[sl], st.dp_size[sl]
+        else:
+            nb = config.stages[longest_stage + 1] if right else config.stages[longest_stage - 1]
+            recompute_ops = [0 for _ in range(num_ops_moved)]
+            tp_size = [nb.tp_size[0] if right else nb.tp_size[-1] for _ in range(num_ops_moved)]
+            dp_size = [nb.dp_size[0] if right else nb.dp_size[-1] for _ in range(num_ops_moved)]
+        return self.predict_stage_time(ops, recompute_ops, tp_size, dp_size, config.micro_bs, algo_list,
+                                       delta=True, on_the_right=right, decrease=decrease)
+
+
+# ---- module-level API with the reference's names -------------------------------------------------
+args = None
+_model: Optional[CostModel] = None
+
+
+def configure(new_args, device="cuda:0"):
+    """Give the module the argparse namespace the reference reads at import (aceso_cost_model.py:10)."""
+    global args, _device
+    args = new_args
+    _device = device
+
+
+_device = "cuda:0"
+
+
+def _m() -> CostModel:
+    if _model is None:
+        raise RuntimeError("read_profiled_time() has not been called")
+    return _model
+
+
+def read_profiled_time(model_name, model_size, time_path):
+    """aceso_cost_model.py:27: load the profile database; returns the number of op types."""
+    global _model
+    if args is None:
+        raise RuntimeError("call configure(args) first")
+    if _model is not None:
+        _model.close()
+    _model = CostModel.from_directory(args, model_name, model_size, time_path, device=_device)
+    return len(_model.db.op_names)
+
+
+def predict_time_breakdown(config, print_time=False, print_memory=False):
+    return _m().predict_time_breakdown(config, print_time, print_memory)
+
+
+def predict_time_breakdown_batch(configs):
+    return _m().predict_time_breakdown_batch(configs)
+
+
+def predict_stage_time(ops, recompute_ops, tp_size, dp_size, base_batch_size, algo_list, delta=False,
+                       on_the_right=False, decrease=True):
+    return _m().predict_stage_time(ops, recompute_ops, tp_size, dp_size, base_batch_size, algo_list, delta,
+                                   on_the_right, decrease)
+
+
+def predict_stage_memory(ops, recompute_ops, tp_size, dp_size, base_batch_size, num_stages_behind, algo_list,
+                         breakdown=False):
+    return _m().predict_stage_memory(ops, recompute_ops, tp_size, dp_size, base_batch_size, num_stages_behind,
+                                     algo_list, breakdown)
+
+
+def predict_value_after_move(config, bottleneck, partner, num_ops_moved, metric, inc_gpus=False, dec_gpus=False, dim=None):
+    return _m().predict_value_after_move(config, bottleneck, partner, num_ops_moved, metric, inc_gpus, dec_gpus, dim)
+
+
+def wrap_predict_delta_time(config, longest_stage, shortest_stage, num_ops_moved, decrease=True):
+    return _m().wrap_predict_delta_time(config, longest_stage, shortest_stage, num_ops_moved, decrease)
+
+
+def predict_stage_time_helper(config, stage_index):
+    return _m().predict_stage_time_helper(config, stage_index)
+
+
+def predict_stage_memory_helper(config, stage_index, ops=None, recompute_ops=None, tp_size=None, dp_size=None,
+                                base_batch_size=None, num_stages_behind=None, algo_list=None):
+    return _m().predict_stage_memory_helper(config, stage_index, ops, recompute_ops, tp_size, dp_size,
+                                            base_batch_size, num_stages_behind, algo_list)
+
+
+def check_recompute(ops, base_batch_size, tp_size, dp_size, num_stages_behind, algo_list):
+    return _m().check_recompute(ops, base_batch_size, tp_size, dp_size, num_stages_behind, algo_list)
+
+
+def update_recompute(config, stage_idx=None):
+    return _m().update_recompute(config, stage_idx)
+
+
+def get_reserved_memory_list(config):
+    return _m().get_reserved_memory_list(config)
+
+
+def get_activation_size(op_name, mbs, tp, algo_index=0):
+    return _m().get_activation_size(op_name, mbs, tp, algo_index)

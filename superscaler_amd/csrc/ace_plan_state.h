@@ -210,7 +210,8 @@ template <bool BD, bool RANGED> struct PlanState {
             ace_d2 ie = lds.ld<ace_d2>(prevrow + g.out_off + iidx * 16u);
             r[ACE_R_IDEAL_FWD] = id_fwd; r[ACE_R_IDEAL_BWD] = id_bwd; r[ACE_R_IDEAL_IN] = id_in;
             r[ACE_R_IDEAL_OUT] = out_cross ? ie.y : ie.x;
-            r[ACE_R_STAGE_MS] = t; r[ACE_R_STAGE_MB] = mem; r[ACE_R_SPARE] = 0.0;
+            r[ACE_R_STAGE_MS] = t; r[ACE_R_STAGE_MB] = mem;
+            r[ACE_R_RESHARD] = rs_f * 1000.0 + rs_b * 1000.0;   // print-only "reshard" column (:355)
         }
     }
 

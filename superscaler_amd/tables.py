@@ -44,7 +44,7 @@ LDS_BYTES = 160 * 1024
 F_RESHARDING, F_RESERVED_MIN, F_NO_RESERVED = 1, 2, 4
 
 (R_FWD, R_BWD, R_IN_COMM, R_OUT_COMM, R_RECOMP, R_WEIGHTS, R_INPUTS, R_ACT, R_SAVED, R_PEAK,
- R_RESERVED, R_IDEAL_FWD, R_IDEAL_BWD, R_IDEAL_IN, R_IDEAL_OUT, R_STAGE_MS, R_STAGE_MB, R_SPARE) = range(18)
+ R_RESERVED, R_IDEAL_FWD, R_IDEAL_BWD, R_IDEAL_IN, R_IDEAL_OUT, R_STAGE_MS, R_STAGE_MB, R_RESHARD) = range(18)
 
 
 class AceTablesStruct(ctypes.Structure):

@@ -166,3 +166,28 @@ def test_full_size_properties(torch_mod):
     _, _, fe_hi, _ = ev.score_host(batch, memory_limit=160000.0)
     assert (fe_lo <= fe).all() and (fe <= fe_hi).all()
     ev.close()
+
+
+def test_known_answers_single_gpu_plans(golden_dir, torch_mod):
+    """The reference tree's own single-GPU plans and published predictions
+    (results/ref/perf_model_{time,mem}_large_{gpt,resnet}.csv), through the GPU path."""
+    from superscaler_amd import aceso_cost_model as acm
+    from superscaler_amd.plan import config_from_json
+    kat = os.path.join(golden_dir, "kat") + "/"
+    st = CostModelSettings(model_name="gpt", micro_batch_size=[1, 2, 4, 8], num_gpus_per_node=1, global_batch_size=1024)
+    m = acm.CostModel.from_directory(st, "gpt", "350M", kat, num_layers=24)
+    cfg = config_from_json(kat + "gpt_350M_mbs8_recomp.json", m.graph.ops)
+    m.predict_time_breakdown(cfg)
+    assert f"{max(cfg.time_list) / 1000:.2f}" == "200.71"
+    assert abs(max(cfg.time_list) - 200712.935038) < 1e-5
+    reserved = m.get_reserved_memory_list(cfg)
+    assert reserved == [5120.0] and abs(cfg.memory_list[0] - 19712.64) < 1e-6
+    m.close()
+    st = CostModelSettings(model_name="resnet", micro_batch_size=[16, 32, 48, 64], num_gpus_per_node=1, global_batch_size=1536)
+    m = acm.CostModel.from_directory(st, "resnet", "500M", kat)
+    cfg = config_from_json(kat + "resnet_500M_mbs64_recomp.json", m.graph.ops)
+    m.predict_time_breakdown(cfg)
+    reserved = m.get_reserved_memory_list(cfg)
+    assert reserved == [3432.0] and int(cfg.memory_list[0] - reserved[0]) == 16519
+    assert abs(max(cfg.time_list) / 1000 - 67.13) / 67.13 < 0.005
+    m.close()

@@ -17,6 +17,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per plan of one scoring-kernel launch on the default workload, from two rocprofv3 --pmc
+# runs (FETCH_SIZE, then WRITE_SIZE) scaled by the readings of a plain 256 MiB copy in the same
+# runs (factors 2.000 and 1.000): 1,266 B read + 844 B written.  See profiles/.
+MEASURED_TRAFFIC_BYTES_PER_PLAN = {("gpt3_13b", 523): 2110.0}
 
 
 def cpu_baseline(tables, batch, budget_s=15.0):
@@ -24,7 +28,7 @@ def cpu_baseline(tables, batch, budget_s=15.0):
     over as many plans of the same batch as fit the time budget."""
     from tests.helpers import oracle_config, oracle_for
     orc = oracle_for(tables)
-    cfgs = [oracle_config(batch, p, tables) for p in range(min(batch.n_plans, 4096))]
+    cfgs = [oracle_config(batch, p, tables) for p in range(min(batch.n_plans, 16384))]
     for c in cfgs[:8]:
         orc.score(c)
     t0 = time.perf_counter()
@@ -48,6 +52,9 @@ def main():
     ap.add_argument("--plans", type=int, default=None)
     ap.add_argument("--topk", type=int, default=64)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibration-copy-mib", type=int, default=0,
+                    help="also run one plain device-to-device copy of this many MiB (a kernel of known "
+                         "traffic, to scale FETCH_SIZE / WRITE_SIZE counter readings)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this evaluator runs on ONE GPU (plans are independent; device counts of the plans "
@@ -109,12 +116,21 @@ def main():
                    "step": "score kernel + device-wide top-k, inputs resident in HBM",
                    "feasible_plans": n_feasible, "best_iter_ms": best, "plan_generation_s": round(gen_s, 1)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
-                     "kernel": "ace_score_kernel<false>", "kernel_ms": kern_ms,
+                     "frac": achieved / HBM_PEAK_GBPS,
+                     "traffic": (MEASURED_TRAFFIC_BYTES_PER_PLAN[(w.name, N)] * P
+                                 if (w.name, N) in MEASURED_TRAFFIC_BYTES_PER_PLAN else None),
+                     "algorithmic_bytes": algo_bytes,
+                     "kernel": "ace_score_kernel<BD=false,RANGED=false,WIN=false,DEFER=true>", "kernel_ms": kern_ms,
                      "algorithmic_bytes_per_plan": 3 * N + 19,
                      "bytes_moved_per_plan": d.bytes_moved_per_plan + 17,
                      "achieved_on_bytes_moved": moved_bytes / (kern_ms * 1e-3) / 1e9},
     }
+    if args.calibration_copy_mib > 0:
+        src = torch.zeros(args.calibration_copy_mib << 20, dtype=torch.uint8, device="cuda:0")
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        out["config"]["calibration_copy_bytes"] = int(src.numel())
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(tables, batch)
     ev.close()

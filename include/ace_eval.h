@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define ACE_ABI_VERSION 1
+#define ACE_ABI_VERSION 2
 #define ACE_MAX_STAGES 16      /* aceso_utils.py:502: end_num_stages = min(num_gpus, 16) */
 #define ACE_STAGE_REC 18       /* doubles per stage record, see ACE_R_* */
 
@@ -76,6 +76,7 @@ typedef struct ace_tables {
     int32_t n_pair_kinds;   /* distinct adjacent-op spec pairings */
     int32_t row_doubles;    /* doubles per type row (even) */
     int32_t hot_off, start_off, out_off, z_off;   /* sub-table offsets inside a row, in doubles */
+    int32_t z_table_doubles; /* doubles per resharding cost table (power of two >= n_diag * C) */
     int32_t n_windows;      /* >= 1; > 1 when the rows do not all fit in LDS */
     int32_t lds_row_bytes;  /* bytes of LDS reserved for resident rows */
     int32_t flags;          /* ACE_F_* */
@@ -83,10 +84,11 @@ typedef struct ace_tables {
     const double *rows;            /* [num_types][row_doubles] */
     const uint32_t *pos_info;      /* [num_ops + 1][2]: row LDS offset / 16 | previous op's row offset / 16 << 16;
                                       pair kind | flags << 8 */
-    const uint8_t *pair_kinds;     /* [n_pair_kinds][n_glog][C][C], C = n_tp * n_algo */
-    const uint32_t *stage_lut;     /* [n_mbs][16]: diag | per-tp mbs-index nibbles << 8 */
+    const uint8_t *pair_kinds;     /* [n_pair_kinds][n_glog][8][8] (previous code, this code) */
+    const uint32_t *stage_lut;     /* [n_mbs][16][2]: hot byte offset of the diag | pair-kind offset << 16;
+                                      diag * C | per-tp mbs-index nibbles << 16 (C = n_tp * n_algo) */
     const double *nb_minus_1;      /* [n_mbs]: global_bs // micro_bs - 1 */
-    const int32_t *win_pos;        /* [n_windows + 1] first position of each window (multiples of 16) */
+    const int32_t *win_pos;        /* [n_windows + 1] first position of each window (multiples of 4) */
     const int32_t *win_row_begin;  /* [n_windows + 1] into win_rows */
     const uint32_t *win_rows;      /* [..][2]: type id, LDS byte offset */
 } ace_tables_t;

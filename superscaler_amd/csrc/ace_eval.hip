@@ -43,13 +43,14 @@ struct AceKernelArgs {
     const uint8_t *pair_kinds;  // -> LDS
     const uint32_t *stage_lut;  // -> LDS
     const double *nbm1;         // [n_mbs]
-    const int32_t *win_pos;     // [n_windows + 1], multiples of 16
+    const int32_t *win_pos;     // [n_windows + 1], multiples of 4
     const int32_t *win_row_begin;
     const uint32_t *win_rows;   // pairs (type, lds byte offset)
     int32_t n_windows, row_doubles, rk_bytes, stg_words;
     double *iter_ms, *peak_mb;
     uint8_t *feasible, *status;
     double *stage_out;
+    double *stage_ws;           // [ceil(P / kBlock) * kBlock][ACE_MAX_STAGES][ACE_WS_REC] for deferred stage tails
 };
 
 // Copy the rows window `w` needs from global memory into LDS (whole workgroup).
@@ -66,8 +67,11 @@ __device__ __forceinline__ void stage_window(const AceKernelArgs &a, unsigned ch
 
 // BD: also write per-stage records.  RANGED: each plan is one stage over an op sub-range.
 // WIN: the rows of all op types do not fit in LDS together; restage at window boundaries.
-template <bool BD, bool RANGED, bool WIN>
+// DEFER: stage tails are stashed in the workspace and evaluated after the op loop, when all lanes
+// are active again (needs every row resident, so never together with WIN).
+template <bool BD, bool RANGED, bool WIN, bool DEFER>
 __global__ __launch_bounds__(kBlock) void ace_score_kernel(const AceKernelArgs a) {
+    static_assert(!DEFER || (!BD && !RANGED && !WIN), "deferred stage tails: plain scoring only");
     extern __shared__ __align__(16) unsigned char lds_raw[];
     const AceGeom &g = a.g;
     const int tid = threadIdx.x;
@@ -83,13 +87,14 @@ __global__ __launch_bounds__(kBlock) void ace_score_kernel(const AceKernelArgs a
     __syncthreads();
 
     AceLds lds{lds_raw};
-    PlanState<BD, RANGED> st;
+    PlanState<BD, RANGED, DEFER> st;
     const ace_u4 h = a.hdr[pl];
     ace_u2 range{0u, 0u};
     if (RANGED) range = a.range[pl];
     st.init(g, lds, h, range);
     const double nbm1 = a.nbm1[st.bidx];
     double *rec = (BD && a.stage_out && active) ? a.stage_out + (size_t)plan * (ACE_MAX_STAGES * ACE_STAGE_REC) : nullptr;
+    if (DEFER) rec = a.stage_ws + (size_t)plan * (ACE_MAX_STAGES * ACE_WS_REC);   // padded lanes own a slot too
 
     int w = 0;
     int next_win = WIN ? a.win_pos[0] : 0x7fffffff;
@@ -103,28 +108,41 @@ __global__ __launch_bounds__(kBlock) void ace_score_kernel(const AceKernelArgs a
             if (q) cw = nxt;
             const int grp = (q >> 2) + 1;
             if (grp < g.G) nxt = a.codes[(size_t)grp * g.P + pl];
-            if (WIN && base == next_win) {
-                // every lane of the workgroup reaches this point together
-                __syncthreads();
-                stage_window(a, lds_raw, w, tid);
-                __syncthreads();
-                ++w;
-                next_win = a.win_pos[w];
-            }
+        }
+        if (WIN && base == next_win) {
+            // every lane of the workgroup reaches this point together
+            __syncthreads();
+            stage_window(a, lds_raw, w, tid);
+            __syncthreads();
+            ++w;
+            next_win = a.win_pos[w];
         }
         const uint32_t word = cw.x;
         cw.x = cw.y; cw.y = cw.z; cw.z = cw.w;
+        // the four position descriptors of this quad in one scalar load (the array is padded)
+        const ace_u4 ia = reinterpret_cast<const ace_u4 *>(a.pos_info)[2 * q];
+        const ace_u4 ib = reinterpret_cast<const ace_u4 *>(a.pos_info)[2 * q + 1];
+        const ace_u2 infos[4] = {{ia.x, ia.y}, {ia.z, ia.w}, {ib.x, ib.y}, {ib.z, ib.w}};
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            const int i = base + k;
-            if (i < g.N) {
+            if (base + k < g.N) {
                 const uint32_t byte = (word >> (8 * k)) & 0xffu;
-                st.step(g, lds, i, byte, pbyte, a.pos_info[i], rec);
+                st.step(g, lds, base + k, byte, pbyte, infos[k], rec);
                 pbyte = byte;
             }
         }
     }
-    if (!RANGED || !st.done) st.finish(g, lds, info_prevrow(a.pos_info[g.N]), pbyte & 7u, rec);
+    if (DEFER) {
+        st.stash(rec, (uint32_t)(g.N - 1), pbyte & 7u);
+        const int n_st = st.s + 1;
+        for (int s2 = 0; s2 < ACE_MAX_STAGES; ++s2) {
+            const bool live = s2 < n_st;
+            if (!__any(live)) break;
+            if (live) st.replay(g, lds, a.pos_info, rec, s2);
+        }
+    } else if (!RANGED || !st.done) {
+        st.finish(g, lds, info_prevrow(a.pos_info[g.N]), pbyte & 7u, rec);
+    }
     double iter, peak;
     uint8_t feas, stat;
     st.result(g, nbm1, iter, peak, feas, stat);
@@ -368,6 +386,8 @@ struct ace_handle {
     double *d_nbm1;
     int32_t *d_win_pos, *d_win_row_begin;
     uint32_t *d_win_rows;
+    double *d_stage_ws;        // grow-only workspace for deferred stage tails
+    size_t stage_ws_plans;     // capacity in plans
 };
 
 extern "C" {
@@ -400,8 +420,8 @@ static int upload(void **dst, const void *src, size_t bytes, size_t alloc_bytes 
 
 }  // extern "C"
 
-template <bool BD, bool RANGED, bool WIN> static int allow_big_lds() {
-    ACE_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&ace_score_kernel<BD, RANGED, WIN>),
+template <bool BD, bool RANGED, bool WIN, bool DEFER> static int allow_big_lds() {
+    ACE_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&ace_score_kernel<BD, RANGED, WIN, DEFER>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
     return ACE_OK;
 }
@@ -414,7 +434,7 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     if (t->abi_version != ACE_ABI_VERSION) return ACE_EVERSION;
     if (t->num_ops <= 0 || t->num_types <= 0 || t->n_mbs <= 0 || t->n_mbs > 15 || t->n_tp <= 0 || t->n_tp > 4 ||
         (t->n_algo != 1 && t->n_algo != 2) || t->n_diag <= 0 || t->n_diag > 254 || t->n_glog <= 0 || t->n_glog > 16 ||
-        t->n_z < 2 || t->n_z > 15 || t->n_pair_kinds <= 0 || t->n_pair_kinds > 255 || t->row_doubles <= 0 ||
+        t->n_z < 0 || t->n_z == 1 || t->n_z > 15 || ((t->flags & ACE_F_RESHARDING) && t->n_z < 2) || t->z_table_doubles <= 0 || (t->z_table_doubles & (t->z_table_doubles - 1)) || t->n_pair_kinds <= 0 || t->n_pair_kinds > 255 || t->row_doubles <= 0 ||
         (t->row_doubles & 1) || t->n_windows <= 0 || t->lds_row_bytes <= 0 || (t->lds_row_bytes & 15) ||
         !t->rows || !t->pos_info || !t->pair_kinds || !t->stage_lut || !t->nb_minus_1 || !t->win_pos ||
         !t->win_row_begin || !t->win_rows)
@@ -424,25 +444,26 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     const int64_t hot_end = (int64_t)t->hot_off + (int64_t)t->n_diag * C * 6;
     const int64_t start_end = (int64_t)t->start_off + (int64_t)t->n_diag * C * 4;
     const int64_t out_end = (int64_t)t->out_off + (int64_t)t->n_mbs * t->n_tp * t->n_algo * 2;
-    const int64_t z_end = (int64_t)t->z_off + (int64_t)t->n_z * t->n_diag * C;
+    const int64_t z_end = (int64_t)t->z_off + (int64_t)t->n_z * t->z_table_doubles;
+    if (t->z_table_doubles < t->n_diag * C) return ACE_EINVAL;
     if ((t->hot_off & 1) || (t->start_off & 1) || (t->out_off & 1) || (t->z_off & 1) || t->hot_off < 0 ||
         t->start_off < 0 || t->out_off < 0 || t->z_off < 0 ||
         hot_end > t->row_doubles || start_end > t->row_doubles || out_end > t->row_doubles || z_end > t->row_doubles)
         return ACE_EINVAL;
     const int64_t row_bytes = (int64_t)t->row_doubles * 8;
     if (row_bytes > t->lds_row_bytes || t->lds_row_bytes > (int32_t)kMaxLds) return ACE_ETOOBIG;
-    const int32_t rk_bytes = t->n_pair_kinds * t->n_glog * C * C;
-    const int32_t stg_words = t->n_mbs * 16;
+    const int32_t rk_bytes = t->n_pair_kinds * t->n_glog * 64;
+    const int32_t stg_words = t->n_mbs * 16 * 2;
     const uint32_t rk_off = (uint32_t)t->lds_row_bytes;
     const uint32_t stg_off = (rk_off + (uint32_t)rk_bytes + 15u) & ~15u;
     const uint32_t lds_bytes = stg_off + (uint32_t)stg_words * 4u;
     if (lds_bytes > kMaxLds) return ACE_ETOOBIG;
-    // window tables: window starts are multiples of 16 ops; every referenced row must fit the
+    // window tables: window starts are multiples of 4 ops; every referenced row must fit the
     // resident region; every position's row offsets must point at a row start inside it
     const int32_t n_win_rows = t->win_row_begin[t->n_windows];
     if (t->win_pos[0] != 0 || t->win_row_begin[0] != 0 || n_win_rows <= 0) return ACE_EINVAL;
     for (int w = 0; w < t->n_windows; ++w) {
-        if (t->win_pos[w + 1] <= t->win_pos[w] || t->win_row_begin[w + 1] < t->win_row_begin[w] || (t->win_pos[w] & 15))
+        if (t->win_pos[w + 1] <= t->win_pos[w] || t->win_row_begin[w + 1] < t->win_row_begin[w] || (t->win_pos[w] & 3))
             return ACE_EINVAL;
     }
     if (t->win_pos[t->n_windows] < t->num_ops) return ACE_EINVAL;
@@ -457,12 +478,16 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
             (pi[1] & 0xffu) >= (uint32_t)t->n_pair_kinds)
             return ACE_EINVAL;
     }
-    for (int j = 0; j < stg_words; ++j) {
-        const uint32_t d = t->stage_lut[j] & 0xffu;
-        if (d != 0xffu && d >= (uint32_t)t->n_diag) return ACE_EINVAL;
+    for (int j = 0; j < stg_words; j += 2) {
+        // (hot offset, diag * C) of every (micro-batch, stage size) pair must address C entries inside the row
+        const int64_t hot_v = t->stage_lut[j] & 0xffffu, rk_v = t->stage_lut[j] >> 16, dc = t->stage_lut[j + 1] & 0xffffu;
+        if ((hot_v & 15) || (int64_t)t->hot_off * 8 + hot_v + (int64_t)C * 48 > row_bytes || dc + C > (int64_t)t->n_diag * C ||
+            (rk_v & 63) || rk_v / 64 >= t->n_glog)
+            return ACE_EINVAL;
     }
     for (int j = 0; j < rk_bytes; ++j) {
-        if ((t->pair_kinds[j] & 15u) >= (uint32_t)t->n_z || (uint32_t)(t->pair_kinds[j] >> 4) >= (uint32_t)t->n_z) return ACE_EINVAL;
+        const uint32_t lim = t->n_z ? (uint32_t)t->n_z : 1u;
+        if ((t->pair_kinds[j] & 15u) >= lim || (uint32_t)(t->pair_kinds[j] >> 4) >= lim) return ACE_EINVAL;
     }
 
     ace_handle *h = new (std::nothrow) ace_handle();
@@ -474,9 +499,10 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     g.n_mbs = t->n_mbs; g.n_tp = t->n_tp; g.n_algo = t->n_algo; g.n_glog = t->n_glog; g.n_pair_kinds = t->n_pair_kinds;
     g.hot_off = (uint32_t)t->hot_off * 8u; g.start_off = (uint32_t)t->start_off * 8u;
     g.out_off = (uint32_t)t->out_off * 8u; g.z_off = (uint32_t)t->z_off * 8u;
-    g.z_stride = (uint32_t)(t->n_diag * C) * 8u;
+    g.z_shift = 3;
+    while ((1 << (g.z_shift - 3)) < t->z_table_doubles) ++g.z_shift;
     g.rk_lds_off = rk_off; g.stg_lds_off = stg_off;
-    g.rk_kind_stride = (uint32_t)(t->n_glog * C * C);
+    g.rk_kind_stride = (uint32_t)(t->n_glog * 64);
     g.flags = t->flags; g.main_params = t->main_params; g.optimizer = t->optimizer;
     g.mem_limit = 0.0; g.strict = 0;
     h->n_windows = t->n_windows; h->row_doubles = t->row_doubles; h->rk_bytes = rk_bytes; h->stg_words = stg_words;
@@ -492,9 +518,10 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
         (rc = upload((void **)&h->d_win_pos, t->win_pos, (size_t)(t->n_windows + 1) * 4)) ||
         (rc = upload((void **)&h->d_win_row_begin, t->win_row_begin, (size_t)(t->n_windows + 1) * 4)) ||
         (rc = upload((void **)&h->d_win_rows, t->win_rows, (size_t)n_win_rows * 8)) ||
-        (rc = allow_big_lds<false, false, false>()) || (rc = allow_big_lds<false, false, true>()) ||
-        (rc = allow_big_lds<true, false, false>()) || (rc = allow_big_lds<true, false, true>()) ||
-        (rc = allow_big_lds<true, true, false>()) || (rc = allow_big_lds<true, true, true>())) {
+        (rc = allow_big_lds<false, false, false, false>()) || (rc = allow_big_lds<false, false, true, false>()) ||
+        (rc = allow_big_lds<false, false, false, true>()) ||
+        (rc = allow_big_lds<true, false, false, false>()) || (rc = allow_big_lds<true, false, true, false>()) ||
+        (rc = allow_big_lds<true, true, false, false>()) || (rc = allow_big_lds<true, true, true, false>())) {
         ace_destroy(h);
         return rc;
     }
@@ -507,6 +534,7 @@ void ace_destroy(ace_handle_t *h) {
     (void)hipFree(h->d_rows); (void)hipFree(h->d_pos_info); (void)hipFree(h->d_pair_kinds);
     (void)hipFree(h->d_stage_lut); (void)hipFree(h->d_nbm1); (void)hipFree(h->d_win_pos);
     (void)hipFree(h->d_win_row_begin); (void)hipFree(h->d_win_rows);
+    if (h->d_stage_ws) (void)hipFree(h->d_stage_ws);
     delete h;
 }
 
@@ -527,6 +555,7 @@ static int fill_args(ace_handle_t *h, const ace_batch_t *b, double memory_limit,
     a->nbm1 = h->d_nbm1; a->win_pos = h->d_win_pos; a->win_row_begin = h->d_win_row_begin; a->win_rows = h->d_win_rows;
     a->n_windows = h->n_windows; a->row_doubles = h->row_doubles; a->rk_bytes = h->rk_bytes; a->stg_words = h->stg_words;
     a->iter_ms = d_iter_ms; a->peak_mb = d_peak_mb; a->feasible = d_feasible; a->status = d_status; a->stage_out = d_stage_out;
+    a->stage_ws = nullptr;
     return ACE_OK;
 }
 
@@ -535,16 +564,35 @@ static int fill_args(ace_handle_t *h, const ace_batch_t *b, double memory_limit,
 template <bool BD, bool RANGED>
 static void launch_score_w(const ace_handle_t *h, const AceKernelArgs &a, hipStream_t s, unsigned blocks) {
     if (h->n_windows > 1)
-        hipLaunchKernelGGL((ace_score_kernel<BD, RANGED, true>), dim3(blocks), dim3(kBlock), h->lds_bytes, s, a);
+        hipLaunchKernelGGL((ace_score_kernel<BD, RANGED, true, false>), dim3(blocks), dim3(kBlock), h->lds_bytes, s, a);
     else
-        hipLaunchKernelGGL((ace_score_kernel<BD, RANGED, false>), dim3(blocks), dim3(kBlock), h->lds_bytes, s, a);
+        hipLaunchKernelGGL((ace_score_kernel<BD, RANGED, false, false>), dim3(blocks), dim3(kBlock), h->lds_bytes, s, a);
 }
 
 static void launch_score(const ace_handle_t *h, const AceKernelArgs &a, hipStream_t s) {
     const unsigned blocks = (unsigned)(((size_t)a.g.P + kBlock - 1) / kBlock);
     if (a.range) launch_score_w<true, true>(h, a, s, blocks);
     else if (a.stage_out) launch_score_w<true, false>(h, a, s, blocks);
+    else if (a.stage_ws)
+        hipLaunchKernelGGL((ace_score_kernel<false, false, false, true>), dim3(blocks), dim3(kBlock), h->lds_bytes, s, a);
     else launch_score_w<false, false>(h, a, s, blocks);
+}
+
+// Plain scoring with every row resident uses the deferred-stage-tail kernel, which needs a
+// per-plan workspace; the handle keeps one and grows it on demand.
+static int ensure_stage_ws(ace_handle_t *h, AceKernelArgs *a) {
+    a->stage_ws = nullptr;
+    if (a->range || a->stage_out || h->n_windows > 1 || h->geom.N >= 65536) return ACE_OK;
+    const size_t need = (((size_t)a->g.P + kBlock - 1) / kBlock) * kBlock;
+    if (need > h->stage_ws_plans) {
+        if (h->d_stage_ws) ACE_HIP(hipFree(h->d_stage_ws));
+        h->d_stage_ws = nullptr;
+        h->stage_ws_plans = 0;
+        ACE_HIP(hipMalloc((void **)&h->d_stage_ws, need * ACE_MAX_STAGES * ACE_WS_REC * sizeof(double)));
+        h->stage_ws_plans = need;
+    }
+    a->stage_ws = h->d_stage_ws;
+    return ACE_OK;
 }
 
 extern "C" {
@@ -554,6 +602,7 @@ int ace_score_batch(ace_handle_t *h, const ace_batch_t *batch, double memory_lim
     AceKernelArgs a;
     int rc = fill_args(h, batch, memory_limit, strict, d_iter_ms, d_peak_mb, d_feasible, d_status, d_stage_out, &a);
     if (rc) return rc;
+    if ((rc = ensure_stage_ws(h, &a))) return rc;
     launch_score(h, a, (hipStream_t)stream);
     ACE_HIP(hipGetLastError());
     return ACE_OK;
@@ -565,6 +614,7 @@ int ace_time_score_kernel(ace_handle_t *h, const ace_batch_t *batch, double memo
     AceKernelArgs a;
     int rc = fill_args(h, batch, memory_limit, strict, d_iter_ms, d_peak_mb, d_feasible, nullptr, nullptr, &a);
     if (rc) return rc;
+    if ((rc = ensure_stage_ws(h, &a))) return rc;
     hipStream_t s = (hipStream_t)stream;
     hipEvent_t e0, e1;
     ACE_HIP(hipEventCreate(&e0));

@@ -56,6 +56,14 @@ ACE_HD double ace_max(double a, double b) {
 }
 #endif
 ACE_HD bool ace_isnan(double a) { return a != a; }
+// product of two values below 2^24 (a single full-rate instruction on the GPU)
+#ifdef ACE_HOST_EMU
+ACE_HD uint32_t ace_mul24(uint32_t a, uint32_t b) { return a * b; }
+ACE_HD double ace_fma(double a, double b, double c) { return std::fma(a, b, c); }
+#else
+ACE_HD uint32_t ace_mul24(uint32_t a, uint32_t b) { return __umul24(a, b); }
+ACE_HD double ace_fma(double a, double b, double c) { return __builtin_fma(a, b, c); }
+#endif
 
 struct alignas(16) ace_d2 { double x, y; };
 struct alignas(16) ace_u4 { uint32_t x, y, z, w; };
@@ -70,9 +78,9 @@ struct AceGeom {
     int32_t C, A_shift;         // codes per diag (n_tp * n_algo), log2(n_algo)
     int32_t n_mbs, n_tp, n_algo, n_glog, n_pair_kinds;
     uint32_t hot_off, start_off, out_off, z_off;   // bytes inside a row
-    uint32_t z_stride;          // bytes of one resharding-cost table inside a row (n_diag * C * 8)
+    uint32_t z_shift;           // log2(bytes of one resharding-cost table inside a row)
     uint32_t rk_lds_off, stg_lds_off;              // LDS byte offsets of the pair-kind and stage LUT regions
-    uint32_t rk_kind_stride;    // bytes of one pair kind (n_glog * C * C)
+    uint32_t rk_kind_stride;    // bytes of one pair kind (n_glog * 64)
     int32_t flags;
     double main_params, optimizer, mem_limit;
     int32_t strict;
@@ -84,7 +92,12 @@ struct AceGeom {
 ACE_HD uint32_t info_row(ace_u2 i) { return (i.x & 0xffffu) << 4; }
 ACE_HD uint32_t info_prevrow(ace_u2 i) { return (i.x >> 16) << 4; }
 
-template <bool BD, bool RANGED> struct PlanState {
+#define ACE_WS_REC 14          // doubles per deferred stage record (see PlanState::stash)
+
+// BD: per-stage records for the caller.  RANGED: one stage over an op sub-range.  DEFER: stage
+// tails are not evaluated where the stage ends (where only the few lanes that cut at this op are
+// active) but stashed to a per-plan workspace and replayed after the op loop with every lane busy.
+template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
     // plan constants
     int S;
     uint32_t bidx;
@@ -94,7 +107,7 @@ template <bool BD, bool RANGED> struct PlanState {
     int lo, hi;                 // RANGED: only ops lo <= i < hi belong to the plan (one stage)
     // stage state
     int s;
-    uint32_t hot_v, z_v, rk_v, mrow;
+    uint32_t hot_v, z_v, rk_v, mrow, dc_v;
     uint32_t t_first;
     bool out_cross;
     double in_comm, inputs, id_in;
@@ -103,6 +116,7 @@ template <bool BD, bool RANGED> struct PlanState {
     double id_fwd, id_bwd;
     bool lastclose;
     bool done;                  // RANGED: the stage was finished inside the op loop
+    uint32_t first_meta;        // DEFER: first op of the current stage: position | code << 16
     // plan accumulators
     double sum_t, max_t, max_mem;
     uint32_t status;
@@ -117,11 +131,11 @@ template <bool BD, bool RANGED> struct PlanState {
         s = -1;
         sum_t = 0.0; max_t = 0.0; max_mem = 0.0;
         status = 0;
-        prev_act = 0.0; lastclose = false; done = false;
+        prev_act = 0.0; lastclose = false; done = false; first_meta = 0;
         fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = pend_rf = pend_rb = rs_f = rs_b = 0.0;
         id_fwd = id_bwd = id_in = 0.0;
         in_comm = inputs = 0.0;
-        hot_v = z_v = rk_v = mrow = t_first = 0;
+        hot_v = z_v = rk_v = mrow = t_first = dc_v = 0;
         out_cross = false;
         ideal_hot_v = ideal_start_v = 0;
         if (bidx >= (uint32_t)g.n_mbs) { status = ACE_PLAN_MALFORMED; bidx = 0; }
@@ -129,33 +143,34 @@ template <bool BD, bool RANGED> struct PlanState {
         if (BD) {
             // the "ideal" pass uses tp = dp = 1 and micro-batch = micro_bs (aceso_cost_model.py:588-590):
             // the diag of (micro_bs, 1 gpu)
-            uint32_t w = lds.ld<uint32_t>(g.stg_lds_off + (bidx * 16u + 0u) * 4u);
-            uint32_t d = w & 0xff;
-            if (d == 0xff) d = 0;
-            ideal_hot_v = d * (uint32_t)g.C * ACE_HOT_STRIDE;
-            ideal_start_v = d * (uint32_t)g.C * ACE_START_STRIDE;
+            ace_u2 w = lds.ld<ace_u2>(g.stg_lds_off + (bidx * 16u + 0u) * 8u);
+            ideal_hot_v = w.x & 0xffffu;
+            ideal_start_v = (w.y & 0xffffu) * ACE_START_STRIDE;
         }
     }
 
-    // Stage head at an op with code `c` whose type row lives at LDS offset `row`.
-    ACE_HD void start(const AceGeom &g, const AceLds &lds, uint32_t row, uint32_t c) {
+    // Stage head, part 1: the per-stage offsets the op loop needs, accumulators back to zero.
+    ACE_HD void start_fast(const AceGeom &g, const AceLds &lds) {
         ++s;
-        uint32_t sidx = (uint32_t)(s < ACE_MAX_STAGES ? s : ACE_MAX_STAGES - 1);
-        if (s >= ACE_MAX_STAGES) status = ACE_PLAN_MALFORMED;
-        uint32_t glog = (uint32_t)(glogs >> (4u * sidx)) & 15u;
-        if (glog >= (uint32_t)g.n_glog) { status |= ACE_PLAN_UNSCORABLE; glog = 0; }
-        uint32_t w = lds.ld<uint32_t>(g.stg_lds_off + (bidx * 16u + glog) * 4u);
-        uint32_t d = w & 0xff;
-        mrow = w >> 8;
-        if (d == 0xff) { status |= ACE_PLAN_UNSCORABLE; d = 0; }
-        uint32_t dc = d * (uint32_t)g.C;
-        hot_v = dc * ACE_HOT_STRIDE;
-        z_v = dc * 8u;
-        rk_v = glog * (uint32_t)(g.C * g.C);
+        // (a plan with more than 16 stage bits is caught by result(): s + 1 != S)
+        uint32_t glog = (uint32_t)(glogs >> (4u * ((uint32_t)s & 15u))) & 15u;
+        ace_u2 w = lds.ld<ace_u2>(g.stg_lds_off + (bidx * 16u + glog) * 8u);
+        hot_v = w.x & 0xffffu;
+        rk_v = w.x >> 16;
+        dc_v = w.y & 0xffffu;
+        mrow = w.y >> 16;
+        z_v = dc_v << 3;
+        fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = pend_rf = pend_rb = rs_f = rs_b = 0.0;
+        lastclose = false;
+    }
+
+    // Stage head, part 2: boundary input of the stage's first op (code `c`, row at LDS offset `row`).
+    ACE_HD void start_lookups(const AceGeom &g, const AceLds &lds, uint32_t row, uint32_t c) {
+        uint32_t sidx = (uint32_t)s & 15u;
         bool in_cross = (cross >> sidx) & 1u;
         out_cross = (cross >> (16u + sidx)) & 1u;
         t_first = c >> g.A_shift;
-        uint32_t a = row + g.start_off + (dc + c) * ACE_START_STRIDE;
+        uint32_t a = row + g.start_off + (dc_v + c) * ACE_START_STRIDE;
         ace_d2 e0 = lds.ld<ace_d2>(a);          // input size, size / intra-node bandwidth
         ace_d2 e1 = lds.ld<ace_d2>(a + 16);     // size / inter-node bandwidth, pad
         inputs = e0.x;
@@ -167,8 +182,40 @@ template <bool BD, bool RANGED> struct PlanState {
             id_in = in_cross ? i1.x : i0.y;
             id_fwd = 0.0; id_bwd = 0.0;
         }
-        fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = pend_rf = pend_rb = rs_f = rs_b = 0.0;
-        lastclose = false;
+    }
+
+    // DEFER: park the finished stage's accumulators in the plan's workspace slot `s`.
+    ACE_HD void stash(double *ws, uint32_t i_last, uint32_t c_last) {
+        if (ws == nullptr || s < 0 || s >= ACE_MAX_STAGES) return;
+        ace_d2 *r = reinterpret_cast<ace_d2 *>(ws + (size_t)s * ACE_WS_REC);
+        uint64_t meta = (uint64_t)(first_meta | (c_last << 19) | ((uint32_t)lastclose << 22)) | ((uint64_t)i_last << 32);
+        double meta_d;
+        __builtin_memcpy(&meta_d, &meta, 8);
+#ifdef ACE_EXP_NOSTORE
+        r[6] = ace_d2{meta_d, fwd + bwd + rcs + W + A + saved + run + peak + rfm + rbm + rs_f + rs_b};
+#else
+        r[0] = ace_d2{fwd, bwd}; r[1] = ace_d2{rcs, W}; r[2] = ace_d2{A, saved}; r[3] = ace_d2{run, peak};
+        r[4] = ace_d2{rfm, rbm}; r[5] = ace_d2{rs_f, rs_b}; r[6] = ace_d2{meta_d, 0.0};
+#endif
+    }
+
+    // DEFER: evaluate stage `s2` from its stashed record (called for s2 = 0, 1, ... in order).
+    ACE_HD void replay(const AceGeom &g, const AceLds &lds, const ace_u2 *pos_info, const double *ws, int s2) {
+        const ace_d2 *r = reinterpret_cast<const ace_d2 *>(ws + (size_t)s2 * ACE_WS_REC);
+        ace_d2 r0 = r[0], r1 = r[1], r2 = r[2], r3 = r[3], r4 = r[4], r5 = r[5], r6 = r[6];
+        s = s2 - 1;
+        start_fast(g, lds);                    // s = s2; per-stage offsets, out_cross, mrow
+        uint64_t meta;
+        __builtin_memcpy(&meta, &r6.x, 8);
+        uint32_t lo32 = (uint32_t)meta, i_last = (uint32_t)(meta >> 32);
+        uint32_t i_first = lo32 & 0xffffu, c_first = (lo32 >> 16) & 7u, c_last = (lo32 >> 19) & 7u;
+        if (i_first >= (uint32_t)g.N) i_first = 0;     // garbage only if the plan was malformed
+        if (i_last >= (uint32_t)g.N) i_last = 0;
+        start_lookups(g, lds, info_row(pos_info[i_first]), c_first);
+        fwd = r0.x; bwd = r0.y; rcs = r1.x; W = r1.y; A = r2.x; saved = r2.y; run = r3.x; peak = r3.y;
+        rfm = r4.x; rbm = r4.y; rs_f = r5.x; rs_b = r5.y;
+        lastclose = (lo32 >> 22) & 1u;
+        finish(g, lds, info_row(pos_info[i_last]), c_last, nullptr);
     }
 
     // Stage tail; `prevrow` is the LDS offset of the row of the stage's last op, `c_last` its code.
@@ -227,8 +274,15 @@ template <bool BD, bool RANGED> struct PlanState {
         const bool ns = (byte >> 4) & 1u;
         const uint32_t row = info_row(info);
         if (ns) {
-            if (s >= 0) finish(g, lds, info_prevrow(info), pbyte & 7u, rec);
-            start(g, lds, row, c);
+            if (DEFER) {
+                if (s >= 0) stash(rec, (uint32_t)(i - 1), pbyte & 7u);
+                start_fast(g, lds);
+                first_meta = (uint32_t)i | (c << 16);
+            } else {
+                if (s >= 0) finish(g, lds, info_prevrow(info), pbyte & 7u, rec);
+                start_fast(g, lds);
+                start_lookups(g, lds, row, c);
+            }
         }
         const uint32_t fl = info.y >> 8;
         uint32_t a = row + g.hot_off + hot_v + c * ACE_HOT_STRIDE;
@@ -242,7 +296,7 @@ template <bool BD, bool RANGED> struct PlanState {
         pend_rb = e2.y;
         fwd += e0.x;
         bwd += e0.y;
-        if (rc) rcs += e0.x;
+        rcs = ace_fma((double)(int)rc, e0.x, rcs);   // rc is 0 or 1: the product is exact, one rounding as in "+="
         W += e1.x;
         A += e1.y;
         if (BD) {
@@ -269,10 +323,11 @@ template <bool BD, bool RANGED> struct PlanState {
             // (the reference raises there)
             uint32_t pk = info.y & 0xffu;
             uint32_t pc = pbyte & 7u;
-            uint32_t r = ns ? 0u : (uint32_t)lds.ld<uint8_t>(g.rk_lds_off + pk * g.rk_kind_stride + rk_v + pc * (uint32_t)g.C + c);
+            uint32_t r = lds.ld<uint8_t>(g.rk_lds_off + ace_mul24(pk, g.rk_kind_stride) + rk_v + ((pc << 3) | c));
+            r = ns ? 0u : r;
             uint32_t za = row + g.z_off + z_v + c * 8u;
-            rs_f += lds.ld<double>(za + (r & 15u) * g.z_stride);
-            rs_b += lds.ld<double>(za + (r >> 4) * g.z_stride);
+            rs_f += lds.ld<double>(za + ((r & 15u) << g.z_shift));
+            rs_b += lds.ld<double>(za + ((r >> 4) << g.z_shift));
         }
     }
 

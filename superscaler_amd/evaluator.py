@@ -59,7 +59,7 @@ def load_library():
     lib.ace_time_score_kernel.argtypes = [ctypes.c_void_p, ctypes.POINTER(AceBatchStruct), ctypes.c_double,
                                           ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                           ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(ctypes.c_double)]
-    if lib.ace_abi_version() != 1:
+    if lib.ace_abi_version() != 2:
         raise AceError("libace_eval.so has a different ABI version")
     _lib = lib
     return lib

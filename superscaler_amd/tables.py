@@ -24,7 +24,9 @@ maxima of table entries:
      ids (0 = the all-zero table: nothing to do, last id = the all-NaN table: the reference would
      raise) for an adjacent op
      pair, from get_op_spec / get_reshard_primitives (model_ops_info.py:92-150, cost_model:185-245)
-  stage_lut[mbs index][glog]  diag | per-tp mbs-index nibbles << 8 (0xF = not profiled)
+  stage_lut[mbs index][glog]  two words: hot-table byte offset of the diag | pair-kind offset of the
+     stage size << 16;  diag * n_codes | per-tp mbs-index nibbles << 16 (0xF = not profiled).
+     Unscorable (micro-batch, stage size) pairs point at one extra diag that is all NaN.
   pos_info[i]  LDS offset / 16 of op i's row | of op i-1's row << 16;  pair kind | flags << 8
 """
 import ctypes
@@ -37,7 +39,7 @@ import numpy as np
 from . import opgraph as og
 from .profile_db import CostModelSettings, ProfileDB
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 MAX_STAGES = 16
 STAGE_REC = 18
 LDS_BYTES = 160 * 1024
@@ -55,7 +57,8 @@ class AceTablesStruct(ctypes.Structure):
         ("n_diag", ctypes.c_int32), ("n_glog", ctypes.c_int32), ("n_z", ctypes.c_int32),
         ("n_pair_kinds", ctypes.c_int32), ("row_doubles", ctypes.c_int32),
         ("hot_off", ctypes.c_int32), ("start_off", ctypes.c_int32), ("out_off", ctypes.c_int32),
-        ("z_off", ctypes.c_int32), ("n_windows", ctypes.c_int32), ("lds_row_bytes", ctypes.c_int32),
+        ("z_off", ctypes.c_int32), ("z_table_doubles", ctypes.c_int32), ("n_windows", ctypes.c_int32),
+        ("lds_row_bytes", ctypes.c_int32),
         ("flags", ctypes.c_int32), ("main_params", ctypes.c_double), ("optimizer", ctypes.c_double),
         ("rows", ctypes.c_void_p), ("pos_info", ctypes.c_void_p), ("pair_kinds", ctypes.c_void_p),
         ("stage_lut", ctypes.c_void_p), ("nb_minus_1", ctypes.c_void_p), ("win_pos", ctypes.c_void_p),
@@ -77,12 +80,13 @@ class CompiledTables:
     start_off: int
     out_off: int
     z_off: int
+    z_table_doubles: int
     lds_row_bytes: int
     flags: int
     rows: np.ndarray            # float64 [n_types, row_doubles]
     pos_info: np.ndarray        # uint32 [N + 1, 2]
-    pair_kinds: np.ndarray      # uint8 [n_pk, n_glog, C, C]
-    stage_lut: np.ndarray       # uint32 [n_mbs, 16]
+    pair_kinds: np.ndarray      # uint8 [n_pk, n_glog, 8, 8]
+    stage_lut: np.ndarray       # uint32 [n_mbs, 16, 2]
     nb_minus_1: np.ndarray      # float64 [n_mbs]
     win_pos: np.ndarray         # int32 [n_win + 1]
     win_row_begin: np.ndarray   # int32 [n_win + 1]
@@ -108,6 +112,7 @@ class CompiledTables:
         s.n_diag, s.n_glog, s.n_z, s.n_pair_kinds = self.n_diag, self.n_glog, self.n_z, self.n_pair_kinds
         s.row_doubles = self.row_doubles
         s.hot_off, s.start_off, s.out_off, s.z_off = self.hot_off, self.start_off, self.out_off, self.z_off
+        s.z_table_doubles = self.z_table_doubles
         s.n_windows = self.n_windows
         s.lds_row_bytes = self.lds_row_bytes
         s.flags = self.flags
@@ -122,10 +127,8 @@ class CompiledTables:
 
     # what a (micro_bs index, log2 stage gpus) pair allows
     def allowed_tp_logs(self, bidx: int, glog: int) -> List[int]:
-        w = int(self.stage_lut[bidx, glog])
-        if (w & 0xff) == 0xff:
-            return []
-        return [t for t in range(len(self.db.tp_list)) if ((w >> (8 + 4 * t)) & 15) != 15]
+        mrow = int(self.stage_lut[bidx, glog, 1]) >> 16
+        return [t for t in range(len(self.db.tp_list)) if ((mrow >> (4 * t)) & 15) != 15]
 
 
 def _mbs_tuple(db: ProfileDB, micro_bs: int, gpus: int) -> Tuple[Optional[int], ...]:
@@ -161,29 +164,32 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
     if M > 15 or T > 4 or A not in (1, 2):
         raise ValueError("table geometry outside what the evaluator encodes (<=15 mbs, <=4 tp, 1-2 algos)")
     C = T * A
+    CP = 8            # codes are 3 bits: pair-kind blocks are always 8 x 8
     tb = db.tables
     shared = settings.consider_shared_space
 
     # ---- diags and the stage LUT -----------------------------------------------------------
     diags: List[List[Optional[int]]] = []
-    stage_lut = np.full((M, 16), 0xFF, dtype=np.uint32)
+    lut_diag = np.full((M, 16), -1, dtype=np.int64)
+    lut_mrow = np.full((M, 16), 0xFFFF, dtype=np.int64)
     n_glog = 1
     for bi, mb in enumerate(db.mbs_list):
         for glog in range(min(16, max_glog)):
             tup = _mbs_tuple(db, mb, 1 << glog)
             if all(x is None or x == 15 for x in tup):
                 continue
-            d = _merge_diag(diags, tup)
-            word = d
+            lut_diag[bi, glog] = _merge_diag(diags, tup)
+            word = 0
             for t in range(4):
                 x = tup[t] if t < T else None
-                word |= (15 if x is None else x) << (8 + 4 * t)
-            stage_lut[bi, glog] = word
+                word |= (15 if x is None else x) << (4 * t)
+            lut_mrow[bi, glog] = word
             n_glog = max(n_glog, glog + 1)
     diag_tuples = [tuple(15 if x is None else x for x in d) for d in diags]
-    ND = len(diag_tuples)
-    if ND == 0 or ND > 254:
+    n_real_diag = len(diag_tuples)
+    if n_real_diag == 0 or n_real_diag > 200:
         raise ValueError("no scorable (micro-batch, stage size) combination")
+    ND = n_real_diag
 
     # ---- adjacent-pair kinds and the collectives in use ----------------------------------------
     z_keys: List[Tuple[int, int]] = []
@@ -207,10 +213,10 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
     pk_of_pos = np.zeros(graph.num_ops + 1, dtype=np.int64)
     kinds = [og.spec_kinds(n) for n in db.op_names]
     pair_cache: Dict[Tuple[int, int], int] = {}
-    zero_block = np.zeros((n_glog, C, C), dtype=np.uint8)
+    zero_block = np.zeros((n_glog, CP, CP), dtype=np.uint8)
 
     def pair_block(tprev: int, tcur: int) -> np.ndarray:
-        blk = np.zeros((n_glog, C, C), dtype=np.uint8)
+        blk = np.zeros((n_glog, CP, CP), dtype=np.uint8)
         if not settings.resharding:
             return blk
         for glog in range(n_glog):
@@ -249,20 +255,45 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
     if len(pk_arrays) > 255:
         raise ValueError("more than 255 distinct adjacent-op spec pairings")
     pair_kinds = np.ascontiguousarray(np.stack(pk_arrays))
-    # cost-table ids: 0 = all zeros, 1..len(z_keys) = real collectives, last = all NaN (errors)
-    NZ = len(z_keys) + 2
-    lo, hi = pair_kinds & 15, pair_kinds >> 4
-    lo = np.where(lo == ERR, NZ - 1, lo)
-    hi = np.where(hi == ERR, NZ - 1, hi)
-    pair_kinds = np.ascontiguousarray((lo | (hi << 4)).astype(np.uint8))
+    # cost-table ids: 0 = all zeros, 1..len(z_keys) = real collectives, last = all NaN (errors);
+    # no tables at all when nothing can ever be paid (resharding off: T5)
+    use_z = bool(settings.resharding and (pair_kinds != 0).any())
+    NZ = len(z_keys) + 2 if use_z else 0
+    if use_z:
+        lo, hi = pair_kinds & 15, pair_kinds >> 4
+        lo = np.where(lo == ERR, NZ - 1, lo)
+        hi = np.where(hi == ERR, NZ - 1, hi)
+        pair_kinds = np.ascontiguousarray((lo | (hi << 4)).astype(np.uint8))
+    else:
+        pair_kinds = np.zeros((1, n_glog, CP, CP), dtype=np.uint8)
+        pk_of_pos[:] = 0
 
     # ---- rows ------------------------------------------------------------------------------
     hot_off = 0
     start_off = hot_off + ND * C * 6
     out_off = start_off + ND * C * 4
     z_off = out_off + M * T * A * 2
-    row_doubles = z_off + NZ * ND * C
+    z_table_doubles = 1
+    while z_table_doubles < ND * C:
+        z_table_doubles *= 2          # one collective's table, padded so its index is a shift
+    # a block of C hot entries that are all NaN: where unscorable (micro-batch, stage size) pairs point
+    nan_off = z_off + NZ * z_table_doubles
+    row_doubles = nan_off + C * 6
     row_doubles += row_doubles & 1
+    if (row_doubles * 8) > 0xFFFF:
+        raise ValueError("an op type's row exceeds what the stage LUT addresses")
+    # stage LUT: [mbs][glog] -> (hot byte offset | pair-kind glog offset << 16, diag * C | mrow << 16)
+    stage_lut = np.zeros((M, 16, 2), dtype=np.uint32)
+    for bi in range(M):
+        for glog in range(16):
+            d = int(lut_diag[bi, glog])
+            rk_v = glog * CP * CP if glog < n_glog else 0
+            if d < 0:
+                stage_lut[bi, glog, 0] = ((nan_off - hot_off) * 8) | (rk_v << 16)
+                stage_lut[bi, glog, 1] = 0 | (0xFFFF << 16)
+            else:
+                stage_lut[bi, glog, 0] = (d * C * 48) | (rk_v << 16)
+                stage_lut[bi, glog, 1] = (d * C) | (int(lut_mrow[bi, glog]) << 16)
     rows = np.zeros((n_types, row_doubles), dtype=np.float64)
     nan = math.nan
     reserved_on = settings.consider_reserved_space
@@ -270,7 +301,7 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
         fl = int(graph.flags[ty])
         hot = np.full((ND, C, 6), nan)
         start = np.full((ND, C, 4), nan)
-        z = np.full((NZ, ND, C), nan)
+        z = np.full((max(NZ, 1), ND, C), nan)
         z[0] = 0.0
         for d, tup in enumerate(diag_tuples):
             for t in range(T):
@@ -301,12 +332,15 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
         rows[ty, hot_off:hot_off + hot.size] = hot.ravel()
         rows[ty, start_off:start_off + start.size] = start.ravel()
         rows[ty, out_off:out_off + out.size] = out.ravel()
-        rows[ty, z_off:z_off + NZ * ND * C] = z.ravel()
+        for k in range(NZ):
+            rows[ty, z_off + k * z_table_doubles:z_off + (k + 1) * z_table_doubles] = nan if k == NZ - 1 else 0.0
+            rows[ty, z_off + k * z_table_doubles:z_off + k * z_table_doubles + ND * C] = z[k].ravel()
+        rows[ty, nan_off:nan_off + C * 6] = nan
 
     # ---- LDS residency: one window if every row fits, else windows over op positions ----------
     row_bytes = row_doubles * 8
     rk_bytes = pair_kinds.size
-    small = ((rk_bytes + 15) & ~15) + M * 16 * 4
+    small = ((rk_bytes + 15) & ~15) + M * 16 * 8
     avail = (lds_budget - small) & ~15
     if avail < 2 * row_bytes:
         raise ValueError(f"one op type's row ({row_bytes} B) does not fit LDS twice ({avail} B available)")
@@ -318,7 +352,7 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
     N = graph.num_ops
     while i < N:
         # a window holds the row of the op just before it (stage tails look back one op) and ends
-        # at a multiple of 16 ops (the kernel restages between 16-op groups) or at the last op
+        # at a multiple of 4 ops (the kernel restages between 4-op words) or at the last op
         slot_of: Dict[int, int] = {}
         if i > 0:
             slot_of[int(tp[i - 1])] = 0
@@ -331,10 +365,10 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
                     break
                 slot_of[ty] = len(slot_of)
             j += 1
-            if j % 16 == 0 or j == N:
+            if j % 4 == 0 or j == N:
                 good = (j, dict(slot_of))
         if good is None:
-            raise ValueError("LDS too small for a 16-op window of this op graph")
+            raise ValueError("LDS too small for a 4-op window of this op graph")
         j, slot_of = good
         for k in range(i, j):
             prev = slot_of[int(tp[k - 1])] if k > 0 else 0
@@ -346,7 +380,7 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
         win_row_begin.append(len(win_rows))
         win_pos.append(j)
         i = j
-    win_pos[-1] = max((win_pos[-1] + 15) // 16 * 16, N + 1)      # never reached: no restaging after the last window
+    win_pos[-1] = max((win_pos[-1] + 3) // 4 * 4, N + 1)      # never reached: no restaging after the last window
     lds_row_bytes = max(off for _, off in win_rows) + row_bytes
 
     # flags about the previous op, seen from position i
@@ -371,7 +405,7 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
     return CompiledTables(
         graph=graph, db=db, settings=settings, n_diag=ND, n_glog=n_glog, n_z=NZ,
         n_pair_kinds=len(pk_arrays), row_doubles=row_doubles, hot_off=hot_off, start_off=start_off,
-        out_off=out_off, z_off=z_off, lds_row_bytes=int(lds_row_bytes), flags=flags,
+        out_off=out_off, z_off=z_off, z_table_doubles=z_table_doubles, lds_row_bytes=int(lds_row_bytes), flags=flags,
         rows=np.ascontiguousarray(rows), pos_info=np.ascontiguousarray(pos_info),
         pair_kinds=pair_kinds, stage_lut=np.ascontiguousarray(stage_lut), nb_minus_1=nbm1,
         win_pos=np.array(win_pos, dtype=np.int32), win_row_begin=np.array(win_row_begin, dtype=np.int32),

@@ -10,14 +10,16 @@
 
 namespace {
 
-template <bool BD, bool RANGED>
+template <bool BD, bool RANGED, bool DEFER = false>
 void score_one(const ace_tables_t *t, const AceGeom &g, std::vector<unsigned char> &lds, uint32_t lds_bytes,
                const uint8_t *codes, ace_u4 h, ace_u2 range, double *rec, double &iter, double &peak, uint8_t &feas,
                uint8_t &st) {
     const size_t row_bytes = (size_t)t->row_doubles * 8;
     const ace_u2 *pos = reinterpret_cast<const ace_u2 *>(t->pos_info);
     AceLds view{lds.data(), lds_bytes};
-    PlanState<BD, RANGED> s;
+    PlanState<BD, RANGED, DEFER> s;
+    std::vector<double> ws(ACE_MAX_STAGES * ACE_WS_REC, __builtin_nan(""));
+    if (DEFER) rec = ws.data();
     s.init(g, view, h, range);
     int w = 0, next_win = t->win_pos[0];
     uint32_t pbyte = 0;
@@ -32,7 +34,13 @@ void score_one(const ace_tables_t *t, const AceGeom &g, std::vector<unsigned cha
         s.step(g, view, i, codes[i], pbyte, pos[i], rec);
         pbyte = codes[i];
     }
-    if (!RANGED || !s.done) s.finish(g, view, info_prevrow(pos[g.N]), pbyte & 7u, rec);
+    if (DEFER) {
+        s.stash(rec, (uint32_t)(g.N - 1), pbyte & 7u);
+        const int n_st = s.s + 1;
+        for (int s2 = 0; s2 < n_st && s2 < ACE_MAX_STAGES; ++s2) s.replay(g, view, pos, rec, s2);
+    } else if (!RANGED || !s.done) {
+        s.finish(g, view, info_prevrow(pos[g.N]), pbyte & 7u, rec);
+    }
     s.result(g, t->nb_minus_1[s.bidx], iter, peak, feas, st);
 }
 
@@ -40,7 +48,7 @@ void score_one(const ace_tables_t *t, const AceGeom &g, std::vector<unsigned cha
 
 extern "C" int ace_emu_score(const ace_tables_t *t, const uint8_t *codes /* [P][N] plan-major */,
                              const uint32_t *hdr /* [P][4] */, const uint32_t *range /* nullable [P][2] */,
-                             long long P, double memory_limit, int strict, double *iter_ms, double *peak_mb,
+                             long long P, double memory_limit, int strict, int defer, double *iter_ms, double *peak_mb,
                              uint8_t *feasible, uint8_t *status, double *stage_out /* nullable [P][16][18] */) {
     const int C = t->n_tp * t->n_algo;
     AceGeom g;
@@ -49,12 +57,13 @@ extern "C" int ace_emu_score(const ace_tables_t *t, const uint8_t *codes /* [P][
     g.C = C; g.A_shift = t->n_algo == 2 ? 1 : 0;
     g.n_mbs = t->n_mbs; g.n_tp = t->n_tp; g.n_algo = t->n_algo; g.n_glog = t->n_glog; g.n_pair_kinds = t->n_pair_kinds;
     g.hot_off = t->hot_off * 8u; g.start_off = t->start_off * 8u; g.out_off = t->out_off * 8u; g.z_off = t->z_off * 8u;
-    g.z_stride = (uint32_t)(t->n_diag * C) * 8u;
-    const int32_t rk_bytes = t->n_pair_kinds * t->n_glog * C * C;
+    g.z_shift = 3;
+    while ((1 << (g.z_shift - 3)) < t->z_table_doubles) ++g.z_shift;
+    const int32_t rk_bytes = t->n_pair_kinds * t->n_glog * 64;
     g.rk_lds_off = (uint32_t)t->lds_row_bytes;
     g.stg_lds_off = (g.rk_lds_off + (uint32_t)rk_bytes + 15u) & ~15u;
-    g.rk_kind_stride = (uint32_t)(t->n_glog * C * C);
-    const uint32_t lds_bytes = g.stg_lds_off + (uint32_t)t->n_mbs * 16u * 4u;
+    g.rk_kind_stride = (uint32_t)(t->n_glog * 64);
+    const uint32_t lds_bytes = g.stg_lds_off + (uint32_t)t->n_mbs * 16u * 8u;
     g.flags = t->flags; g.main_params = t->main_params; g.optimizer = t->optimizer;
     g.mem_limit = memory_limit; g.strict = strict ? 1 : 0;
     if (range && !stage_out) return -1;
@@ -63,7 +72,7 @@ extern "C" int ace_emu_score(const ace_tables_t *t, const uint8_t *codes /* [P][
     for (long long p = 0; p < P; ++p) {
         memset(lds.data(), 0xff, lds.size());
         memcpy(lds.data() + g.rk_lds_off, t->pair_kinds, rk_bytes);
-        memcpy(lds.data() + g.stg_lds_off, t->stage_lut, (size_t)t->n_mbs * 16 * 4);
+        memcpy(lds.data() + g.stg_lds_off, t->stage_lut, (size_t)t->n_mbs * 16 * 8);
         ace_u4 h;
         memcpy(&h, hdr + 4 * p, 16);
         ace_u2 rg{0u, 0u};
@@ -74,6 +83,7 @@ extern "C" int ace_emu_score(const ace_tables_t *t, const uint8_t *codes /* [P][
         uint8_t feas, st;
         if (range) score_one<true, true>(t, g, lds, lds_bytes, c, h, rg, rec, iter, peak, feas, st);
         else if (stage_out) score_one<true, false>(t, g, lds, lds_bytes, c, h, rg, rec, iter, peak, feas, st);
+        else if (defer && t->n_windows == 1) score_one<false, false, true>(t, g, lds, lds_bytes, c, h, rg, rec, iter, peak, feas, st);
         else score_one<false, false>(t, g, lds, lds_bytes, c, h, rg, rec, iter, peak, feas, st);
         iter_ms[p] = iter; peak_mb[p] = peak; feasible[p] = feas;
         if (status) status[p] = st;

@@ -64,7 +64,7 @@ def emu_lib():
     return _emu
 
 
-def emu_score(tables, batch, memory_limit=None, strict=False, breakdown=False, ranges=None):
+def emu_score(tables, batch, memory_limit=None, strict=False, breakdown=False, ranges=None, defer=True):
     lib = emu_lib()
     ts = tables.as_struct()
     P = batch.n_plans
@@ -78,7 +78,7 @@ def emu_score(tables, batch, memory_limit=None, strict=False, breakdown=False, r
         ranges = np.ascontiguousarray(ranges, dtype=np.uint32)
         breakdown = True
     rc = lib.ace_emu_score(ctypes.byref(ts), codes.ctypes.data_as(ctypes.c_void_p), hdr.ctypes.data_as(ctypes.c_void_p),
-                           ranges.ctypes.data_as(ctypes.c_void_p) if ranges is not None else None, ctypes.c_longlong(P), ctypes.c_double(limit), ctypes.c_int(int(strict)),
+                           ranges.ctypes.data_as(ctypes.c_void_p) if ranges is not None else None, ctypes.c_longlong(P), ctypes.c_double(limit), ctypes.c_int(int(strict)), ctypes.c_int(int(defer)),
                            it.ctypes.data_as(ctypes.c_void_p), pk.ctypes.data_as(ctypes.c_void_p),
                            fe.ctypes.data_as(ctypes.c_void_p), st.ctypes.data_as(ctypes.c_void_p),
                            rec.ctypes.data_as(ctypes.c_void_p) if breakdown else None)

@@ -23,12 +23,13 @@ def case(request):
 
 def test_scores_bit_exact(case):
     w, tables, batch, orc = case
-    it, pk, fe, st, _ = emu_score(tables, batch)
     oit, opk, ofe, _ = oracle_scores(orc, batch, tables)
-    assert (st == 0).all()
-    assert np.array_equal(it, oit)
-    assert np.array_equal(pk, opk)
-    assert np.array_equal(fe, ofe)
+    for defer in (False, True):     # stage tails evaluated in place / stashed and replayed after the op loop
+        it, pk, fe, st, _ = emu_score(tables, batch, defer=defer)
+        assert (st == 0).all()
+        assert np.array_equal(it, oit)
+        assert np.array_equal(pk, opk)
+        assert np.array_equal(fe, ofe)
     # strict comparison flips only plans that sit exactly on the limit
     it2, pk2, fe2, _, _ = emu_score(tables, batch, memory_limit=float(np.median(opk)), strict=True)
     assert np.array_equal(fe2, (opk < float(np.median(opk))).astype(np.uint8))

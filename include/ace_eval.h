@@ -82,8 +82,8 @@ typedef struct ace_tables {
     int32_t flags;          /* ACE_F_* */
     double main_params, optimizer;   /* aceso_utils.py:48-52 */
     const double *rows;            /* [num_types][row_doubles] */
-    const uint32_t *pos_info;      /* [num_ops + 1][2]: row LDS offset / 16 | previous op's row offset / 16 << 16;
-                                      pair kind | flags << 8 */
+    const uint32_t *pos_info;      /* [num_ops + 1]: LDS slot of the op's row | slot of the previous op's row << 8 |
+                                      pair kind << 16 | flags << 24 (a slot is row_doubles * 8 bytes) */
     const uint8_t *pair_kinds;     /* [n_pair_kinds][n_glog][8][8] (previous code, this code) */
     const uint32_t *stage_lut;     /* [n_mbs][16][2]: hot byte offset of the diag | pair-kind offset << 16;
                                       diag * C | per-tp mbs-index nibbles << 16 (C = n_tp * n_algo) */

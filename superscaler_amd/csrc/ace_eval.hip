@@ -39,7 +39,7 @@ struct AceKernelArgs {
     const ace_u4 *hdr;          // [P]
     const ace_u2 *range;        // [P] (first op, one past the last op) or null
     const double *rows;         // [n_types][row_doubles]
-    const ace_u2 *pos_info;     // [N + 1], padded to a multiple of 4 entries
+    const uint32_t *pos_info;   // [N + 1], padded to 16 * G + 16 entries
     const uint8_t *pair_kinds;  // -> LDS
     const uint32_t *stage_lut;  // -> LDS
     const double *nbm1;         // [n_mbs]
@@ -98,39 +98,39 @@ __global__ __launch_bounds__(kBlock) void ace_score_kernel(const AceKernelArgs a
 
     int w = 0;
     int next_win = WIN ? a.win_pos[0] : 0x7fffffff;
-    ace_u4 cw = a.codes[pl];                 // sixteen op bytes; consumed one 32-bit word (4 ops) at a time
-    ace_u4 nxt = cw;
+    ace_u4 cw = a.codes[pl];                 // sixteen op bytes of this plan
     uint32_t pbyte = 0;                      // code byte of the previous op
-    const int quads = (g.N + 3) >> 2;
-    for (int q = 0; q < quads; ++q) {
-        const int base = q << 2;
-        if ((q & 3) == 0) {
-            if (q) cw = nxt;
-            const int grp = (q >> 2) + 1;
-            if (grp < g.G) nxt = a.codes[(size_t)grp * g.P + pl];
-        }
-        if (WIN && base == next_win) {
-            // every lane of the workgroup reaches this point together
-            __syncthreads();
-            stage_window(a, lds_raw, w, tid);
-            __syncthreads();
-            ++w;
-            next_win = a.win_pos[w];
-        }
-        const uint32_t word = cw.x;
-        cw.x = cw.y; cw.y = cw.z; cw.z = cw.w;
-        // the four position descriptors of this quad in one scalar load (the array is padded)
-        const ace_u4 ia = reinterpret_cast<const ace_u4 *>(a.pos_info)[2 * q];
-        const ace_u4 ib = reinterpret_cast<const ace_u4 *>(a.pos_info)[2 * q + 1];
-        const ace_u2 infos[4] = {{ia.x, ia.y}, {ia.z, ia.w}, {ib.x, ib.y}, {ib.z, ib.w}};
+    for (int grp = 0; grp < g.G; ++grp) {
+        const int base = grp << 4;
+        // the sixteen position descriptors of this group and the first one of the next: scalar loads
+        // (the array is padded)
+        const ace_u4 *ip = reinterpret_cast<const ace_u4 *>(a.pos_info + base);
+        const ace_u4 i0 = ip[0], i1 = ip[1], i2 = ip[2], i3 = ip[3];
+        const uint32_t infos[17] = {i0.x, i0.y, i0.z, i0.w, i1.x, i1.y, i1.z, i1.w,
+                                    i2.x, i2.y, i2.z, i2.w, i3.x, i3.y, i3.z, i3.w, a.pos_info[base + 16]};
+        ace_u4 nxt = cw;
+        if (grp + 1 < g.G) nxt = a.codes[(size_t)(grp + 1) * g.P + pl];
+        const uint32_t words[5] = {cw.x, cw.y, cw.z, cw.w, nxt.x};
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            if (base + k < g.N) {
-                const uint32_t byte = (word >> (8 * k)) & 0xffu;
-                st.step(g, lds, base + k, byte, pbyte, infos[k], rec);
+        for (int k = 0; k < 16; ++k) {
+            const int i = base + k;
+            if (WIN && (k & 3) == 0 && i == next_win) {
+                // every lane of the workgroup reaches this point together
+                __syncthreads();
+                stage_window(a, lds_raw, w, tid);
+                __syncthreads();
+                ++w;
+                next_win = a.win_pos[w];
+            }
+            if (i < g.N) {
+                const uint32_t byte = (words[k >> 2] >> (8 * (k & 3))) & 0xffu;
+                uint32_t nbyte = (words[(k + 1) >> 2] >> (8 * ((k + 1) & 3))) & 0xffu;
+                if (i + 1 >= g.N) nbyte = 0x10u;
+                st.step(g, lds, i, byte, pbyte, nbyte, infos[k], infos[k + 1], rec);
                 pbyte = byte;
             }
         }
+        cw = nxt;
     }
     if (DEFER) {
         st.stash(rec, (uint32_t)(g.N - 1), pbyte & 7u);
@@ -141,7 +141,7 @@ __global__ __launch_bounds__(kBlock) void ace_score_kernel(const AceKernelArgs a
             if (live) st.replay(g, lds, a.pos_info, rec, s2);
         }
     } else if (!RANGED || !st.done) {
-        st.finish(g, lds, info_prevrow(a.pos_info[g.N]), pbyte & 7u, rec);
+        st.finish(g, lds, info_prevrow(g, a.pos_info[g.N]), pbyte & 7u, rec);
     }
     double iter, peak;
     uint8_t feas, stat;
@@ -380,7 +380,7 @@ struct ace_handle {
     uint32_t lds_bytes;
     // device copies
     double *d_rows;
-    ace_u2 *d_pos_info;
+    uint32_t *d_pos_info;
     uint8_t *d_pair_kinds;
     uint32_t *d_stage_lut;
     double *d_nbm1;
@@ -472,10 +472,9 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
         if ((int64_t)t->win_rows[2 * r + 1] + row_bytes > t->lds_row_bytes || (t->win_rows[2 * r + 1] & 15u)) return ACE_EINVAL;
     }
     for (int i = 0; i <= t->num_ops; ++i) {
-        const uint32_t *pi = t->pos_info + 2 * (size_t)i;
-        const int64_t row = (int64_t)(pi[0] & 0xffffu) * 16, prow = (int64_t)(pi[0] >> 16) * 16;
-        if (row + row_bytes > t->lds_row_bytes || prow + row_bytes > t->lds_row_bytes ||
-            (pi[1] & 0xffu) >= (uint32_t)t->n_pair_kinds)
+        const uint32_t pi = t->pos_info[i];
+        if ((int64_t)((pi & 0xffu) + 1) * row_bytes > t->lds_row_bytes || (int64_t)(((pi >> 8) & 0xffu) + 1) * row_bytes > t->lds_row_bytes ||
+            ((pi >> 16) & 0xffu) >= (uint32_t)t->n_pair_kinds)
             return ACE_EINVAL;
     }
     for (int j = 0; j < stg_words; j += 2) {
@@ -503,15 +502,16 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     while ((1 << (g.z_shift - 3)) < t->z_table_doubles) ++g.z_shift;
     g.rk_lds_off = rk_off; g.stg_lds_off = stg_off;
     g.rk_kind_stride = (uint32_t)(t->n_glog * 64);
+    g.row_bytes = (uint32_t)row_bytes;
     g.flags = t->flags; g.main_params = t->main_params; g.optimizer = t->optimizer;
     g.mem_limit = 0.0; g.strict = 0;
     h->n_windows = t->n_windows; h->row_doubles = t->row_doubles; h->rk_bytes = rk_bytes; h->stg_words = stg_words;
     h->num_types = t->num_types; h->lds_bytes = lds_bytes;
-    const size_t pos_entries = ((size_t)t->num_ops + 1 + 3) & ~(size_t)3;
+    const size_t pos_entries = (size_t)((t->num_ops + 15) / 16) * 16 + 16;
     int rc;
     if ((rc = hipGetDevice(&h->device) == hipSuccess ? ACE_OK : ACE_EHIP) ||
         (rc = upload((void **)&h->d_rows, t->rows, (size_t)t->num_types * row_bytes)) ||
-        (rc = upload((void **)&h->d_pos_info, t->pos_info, (size_t)(t->num_ops + 1) * 8, pos_entries * 8)) ||
+        (rc = upload((void **)&h->d_pos_info, t->pos_info, (size_t)(t->num_ops + 1) * 4, pos_entries * 4)) ||
         (rc = upload((void **)&h->d_pair_kinds, t->pair_kinds, (size_t)rk_bytes)) ||
         (rc = upload((void **)&h->d_stage_lut, t->stage_lut, (size_t)stg_words * 4)) ||
         (rc = upload((void **)&h->d_nbm1, t->nb_minus_1, (size_t)t->n_mbs * 8)) ||

@@ -81,16 +81,17 @@ struct AceGeom {
     uint32_t z_shift;           // log2(bytes of one resharding-cost table inside a row)
     uint32_t rk_lds_off, stg_lds_off;              // LDS byte offsets of the pair-kind and stage LUT regions
     uint32_t rk_kind_stride;    // bytes of one pair kind (n_glog * 64)
+    uint32_t row_bytes;         // bytes of one op type's row
     int32_t flags;
     double main_params, optimizer, mem_limit;
     int32_t strict;
 };
 
-// position descriptor (wave-uniform): x = row offset / 16 | previous op's row offset / 16 << 16,
-// y = pair kind | flags << 8 (bit 0: previous op is an ordinary op followed by a layer start;
-// bit 1: previous op is an ordinary op)
-ACE_HD uint32_t info_row(ace_u2 i) { return (i.x & 0xffffu) << 4; }
-ACE_HD uint32_t info_prevrow(ace_u2 i) { return (i.x >> 16) << 4; }
+// position descriptor (wave-uniform), one word: bits 0-7 LDS slot of the op's row, 8-15 slot of the
+// previous op's row, 16-23 pair kind, bit 24: the previous op is an ordinary op followed by a layer
+// start, bit 25: the previous op is an ordinary op
+ACE_HD uint32_t info_row(const AceGeom &g, uint32_t i) { return (i & 0xffu) * g.row_bytes; }
+ACE_HD uint32_t info_prevrow(const AceGeom &g, uint32_t i) { return ((i >> 8) & 0xffu) * g.row_bytes; }
 
 #define ACE_WS_REC 14          // doubles per deferred stage record (see PlanState::stash)
 
@@ -117,6 +118,8 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
     bool lastclose;
     bool done;                  // RANGED: the stage was finished inside the op loop
     uint32_t first_meta;        // DEFER: first op of the current stage: position | code << 16
+    ace_u2 lut_next;            // stage LUT entry of the NEXT stage, fetched one stage ahead
+    uint32_t r_next;            // collective ids of the (this op, next op) pair, fetched one op ahead
     // plan accumulators
     double sum_t, max_t, max_mem;
     uint32_t status;
@@ -131,7 +134,8 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         s = -1;
         sum_t = 0.0; max_t = 0.0; max_mem = 0.0;
         status = 0;
-        prev_act = 0.0; lastclose = false; done = false; first_meta = 0;
+        prev_act = 0.0; lastclose = false; done = false; first_meta = 0; r_next = 0;
+        lut_next = ace_u2{0u, 0u};
         fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = pend_rf = pend_rb = rs_f = rs_b = 0.0;
         id_fwd = id_bwd = id_in = 0.0;
         in_comm = inputs = 0.0;
@@ -140,6 +144,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         ideal_hot_v = ideal_start_v = 0;
         if (bidx >= (uint32_t)g.n_mbs) { status = ACE_PLAN_MALFORMED; bidx = 0; }
         if (RANGED && (lo < 0 || hi > g.N || lo >= hi)) { status = ACE_PLAN_MALFORMED; lo = 0; hi = 1; }
+        lut_next = lds.ld<ace_u2>(g.stg_lds_off + (bidx * 16u + ((uint32_t)glogs & 15u)) * 8u);
         if (BD) {
             // the "ideal" pass uses tp = dp = 1 and micro-batch = micro_bs (aceso_cost_model.py:588-590):
             // the diag of (micro_bs, 1 gpu)
@@ -150,11 +155,19 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
     }
 
     // Stage head, part 1: the per-stage offsets the op loop needs, accumulators back to zero.
-    ACE_HD void start_fast(const AceGeom &g, const AceLds &lds) {
+    ACE_HD void start_fast(const AceGeom &g, const AceLds &lds, bool pipelined) {
         ++s;
         // (a plan with more than 16 stage bits is caught by result(): s + 1 != S)
-        uint32_t glog = (uint32_t)(glogs >> (4u * ((uint32_t)s & 15u))) & 15u;
-        ace_u2 w = lds.ld<ace_u2>(g.stg_lds_off + (bidx * 16u + glog) * 8u);
+        ace_u2 w;
+        if (pipelined) {
+            // this stage's LUT entry was fetched when the previous stage began; fetch the next one now
+            w = lut_next;
+            uint32_t glog_n = (uint32_t)(glogs >> (4u * ((uint32_t)(s + 1) & 15u))) & 15u;
+            lut_next = lds.ld<ace_u2>(g.stg_lds_off + (bidx * 16u + glog_n) * 8u);
+        } else {
+            uint32_t glog = (uint32_t)(glogs >> (4u * ((uint32_t)s & 15u))) & 15u;
+            w = lds.ld<ace_u2>(g.stg_lds_off + (bidx * 16u + glog) * 8u);
+        }
         hot_v = w.x & 0xffffu;
         rk_v = w.x >> 16;
         dc_v = w.y & 0xffffu;
@@ -200,22 +213,22 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
     }
 
     // DEFER: evaluate stage `s2` from its stashed record (called for s2 = 0, 1, ... in order).
-    ACE_HD void replay(const AceGeom &g, const AceLds &lds, const ace_u2 *pos_info, const double *ws, int s2) {
+    ACE_HD void replay(const AceGeom &g, const AceLds &lds, const uint32_t *pos_info, const double *ws, int s2) {
         const ace_d2 *r = reinterpret_cast<const ace_d2 *>(ws + (size_t)s2 * ACE_WS_REC);
         ace_d2 r0 = r[0], r1 = r[1], r2 = r[2], r3 = r[3], r4 = r[4], r5 = r[5], r6 = r[6];
         s = s2 - 1;
-        start_fast(g, lds);                    // s = s2; per-stage offsets, out_cross, mrow
+        start_fast(g, lds, false);             // s = s2; per-stage offsets, mrow
         uint64_t meta;
         __builtin_memcpy(&meta, &r6.x, 8);
         uint32_t lo32 = (uint32_t)meta, i_last = (uint32_t)(meta >> 32);
         uint32_t i_first = lo32 & 0xffffu, c_first = (lo32 >> 16) & 7u, c_last = (lo32 >> 19) & 7u;
         if (i_first >= (uint32_t)g.N) i_first = 0;     // garbage only if the plan was malformed
         if (i_last >= (uint32_t)g.N) i_last = 0;
-        start_lookups(g, lds, info_row(pos_info[i_first]), c_first);
+        start_lookups(g, lds, info_row(g, pos_info[i_first]), c_first);
         fwd = r0.x; bwd = r0.y; rcs = r1.x; W = r1.y; A = r2.x; saved = r2.y; run = r3.x; peak = r3.y;
         rfm = r4.x; rbm = r4.y; rs_f = r5.x; rs_b = r5.y;
         lastclose = (lo32 >> 22) & 1u;
-        finish(g, lds, info_row(pos_info[i_last]), c_last, nullptr);
+        finish(g, lds, info_row(g, pos_info[i_last]), c_last, nullptr);
     }
 
     // Stage tail; `prevrow` is the LDS offset of the row of the stage's last op, `c_last` its code.
@@ -262,29 +275,31 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         }
     }
 
-    // One op at position i.  `byte` is its code byte, `pbyte` the previous op's, `info` the
-    // position's (wave-uniform) descriptor.
-    ACE_HD void step(const AceGeom &g, const AceLds &lds, int i, uint32_t byte, uint32_t pbyte, ace_u2 info, double *rec) {
+    // One op at position i.  `byte` is its code byte, `pbyte` / `nbyte` the previous / next op's
+    // (nbyte = 0x10 after the last op), `info` / `ninfo` this and the next position's (wave-uniform)
+    // descriptors.
+    ACE_HD void step(const AceGeom &g, const AceLds &lds, int i, uint32_t byte, uint32_t pbyte, uint32_t nbyte,
+                     uint32_t info, uint32_t ninfo, double *rec) {
         if (RANGED) {
-            if (i == hi) { finish(g, lds, info_prevrow(info), pbyte & 7u, rec); done = true; }
+            if (i == hi) { finish(g, lds, info_prevrow(g, info), pbyte & 7u, rec); done = true; }
             if (i < lo || i >= hi) return;
         }
         const uint32_t c = byte & 7u;
         const bool rc = (byte >> 3) & 1u;
         const bool ns = (byte >> 4) & 1u;
-        const uint32_t row = info_row(info);
+        const uint32_t row = info_row(g, info);
         if (ns) {
             if (DEFER) {
                 if (s >= 0) stash(rec, (uint32_t)(i - 1), pbyte & 7u);
-                start_fast(g, lds);
+                start_fast(g, lds, true);
                 first_meta = (uint32_t)i | (c << 16);
             } else {
-                if (s >= 0) finish(g, lds, info_prevrow(info), pbyte & 7u, rec);
-                start_fast(g, lds);
+                if (s >= 0) finish(g, lds, info_prevrow(g, info), pbyte & 7u, rec);
+                start_fast(g, lds, true);
                 start_lookups(g, lds, row, c);
             }
         }
-        const uint32_t fl = info.y >> 8;
+        const uint32_t fl = info >> 24;
         uint32_t a = row + g.hot_off + hot_v + c * ACE_HOT_STRIDE;
         ace_d2 e0 = lds.ld<ace_d2>(a);         // fwd us, bwd us
         ace_d2 e1 = lds.ld<ace_d2>(a + 16);    // weights MB, activations MB (shared-buffer rule applied)
@@ -305,7 +320,11 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
             id_bwd += ie.y;
         }
         // (previous op, this op) both recomputed and in one stage
+#ifdef ACE_EXP_NOPAIR
+        const bool pair = false;
+#else
         const bool pair = ((byte & pbyte) >> 3) & ~(byte >> 4) & 1u;
+#endif
         const bool savez = fl & 1u;     // previous op is an ordinary op followed by a layer start
         if (pair) {
             run += prev_act;
@@ -317,18 +336,20 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         }
         lastclose = pair && (fl & 2u);
         prev_act = e1.y;
+#ifndef ACE_EXP_NORESHARD
         if (g.flags & ACE_F_RESHARDING) {
             // collective ids of the (previous, this) op pair; id 0 is an all-zero cost table, so a
             // pair that needs nothing adds 0.0, and the id past the last real table is all NaN
             // (the reference raises there)
-            uint32_t pk = info.y & 0xffu;
-            uint32_t pc = pbyte & 7u;
-            uint32_t r = lds.ld<uint8_t>(g.rk_lds_off + ace_mul24(pk, g.rk_kind_stride) + rk_v + ((pc << 3) | c));
-            r = ns ? 0u : r;
+            // (fetched while the previous op was processed; a stage's first op pays nothing)
+            uint32_t r = ns ? 0u : r_next;
+            uint32_t npk = (ninfo >> 16) & 0xffu;
+            r_next = lds.ld<uint8_t>(g.rk_lds_off + ace_mul24(npk, g.rk_kind_stride) + rk_v + ((c << 3) | (nbyte & 7u)));
             uint32_t za = row + g.z_off + z_v + c * 8u;
             rs_f += lds.ld<double>(za + ((r & 15u) << g.z_shift));
             rs_b += lds.ld<double>(za + ((r >> 4) << g.z_shift));
         }
+#endif
     }
 
     ACE_HD void result(const AceGeom &g, double nbm1, double &iter_ms, double &peak_mb, uint8_t &feasible, uint8_t &st) {

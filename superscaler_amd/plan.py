@@ -222,3 +222,76 @@ def validate_batch(batch: PlanBatch, tables: CompiledTables) -> Optional[str]:
     if np.any((batch.codes & 7) >= tables.C):
         return "tp/algo code outside the profile database"
     return None
+
+
+# model_size -> (num_layers, seq_len, hidden, ffn_hidden, heads, kv_channels, vocab)  (aceso_utils.py:27-34)
+GPT_CONFIGS = {
+    "350M": (24, 2048, 1024, 4096, 16, 64, 51200), "1_3B": (24, 2048, 2048, 8192, 32, 64, 51200),
+    "2_6B": (32, 2048, 2560, 10240, 32, 80, 51200), "6_7B": (32, 2048, 4096, 16384, 32, 128, 51200),
+    "13B": (40, 2048, 5120, 20480, 40, 128, 51200), "scale-layer": (1, 2048, 512, 2048, 8, 64, 51200),
+}
+# model_size -> (num_layers, enc_seq, dec_seq, hidden, ffn_hidden, heads, kv_channels, vocab)  (aceso_utils.py:38-45)
+T5_CONFIGS = {
+    "770M": (24, 2048, 512, 1024, 4096, 16, 64, 30592), "3B": (24, 2048, 512, 1024, 16384, 32, 128, 30592),
+    "6B": (24, 2048, 512, 1024, 32768, 64, 128, 30592), "11B": (24, 2048, 512, 1024, 65536, 128, 128, 30592),
+    "22B": (48, 2048, 512, 1024, 65536, 128, 128, 30592),
+}
+# model_size -> (blocks per stage, in_channels, width_factor)  (aceso_utils.py:16-24)
+RESNET_CONFIGS = {
+    "250M": ([3, 4, 6, 3], 160, 2), "500M": ([3, 4, 6, 3], 224, 2), "1B": ([3, 4, 6, 3], 320, 2),
+    "2B": ([3, 4, 6, 3], 448, 2), "4B": ([3, 4, 6, 3], 640, 2), "6_8B": ([3, 4, 6, 3], 320, 16),
+    "13B": ([3, 4, 23, 3], 320, 16),
+}
+
+
+def config_to_json_dict(config, model_name: str, model_size: str, num_layers=None) -> dict:
+    """The plan JSON the training runtime consumes (aceso_utils.py:137-211), as a dict."""
+    if model_name == "scale-layer":
+        model_name, model_size = "gpt", "scale-layer"
+    d = {"model_name": model_name, "model_size": model_size}
+    if model_name == "resnet":
+        layers, in_channels, width = RESNET_CONFIGS[model_size]
+        d.update(num_layers=layers, in_channels=in_channels, width_factor=width)
+    elif model_name == "gpt":
+        n, seq, hidden, _, heads, _, _ = GPT_CONFIGS[model_size]
+        d.update(num_layers=num_layers if num_layers is not None else n, seq_length=seq,
+                 max_position_embeddings=seq, num_attention_heads=heads, hidden_size=hidden)
+    elif model_name == "t5":
+        n, enc, dec, hidden, ffn, heads, kv, _ = T5_CONFIGS[model_size]
+        d.update(num_layers=num_layers if num_layers is not None else n, encoder_seq_length=enc,
+                 decoder_seq_length=dec, max_position_embeddings=enc, num_attention_heads=heads, kv_channels=kv,
+                 hidden_size=hidden, ffn_hidden_size=ffn)
+    else:
+        raise RuntimeError(f"{model_name} not supportted.")
+    d["global_batch_size"] = config.global_bs
+    d["micro_batch_size"] = config.micro_bs
+    d["num_stages"] = config.num_stages
+    d["num_gpus"] = [st.num_gpus for st in config.stages]
+    d["checkpoint_activations"] = [max(st.recompute_ops) > 0 for st in config.stages]
+    d["resharding_stages"] = [max(st.tp_size) != min(st.tp_size) or max(st.dp_size) != min(st.dp_size) or
+                              max(st.algo) != min(st.algo) for st in config.stages]
+    d["num_ops_in_each_stage"] = [len(st.ops) for st in config.stages]
+    d["model_parallel_size_of_each_op"] = [list(st.tp_size) for st in config.stages]
+    d["data_parallel_size_of_each_op"] = [list(st.dp_size) for st in config.stages]
+    d["recompute_ops"] = [list(st.recompute_ops) for st in config.stages]
+    d["algo_of_each_op"] = [list(st.algo) for st in config.stages]
+    return d
+
+
+def dump_config_to_json(config, file_name: str, model_name: str, model_size: str, num_layers=None) -> None:
+    with open(file_name, "w") as f:
+        json.dump(config_to_json_dict(config, model_name, model_size, num_layers), f, indent=4)
+
+
+def check_legality(config, num_gpus: int, num_gpus_per_node: int, num_nodes: int) -> bool:
+    """aceso_utils.py:760-774: stage sizes in {1,2,4,8}, all devices used, node boundaries fall on
+    stage boundaries."""
+    total, from_start = 0, []
+    for st in config.stages:
+        if st.num_gpus not in (1, 2, 4, 8):
+            return False
+        total += st.num_gpus
+        from_start.append(total)
+    if total != num_gpus:
+        return False
+    return all(num_gpus_per_node * i in from_start for i in range(1, num_nodes + 1))

@@ -27,7 +27,7 @@ maxima of table entries:
   stage_lut[mbs index][glog]  two words: hot-table byte offset of the diag | pair-kind offset of the
      stage size << 16;  diag * n_codes | per-tp mbs-index nibbles << 16 (0xF = not profiled).
      Unscorable (micro-batch, stage size) pairs point at one extra diag that is all NaN.
-  pos_info[i]  LDS offset / 16 of op i's row | of op i-1's row << 16;  pair kind | flags << 8
+  pos_info[i]  LDS slot of op i's row | slot of op i-1's row << 8 | pair kind << 16 | flags << 24
 """
 import ctypes
 import math
@@ -84,7 +84,7 @@ class CompiledTables:
     lds_row_bytes: int
     flags: int
     rows: np.ndarray            # float64 [n_types, row_doubles]
-    pos_info: np.ndarray        # uint32 [N + 1, 2]
+    pos_info: np.ndarray        # uint32 [N + 1]
     pair_kinds: np.ndarray      # uint8 [n_pk, n_glog, 8, 8]
     stage_lut: np.ndarray       # uint32 [n_mbs, 16, 2]
     nb_minus_1: np.ndarray      # float64 [n_mbs]
@@ -345,7 +345,9 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
     if avail < 2 * row_bytes:
         raise ValueError(f"one op type's row ({row_bytes} B) does not fit LDS twice ({avail} B available)")
     slots = avail // row_bytes
-    pos_info = np.zeros((graph.num_ops + 1, 2), dtype=np.uint32)
+    if slots > 255:
+        slots = 255
+    pos_info = np.zeros(graph.num_ops + 1, dtype=np.uint32)
     win_pos, win_row_begin, win_rows = [0], [0], []
     tp = graph.type_of_pos
     i = 0
@@ -372,9 +374,9 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
         j, slot_of = good
         for k in range(i, j):
             prev = slot_of[int(tp[k - 1])] if k > 0 else 0
-            pos_info[k, 0] = (slot_of[int(tp[k])] * row_bytes // 16) | ((prev * row_bytes // 16) << 16)
+            pos_info[k] = slot_of[int(tp[k])] | (prev << 8)
         if j == N:
-            pos_info[N, 0] = (slot_of[int(tp[N - 1])] * row_bytes // 16) << 16
+            pos_info[N] = slot_of[int(tp[N - 1])] << 8
         for ty, sl in slot_of.items():
             win_rows.append((ty, sl * row_bytes))
         win_row_begin.append(len(win_rows))
@@ -392,7 +394,7 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
             fl |= 1      # ordinary op right before a layer start: saved += 0, peak segment closes
         if normal[prev_t]:
             fl |= 2      # ordinary op: closes the last segment when the pair ends the stage
-        pos_info[k, 1] = int(pk_of_pos[k]) | (fl << 8)
+        pos_info[k] |= (int(pk_of_pos[k]) << 16) | (fl << 24)
 
     flags = 0
     if settings.resharding and (pair_kinds != 0).any():

@@ -15,7 +15,7 @@ void score_one(const ace_tables_t *t, const AceGeom &g, std::vector<unsigned cha
                const uint8_t *codes, ace_u4 h, ace_u2 range, double *rec, double &iter, double &peak, uint8_t &feas,
                uint8_t &st) {
     const size_t row_bytes = (size_t)t->row_doubles * 8;
-    const ace_u2 *pos = reinterpret_cast<const ace_u2 *>(t->pos_info);
+    const uint32_t *pos = t->pos_info;
     AceLds view{lds.data(), lds_bytes};
     PlanState<BD, RANGED, DEFER> s;
     std::vector<double> ws(ACE_MAX_STAGES * ACE_WS_REC, __builtin_nan(""));
@@ -31,7 +31,7 @@ void score_one(const ace_tables_t *t, const AceGeom &g, std::vector<unsigned cha
                 memcpy(lds.data() + t->win_rows[2 * r + 1], t->rows + (size_t)t->win_rows[2 * r] * t->row_doubles, row_bytes);
             next_win = t->win_pos[++w];
         }
-        s.step(g, view, i, codes[i], pbyte, pos[i], rec);
+        s.step(g, view, i, codes[i], pbyte, i + 1 < g.N ? codes[i + 1] : 0x10u, pos[i], pos[i + 1], rec);
         pbyte = codes[i];
     }
     if (DEFER) {
@@ -39,7 +39,7 @@ void score_one(const ace_tables_t *t, const AceGeom &g, std::vector<unsigned cha
         const int n_st = s.s + 1;
         for (int s2 = 0; s2 < n_st && s2 < ACE_MAX_STAGES; ++s2) s.replay(g, view, pos, rec, s2);
     } else if (!RANGED || !s.done) {
-        s.finish(g, view, info_prevrow(pos[g.N]), pbyte & 7u, rec);
+        s.finish(g, view, info_prevrow(g, pos[g.N]), pbyte & 7u, rec);
     }
     s.result(g, t->nb_minus_1[s.bidx], iter, peak, feas, st);
 }
@@ -63,6 +63,7 @@ extern "C" int ace_emu_score(const ace_tables_t *t, const uint8_t *codes /* [P][
     g.rk_lds_off = (uint32_t)t->lds_row_bytes;
     g.stg_lds_off = (g.rk_lds_off + (uint32_t)rk_bytes + 15u) & ~15u;
     g.rk_kind_stride = (uint32_t)(t->n_glog * 64);
+    g.row_bytes = (uint32_t)t->row_doubles * 8u;
     const uint32_t lds_bytes = g.stg_lds_off + (uint32_t)t->n_mbs * 16u * 8u;
     g.flags = t->flags; g.main_params = t->main_params; g.optimizer = t->optimizer;
     g.mem_limit = memory_limit; g.strict = strict ? 1 : 0;

@@ -125,3 +125,41 @@ def test_module_level_api_requires_configuration():
     acm._model = None
     with pytest.raises(RuntimeError):
         acm.predict_time_breakdown(None)
+
+
+# ---- uniform plan grid (the batched form of search/gen_megatron_plan.py) -----------------------
+def _grid_check(golden_dir, backend):
+    from superscaler_amd.megatron_grid import best_uniform_plans, enumerate_grid
+    from tests.helpers import oracle_for
+    g, m = make_model(golden_dir, "gpt_1_3B", backend)
+    try:
+        num_gpus = g["num_nodes"] * g["num_gpus_per_node"]
+        configs = enumerate_grid(m, num_gpus, g["num_layers"])
+        assert len(configs) > 20
+        got = best_uniform_plans(m, num_gpus, g["num_layers"], num_saved=5)
+        # the reference's selection (gen_megatron_plan.py:101-135) on the oracle's numbers
+        orc = oracle_for(m.tables)
+        from oracle.aceso_oracle import get_config as oget
+        feasible = {}
+        for c in configs:
+            flat = lambda key: [x for st in c.stages for x in getattr(st, key)]
+            oc = oget([len(st.ops) for st in c.stages], flat("tp_size"), flat("dp_size"), flat("recompute_ops"),
+                      c.micro_bs, c.global_bs, m.graph.ops, flat("algo"))
+            orc.predict_time_breakdown(oc)
+            t, mem = max(oc.time_list), max(oc.memory_list)
+            if mem < g["memory_limit"]:
+                if t not in feasible or mem < feasible[t]:
+                    feasible[t] = mem
+        want = [(t, feasible[t]) for t in sorted(feasible)[:5]]
+        assert [(t, mem) for t, mem, _ in got] == want and len(want) > 0
+    finally:
+        m.close()
+
+
+def test_uniform_grid_emu(golden_dir):
+    _grid_check(golden_dir, "emu")
+
+
+@pytest.mark.gpu
+def test_uniform_grid_gpu(golden_dir):
+    _grid_check(golden_dir, "gpu")

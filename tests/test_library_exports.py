@@ -1,0 +1,68 @@
+"""The C-ABI library loads without a GPU and exports every function include/ace_eval.h declares;
+argument checking that needs no device is exercised too (no kernel is launched here)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from superscaler_amd import evaluator, synth
+from superscaler_amd.tables import AceTablesStruct
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "ace_eval.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ace_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported():
+    lib = evaluator.load_library()
+    names = declared_functions()
+    assert {"ace_create", "ace_destroy", "ace_score_batch", "ace_topk", "ace_strerror"} <= set(names)
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in include/ace_eval.h but not exported"
+    assert sorted(evaluator.EXPORTS) == names
+    assert lib.ace_abi_version() == 2
+
+
+def test_error_strings_and_argument_checks():
+    lib = evaluator.load_library()
+    assert lib.ace_strerror(0) == b"ok"
+    assert lib.ace_strerror(-1) == b"invalid argument"
+    assert lib.ace_strerror(-99) == b"unknown error"
+    h = ctypes.c_void_p()
+    assert lib.ace_create(None, ctypes.byref(h)) == -1          # null tables
+    ts = AceTablesStruct()
+    ts.abi_version = 1
+    assert lib.ace_create(ctypes.byref(ts), ctypes.byref(h)) == -5   # ABI version mismatch
+    tables = synth.make_tables(synth.WORKLOADS["gpt3_1_3b"])
+    bad = tables.as_struct()
+    bad.n_tp = 9
+    assert lib.ace_create(ctypes.byref(bad), ctypes.byref(h)) == -1  # geometry the encoding cannot hold
+    bad = tables.as_struct()
+    lut = tables.stage_lut.copy()
+    lut[0, 0, 0] = 0xFFF0                                           # hot offset far outside the row
+    bad.stage_lut = lut.ctypes.data
+    assert lib.ace_create(ctypes.byref(bad), ctypes.byref(h)) == -1
+    assert lib.ace_topk_workspace_bytes(1 << 20, 64) > 0
+    assert lib.ace_topk_workspace_bytes(1 << 20, 0) == 0
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(evaluator, "_lib", None)
+    monkeypatch.setattr(evaluator, "_LIB_PATH", "/nonexistent/libace_eval.so")
+    with pytest.raises(evaluator.AceError):
+        evaluator.load_library()
+
+
+def test_no_gpu_means_no_scoring():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    tables = synth.make_tables(synth.WORKLOADS["gpt3_1_3b"])
+    with pytest.raises(evaluator.AceError):
+        evaluator.PlanEvaluator(tables)

@@ -407,12 +407,81 @@ class CostModel:
             current_peak = new_peak
         return recompute_ops
 
+    def check_recompute_batch(self, queries):
+        """check_recompute for many stages at once: the greedy passes advance in lockstep and every
+        round costs ONE launch for all stages still above the limit.
+        queries: [(ops, micro_bs, tp_size, dp_size, num_stages_behind, algo_list)]; returns the
+        recompute lists in the same order, identical to check_recompute called one by one."""
+        args = self.settings
+        n = len(queries)
+        if not args.flex_recompute:
+            return [[1] * len(q[0]) for q in queries]
+        rcs = [[0] * len(q[0]) for q in queries]
+        if n == 0:
+            return rcs
+        rec = self._stage_records([(q[0], rcs[k], q[2], q[3], q[1], q[4], q[5]) for k, q in enumerate(queries)])
+        state = []
+        for k, (ops, micro_bs, tp_size, dp_size, nsb, algo_list) in enumerate(queries):
+            mw, mg, mo, ma, mp, mr = self._memory_breakdown([float(x) for x in rec[k]], nsb)
+            stage_memory = (mw + mg + mo + ma + mp + mr) + args.peak_mem_in_backward
+            st = {"mem": stage_memory, "saved": 0, "peak": 0, "groups": None, "active": stage_memory - args.memory_limit > 0}
+            if st["active"]:
+                groups = {}
+                for index in range(len(ops)):
+                    g = groups.setdefault(ops[index], {"index": [], "activation_size": [], "recomputed": False, "sum_size": 0})
+                    g["index"].append(index)
+                    sz = self.get_activation_size(ops[index], micro_bs // dp_size[index], tp_size[index],
+                                                  algo_list[index]) * (nsb + 1)
+                    g["activation_size"].append(sz)
+                    g["sum_size"] += sz
+                st["groups"] = groups
+            state.append(st)
+        while True:
+            todo = []
+            for k, st in enumerate(state):
+                if not st["active"]:
+                    continue
+                ops = queries[k][0]
+                idx_group, _ = self._next_recompute_op_group(ops, st["groups"], st["mem"] - args.memory_limit)
+                if idx_group is None:
+                    st["active"] = False
+                    continue
+                for si in idx_group:
+                    if si < 0:
+                        break
+                    rcs[k][si] = 1
+                    if si < len(ops) - 1:
+                        rcs[k][si + 1] = 1
+                todo.append(k)
+            if not todo:
+                return rcs
+            rec = self._stage_records([(queries[k][0], rcs[k], queries[k][2], queries[k][3], queries[k][1],
+                                        queries[k][4], queries[k][5]) for k in todo])
+            for j, k in enumerate(todo):
+                st, nsb = state[k], queries[k][4]
+                new_saved, new_peak = float(rec[j, R_SAVED]), float(rec[j, R_PEAK])
+                st["mem"] -= (new_saved - st["saved"]) * (nsb + 1)
+                st["saved"] = new_saved
+                st["mem"] += (new_peak - st["peak"])
+                st["peak"] = new_peak
+                st["active"] = st["mem"] - args.memory_limit > 0
+
     def update_recompute(self, config, stage_idx=None):
         """aceso_cost_model.py:874-883."""
         for k in ([stage_idx] if stage_idx is not None else range(config.num_stages)):
             st = config.stages[k]
             st.recompute_ops = self.check_recompute(st.ops, config.micro_bs, st.tp_size, st.dp_size,
                                                     st.num_stages_behind, st.algo)
+
+    def update_recompute_batch(self, configs) -> None:
+        """update_recompute(config) for every stage of every plan, in lockstep on the GPU."""
+        qs, where = [], []
+        for c in configs:
+            for st in c.stages:
+                qs.append((st.ops, c.micro_bs, st.tp_size, st.dp_size, st.num_stages_behind, st.algo))
+                where.append(st)
+        for st, rc in zip(where, self.check_recompute_batch(qs)):
+            st.recompute_ops = rc
 
     def predict_value_after_move(self, config, bottleneck, partner, num_ops_moved, metric, inc_gpus=False,
                                  dec_gpus=False, dim=None):

@@ -1,0 +1,171 @@
+"""Neighbour generation in array form and a batched local search on top of it.
+
+The reference's move primitives (search/aceso_prims.py:812-826: op migration `dec_op`, `inc/dec_tp`,
+`inc/dec_dp`, `inc/dec_mbs`, recompute and algorithm fine-tuning) rebuild Python objects with
+copy.deepcopy for every candidate.  Here a move is a byte edit on a copy of the base plan's code
+row / header, so thousands of neighbours of one plan are produced with a few numpy operations and
+scored by one kernel launch.  The search policy of the reference (aceso_policy.py) is not
+reproduced: `hill_climb` is a plain best-neighbour descent used to exercise the batched path.
+"""
+from typing import Tuple
+
+import numpy as np
+
+from . import opgraph as og
+from .plan import PlanBatch
+from .tables import CompiledTables
+
+
+def _stage_bounds(codes_row: np.ndarray):
+    starts = np.flatnonzero(codes_row & 16)
+    return starts, np.append(starts[1:], len(codes_row))
+
+
+def _set_header(hdr_row, S, bidx, glogs, gpn):
+    gword, cross, till = 0, 0, 0
+    for s in range(S):
+        gword |= int(glogs[s]) << (4 * s)
+        if till % gpn == 0 and till > 0:
+            cross |= 1 << s
+        till += 1 << int(glogs[s])
+        if till % gpn == 0:
+            cross |= 1 << (16 + s)
+    hdr_row[0] = S | (bidx << 8)
+    hdr_row[1] = gword & 0xFFFFFFFF
+    hdr_row[2] = gword >> 32
+    hdr_row[3] = cross
+
+
+def make_neighbours(base: PlanBatch, tables: CompiledTables, n: int, rng: np.random.Generator,
+                    max_move: int = 8) -> PlanBatch:
+    """n single-move neighbours of base plan 0 (moves that would leave the profiled grid are replaced
+    by a copy of the base plan, so the batch always has n valid rows)."""
+    A = tables.db.n_algo
+    N = tables.graph.num_ops
+    gpn = tables.settings.num_gpus_per_node
+    row0, hdr0 = base.codes[0], base.hdr[0]
+    S = int(hdr0[0] & 0xff)
+    bidx = int(hdr0[0] >> 8) & 0xff
+    gword = int(hdr0[1]) | (int(hdr0[2]) << 32)
+    glogs = np.array([(gword >> (4 * s)) & 15 for s in range(S)])
+    starts, ends = _stage_bounds(row0)
+    tunable = (tables.graph.flags[tables.graph.type_of_pos] & og.F_TUNABLE) != 0
+    M = len(tables.db.mbs_list)
+    codes = np.repeat(row0[None, :], n, axis=0)
+    hdr = np.repeat(hdr0[None, :], n, axis=0)
+    kinds = rng.integers(0, 6, size=n)
+
+    def allowed(b, gl):
+        return tables.allowed_tp_logs(b, gl)
+
+    def tp_logs(seg):
+        return (seg.astype(np.int64) & 7) // A
+
+    def with_tp(seg, t):
+        """The code bytes `seg` with their tp replaced by t (algo, recompute and stage bits kept)."""
+        return ((seg & 0xF8) | (np.asarray(t, dtype=np.int64) * A + (seg.astype(np.int64) & 7) % A).astype(np.uint8))
+
+    for k in range(n):
+        kind = kinds[k]
+        row = codes[k]
+        if kind == 0 and S > 1:
+            # op migration: move a stage boundary by up to max_move ops; the ops that change stage
+            # take the tp of the op they now follow / precede in the receiving stage
+            j = int(rng.integers(1, S))
+            d = int(rng.integers(1, max_move + 1)) * (1 if rng.random() < 0.5 else -1)
+            cut = int(starts[j])
+            new_cut = cut + d
+            if new_cut <= starts[j - 1] or new_cut >= ends[j]:
+                continue
+            row[cut] &= 0xEF
+            if d > 0:      # stage j-1 grows: ops [cut, new_cut) join it with the tp of op cut-1
+                row[cut:new_cut] = with_tp(row[cut:new_cut], int(tp_logs(row[cut - 1:cut])[0]))
+            else:          # stage j grows to the left with the tp of its former first op
+                row[new_cut:cut] = with_tp(row[new_cut:cut], int(tp_logs(row[cut:cut + 1])[0]))
+            row[new_cut] |= 16
+        elif kind == 1:
+            # tp <-> dp inside one stage: all ops one step up or down, if the stage allows it
+            s = int(rng.integers(0, S))
+            step = 1 if rng.random() < 0.5 else -1
+            lo, hi = int(starts[s]), int(ends[s])
+            t = tp_logs(row[lo:hi]) + step
+            ok = allowed(bidx, int(glogs[s]))
+            if t.min() < 0 or not np.all(np.isin(t, ok)):
+                continue
+            row[lo:hi] = with_tp(row[lo:hi], t)
+        elif kind == 2:
+            # micro-batch size one step up or down, if every op stays on the profiled grid
+            b2 = bidx + (1 if rng.random() < 0.5 else -1)
+            if b2 < 0 or b2 >= M:
+                continue
+            good = True
+            for s in range(S):
+                t = tp_logs(row[starts[s]:ends[s]])
+                if not np.all(np.isin(t, allowed(b2, int(glogs[s])))):
+                    good = False
+                    break
+            if not good:
+                continue
+            hdr[k, 0] = S | (b2 << 8)
+        elif kind == 3:
+            # recompute: toggle a short run of ops
+            lo = int(rng.integers(0, N))
+            hi = min(N, lo + int(rng.integers(1, 14)))
+            row[lo:hi] ^= 8
+        elif kind == 4 and A == 2:
+            # partition algorithm of one tunable op
+            cand = np.flatnonzero(tunable)
+            i = int(cand[rng.integers(0, len(cand))])
+            row[i] ^= 1
+        elif kind == 5 and S > 1:
+            # move half of stage a's devices to a stage b that has exactly that many (sizes stay powers
+            # of two and the total is unchanged)
+            a, b = rng.choice(S, size=2, replace=False)
+            if glogs[a] - 1 != glogs[b]:
+                continue
+            g2 = glogs.copy()
+            g2[a] -= 1
+            g2[b] += 1
+            if not allowed(bidx, int(g2[a])) or not allowed(bidx, int(g2[b])):
+                continue
+            good = True
+            for s in (a, b):
+                ok = allowed(bidx, int(g2[s]))
+                lo, hi = int(starts[s]), int(ends[s])
+                t = np.clip(tp_logs(row[lo:hi]), min(ok), max(ok))
+                if not np.all(np.isin(t, ok)):
+                    good = False
+                    break
+                row[lo:hi] = with_tp(row[lo:hi], t)
+            if not good:
+                codes[k] = row0
+                continue
+            _set_header(hdr[k], S, bidx, g2, gpn)
+    return PlanBatch(codes, hdr)
+
+
+def hill_climb(cm, start: PlanBatch, steps: int, n_neighbours: int, seed: int = 0, max_move: int = 8,
+               on_step=None) -> Tuple[PlanBatch, float, float]:
+    """Best-neighbour descent: at every step n_neighbours single-move neighbours of the current plan
+    are scored in one launch and the fastest feasible one replaces it if it is faster.
+    Returns (plan, iteration ms, peak MB)."""
+    rng = np.random.default_rng(seed)
+    tables = cm.tables
+    ev = cm.evaluator
+    cur = start.slice(0, 1)
+    it, pk, fe, st = ev.score_host(cur)
+    cur_t = float(it[0]) if fe[0] else float("inf")
+    cur_m = float(pk[0])
+    for step in range(steps):
+        nb = make_neighbours(cur, tables, n_neighbours, rng, max_move)
+        d = ev.upload(nb, validate=False)
+        it, pk, fe, st = ev.score(d)
+        idx, val, cnt = ev.topk(it, fe, 1)
+        if int(cnt.item()) == 1:
+            best_i, best_t = int(idx[0].item()), float(val[0].item())
+            if best_t < cur_t:
+                cur = nb.slice(best_i, best_i + 1)
+                cur_t, cur_m = best_t, float(pk[best_i].item())
+        if on_step is not None:
+            on_step(step, cur_t, cur_m)
+    return cur, cur_t, cur_m

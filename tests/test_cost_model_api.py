@@ -83,6 +83,16 @@ def _run_all(g, m):
             assert gv == v and list(gr) == r
         for b, partner, k, dec, v in p["delta_time"]:
             assert m.wrap_predict_delta_time(c, b, partner, k, decrease=dec) == v
+    # the lockstep batched greedy pass gives the same lists as the one-by-one calls
+    qs, want = [], []
+    for c, p in list(zip(cfgs, g["plans"]))[:8]:
+        for s, st in enumerate(c.stages):
+            qs.append((st.ops, p["micro_batch_size"], st.tp_size, st.dp_size, st.num_stages_behind, st.algo))
+            want.append(p["check_recompute"][s])
+    assert m.check_recompute_batch(qs) == want
+    cs = [cfg_of(g, m, p) for p in g["plans"][:4]]
+    m.update_recompute_batch(cs)
+    assert [[st.recompute_ops for st in c.stages] for c in cs] == [p["check_recompute"] for p in g["plans"][:4]]
     # update_recompute rewrites the stages' recompute lists with check_recompute's answer
     c = cfg_of(g, m, g["plans"][1])
     m.update_recompute(c)

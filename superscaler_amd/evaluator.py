@@ -192,6 +192,45 @@ class PlanEvaluator:
         _check(self.lib, rc, "ace_time_score_kernel")
         return ms.value
 
+    def score_stream(self, batches, k: int, memory_limit: Optional[float] = None, strict: bool = False):
+        """Score host-resident batches one after the other while the next one is uploaded: uploads run
+        on a second stream (same priority) into the buffers of the batch before last, scoring and the
+        per-batch top-k on the current stream.  Returns (global plan indices, times) of the k fastest
+        feasible plans over all batches (ascending, ties -> lower global index) and the number of
+        plans seen."""
+        torch = self._torch
+        copy_stream = torch.cuda.Stream(device=self.device)
+        main = torch.cuda.current_stream(self.device)
+        best_idx = np.empty(0, dtype=np.int64)
+        best_val = np.empty(0, dtype=np.float64)
+        offset = 0
+        it = iter(batches)
+
+        def upload(b):
+            with torch.cuda.stream(copy_stream):
+                d = self.upload(b)
+                ev = torch.cuda.Event()
+                ev.record(copy_stream)
+            return d, ev
+
+        nxt = next(it, None)
+        pending = upload(nxt) if nxt is not None else None
+        while pending is not None:
+            d, ready = pending
+            nxt = next(it, None)
+            pending = upload(nxt) if nxt is not None else None     # overlaps with the scoring below
+            main.wait_event(ready)
+            t, pk, fe, st = self.score(d, memory_limit, strict)
+            idx, val, cnt = self.topk(t, fe, k)
+            n = int(cnt.item())                                      # synchronises this batch
+            best_idx = np.concatenate([best_idx, idx[:n].cpu().numpy() + offset])
+            best_val = np.concatenate([best_val, val[:n].cpu().numpy()])
+            order = np.lexsort((best_idx, best_val))[:k]
+            best_idx, best_val = best_idx[order], best_val[order]
+            offset += d.n_plans
+            del d
+        return best_idx, best_val, offset
+
     # convenience: host in, host out
     def score_host(self, batch: PlanBatch, memory_limit=None, strict=False, breakdown=False, ranges=None):
         d = self.upload(batch, ranges=ranges)

@@ -191,3 +191,82 @@ def test_known_answers_single_gpu_plans(golden_dir, torch_mod):
     assert reserved == [3432.0] and int(cfg.memory_list[0] - reserved[0]) == 16519
     assert abs(max(cfg.time_list) / 1000 - 67.13) / 67.13 < 0.005
     m.close()
+
+
+def _tiny_gpt(num_layers, pp_choices, num_gpus=16):
+    import dataclasses
+    w = dataclasses.replace(synth.WORKLOADS["gpt3_13b"], name=f"tiny{num_layers}", num_layers=num_layers,
+                            num_gpus=num_gpus, pp_choices=pp_choices, memory_limit=30000.0)
+    tables = synth.make_tables(w)
+    return w, tables
+
+
+@pytest.mark.parametrize("layers,pp,n_plans", [(1, [16], 1), (1, [16], 1025), (1, [1, 2], 64), (5, [1, 4, 16], 3000)])
+def test_edge_shapes(layers, pp, n_plans, torch_mod):
+    """Op count a multiple of 16 (one layer = 16 ops), every op its own stage (16 stages on 16 ops),
+    a single plan, a plan count that is not a multiple of the workgroup size."""
+    from superscaler_amd.evaluator import PlanEvaluator
+    w, tables = _tiny_gpt(layers, pp)
+    assert tables.graph.num_ops == 13 * layers + 3
+    batch = synth.make_plans(w, tables, n_plans=n_plans)
+    ev = PlanEvaluator(tables)
+    it, pk, fe, st = ev.score_host(batch)
+    it2, pk2, fe2, st2, rec = ev.score_host(batch, breakdown=True)
+    orc = oracle_for(tables)
+    n = min(n_plans, 200)
+    oit, opk, ofe, _ = oracle_scores(orc, batch, tables, idx=range(n))
+    assert (st == 0).all()
+    assert np.array_equal(it[:n], oit) and np.array_equal(pk[:n], opk) and np.array_equal(fe[:n], ofe)
+    assert np.array_equal(it, it2) and np.array_equal(pk, pk2) and np.array_equal(fe, fe2)
+    eit, epk, efe, _, _ = emu_score(tables, batch)
+    assert np.array_equal(it, eit) and np.array_equal(pk, epk)
+    d = ev.upload(batch)
+    dit, dpk, dfe, dst = ev.score(d)
+    idx, val, cnt = ev.topk(dit, dfe, 5)
+    order = np.lexsort((np.arange(n_plans), np.where(fe > 0, it, np.inf)))[:min(5, int(fe.sum()))]
+    assert np.array_equal(idx.cpu().numpy()[:len(order)], order)
+    ev.close()
+
+
+def test_unscorable_and_malformed_plans_are_flagged(torch_mod):
+    """A micro-batch / stage-size pair outside the profiled grid gives NaN + status 1 (the reference
+    raises KeyError); inconsistent stage bits give status 3; neighbours in the batch are unaffected."""
+    from superscaler_amd.evaluator import PlanEvaluator
+    w, tables = _tiny_gpt(5, [1, 2, 4])
+    batch = synth.make_plans(w, tables, n_plans=64)
+    ev = PlanEvaluator(tables)
+    it0, pk0, fe0, st0 = ev.score_host(batch)
+    bad = PlanBatch(batch.codes.copy(), batch.hdr.copy())
+    bad.hdr[3, 0] = (bad.hdr[3, 0] & 0xff) | (0 << 8)      # micro-batch 1 ...
+    bad.hdr[3, 1] = 0x4444                                  # ... on 16-device stages: 1 // dp is not profiled
+    bad.hdr[3, 0] = 4                                       # (and claim four stages)
+    bad.codes[3] &= 0xEF
+    bad.codes[3, [0, 10, 20, 30]] |= 16
+    bad.codes[7, 5] |= 16                                   # one stage bit more than num_stages says
+    d = ev.upload(bad, validate=False)
+    it, pk, fe, st = [t.cpu().numpy() for t in ev.score(d)]
+    assert st[3] == 1 and np.isnan(it[3]) and np.isnan(pk[3]) and fe[3] == 0
+    assert st[7] == 3 and fe[7] == 0
+    keep = np.ones(64, dtype=bool)
+    keep[[3, 7]] = False
+    assert (st[keep] == 0).all() and np.array_equal(it[keep], it0[keep]) and np.array_equal(fe[keep], fe0[keep])
+    ev.close()
+
+
+def test_streamed_batches_match_one_shot(torch_mod):
+    """GPT-3 175B-shaped graph (1,251 ops), plans streamed in batches with overlapped upload: the
+    merged top-k equals the top-k of the same plans scored in one piece."""
+    from superscaler_amd.evaluator import PlanEvaluator
+    w = synth.WORKLOADS["gpt3_175b"]
+    tables = synth.make_tables(w)
+    ev = PlanEvaluator(tables)
+    parts = [synth.make_plans(w, tables, n_plans=8192, seed_offset=100 + j) for j in range(4)]
+    limit = 400000.0        # a cap that leaves some of these 64-GPU-per-stage plans feasible
+    idx, val, seen = ev.score_stream(iter(parts), k=32, memory_limit=limit)
+    assert seen == 4 * 8192
+    whole = PlanBatch.concat(parts)
+    it, pk, fe, st = ev.score_host(whole, memory_limit=limit)
+    order = np.lexsort((np.arange(len(it)), np.where(fe > 0, it, np.inf)))[:min(32, int(fe.sum()))]
+    assert int(fe.sum()) > 0
+    assert np.array_equal(idx, order) and np.array_equal(val, it[order])
+    ev.close()

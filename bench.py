@@ -52,6 +52,8 @@ def main():
     ap.add_argument("--plans", type=int, default=None)
     ap.add_argument("--topk", type=int, default=64)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pp", type=int, nargs="+", default=None,
+                    help="restrict the pipeline depths the plans are drawn from (profiling aid)")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="also run one plain device-to-device copy of this many MiB (a kernel of known "
                          "traffic, to scale FETCH_SIZE / WRITE_SIZE counter readings)")
@@ -69,6 +71,9 @@ def main():
         sys.exit(3)
 
     w = synth.WORKLOADS[args.workload]
+    if args.pp:
+        import dataclasses
+        w = dataclasses.replace(w, pp_choices=list(args.pp))
     n_plans = args.plans or w.n_plans
     tables = synth.make_tables(w)
     t0 = time.perf_counter()

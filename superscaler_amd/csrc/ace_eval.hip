@@ -19,7 +19,10 @@
 
 namespace {
 
-constexpr int kBlock = 1024;             // lanes (= plans) per workgroup: 16 wavefronts, 4 per SIMD
+#ifndef ACE_BLOCK
+#define ACE_BLOCK 1024
+#endif
+constexpr int kBlock = ACE_BLOCK;        // lanes (= plans) per workgroup: 16 wavefronts, 4 per SIMD
 constexpr uint32_t kMaxLds = 160 * 1024;  // CDNA4 LDS per workgroup
 
 thread_local char g_hip_err[256] = "";
@@ -124,8 +127,8 @@ __global__ __launch_bounds__(kBlock) void ace_score_kernel(const AceKernelArgs a
             }
             if (i < g.N) {
                 const uint32_t byte = (words[k >> 2] >> (8 * (k & 3))) & 0xffu;
-                uint32_t nbyte = (words[(k + 1) >> 2] >> (8 * ((k + 1) & 3))) & 0xffu;
-                if (i + 1 >= g.N) nbyte = 0x10u;
+                // (past the last op the code bytes are zero padding: a harmless code 0)
+                const uint32_t nbyte = (words[(k + 1) >> 2] >> (8 * ((k + 1) & 3))) & 0xffu;
                 st.step(g, lds, i, byte, pbyte, nbyte, infos[k], infos[k + 1], rec);
                 pbyte = byte;
             }

@@ -326,14 +326,15 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         const bool pair = ((byte & pbyte) >> 3) & ~(byte >> 4) & 1u;
 #endif
         const bool savez = fl & 1u;     // previous op is an ordinary op followed by a layer start
-        if (pair) {
-            run += prev_act;
-            if (!savez) saved += prev_act;
-        }
-        if (!pair || savez) {
-            peak = ace_max(peak, run);
-            run = 0.0;
-        }
+        // All of this is arithmetic on 0.0 / 1.0 factors instead of selects: x*1.0 and x+0.0 are exact,
+        // so every value is the one the reference computes.
+        const double pairf = (double)(int)pair;
+        const double keepf = pairf * (savez ? 0.0 : 1.0);         // 1.0 iff the pair continues the running segment
+        run = ace_fma(pairf, prev_act, run);                      // run += prev_act        if pair
+        saved = ace_fma(keepf, prev_act, saved);                  // saved += prev_act      if pair and not savez
+        const double closed = run * (1.0 - keepf);                // run if the segment closes here, else 0.0
+        peak = ace_max(peak, closed);                             // max(peak, 0.0) leaves peak (>= 0) alone
+        run = run - closed;                                       // 0.0 if closed, else run
         lastclose = pair && (fl & 2u);
         prev_act = e1.y;
 #ifndef ACE_EXP_NORESHARD

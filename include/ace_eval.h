@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define ACE_ABI_VERSION 2
+#define ACE_ABI_VERSION 3
 #define ACE_MAX_STAGES 16      /* aceso_utils.py:502: end_num_stages = min(num_gpus, 16) */
 #define ACE_STAGE_REC 18       /* doubles per stage record, see ACE_R_* */
 
@@ -82,9 +82,11 @@ typedef struct ace_tables {
     int32_t flags;          /* ACE_F_* */
     double main_params, optimizer;   /* aceso_utils.py:48-52 */
     const double *rows;            /* [num_types][row_doubles] */
-    const uint32_t *pos_info;      /* [num_ops + 1]: LDS slot of the op's row | slot of the previous op's row << 8 |
-                                      pair kind << 16 | flags << 24 (a slot is row_doubles * 8 bytes) */
-    const uint8_t *pair_kinds;     /* [n_pair_kinds][n_glog][8][8] (previous code, this code) */
+    const uint32_t *pos_info;      /* [num_ops + 1]: LDS slot of the op's row | slot of the next op's row << 8 |
+                                      kind of the (this op, next op) pair << 16 | flags << 24: bit 24 = an
+                                      ordinary op followed by a layer start, bit 25 = an ordinary op
+                                      (a slot is row_doubles * 8 bytes; the last entry is unused) */
+    const uint8_t *pair_kinds;     /* [n_pair_kinds][n_glog][8][8] (first op's code, second op's code) */
     const uint32_t *stage_lut;     /* [n_mbs][16][2]: hot byte offset of the diag | pair-kind offset << 16;
                                       diag * C | per-tp mbs-index nibbles << 16 (C = n_tp * n_algo) */
     const double *nb_minus_1;      /* [n_mbs]: global_bs // micro_bs - 1 */

@@ -86,7 +86,7 @@ __global__ __launch_bounds__(kBlock) void ace_score_kernel(const AceKernelArgs a
     for (int j = tid; j < a.rk_bytes; j += kBlock) lds_raw[g.rk_lds_off + j] = a.pair_kinds[j];
     for (int j = tid; j < a.stg_words; j += kBlock)
         reinterpret_cast<uint32_t *>(lds_raw + g.stg_lds_off)[j] = a.stage_lut[j];
-    if (!WIN) stage_window(a, lds_raw, 0, tid);
+    stage_window(a, lds_raw, 0, tid);        // every row, or the first window's
     __syncthreads();
 
     AceLds lds{lds_raw};
@@ -99,21 +99,25 @@ __global__ __launch_bounds__(kBlock) void ace_score_kernel(const AceKernelArgs a
     double *rec = (BD && a.stage_out && active) ? a.stage_out + (size_t)plan * (ACE_MAX_STAGES * ACE_STAGE_REC) : nullptr;
     if (DEFER) rec = a.stage_ws + (size_t)plan * (ACE_MAX_STAGES * ACE_WS_REC);   // padded lanes own a slot too
 
-    int w = 0;
-    int next_win = WIN ? a.win_pos[0] : 0x7fffffff;
+    int w = 1;
+    int next_win = WIN ? a.win_pos[1] : 0x7fffffff;
     ace_u4 cw = a.codes[pl];                 // sixteen op bytes of this plan
-    uint32_t pbyte = 0;                      // code byte of the previous op
+    if (!RANGED) st.begin(g, lds, 0, cw.x & 0xffu, a.pos_info[0]);
+    // the byte after the last op reads as "a stage starts here": that is what ends the last stage
+    const int end_word = g.N >> 2;
+    const uint32_t end_bit = 0x10u << (8 * (g.N & 3));
     for (int grp = 0; grp < g.G; ++grp) {
         const int base = grp << 4;
-        // the sixteen position descriptors of this group and the first one of the next: scalar loads
-        // (the array is padded)
+        // the sixteen position descriptors of this group: scalar loads (the array is padded)
         const ace_u4 *ip = reinterpret_cast<const ace_u4 *>(a.pos_info + base);
         const ace_u4 i0 = ip[0], i1 = ip[1], i2 = ip[2], i3 = ip[3];
-        const uint32_t infos[17] = {i0.x, i0.y, i0.z, i0.w, i1.x, i1.y, i1.z, i1.w,
-                                    i2.x, i2.y, i2.z, i2.w, i3.x, i3.y, i3.z, i3.w, a.pos_info[base + 16]};
-        ace_u4 nxt = cw;
+        const uint32_t infos[16] = {i0.x, i0.y, i0.z, i0.w, i1.x, i1.y, i1.z, i1.w,
+                                    i2.x, i2.y, i2.z, i2.w, i3.x, i3.y, i3.z, i3.w};
+        ace_u4 nxt = ace_u4{0u, 0u, 0u, 0u};
         if (grp + 1 < g.G) nxt = a.codes[(size_t)(grp + 1) * g.P + pl];
-        const uint32_t words[5] = {cw.x, cw.y, cw.z, cw.w, nxt.x};
+        uint32_t words[5] = {cw.x, cw.y, cw.z, cw.w, nxt.x};
+#pragma unroll
+        for (int j = 0; j < 5; ++j) words[j] |= ((base >> 2) + j == end_word) ? end_bit : 0u;
 #pragma unroll
         for (int k = 0; k < 16; ++k) {
             const int i = base + k;
@@ -127,24 +131,20 @@ __global__ __launch_bounds__(kBlock) void ace_score_kernel(const AceKernelArgs a
             }
             if (i < g.N) {
                 const uint32_t byte = (words[k >> 2] >> (8 * (k & 3))) & 0xffu;
-                // (past the last op the code bytes are zero padding: a harmless code 0)
                 const uint32_t nbyte = (words[(k + 1) >> 2] >> (8 * ((k + 1) & 3))) & 0xffu;
-                st.step(g, lds, i, byte, pbyte, nbyte, infos[k], infos[k + 1], rec);
-                pbyte = byte;
+                st.step(g, lds, i, byte, nbyte, infos[k], rec);
             }
         }
         cw = nxt;
     }
     if (DEFER) {
-        st.stash(rec, (uint32_t)(g.N - 1), pbyte & 7u);
-        const int n_st = st.s + 1;
+        const int n_st = st.s;
         for (int s2 = 0; s2 < ACE_MAX_STAGES; ++s2) {
             const bool live = s2 < n_st;
             if (!__any(live)) break;
             if (live) st.replay(g, lds, a.pos_info, rec, s2);
         }
-    } else if (!RANGED || !st.done) {
-        st.finish(g, lds, info_prevrow(g, a.pos_info[g.N]), pbyte & 7u, rec);
+        st.s = n_st;             // replay() walks s again; result() checks the count of the op loop
     }
     double iter, peak;
     uint8_t feas, stat;

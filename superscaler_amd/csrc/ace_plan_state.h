@@ -3,6 +3,7 @@
 // One instance scores one plan, op by op, in op order, with exactly the floating-point
 // operations (and their association) of the reference's search/aceso_cost_model.py, so the
 // results are bit-identical to the reference's Python floats:
+//   begin()   head of the first stage
 //   step()    one op: get_time_v3 sums (:307-313), resharding of the (previous, this) op pair
 //             (:340-350), get_recompute_time_v3 (:365-371), get_memory_v3 (:382-392),
 //             get_activations_v3 (:403-415), get_peak_activations (:428-445),
@@ -88,10 +89,10 @@ struct AceGeom {
 };
 
 // position descriptor (wave-uniform), one word: bits 0-7 LDS slot of the op's row, 8-15 slot of the
-// previous op's row, 16-23 pair kind, bit 24: the previous op is an ordinary op followed by a layer
-// start, bit 25: the previous op is an ordinary op
+// next op's row (while this op's window is resident), 16-23 kind of the (this op, next op) pair,
+// bit 24: this is an ordinary op followed by a layer start, bit 25: this is an ordinary op
 ACE_HD uint32_t info_row(const AceGeom &g, uint32_t i) { return (i & 0xffu) * g.row_bytes; }
-ACE_HD uint32_t info_prevrow(const AceGeom &g, uint32_t i) { return ((i >> 8) & 0xffu) * g.row_bytes; }
+ACE_HD uint32_t info_nextrow(const AceGeom &g, uint32_t i) { return ((i >> 8) & 0xffu) * g.row_bytes; }
 
 #define ACE_WS_REC 14          // doubles per deferred stage record (see PlanState::stash)
 
@@ -113,13 +114,12 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
     bool out_cross;
     double in_comm, inputs, id_in;
     // per-op accumulators (reset at every stage head)
-    double fwd, bwd, rcs, W, A, saved, run, peak, rfm, rbm, pend_rf, pend_rb, rs_f, rs_b, prev_act;
+    double fwd, bwd, rcs, W, A, saved, run, peak, rfm, rbm, rs_f, rs_b;
     double id_fwd, id_bwd;
     bool lastclose;
-    bool done;                  // RANGED: the stage was finished inside the op loop
     uint32_t first_meta;        // DEFER: first op of the current stage: position | code << 16
     ace_u2 lut_next;            // stage LUT entry of the NEXT stage, fetched one stage ahead
-    uint32_t r_next;            // collective ids of the (this op, next op) pair, fetched one op ahead
+    uint32_t r_next;            // collective ids of the (previous op, this op) pair, fetched one op ahead
     // plan accumulators
     double sum_t, max_t, max_mem;
     uint32_t status;
@@ -134,9 +134,9 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         s = -1;
         sum_t = 0.0; max_t = 0.0; max_mem = 0.0;
         status = 0;
-        prev_act = 0.0; lastclose = false; done = false; first_meta = 0; r_next = 0;
+        lastclose = false; first_meta = 0; r_next = 0;
         lut_next = ace_u2{0u, 0u};
-        fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = pend_rf = pend_rb = rs_f = rs_b = 0.0;
+        fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = rs_f = rs_b = 0.0;
         id_fwd = id_bwd = id_in = 0.0;
         in_comm = inputs = 0.0;
         hot_v = z_v = rk_v = mrow = t_first = dc_v = 0;
@@ -173,8 +173,9 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         dc_v = w.y & 0xffffu;
         mrow = w.y >> 16;
         z_v = dc_v << 3;
-        fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = pend_rf = pend_rb = rs_f = rs_b = 0.0;
+        fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = rs_f = rs_b = 0.0;
         lastclose = false;
+        r_next = 0;             // a stage's first op pays no resharding
     }
 
     // Stage head, part 2: boundary input of the stage's first op (code `c`, row at LDS offset `row`).
@@ -204,12 +205,8 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         uint64_t meta = (uint64_t)(first_meta | (c_last << 19) | ((uint32_t)lastclose << 22)) | ((uint64_t)i_last << 32);
         double meta_d;
         __builtin_memcpy(&meta_d, &meta, 8);
-#ifdef ACE_EXP_NOSTORE
-        r[6] = ace_d2{meta_d, fwd + bwd + rcs + W + A + saved + run + peak + rfm + rbm + rs_f + rs_b};
-#else
         r[0] = ace_d2{fwd, bwd}; r[1] = ace_d2{rcs, W}; r[2] = ace_d2{A, saved}; r[3] = ace_d2{run, peak};
         r[4] = ace_d2{rfm, rbm}; r[5] = ace_d2{rs_f, rs_b}; r[6] = ace_d2{meta_d, 0.0};
-#endif
     }
 
     // DEFER: evaluate stage `s2` from its stashed record (called for s2 = 0, 1, ... in order).
@@ -275,40 +272,33 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         }
     }
 
-    // One op at position i.  `byte` is its code byte, `pbyte` / `nbyte` the previous / next op's
-    // (nbyte = 0x10 after the last op), `info` / `ninfo` this and the next position's (wave-uniform)
-    // descriptors.
-    ACE_HD void step(const AceGeom &g, const AceLds &lds, int i, uint32_t byte, uint32_t pbyte, uint32_t nbyte,
-                     uint32_t info, uint32_t ninfo, double *rec) {
+    // Head of the plan's first stage (RANGED: of the queried stage); `byte` / `info` belong to its first op.
+    ACE_HD void begin(const AceGeom &g, const AceLds &lds, int i, uint32_t byte, uint32_t info) {
+        if (!(byte & 0x10u)) status = ACE_PLAN_MALFORMED;    // the first op must open a stage
+        start_fast(g, lds, true);
+        if (DEFER) first_meta = (uint32_t)i | ((byte & 7u) << 16);
+        else start_lookups(g, lds, info_row(g, info), byte & 7u);
+    }
+
+    // One op at position i.  `byte` is its code byte, `nbyte` the next op's (0x10 after the last op: the plan's last stage ends there),
+    // `info` the position's (wave-uniform) descriptor.  Everything that concerns the (this op, next op)
+    // pair is handled here too, so nothing but the accumulators is carried from op to op; a stage
+    // that ends with this op is closed (and the next one opened) in the middle of the step.
+    ACE_HD void step(const AceGeom &g, const AceLds &lds, int i, uint32_t byte, uint32_t nbyte, uint32_t info,
+                     double *rec) {
         if (RANGED) {
-            if (i == hi) { finish(g, lds, info_prevrow(g, info), pbyte & 7u, rec); done = true; }
             if (i < lo || i >= hi) return;
+            if (i == lo) begin(g, lds, i, byte, info);
         }
         const uint32_t c = byte & 7u;
+        const uint32_t nc = nbyte & 7u;
         const bool rc = (byte >> 3) & 1u;
-        const bool ns = (byte >> 4) & 1u;
         const uint32_t row = info_row(g, info);
-        if (ns) {
-            if (DEFER) {
-                if (s >= 0) stash(rec, (uint32_t)(i - 1), pbyte & 7u);
-                start_fast(g, lds, true);
-                first_meta = (uint32_t)i | (c << 16);
-            } else {
-                if (s >= 0) finish(g, lds, info_prevrow(g, info), pbyte & 7u, rec);
-                start_fast(g, lds, true);
-                start_lookups(g, lds, row, c);
-            }
-        }
         const uint32_t fl = info >> 24;
         uint32_t a = row + g.hot_off + hot_v + c * ACE_HOT_STRIDE;
         ace_d2 e0 = lds.ld<ace_d2>(a);         // fwd us, bwd us
         ace_d2 e1 = lds.ld<ace_d2>(a + 16);    // weights MB, activations MB (shared-buffer rule applied)
         ace_d2 e2 = lds.ld<ace_d2>(a + 32);    // fwd / bwd reserved MB
-        // reserved maxima run over every op but the stage's last: fold the previous op now
-        rfm = ace_max(rfm, pend_rf);
-        rbm = ace_max(rbm, pend_rb);
-        pend_rf = e2.x;
-        pend_rb = e2.y;
         fwd += e0.x;
         bwd += e0.y;
         rcs = ace_fma((double)(int)rc, e0.x, rcs);   // rc is 0 or 1: the product is exact, one rounding as in "+="
@@ -319,42 +309,51 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
             id_fwd += ie.x;
             id_bwd += ie.y;
         }
-        // (previous op, this op) both recomputed and in one stage
-#ifdef ACE_EXP_NOPAIR
-        const bool pair = false;
-#else
-        const bool pair = ((byte & pbyte) >> 3) & ~(byte >> 4) & 1u;
-#endif
-        const bool savez = fl & 1u;     // previous op is an ordinary op followed by a layer start
+        if (g.flags & ACE_F_RESHARDING) {
+            // collective ids of the (previous, this) op pair, fetched while the previous op was
+            // processed; id 0 is an all-zero cost table, so a pair that needs nothing (and a stage's
+            // first op) adds 0.0, and the id past the last real table is all NaN (the reference raises there)
+            const uint32_t r = r_next;
+            const uint32_t pk = (info >> 16) & 0xffu;
+            r_next = lds.ld<uint8_t>(g.rk_lds_off + ace_mul24(pk, g.rk_kind_stride) + rk_v + ((c << 3) | nc));
+            const uint32_t za = row + g.z_off + z_v + c * 8u;
+            rs_f += lds.ld<double>(za + ((r & 15u) << g.z_shift));
+            rs_b += lds.ld<double>(za + ((r >> 4) << g.z_shift));
+        }
+        // the stage ends with this op
+        const bool last = RANGED ? (i + 1 == hi) : (bool)((nbyte >> 4) & 1u);
+        if (last) {
+            if (DEFER) stash(rec, (uint32_t)i, c);
+            else finish(g, lds, row, c, rec);
+            if (!RANGED) {
+                // (after the plan's last op this opens a stage that stays empty: s == S in the end)
+                start_fast(g, lds, true);
+                if (DEFER) first_meta = (uint32_t)(i + 1) | (nc << 16);
+                else if (i + 1 < g.N) start_lookups(g, lds, info_nextrow(g, info), nc);
+            }
+            // the reserved maxima run over every op but the stage's last (get_reserved_memory :453-460)
+            e2 = ace_d2{0.0, 0.0};
+        }
+        rfm = ace_max(rfm, e2.x);
+        rbm = ace_max(rbm, e2.y);
+        // (this op, next op) both recomputed and in one stage
+        const bool pair = ((byte & nbyte) >> 3) & ~(nbyte >> 4) & 1u;
+        const bool savez = fl & 1u;     // this is an ordinary op followed by a layer start
         // All of this is arithmetic on 0.0 / 1.0 factors instead of selects: x*1.0 and x+0.0 are exact,
-        // so every value is the one the reference computes.
+        // so every value is the one the reference computes.  (After a stage end the accumulators
+        // are zero and pair is false: nothing happens.)
         const double pairf = (double)(int)pair;
         const double keepf = pairf * (savez ? 0.0 : 1.0);         // 1.0 iff the pair continues the running segment
-        run = ace_fma(pairf, prev_act, run);                      // run += prev_act        if pair
-        saved = ace_fma(keepf, prev_act, saved);                  // saved += prev_act      if pair and not savez
+        run = ace_fma(pairf, e1.y, run);                          // run += act             if pair
+        saved = ace_fma(keepf, e1.y, saved);                      // saved += act           if pair and not savez
         const double closed = run * (1.0 - keepf);                // run if the segment closes here, else 0.0
         peak = ace_max(peak, closed);                             // max(peak, 0.0) leaves peak (>= 0) alone
         run = run - closed;                                       // 0.0 if closed, else run
         lastclose = pair && (fl & 2u);
-        prev_act = e1.y;
-#ifndef ACE_EXP_NORESHARD
-        if (g.flags & ACE_F_RESHARDING) {
-            // collective ids of the (previous, this) op pair; id 0 is an all-zero cost table, so a
-            // pair that needs nothing adds 0.0, and the id past the last real table is all NaN
-            // (the reference raises there)
-            // (fetched while the previous op was processed; a stage's first op pays nothing)
-            uint32_t r = ns ? 0u : r_next;
-            uint32_t npk = (ninfo >> 16) & 0xffu;
-            r_next = lds.ld<uint8_t>(g.rk_lds_off + ace_mul24(npk, g.rk_kind_stride) + rk_v + ((c << 3) | (nbyte & 7u)));
-            uint32_t za = row + g.z_off + z_v + c * 8u;
-            rs_f += lds.ld<double>(za + ((r & 15u) << g.z_shift));
-            rs_b += lds.ld<double>(za + ((r >> 4) << g.z_shift));
-        }
-#endif
     }
 
     ACE_HD void result(const AceGeom &g, double nbm1, double &iter_ms, double &peak_mb, uint8_t &feasible, uint8_t &st) {
-        if (!RANGED && s + 1 != S) status = ACE_PLAN_MALFORMED;
+        if (!RANGED && s != S) status = ACE_PLAN_MALFORMED;   // every stage end also opened the next stage
         // max over stages of t_s*(nb-1) + sum(t): rounding is monotonic, so the maximum is attained
         // at the largest t_s and equals this expression bit for bit
         iter_ms = max_t * nbm1 + sum_t;

@@ -10,7 +10,7 @@ from typing import Optional, Sequence, Tuple
 import numpy as np
 
 from .plan import PlanBatch, validate_batch
-from .tables import MAX_STAGES, STAGE_REC, AceTablesStruct, CompiledTables
+from .tables import ABI_VERSION, MAX_STAGES, STAGE_REC, AceTablesStruct, CompiledTables
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libace_eval.so")
 _lib = None
@@ -59,7 +59,7 @@ def load_library():
     lib.ace_time_score_kernel.argtypes = [ctypes.c_void_p, ctypes.POINTER(AceBatchStruct), ctypes.c_double,
                                           ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                           ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(ctypes.c_double)]
-    if lib.ace_abi_version() != 2:
+    if lib.ace_abi_version() != ABI_VERSION:
         raise AceError("libace_eval.so has a different ABI version")
     _lib = lib
     return lib

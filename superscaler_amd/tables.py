@@ -27,7 +27,7 @@ maxima of table entries:
   stage_lut[mbs index][glog]  two words: hot-table byte offset of the diag | pair-kind offset of the
      stage size << 16;  diag * n_codes | per-tp mbs-index nibbles << 16 (0xF = not profiled).
      Unscorable (micro-batch, stage size) pairs point at one extra diag that is all NaN.
-  pos_info[i]  LDS slot of op i's row | slot of op i-1's row << 8 | pair kind << 16 | flags << 24
+  pos_info[i]  LDS slot of op i's row | slot of op i+1's row << 8 | kind of the (i, i+1) pair << 16 | flags << 24
 """
 import ctypes
 import math
@@ -39,7 +39,7 @@ import numpy as np
 from . import opgraph as og
 from .profile_db import CostModelSettings, ProfileDB
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 MAX_STAGES = 16
 STAGE_REC = 18
 LDS_BYTES = 160 * 1024
@@ -353,11 +353,10 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
     i = 0
     N = graph.num_ops
     while i < N:
-        # a window holds the row of the op just before it (stage tails look back one op) and ends
-        # at a multiple of 4 ops (the kernel restages between 4-op words) or at the last op
+        # a window also holds the row of the op right after it (a stage that ends with the window's
+        # last op opens the next stage there) and ends at a multiple of 4 ops (the kernel restages
+        # between 4-op words) or at the last op
         slot_of: Dict[int, int] = {}
-        if i > 0:
-            slot_of[int(tp[i - 1])] = 0
         j = i
         good = None
         while j < N:
@@ -367,16 +366,23 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
                     break
                 slot_of[ty] = len(slot_of)
             j += 1
-            if j % 4 == 0 or j == N:
+            if j == N:
                 good = (j, dict(slot_of))
+            elif j % 4 == 0:
+                nt = int(tp[j])
+                if nt in slot_of:
+                    good = (j, dict(slot_of))
+                elif len(slot_of) < slots:
+                    snap = dict(slot_of)
+                    snap[nt] = len(snap)
+                    good = (j, snap)
         if good is None:
             raise ValueError("LDS too small for a 4-op window of this op graph")
         j, slot_of = good
         for k in range(i, j):
-            prev = slot_of[int(tp[k - 1])] if k > 0 else 0
-            pos_info[k] = slot_of[int(tp[k])] | (prev << 8)
-        if j == N:
-            pos_info[N] = slot_of[int(tp[N - 1])] << 8
+            own = slot_of[int(tp[k])]
+            nxt = slot_of[int(tp[k + 1])] if k + 1 < N else own
+            pos_info[k] = own | (nxt << 8)
         for ty, sl in slot_of.items():
             win_rows.append((ty, sl * row_bytes))
         win_row_begin.append(len(win_rows))
@@ -385,16 +391,16 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
     win_pos[-1] = max((win_pos[-1] + 3) // 4 * 4, N + 1)      # never reached: no restaging after the last window
     lds_row_bytes = max(off for _, off in win_rows) + row_bytes
 
-    # flags about the previous op, seen from position i
+    # the (op k, op k + 1) pair, seen from position k
     normal = [not (shared and (int(graph.flags[t]) & (og.F_ACT_X1_5 | og.F_ACT_ZERO))) for t in range(n_types)]
-    for k in range(1, N):
-        prev_t, cur_t = int(tp[k - 1]), int(tp[k])
+    for k in range(N - 1):
+        cur_t, next_t = int(tp[k]), int(tp[k + 1])
         fl = 0
-        if normal[prev_t] and (int(graph.flags[cur_t]) & og.F_LAYER_START):
+        if normal[cur_t] and (int(graph.flags[next_t]) & og.F_LAYER_START):
             fl |= 1      # ordinary op right before a layer start: saved += 0, peak segment closes
-        if normal[prev_t]:
+        if normal[cur_t]:
             fl |= 2      # ordinary op: closes the last segment when the pair ends the stage
-        pos_info[k] |= (int(pk_of_pos[k]) << 16) | (fl << 24)
+        pos_info[k] |= (int(pk_of_pos[k + 1]) << 16) | (fl << 24)
 
     flags = 0
     if settings.resharding and (pair_kinds != 0).any():

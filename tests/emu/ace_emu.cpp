@@ -22,7 +22,6 @@ void score_one(const ace_tables_t *t, const AceGeom &g, std::vector<unsigned cha
     if (DEFER) rec = ws.data();
     s.init(g, view, h, range);
     int w = 0, next_win = t->win_pos[0];
-    uint32_t pbyte = 0;
     for (int i = 0; i < g.N; ++i) {
         if (i == next_win) {
             // poison, then stage exactly the rows the window lists: a read of any other row yields NaN
@@ -31,15 +30,13 @@ void score_one(const ace_tables_t *t, const AceGeom &g, std::vector<unsigned cha
                 memcpy(lds.data() + t->win_rows[2 * r + 1], t->rows + (size_t)t->win_rows[2 * r] * t->row_doubles, row_bytes);
             next_win = t->win_pos[++w];
         }
-        s.step(g, view, i, codes[i], pbyte, i + 1 < g.N ? codes[i + 1] : 0x10u, pos[i], pos[i + 1], rec);
-        pbyte = codes[i];
+        if (!RANGED && i == 0) s.begin(g, view, 0, codes[0], pos[0]);
+        s.step(g, view, i, codes[i], i + 1 < g.N ? codes[i + 1] : 0x10u, pos[i], rec);
     }
     if (DEFER) {
-        s.stash(rec, (uint32_t)(g.N - 1), pbyte & 7u);
-        const int n_st = s.s + 1;
+        const int n_st = s.s;
         for (int s2 = 0; s2 < n_st && s2 < ACE_MAX_STAGES; ++s2) s.replay(g, view, pos, rec, s2);
-    } else if (!RANGED || !s.done) {
-        s.finish(g, view, info_prevrow(g, pos[g.N]), pbyte & 7u, rec);
+        s.s = n_st;              // replay() walks s again; result() checks the count of the op loop
     }
     s.result(g, t->nb_minus_1[s.bidx], iter, peak, feas, st);
 }

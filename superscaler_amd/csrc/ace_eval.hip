@@ -103,9 +103,7 @@ __global__ __launch_bounds__(kBlock) void ace_score_kernel(const AceKernelArgs a
     int next_win = WIN ? a.win_pos[1] : 0x7fffffff;
     ace_u4 cw = a.codes[pl];                 // sixteen op bytes of this plan
     if (!RANGED) st.begin(g, lds, 0, cw.x & 0xffu, a.pos_info[0]);
-    // the byte after the last op reads as "a stage starts here": that is what ends the last stage
-    const int end_word = g.N >> 2;
-    const uint32_t end_bit = 0x10u << (8 * (g.N & 3));
+    uint32_t pinfo = 0;                      // descriptor of the previous group's last position
     for (int grp = 0; grp < g.G; ++grp) {
         const int base = grp << 4;
         // the sixteen position descriptors of this group: scalar loads (the array is padded)
@@ -115,9 +113,14 @@ __global__ __launch_bounds__(kBlock) void ace_score_kernel(const AceKernelArgs a
                                     i2.x, i2.y, i2.z, i2.w, i3.x, i3.y, i3.z, i3.w};
         ace_u4 nxt = ace_u4{0u, 0u, 0u, 0u};
         if (grp + 1 < g.G) nxt = a.codes[(size_t)(grp + 1) * g.P + pl];
-        uint32_t words[5] = {cw.x, cw.y, cw.z, cw.w, nxt.x};
+        const uint32_t words[5] = {cw.x, cw.y, cw.z, cw.w, nxt.x};
+        // pair_bit() of the sixteen (op, next op) pairs, four at a time: bit 0 of each byte
+        uint32_t pairs[4];
 #pragma unroll
-        for (int j = 0; j < 5; ++j) words[j] |= ((base >> 2) + j == end_word) ? end_bit : 0u;
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t nw = (words[j] >> 8) | (words[j + 1] << 24);      // the next-op bytes of word j
+            pairs[j] = ((words[j] & nw) >> 3) & ~(nw >> 4) & 0x01010101u;
+        }
 #pragma unroll
         for (int k = 0; k < 16; ++k) {
             const int i = base + k;
@@ -131,10 +134,13 @@ __global__ __launch_bounds__(kBlock) void ace_score_kernel(const AceKernelArgs a
             }
             if (i < g.N) {
                 const uint32_t byte = (words[k >> 2] >> (8 * (k & 3))) & 0xffu;
+                // (past the last op the code bytes are zero padding)
                 const uint32_t nbyte = (words[(k + 1) >> 2] >> (8 * ((k + 1) & 3))) & 0xffu;
-                st.step(g, lds, i, byte, nbyte, infos[k], rec);
+                const uint32_t pair = (pairs[k >> 2] >> (8 * (k & 3))) & 1u;
+                st.step(g, lds, i, byte, nbyte, pair, infos[k], k ? infos[k - 1] : pinfo, i + 1 == g.N, rec);
             }
         }
+        pinfo = infos[15];
         cw = nxt;
     }
     if (DEFER) {

@@ -60,11 +60,20 @@ ACE_HD bool ace_isnan(double a) { return a != a; }
 // product of two values below 2^24 (a single full-rate instruction on the GPU)
 #ifdef ACE_HOST_EMU
 ACE_HD uint32_t ace_mul24(uint32_t a, uint32_t b) { return a * b; }
+ACE_HD uint32_t ace_mad24(uint32_t a, uint32_t b, uint32_t c) { return a * b + c; }
 ACE_HD double ace_fma(double a, double b, double c) { return std::fma(a, b, c); }
 #else
 ACE_HD uint32_t ace_mul24(uint32_t a, uint32_t b) { return __umul24(a, b); }
+ACE_HD uint32_t ace_mad24(uint32_t a, uint32_t b, uint32_t c) { return __umul24(a, b) + c; }
 ACE_HD double ace_fma(double a, double b, double c) { return __builtin_fma(a, b, c); }
 #endif
+// 1.0 or 0.0 from a wave-uniform flag, built from integer words so that it stays in scalar registers
+ACE_HD double ace_scalar_01(bool one) {
+    const uint64_t bits = (uint64_t)(one ? 0x3ff00000u : 0u) << 32;
+    double d;
+    __builtin_memcpy(&d, &bits, 8);
+    return d;
+}
 
 struct alignas(16) ace_d2 { double x, y; };
 struct alignas(16) ace_u4 { uint32_t x, y, z, w; };
@@ -120,6 +129,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
     uint32_t first_meta;        // DEFER: first op of the current stage: position | code << 16
     ace_u2 lut_next;            // stage LUT entry of the NEXT stage, fetched one stage ahead
     uint32_t r_next;            // collective ids of the (previous op, this op) pair, fetched one op ahead
+    uint32_t pair_prev;         // pair_bit of the (previous op, this op) pair
     // plan accumulators
     double sum_t, max_t, max_mem;
     uint32_t status;
@@ -134,7 +144,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         s = -1;
         sum_t = 0.0; max_t = 0.0; max_mem = 0.0;
         status = 0;
-        lastclose = false; first_meta = 0; r_next = 0;
+        lastclose = false; first_meta = 0; r_next = 0; pair_prev = 0;
         lut_next = ace_u2{0u, 0u};
         fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = rs_f = rs_b = 0.0;
         id_fwd = id_bwd = id_in = 0.0;
@@ -280,12 +290,12 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         else start_lookups(g, lds, info_row(g, info), byte & 7u);
     }
 
-    // One op at position i.  `byte` is its code byte, `nbyte` the next op's (0x10 after the last op: the plan's last stage ends there),
-    // `info` the position's (wave-uniform) descriptor.  Everything that concerns the (this op, next op)
+    // One op at position i.  `byte` is its code byte, `nbyte` the next op's (0 after the last op, where `plan_end` is set instead),
+    // `pair` = pair_bit(byte, nbyte), `info` / `pinfo` this and the previous position's (wave-uniform) descriptors.  Everything that concerns the (this op, next op)
     // pair is handled here too, so nothing but the accumulators is carried from op to op; a stage
     // that ends with this op is closed (and the next one opened) in the middle of the step.
-    ACE_HD void step(const AceGeom &g, const AceLds &lds, int i, uint32_t byte, uint32_t nbyte, uint32_t info,
-                     double *rec) {
+    ACE_HD void step(const AceGeom &g, const AceLds &lds, int i, uint32_t byte, uint32_t nbyte, uint32_t pair,
+                     uint32_t info, uint32_t pinfo, bool plan_end, double *rec) {
         if (RANGED) {
             if (i < lo || i >= hi) return;
             if (i == lo) begin(g, lds, i, byte, info);
@@ -294,8 +304,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         const uint32_t nc = nbyte & 7u;
         const bool rc = (byte >> 3) & 1u;
         const uint32_t row = info_row(g, info);
-        const uint32_t fl = info >> 24;
-        uint32_t a = row + g.hot_off + hot_v + c * ACE_HOT_STRIDE;
+        const uint32_t a = (row + g.hot_off) + ace_mad24(c, ACE_HOT_STRIDE, hot_v);
         ace_d2 e0 = lds.ld<ace_d2>(a);         // fwd us, bwd us
         ace_d2 e1 = lds.ld<ace_d2>(a + 16);    // weights MB, activations MB (shared-buffer rule applied)
         ace_d2 e2 = lds.ld<ace_d2>(a + 32);    // fwd / bwd reserved MB
@@ -315,14 +324,16 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
             // first op) adds 0.0, and the id past the last real table is all NaN (the reference raises there)
             const uint32_t r = r_next;
             const uint32_t pk = (info >> 16) & 0xffu;
-            r_next = lds.ld<uint8_t>(g.rk_lds_off + ace_mul24(pk, g.rk_kind_stride) + rk_v + ((c << 3) | nc));
-            const uint32_t za = row + g.z_off + z_v + c * 8u;
+            r_next = lds.ld<uint8_t>((g.rk_lds_off + ace_mul24(pk, g.rk_kind_stride)) + (rk_v + ((c << 3) | nc)));
+            const uint32_t za = (row + g.z_off) + (z_v + c * 8u);
             rs_f += lds.ld<double>(za + ((r & 15u) << g.z_shift));
             rs_b += lds.ld<double>(za + ((r >> 4) << g.z_shift));
         }
         // the stage ends with this op
-        const bool last = RANGED ? (i + 1 == hi) : (bool)((nbyte >> 4) & 1u);
+        const bool last = RANGED ? (i + 1 == hi) : (((nbyte >> 4) & 1u) || plan_end);
         if (last) {
+            // :439 "i + 1 == len(ops) - 1": the (previous, this) pair closes the last segment
+            lastclose = pair_prev & (pinfo >> 25) & 1u;
             if (DEFER) stash(rec, (uint32_t)i, c);
             else finish(g, lds, row, c, rec);
             if (!RANGED) {
@@ -336,20 +347,19 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         }
         rfm = ace_max(rfm, e2.x);
         rbm = ace_max(rbm, e2.y);
-        // (this op, next op) both recomputed and in one stage
-        const bool pair = ((byte & nbyte) >> 3) & ~(nbyte >> 4) & 1u;
-        const bool savez = fl & 1u;     // this is an ordinary op followed by a layer start
+        // pair: (this op, next op) both recomputed and in one stage
+        const bool savez = (info >> 24) & 1u;     // this is an ordinary op followed by a layer start
         // All of this is arithmetic on 0.0 / 1.0 factors instead of selects: x*1.0 and x+0.0 are exact,
         // so every value is the one the reference computes.  (After a stage end the accumulators
         // are zero and pair is false: nothing happens.)
         const double pairf = (double)(int)pair;
-        const double keepf = pairf * (savez ? 0.0 : 1.0);         // 1.0 iff the pair continues the running segment
+        const double keepf = pairf * ace_scalar_01(!savez);       // 1.0 iff the pair continues the running segment
         run = ace_fma(pairf, e1.y, run);                          // run += act             if pair
         saved = ace_fma(keepf, e1.y, saved);                      // saved += act           if pair and not savez
         const double closed = run * (1.0 - keepf);                // run if the segment closes here, else 0.0
         peak = ace_max(peak, closed);                             // max(peak, 0.0) leaves peak (>= 0) alone
         run = run - closed;                                       // 0.0 if closed, else run
-        lastclose = pair && (fl & 2u);
+        pair_prev = pair;
     }
 
     ACE_HD void result(const AceGeom &g, double nbm1, double &iter_ms, double &peak_mb, uint8_t &feasible, uint8_t &st) {
@@ -369,6 +379,9 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         }
     }
 };
+
+// 1 iff two consecutive ops (code bytes a, b) are both recomputed and b does not start a stage
+ACE_HD uint32_t pair_bit(uint32_t a, uint32_t b) { return ((a & b) >> 3) & ~(b >> 4) & 1u; }
 
 // byte k (0..15) of a 16-op group held in four 32-bit words
 ACE_HD uint32_t group_byte(const uint32_t w[4], int k) { return (w[k >> 2] >> ((k & 3) * 8)) & 0xffu; }

@@ -31,7 +31,8 @@ void score_one(const ace_tables_t *t, const AceGeom &g, std::vector<unsigned cha
             next_win = t->win_pos[++w];
         }
         if (!RANGED && i == 0) s.begin(g, view, 0, codes[0], pos[0]);
-        s.step(g, view, i, codes[i], i + 1 < g.N ? codes[i + 1] : 0x10u, pos[i], rec);
+        const uint32_t nbyte = i + 1 < g.N ? codes[i + 1] : 0u;
+        s.step(g, view, i, codes[i], nbyte, pair_bit(codes[i], nbyte), pos[i], i > 0 ? pos[i - 1] : 0u, i + 1 == g.N, rec);
     }
     if (DEFER) {
         const int n_st = s.s;

@@ -69,7 +69,8 @@ typedef struct ace_tables {
     int32_t num_ops;        /* N: positions in the op sequence */
     int32_t num_types;      /* distinct op names (table rows) */
     int32_t n_mbs, n_tp, n_algo;
-    int32_t n_diag;         /* distinct (micro_bs, stage gpus) -> per-tp micro-batch index maps */
+    int32_t n_diag;         /* distinct (micro_bs, stage gpus) -> per-tp micro-batch index maps, at most 14;
+                               the hot sub-table holds n_diag + 1 (the last one all NaN) */
     int32_t n_glog;         /* stage device counts 2^0 .. 2^(n_glog-1) */
     int32_t n_z;            /* resharding cost tables: table 0 is all zeros (nothing to pay), then one per
                                (collective, group size) in use, the last one all NaN (the reference raises) */
@@ -87,8 +88,9 @@ typedef struct ace_tables {
                                       ordinary op followed by a layer start, bit 25 = an ordinary op
                                       (a slot is row_doubles * 8 bytes; the last entry is unused) */
     const uint8_t *pair_kinds;     /* [n_pair_kinds][n_glog][8][8] (first op's code, second op's code) */
-    const uint32_t *stage_lut;     /* [n_mbs][16][2]: hot byte offset of the diag | pair-kind offset << 16;
-                                      diag * C | per-tp mbs-index nibbles << 16 (C = n_tp * n_algo) */
+    const uint32_t *stage_lut;     /* [n_mbs][16] by log2(stage gpus): diag | per-tp mbs-index nibbles << 16;
+                                      diag n_diag = the all-NaN entries after the hot sub-table (a pair the
+                                      reference raises KeyError for) */
     const double *nb_minus_1;      /* [n_mbs]: global_bs // micro_bs - 1 */
     const int32_t *win_pos;        /* [n_windows + 1] first position of each window (multiples of 4) */
     const int32_t *win_row_begin;  /* [n_windows + 1] into win_rows */

@@ -442,7 +442,7 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     *out = nullptr;
     if (t->abi_version != ACE_ABI_VERSION) return ACE_EVERSION;
     if (t->num_ops <= 0 || t->num_types <= 0 || t->n_mbs <= 0 || t->n_mbs > 15 || t->n_tp <= 0 || t->n_tp > 4 ||
-        (t->n_algo != 1 && t->n_algo != 2) || t->n_diag <= 0 || t->n_diag > 254 || t->n_glog <= 0 || t->n_glog > 16 ||
+        (t->n_algo != 1 && t->n_algo != 2) || t->n_diag <= 0 || t->n_diag > 14 || t->n_glog <= 0 || t->n_glog > 16 ||
         t->n_z < 0 || t->n_z == 1 || t->n_z > 15 || ((t->flags & ACE_F_RESHARDING) && t->n_z < 2) || t->z_table_doubles <= 0 || (t->z_table_doubles & (t->z_table_doubles - 1)) || t->n_pair_kinds <= 0 || t->n_pair_kinds > 255 || t->row_doubles <= 0 ||
         (t->row_doubles & 1) || t->n_windows <= 0 || t->lds_row_bytes <= 0 || (t->lds_row_bytes & 15) ||
         !t->rows || !t->pos_info || !t->pair_kinds || !t->stage_lut || !t->nb_minus_1 || !t->win_pos ||
@@ -450,7 +450,7 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
         return ACE_EINVAL;
     const int C = t->n_tp * t->n_algo;
     // sub-tables must lie inside a row and be 16-byte aligned
-    const int64_t hot_end = (int64_t)t->hot_off + (int64_t)t->n_diag * C * 6;
+    const int64_t hot_end = (int64_t)t->hot_off + (int64_t)(t->n_diag + 1) * C * 6;
     const int64_t start_end = (int64_t)t->start_off + (int64_t)t->n_diag * C * 4;
     const int64_t out_end = (int64_t)t->out_off + (int64_t)t->n_mbs * t->n_tp * t->n_algo * 2;
     const int64_t z_end = (int64_t)t->z_off + (int64_t)t->n_z * t->z_table_doubles;
@@ -462,7 +462,7 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     const int64_t row_bytes = (int64_t)t->row_doubles * 8;
     if (row_bytes > t->lds_row_bytes || t->lds_row_bytes > (int32_t)kMaxLds) return ACE_ETOOBIG;
     const int32_t rk_bytes = t->n_pair_kinds * t->n_glog * 64;
-    const int32_t stg_words = t->n_mbs * 16 * 2;
+    const int32_t stg_words = t->n_mbs * 16;
     const uint32_t rk_off = (uint32_t)t->lds_row_bytes;
     const uint32_t stg_off = (rk_off + (uint32_t)rk_bytes + 15u) & ~15u;
     const uint32_t lds_bytes = stg_off + (uint32_t)stg_words * 4u;
@@ -486,12 +486,9 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
             ((pi >> 16) & 0xffu) >= (uint32_t)t->n_pair_kinds)
             return ACE_EINVAL;
     }
-    for (int j = 0; j < stg_words; j += 2) {
-        // (hot offset, diag * C) of every (micro-batch, stage size) pair must address C entries inside the row
-        const int64_t hot_v = t->stage_lut[j] & 0xffffu, rk_v = t->stage_lut[j] >> 16, dc = t->stage_lut[j + 1] & 0xffffu;
-        if ((hot_v & 15) || (int64_t)t->hot_off * 8 + hot_v + (int64_t)C * 48 > row_bytes || dc + C > (int64_t)t->n_diag * C ||
-            (rk_v & 63) || rk_v / 64 >= t->n_glog)
-            return ACE_EINVAL;
+    for (int j = 0; j < stg_words; ++j) {
+        // the diag of every (micro-batch, stage size) pair must exist (n_diag = the all-NaN one)
+        if ((t->stage_lut[j] & 0xffffu) > (uint32_t)t->n_diag) return ACE_EINVAL;
     }
     for (int j = 0; j < rk_bytes; ++j) {
         const uint32_t lim = t->n_z ? (uint32_t)t->n_z : 1u;

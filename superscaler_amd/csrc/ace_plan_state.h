@@ -64,12 +64,20 @@ ACE_HD uint32_t ace_mad24(uint32_t a, uint32_t b, uint32_t c) { return a * b + c
 ACE_HD double ace_fma(double a, double b, double c) { return std::fma(a, b, c); }
 #else
 ACE_HD uint32_t ace_mul24(uint32_t a, uint32_t b) { return __umul24(a, b); }
-ACE_HD uint32_t ace_mad24(uint32_t a, uint32_t b, uint32_t c) { return __umul24(a, b) + c; }
+ACE_HD uint32_t ace_mad24(uint32_t a, uint32_t b, uint32_t c) {
+    uint32_t r = __umul24(a, b) + c;
+    asm("" : "+v"(r));          // one v_mad_u32_u24; without this the sum is re-associated into three instructions
+    return r;
+}
 ACE_HD double ace_fma(double a, double b, double c) { return __builtin_fma(a, b, c); }
 #endif
 // 1.0 or 0.0 from a wave-uniform flag, built from integer words so that it stays in scalar registers
 ACE_HD double ace_scalar_01(bool one) {
-    const uint64_t bits = (uint64_t)(one ? 0x3ff00000u : 0u) << 32;
+    uint32_t hi = one ? 0x3ff00000u : 0u;
+#ifndef ACE_HOST_EMU
+    asm("" : "+s"(hi));         // keeps the compiler from turning the product below into per-lane selects
+#endif
+    const uint64_t bits = (uint64_t)hi << 32;
     double d;
     __builtin_memcpy(&d, &bits, 8);
     return d;
@@ -127,7 +135,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
     double id_fwd, id_bwd;
     bool lastclose;
     uint32_t first_meta;        // DEFER: first op of the current stage: position | code << 16
-    ace_u2 lut_next;            // stage LUT entry of the NEXT stage, fetched one stage ahead
+    uint64_t diags;             // the diag of every stage, 4 bits each, looked up once per plan
     uint32_t r_next;            // collective ids of the (previous op, this op) pair, fetched one op ahead
     uint32_t pair_prev;         // pair_bit of the (previous op, this op) pair
     // plan accumulators
@@ -145,7 +153,6 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         sum_t = 0.0; max_t = 0.0; max_mem = 0.0;
         status = 0;
         lastclose = false; first_meta = 0; r_next = 0; pair_prev = 0;
-        lut_next = ace_u2{0u, 0u};
         fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = rs_f = rs_b = 0.0;
         id_fwd = id_bwd = id_in = 0.0;
         in_comm = inputs = 0.0;
@@ -154,35 +161,37 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         ideal_hot_v = ideal_start_v = 0;
         if (bidx >= (uint32_t)g.n_mbs) { status = ACE_PLAN_MALFORMED; bidx = 0; }
         if (RANGED && (lo < 0 || hi > g.N || lo >= hi)) { status = ACE_PLAN_MALFORMED; lo = 0; hi = 1; }
-        lut_next = lds.ld<ace_u2>(g.stg_lds_off + (bidx * 16u + ((uint32_t)glogs & 15u)) * 8u);
+        // one LUT read per possible stage now, none where a stage begins (where few lanes are active)
+        diags = 0;
+        for (uint32_t k = 0; k < ACE_MAX_STAGES; ++k) {
+            uint32_t glog = (uint32_t)(glogs >> (4u * k)) & 15u;
+            uint32_t w = lds.ld<uint32_t>(g.stg_lds_off + (bidx * 16u + glog) * 4u);
+            diags |= (uint64_t)(w & 15u) << (4u * k);
+        }
         if (BD) {
             // the "ideal" pass uses tp = dp = 1 and micro-batch = micro_bs (aceso_cost_model.py:588-590):
             // the diag of (micro_bs, 1 gpu)
-            ace_u2 w = lds.ld<ace_u2>(g.stg_lds_off + (bidx * 16u + 0u) * 8u);
-            ideal_hot_v = w.x & 0xffffu;
-            ideal_start_v = (w.y & 0xffffu) * ACE_START_STRIDE;
+            uint32_t d = lds.ld<uint32_t>(g.stg_lds_off + (bidx * 16u + 0u) * 4u) & 15u;
+            ideal_hot_v = ace_mul24(d, (uint32_t)g.C * ACE_HOT_STRIDE);
+            ideal_start_v = ace_mul24(d, (uint32_t)g.C * ACE_START_STRIDE);
         }
     }
 
     // Stage head, part 1: the per-stage offsets the op loop needs, accumulators back to zero.
-    ACE_HD void start_fast(const AceGeom &g, const AceLds &lds, bool pipelined) {
+    // `tail`: also what only finish() uses (one LDS read).
+    ACE_HD void start_fast(const AceGeom &g, const AceLds &lds, bool tail) {
         ++s;
-        // (a plan with more than 16 stage bits is caught by result(): s + 1 != S)
-        ace_u2 w;
-        if (pipelined) {
-            // this stage's LUT entry was fetched when the previous stage began; fetch the next one now
-            w = lut_next;
-            uint32_t glog_n = (uint32_t)(glogs >> (4u * ((uint32_t)(s + 1) & 15u))) & 15u;
-            lut_next = lds.ld<ace_u2>(g.stg_lds_off + (bidx * 16u + glog_n) * 8u);
-        } else {
-            uint32_t glog = (uint32_t)(glogs >> (4u * ((uint32_t)s & 15u))) & 15u;
-            w = lds.ld<ace_u2>(g.stg_lds_off + (bidx * 16u + glog) * 8u);
+        // (a plan with more than 16 stage bits is caught by result())
+        const uint32_t sh = 4u * ((uint32_t)s & 15u);
+        const uint32_t d = (uint32_t)(diags >> sh) & 15u;
+        const uint32_t glog = (uint32_t)(glogs >> sh) & 15u;
+        hot_v = ace_mul24(d, (uint32_t)g.C * ACE_HOT_STRIDE);
+        z_v = ace_mul24(d, (uint32_t)g.C * 8u);
+        rk_v = glog << 6;
+        if (tail) {
+            dc_v = ace_mul24(d, (uint32_t)g.C);
+            mrow = lds.ld<uint32_t>(g.stg_lds_off + (bidx * 16u + glog) * 4u) >> 16;
         }
-        hot_v = w.x & 0xffffu;
-        rk_v = w.x >> 16;
-        dc_v = w.y & 0xffffu;
-        mrow = w.y >> 16;
-        z_v = dc_v << 3;
         fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = rs_f = rs_b = 0.0;
         lastclose = false;
         r_next = 0;             // a stage's first op pays no resharding
@@ -224,7 +233,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         const ace_d2 *r = reinterpret_cast<const ace_d2 *>(ws + (size_t)s2 * ACE_WS_REC);
         ace_d2 r0 = r[0], r1 = r[1], r2 = r[2], r3 = r[3], r4 = r[4], r5 = r[5], r6 = r[6];
         s = s2 - 1;
-        start_fast(g, lds, false);             // s = s2; per-stage offsets, mrow
+        start_fast(g, lds, true);              // s = s2; per-stage offsets, mrow
         uint64_t meta;
         __builtin_memcpy(&meta, &r6.x, 8);
         uint32_t lo32 = (uint32_t)meta, i_last = (uint32_t)(meta >> 32);
@@ -285,7 +294,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
     // Head of the plan's first stage (RANGED: of the queried stage); `byte` / `info` belong to its first op.
     ACE_HD void begin(const AceGeom &g, const AceLds &lds, int i, uint32_t byte, uint32_t info) {
         if (!(byte & 0x10u)) status = ACE_PLAN_MALFORMED;    // the first op must open a stage
-        start_fast(g, lds, true);
+        start_fast(g, lds, !DEFER);
         if (DEFER) first_meta = (uint32_t)i | ((byte & 7u) << 16);
         else start_lookups(g, lds, info_row(g, info), byte & 7u);
     }
@@ -338,7 +347,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
             else finish(g, lds, row, c, rec);
             if (!RANGED) {
                 // (after the plan's last op this opens a stage that stays empty: s == S in the end)
-                start_fast(g, lds, true);
+                start_fast(g, lds, !DEFER);
                 if (DEFER) first_meta = (uint32_t)(i + 1) | (nc << 16);
                 else if (i + 1 < g.N) start_lookups(g, lds, info_nextrow(g, info), nc);
             }

@@ -24,9 +24,8 @@ maxima of table entries:
      ids (0 = the all-zero table: nothing to do, last id = the all-NaN table: the reference would
      raise) for an adjacent op
      pair, from get_op_spec / get_reshard_primitives (model_ops_info.py:92-150, cost_model:185-245)
-  stage_lut[mbs index][glog]  two words: hot-table byte offset of the diag | pair-kind offset of the
-     stage size << 16;  diag * n_codes | per-tp mbs-index nibbles << 16 (0xF = not profiled).
-     Unscorable (micro-batch, stage size) pairs point at one extra diag that is all NaN.
+  stage_lut[mbs index][glog]  diag | per-tp mbs-index nibbles << 16 (0xF = not profiled).
+     Unscorable (micro-batch, stage size) pairs point at diag n_diag, whose hot entries are all NaN.
   pos_info[i]  LDS slot of op i's row | slot of op i+1's row << 8 | kind of the (i, i+1) pair << 16 | flags << 24
 """
 import ctypes
@@ -86,7 +85,7 @@ class CompiledTables:
     rows: np.ndarray            # float64 [n_types, row_doubles]
     pos_info: np.ndarray        # uint32 [N + 1]
     pair_kinds: np.ndarray      # uint8 [n_pk, n_glog, 8, 8]
-    stage_lut: np.ndarray       # uint32 [n_mbs, 16, 2]
+    stage_lut: np.ndarray       # uint32 [n_mbs, 16]
     nb_minus_1: np.ndarray      # float64 [n_mbs]
     win_pos: np.ndarray         # int32 [n_win + 1]
     win_row_begin: np.ndarray   # int32 [n_win + 1]
@@ -127,7 +126,7 @@ class CompiledTables:
 
     # what a (micro_bs index, log2 stage gpus) pair allows
     def allowed_tp_logs(self, bidx: int, glog: int) -> List[int]:
-        mrow = int(self.stage_lut[bidx, glog, 1]) >> 16
+        mrow = int(self.stage_lut[bidx, glog]) >> 16
         return [t for t in range(len(self.db.tp_list)) if ((mrow >> (4 * t)) & 15) != 15]
 
 
@@ -270,36 +269,31 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
 
     # ---- rows ------------------------------------------------------------------------------
     hot_off = 0
-    start_off = hot_off + ND * C * 6
+    start_off = hot_off + (ND + 1) * C * 6      # diag ND: all NaN, where unscorable (micro-batch, stage size) pairs point
     out_off = start_off + ND * C * 4
     z_off = out_off + M * T * A * 2
     z_table_doubles = 1
     while z_table_doubles < ND * C:
         z_table_doubles *= 2          # one collective's table, padded so its index is a shift
-    # a block of C hot entries that are all NaN: where unscorable (micro-batch, stage size) pairs point
-    nan_off = z_off + NZ * z_table_doubles
-    row_doubles = nan_off + C * 6
+    row_doubles = z_off + NZ * z_table_doubles
     row_doubles += row_doubles & 1
-    if (row_doubles * 8) > 0xFFFF:
-        raise ValueError("an op type's row exceeds what the stage LUT addresses")
-    # stage LUT: [mbs][glog] -> (hot byte offset | pair-kind glog offset << 16, diag * C | mrow << 16)
-    stage_lut = np.zeros((M, 16, 2), dtype=np.uint32)
+    if ND > 14:
+        raise ValueError("more than 14 distinct micro-batch maps: a plan packs one 4-bit diag per stage")
+    # stage LUT: [mbs][glog] -> diag | mrow << 16
+    stage_lut = np.zeros((M, 16), dtype=np.uint32)
     for bi in range(M):
         for glog in range(16):
             d = int(lut_diag[bi, glog])
-            rk_v = glog * CP * CP if glog < n_glog else 0
             if d < 0:
-                stage_lut[bi, glog, 0] = ((nan_off - hot_off) * 8) | (rk_v << 16)
-                stage_lut[bi, glog, 1] = 0 | (0xFFFF << 16)
+                stage_lut[bi, glog] = ND | (0xFFFF << 16)
             else:
-                stage_lut[bi, glog, 0] = (d * C * 48) | (rk_v << 16)
-                stage_lut[bi, glog, 1] = (d * C) | (int(lut_mrow[bi, glog]) << 16)
+                stage_lut[bi, glog] = d | (int(lut_mrow[bi, glog]) << 16)
     rows = np.zeros((n_types, row_doubles), dtype=np.float64)
     nan = math.nan
     reserved_on = settings.consider_reserved_space
     for ty, name in enumerate(db.op_names):
         fl = int(graph.flags[ty])
-        hot = np.full((ND, C, 6), nan)
+        hot = np.full((ND + 1, C, 6), nan)
         start = np.full((ND, C, 4), nan)
         z = np.full((max(NZ, 1), ND, C), nan)
         z[0] = 0.0
@@ -335,7 +329,6 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
         for k in range(NZ):
             rows[ty, z_off + k * z_table_doubles:z_off + (k + 1) * z_table_doubles] = nan if k == NZ - 1 else 0.0
             rows[ty, z_off + k * z_table_doubles:z_off + k * z_table_doubles + ND * C] = z[k].ravel()
-        rows[ty, nan_off:nan_off + C * 6] = nan
 
     # ---- LDS residency: one window if every row fits, else windows over op positions ----------
     row_bytes = row_doubles * 8

@@ -62,7 +62,7 @@ extern "C" int ace_emu_score(const ace_tables_t *t, const uint8_t *codes /* [P][
     g.stg_lds_off = (g.rk_lds_off + (uint32_t)rk_bytes + 15u) & ~15u;
     g.rk_kind_stride = (uint32_t)(t->n_glog * 64);
     g.row_bytes = (uint32_t)t->row_doubles * 8u;
-    const uint32_t lds_bytes = g.stg_lds_off + (uint32_t)t->n_mbs * 16u * 8u;
+    const uint32_t lds_bytes = g.stg_lds_off + (uint32_t)t->n_mbs * 16u * 4u;
     g.flags = t->flags; g.main_params = t->main_params; g.optimizer = t->optimizer;
     g.mem_limit = memory_limit; g.strict = strict ? 1 : 0;
     if (range && !stage_out) return -1;
@@ -71,7 +71,7 @@ extern "C" int ace_emu_score(const ace_tables_t *t, const uint8_t *codes /* [P][
     for (long long p = 0; p < P; ++p) {
         memset(lds.data(), 0xff, lds.size());
         memcpy(lds.data() + g.rk_lds_off, t->pair_kinds, rk_bytes);
-        memcpy(lds.data() + g.stg_lds_off, t->stage_lut, (size_t)t->n_mbs * 16 * 8);
+        memcpy(lds.data() + g.stg_lds_off, t->stage_lut, (size_t)t->n_mbs * 16 * 4);
         ace_u4 h;
         memcpy(&h, hdr + 4 * p, 16);
         ace_u2 rg{0u, 0u};

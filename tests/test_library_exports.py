@@ -45,7 +45,7 @@ def test_error_strings_and_argument_checks():
     assert lib.ace_create(ctypes.byref(bad), ctypes.byref(h)) == -1  # geometry the encoding cannot hold
     bad = tables.as_struct()
     lut = tables.stage_lut.copy()
-    lut[0, 0, 0] = 0xFFF0                                           # hot offset far outside the row
+    lut[0, 0] = 0xFFF0                                              # a diag the tables do not have
     bad.stage_lut = lut.ctypes.data
     assert lib.ace_create(ctypes.byref(bad), ctypes.byref(h)) == -1
     assert lib.ace_topk_workspace_bytes(1 << 20, 64) > 0

@@ -144,11 +144,51 @@ def make_neighbours(base: PlanBatch, tables: CompiledTables, n: int, rng: np.ran
     return PlanBatch(codes, hdr)
 
 
+class VisitedPlans:
+    """The search's visited set (aceso_search.py:47,105 over aceso_utils.py:831-844) in array form.
+
+    The reference keys on the config_details string: per-stage op counts, tp, dp, recompute flags,
+    algos and the micro-batch size.  For one op graph the encoded bytes of a plan (its code row and
+    the first three header words; the fourth, the cross-node bits, follows from them) carry exactly
+    that information, so two plans have the same string iff these bytes are equal."""
+
+    def __init__(self):
+        self._seen = set()
+
+    def __len__(self):
+        return len(self._seen)
+
+    @staticmethod
+    def keys(batch: PlanBatch) -> np.ndarray:
+        """One fixed-size bytes key per plan (a numpy void array; equal keys = equal plans)."""
+        raw = np.concatenate([np.ascontiguousarray(batch.codes),
+                              np.ascontiguousarray(batch.hdr[:, :3]).view(np.uint8).reshape(batch.n_plans, 12)], axis=1)
+        return np.ascontiguousarray(raw).view(np.dtype((np.void, raw.shape[1]))).ravel()
+
+    def unseen(self, batch: PlanBatch) -> np.ndarray:
+        """Mask of the plans that were not marked before and do not repeat an earlier row of this batch."""
+        keys = self.keys(batch)
+        _, first = np.unique(keys, return_index=True)
+        mask = np.zeros(batch.n_plans, dtype=bool)
+        mask[first] = True
+        if self._seen:
+            for p in np.flatnonzero(mask):
+                if keys[p].tobytes() in self._seen:
+                    mask[p] = False
+        return mask
+
+    def mark(self, batch: PlanBatch, rows=None) -> None:
+        keys = self.keys(batch)
+        for p in (range(batch.n_plans) if rows is None else rows):
+            self._seen.add(keys[int(p)].tobytes())
+
+
 def hill_climb(cm, start: PlanBatch, steps: int, n_neighbours: int, seed: int = 0, max_move: int = 8,
-               on_step=None) -> Tuple[PlanBatch, float, float]:
+               on_step=None, visited: VisitedPlans = None) -> Tuple[PlanBatch, float, float]:
     """Best-neighbour descent: at every step n_neighbours single-move neighbours of the current plan
-    are scored in one launch and the fastest feasible one replaces it if it is faster.
-    Returns (plan, iteration ms, peak MB)."""
+    are scored in one launch and the fastest feasible one replaces it if it is faster.  With a
+    `visited` set, neighbours seen in an earlier step (or twice in one step) are dropped before
+    scoring, as aceso_search.py:47 does.  Returns (plan, iteration ms, peak MB)."""
     rng = np.random.default_rng(seed)
     tables = cm.tables
     ev = cm.evaluator
@@ -156,8 +196,18 @@ def hill_climb(cm, start: PlanBatch, steps: int, n_neighbours: int, seed: int = 
     it, pk, fe, st = ev.score_host(cur)
     cur_t = float(it[0]) if fe[0] else float("inf")
     cur_m = float(pk[0])
+    if visited is not None:
+        visited.mark(cur)
     for step in range(steps):
         nb = make_neighbours(cur, tables, n_neighbours, rng, max_move)
+        if visited is not None:
+            keep = np.flatnonzero(visited.unseen(nb))
+            if len(keep) == 0:
+                if on_step is not None:
+                    on_step(step, cur_t, cur_m)
+                continue
+            nb = PlanBatch(np.ascontiguousarray(nb.codes[keep]), np.ascontiguousarray(nb.hdr[keep]))
+            visited.mark(nb)
         d = ev.upload(nb, validate=False)
         it, pk, fe, st = ev.score(d)
         idx, val, cnt = ev.topk(it, fe, 1)

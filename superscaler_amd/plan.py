@@ -80,6 +80,36 @@ def config_from_json(path_or_dict, full_op_list) -> AcesoConfig:
                       d["micro_batch_size"], d["global_batch_size"], full_op_list, flat(d["algo_of_each_op"]))
 
 
+def config_details(config, get_string=False):
+    """Per-stage op counts, tp, dp, recompute, micro-batch and algo of a plan, as the reference's
+    visited sets key on (aceso_utils.py:117-135; same string when get_string is set)."""
+    if config is None:
+        return ""
+    num_ops_stage = [len(st.ops) for st in config.stages[:config.num_stages]]
+    tp_size_list = [st.tp_size for st in config.stages[:config.num_stages]]
+    dp_size_list = [st.dp_size for st in config.stages[:config.num_stages]]
+    recompute_ops = [st.recompute_ops for st in config.stages[:config.num_stages]]
+    algo_list = [st.algo for st in config.stages[:config.num_stages]]
+    if get_string:
+        return f"{num_ops_stage}, {tp_size_list}, {dp_size_list}, {recompute_ops}, {config.micro_bs}, {algo_list}"
+    return num_ops_stage, tp_size_list, dp_size_list, recompute_ops, config.micro_bs, algo_list
+
+
+def is_visited(visited_set, hash_str, target=""):
+    """aceso_utils.py:831-838"""
+    return hash_str in visited_set and target in visited_set[hash_str]
+
+
+def mark_visited(visited_set, hash_str, target=""):
+    """aceso_utils.py:840-844"""
+    visited_set.setdefault(hash_str, []).append(target)
+
+
+def num_visited(visited_set, hash_str):
+    """aceso_utils.py:846-850"""
+    return len(visited_set.get(hash_str, ()))
+
+
 def cross_node_bits(stage_gpus: Sequence[int], gpus_per_node: int) -> int:
     """in/out cross-node flags of every stage (aceso_cost_model.py:572-574)."""
     bits, till_now = 0, 0

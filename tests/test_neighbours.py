@@ -4,8 +4,8 @@ import numpy as np
 import pytest
 
 from superscaler_amd import synth
-from superscaler_amd.neighbours import hill_climb, make_neighbours
-from superscaler_amd.plan import validate_batch
+from superscaler_amd.neighbours import VisitedPlans, hill_climb, make_neighbours
+from superscaler_amd.plan import PlanBatch, config_details, is_visited, mark_visited, num_visited, validate_batch
 from tests.helpers import emu_score, oracle_for, oracle_scores
 
 
@@ -31,6 +31,38 @@ def test_neighbours_are_valid_and_score_like_the_oracle(name):
     assert changed > 100
 
 
+def test_visited_set_matches_the_reference_string_key():
+    """Two plans share a key iff their config_details strings (the reference's visited key) are equal."""
+    w = synth.WORKLOADS["gpt3_1_3b"]
+    tables = synth.make_tables(w)
+    base = synth.make_plans(w, tables, n_plans=2, seed_offset=7)
+    nb = make_neighbours(base.slice(0, 1), tables, 300, np.random.default_rng(2))
+    batch = PlanBatch.concat([base, nb])
+    strings = [config_details(batch.to_config(p, tables), get_string=True) for p in range(batch.n_plans)]
+    keys = [k.tobytes() for k in VisitedPlans.keys(batch)]
+    for a in range(0, batch.n_plans, 7):
+        for b in range(batch.n_plans):
+            assert (strings[a] == strings[b]) == (keys[a] == keys[b])
+    assert len(set(strings)) < batch.n_plans      # the sample does contain repeats
+    vs = VisitedPlans()
+    first = vs.unseen(batch)
+    assert first.sum() == len(set(strings)) and first[0]
+    seen = set()
+    for p in range(batch.n_plans):                # exactly the first occurrence of every string is kept
+        assert first[p] == (strings[p] not in seen)
+        seen.add(strings[p])
+    vs.mark(batch, rows=np.flatnonzero(first)[:10])
+    again = vs.unseen(batch)
+    assert again.sum() == first.sum() - 10 and len(vs) == 10
+    # the reference's dict-of-lists helpers
+    d = {}
+    assert not is_visited(d, "k", 1) and num_visited(d, "k") == 0
+    mark_visited(d, "k", 1)
+    mark_visited(d, "k", 2)
+    assert is_visited(d, "k", 2) and not is_visited(d, "k", 3) and num_visited(d, "k") == 2
+    assert config_details(None) == ""
+
+
 @pytest.mark.gpu
 def test_hill_climb_improves_and_agrees_with_the_oracle():
     from superscaler_amd.aceso_cost_model import CostModel
@@ -39,7 +71,10 @@ def test_hill_climb_improves_and_agrees_with_the_oracle():
     cm = CostModel(synth.make_settings(w), synth.make_db(w, graph), graph)
     start = synth.make_plans(w, cm.tables, n_plans=1, seed_offset=11)
     trace = []
-    plan, t, m = hill_climb(cm, start, steps=20, n_neighbours=2048, seed=1, on_step=lambda s, t, m: trace.append(t))
+    visited = VisitedPlans()
+    plan, t, m = hill_climb(cm, start, steps=20, n_neighbours=2048, seed=1, on_step=lambda s, t, m: trace.append(t),
+                            visited=visited)
+    assert len(visited) > 20
     orc = oracle_for(cm.tables)
     (t0,), _, (f0,), _ = oracle_scores(orc, start, cm.tables)
     (t1,), (m1,), (f1,), _ = oracle_scores(orc, plan, cm.tables)

@@ -138,13 +138,28 @@ def test_reference_golden_vectors(name, golden_dir, torch_mod):
 
 
 def test_full_size_properties(torch_mod):
-    """GPT-3 13B at a size the oracle cannot cover: size-independent properties."""
+    """GPT-3 13B at the benchmark's full size (1,048,576 plans), which the oracle cannot cover:
+    size-independent properties, an oracle spot check and the top-k against a stable sort."""
     from superscaler_amd.evaluator import PlanEvaluator
     w = synth.WORKLOADS["gpt3_13b"]
     tables = synth.make_tables(w)
     ev = PlanEvaluator(tables)
-    n = 262144
-    batch = synth.make_plans(w, tables, n_plans=n, seed_offset=7)
+    n = w.n_plans
+    assert n == 1048576
+    batch = synth.make_plans(w, tables, n_plans=n, seed_offset=7, workers=8)
+    # 48 plans spread over the batch against the oracle, bit for bit
+    sample = np.random.Generator(np.random.PCG64(3)).choice(n, size=48, replace=False)
+    d = ev.upload(batch)
+    t_it, t_pk, t_fe, t_st = ev.score(d)
+    oit, opk, ofe, _ = oracle_scores(oracle_for(tables), batch, tables, idx=sample)
+    assert np.array_equal(t_it.cpu().numpy()[sample], oit) and np.array_equal(t_pk.cpu().numpy()[sample], opk)
+    assert np.array_equal(t_fe.cpu().numpy()[sample], ofe)
+    # top-64 = the first 64 of a stable ascending sort of the feasible plans
+    idx, val, cnt = ev.topk(t_it, t_fe, 64)
+    h_it, h_fe = t_it.cpu().numpy(), t_fe.cpu().numpy()
+    feas = np.flatnonzero(h_fe)
+    order = feas[np.argsort(h_it[feas], kind="stable")][:64]
+    assert int(cnt.item()) == 64 and np.array_equal(idx.cpu().numpy(), order) and np.array_equal(val.cpu().numpy(), h_it[order])
     # duplicated plans score identically; a permuted batch gives permuted results
     perm = np.random.Generator(np.random.PCG64(1)).permutation(n)
     it, pk, fe, st = ev.score_host(batch)

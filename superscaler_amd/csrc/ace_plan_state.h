@@ -8,7 +8,10 @@
 //             (:340-350), get_recompute_time_v3 (:365-371), get_memory_v3 (:382-392),
 //             get_activations_v3 (:403-415), get_peak_activations (:428-445),
 //             get_reserved_memory maxima (:453-460)
-//   start()   stage head: boundary input size / p2p time (:319-331), per-stage lookup offsets
+//   start_fast() / start_lookups()  stage head: per-stage lookup offsets; boundary input size /
+//             p2p time (:319-331)
+//   stash() / replay()  deferred stage tails: a finished stage's accumulators are parked in a
+//             workspace and its tail is evaluated after the op loop
 //   finish()  stage tail: output p2p (:321-336), stage time (:352-353, :579), stage memory
 //             (predict_stage_memory :514-539, get_reserved_memory :480-483), running
 //             sum / max for the 1F1B composition (:613-619)
@@ -247,15 +250,15 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         finish(g, lds, info_row(g, pos_info[i_last]), c_last, nullptr);
     }
 
-    // Stage tail; `prevrow` is the LDS offset of the row of the stage's last op, `c_last` its code.
-    ACE_HD void finish(const AceGeom &g, const AceLds &lds, uint32_t prevrow, uint32_t c_last, double *rec) {
+    // Stage tail; `lastrow` is the LDS offset of the row of the stage's last op, `c_last` its code.
+    ACE_HD void finish(const AceGeom &g, const AceLds &lds, uint32_t lastrow, uint32_t c_last, double *rec) {
         uint32_t t_last = c_last >> g.A_shift;
         uint32_t a_last = c_last & (uint32_t)(g.n_algo - 1);
         uint32_t m_last = (mrow >> (4u * t_last)) & 15u;
         if (m_last >= (uint32_t)g.n_mbs) m_last = 0;   // only for plans whose sums are NaN already
         // output_size[ops[-1]][mbs[-1]][tp[0]][algo[-1]]  (sic, aceso_cost_model.py:321-326)
         uint32_t oidx = ((m_last * (uint32_t)g.n_tp + t_first) << g.A_shift) + a_last;
-        ace_d2 oe = lds.ld<ace_d2>(prevrow + g.out_off + oidx * 16u);
+        ace_d2 oe = lds.ld<ace_d2>(lastrow + g.out_off + oidx * 16u);
         double out_comm = out_cross ? oe.y : oe.x;
         double in_c = in_comm + rs_f * 1000.0;      // :352
         double out_c = out_comm + rs_b * 1000.0;    // :353
@@ -283,7 +286,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
             r[ACE_R_SAVED] = saved; r[ACE_R_PEAK] = peak; r[ACE_R_RESERVED] = reserved;
             // ideal pass: output_size[ops[-1]][mbs index of micro_bs][tp index 0][algo[-1]]
             uint32_t iidx = ((bidx * (uint32_t)g.n_tp + 0u) << g.A_shift) + a_last;
-            ace_d2 ie = lds.ld<ace_d2>(prevrow + g.out_off + iidx * 16u);
+            ace_d2 ie = lds.ld<ace_d2>(lastrow + g.out_off + iidx * 16u);
             r[ACE_R_IDEAL_FWD] = id_fwd; r[ACE_R_IDEAL_BWD] = id_bwd; r[ACE_R_IDEAL_IN] = id_in;
             r[ACE_R_IDEAL_OUT] = out_cross ? ie.y : ie.x;
             r[ACE_R_STAGE_MS] = t; r[ACE_R_STAGE_MB] = mem;

@@ -483,6 +483,12 @@ class CostModel:
         for st, rc in zip(where, self.check_recompute_batch(qs)):
             st.recompute_ops = rc
 
+    def update_recompute_arrays(self, batch: PlanBatch) -> PlanBatch:
+        """update_recompute for every stage of every plan of an encoded batch, without Python objects:
+        a copy of the batch with the recompute bits check_recompute chooses (see recompute.py)."""
+        from .recompute import update_recompute_arrays
+        return update_recompute_arrays(self, batch)
+
     def predict_value_after_move(self, config, bottleneck, partner, num_ops_moved, metric, inc_gpus=False,
                                  dec_gpus=False, dim=None):
         """aceso_cost_model.py:693-739."""

@@ -99,6 +99,47 @@ def _run_all(g, m):
     assert [st.recompute_ops for st in c.stages] == g["plans"][1]["check_recompute"]
 
 
+def _check_arrays_recompute(g, m):
+    """update_recompute on encoded plans reproduces the reference's check_recompute for every stage."""
+    cfgs = [cfg_of(g, m, p) for p in g["plans"]]
+    batch = m.encode(cfgs)
+    out = m.update_recompute_arrays(batch)
+    assert np.array_equal(out.hdr, batch.hdr) and np.array_equal(out.codes & 0xF7, batch.codes & 0xF7)
+    for k, p in enumerate(g["plans"]):
+        got = out.to_config(k, m.tables)
+        assert [st.recompute_ops for st in got.stages] == p["check_recompute"]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_recompute_arrays_match_reference_emu(golden_dir, case):
+    g, m = make_model(golden_dir, case, "emu")
+    _check_arrays_recompute(g, m)
+
+
+@pytest.mark.parametrize("name,limit", [("gpt3_1_3b", 9000.0), ("t5_770m", 6000.0), ("wresnet_1b", 1500.0)])
+def test_recompute_arrays_match_the_staged_loop(name, limit):
+    """On synthetic plans far above the memory limit (many greedy rounds, partial groups) the
+    array form equals check_recompute_batch, which the reference's own vectors pin."""
+    import dataclasses
+    from superscaler_amd import synth
+    w = synth.WORKLOADS[name]
+    graph = synth.make_graph(w)
+    st = dataclasses.replace(synth.make_settings(w), memory_limit=limit)
+    m = acm.CostModel(st, synth.make_db(w, graph), graph)
+    m._evaluator = EmuEvaluator(m.tables)
+    batch = synth.make_plans(w, m.tables, n_plans=24, seed_offset=5)
+    out = m.update_recompute_arrays(batch)
+    rounds = 0
+    for k in range(batch.n_plans):
+        c = batch.to_config(k, m.tables)
+        qs = [(s.ops, c.micro_bs, s.tp_size, s.dp_size, s.num_stages_behind, s.algo) for s in c.stages]
+        want = m.check_recompute_batch(qs)
+        got = [s.recompute_ops for s in out.to_config(k, m.tables).stages]
+        assert got == want
+        rounds += sum(1 for r in want if 0 < sum(r) < len(r))
+    assert rounds > 10, "the limit should force partial recomputation in many stages"
+
+
 @pytest.mark.parametrize("case", CASES)
 def test_api_matches_reference_emu(golden_dir, case):
     g, m = make_model(golden_dir, case, "emu")
@@ -111,6 +152,7 @@ def test_api_matches_reference_gpu(golden_dir, case):
     g, m = make_model(golden_dir, case, "gpu")
     try:
         _run_all(g, m)
+        _check_arrays_recompute(g, m)
     finally:
         m.close()
 
@@ -173,3 +215,26 @@ def test_uniform_grid_emu(golden_dir):
 @pytest.mark.gpu
 def test_uniform_grid_gpu(golden_dir):
     _grid_check(golden_dir, "gpu")
+
+
+@pytest.mark.gpu
+def test_recompute_arrays_gpu_equals_cpu_build():
+    """2,048 GPT-3 13B plans under a 40 GB cap: the array-form greedy loop gives the same bits whether
+    its stage records come from the GPU or from the CPU build of the kernel source."""
+    import dataclasses
+    from superscaler_amd import synth
+    w = synth.WORKLOADS["gpt3_13b"]
+    graph = synth.make_graph(w)
+    st = dataclasses.replace(synth.make_settings(w), memory_limit=40000.0)
+    m = acm.CostModel(st, synth.make_db(w, graph), graph)
+    try:
+        batch = synth.make_plans(w, m.tables, n_plans=2048, seed_offset=9)
+        on_gpu = m.update_recompute_arrays(batch)
+        real, m._evaluator = m._evaluator, EmuEvaluator(m.tables)
+        on_cpu = m.update_recompute_arrays(batch)
+        m._evaluator = real
+        assert np.array_equal(on_gpu.codes, on_cpu.codes)
+        frac = (on_gpu.codes & 8).astype(bool).mean()
+        assert 0.1 < frac < 0.9
+    finally:
+        m.close()

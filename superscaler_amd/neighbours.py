@@ -184,11 +184,13 @@ class VisitedPlans:
 
 
 def hill_climb(cm, start: PlanBatch, steps: int, n_neighbours: int, seed: int = 0, max_move: int = 8,
-               on_step=None, visited: VisitedPlans = None) -> Tuple[PlanBatch, float, float]:
+               on_step=None, visited: VisitedPlans = None, greedy_recompute: bool = False) -> Tuple[PlanBatch, float, float]:
     """Best-neighbour descent: at every step n_neighbours single-move neighbours of the current plan
     are scored in one launch and the fastest feasible one replaces it if it is faster.  With a
     `visited` set, neighbours seen in an earlier step (or twice in one step) are dropped before
-    scoring, as aceso_search.py:47 does.  Returns (plan, iteration ms, peak MB)."""
+    scoring, as aceso_search.py:47 does.  With `greedy_recompute` every neighbour's recompute bits are
+    replaced by check_recompute's choice before it is scored, as the reference's primitives do
+    (aceso_prims.py:107-108).  Returns (plan, iteration ms, peak MB)."""
     rng = np.random.default_rng(seed)
     tables = cm.tables
     ev = cm.evaluator
@@ -208,6 +210,8 @@ def hill_climb(cm, start: PlanBatch, steps: int, n_neighbours: int, seed: int = 
                 continue
             nb = PlanBatch(np.ascontiguousarray(nb.codes[keep]), np.ascontiguousarray(nb.hdr[keep]))
             visited.mark(nb)
+        if greedy_recompute:
+            nb = cm.update_recompute_arrays(nb)
         d = ev.upload(nb, validate=False)
         it, pk, fe, st = ev.score(d)
         idx, val, cnt = ev.topk(it, fe, 1)

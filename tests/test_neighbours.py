@@ -81,4 +81,9 @@ def test_hill_climb_improves_and_agrees_with_the_oracle():
     assert f1 == 1 and t1 == t and m1 == m
     assert t1 < t0 or not f0
     assert all(a >= b for a, b in zip(trace, trace[1:]))
+    # with check_recompute applied to every neighbour the accepted plan carries exactly those bits
+    plan2, t2, m2 = hill_climb(cm, start, steps=6, n_neighbours=512, seed=2, greedy_recompute=True)
+    assert np.array_equal(cm.update_recompute_arrays(plan2).codes, plan2.codes) or t2 == (t0 if f0 else float("inf"))
+    (t3,), (m3,), (f3,), _ = oracle_scores(orc, plan2, cm.tables)
+    assert (f3 == 1 and t3 == t2 and m3 == m2) or t2 == float("inf")
     cm.close()

@@ -190,7 +190,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         const uint32_t glog = (uint32_t)(glogs >> sh) & 15u;
         hot_v = ace_mul24(d, (uint32_t)g.C * ACE_HOT_STRIDE);
         z_v = ace_mul24(d, (uint32_t)g.C * 8u);
-        rk_v = glog << 6;
+        rk_v = (glog < (uint32_t)g.n_glog ? glog : 0u) << 6;   // (a stage size outside the tables is unscorable anyway)
         if (tail) {
             dc_v = ace_mul24(d, (uint32_t)g.C);
             mrow = lds.ld<uint32_t>(g.stg_lds_off + (bidx * 16u + glog) * 4u) >> 16;

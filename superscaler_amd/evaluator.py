@@ -75,13 +75,21 @@ def _check(lib, rc, what):
 class DeviceBatch:
     """A PlanBatch resident in HBM in the layout the kernel streams."""
 
-    def __init__(self, batch: PlanBatch, device="cuda:0", ranges: Optional[np.ndarray] = None):
+    def __init__(self, batch: PlanBatch, device="cuda:0", ranges: Optional[np.ndarray] = None, staging=None):
+        """`staging`: a pinned uint8 host tensor of at least P * N bytes; the plan bytes then go through
+        it and the copy to the device does not block the host (the caller must not reuse the tensor
+        before that copy has completed)."""
         import torch
         self.n_plans = batch.n_plans
         self.num_ops = batch.num_ops
         P, N = batch.codes.shape
         G = (N + 15) // 16
-        codes = torch.from_numpy(np.ascontiguousarray(batch.codes)).to(device)
+        if staging is not None:
+            stage = staging[:P * N].view(P, N)
+            stage.copy_(torch.from_numpy(np.ascontiguousarray(batch.codes)))
+            codes = stage.to(device, non_blocking=True)
+        else:
+            codes = torch.from_numpy(np.ascontiguousarray(batch.codes)).to(device)
         if G * 16 != N:
             codes = torch.nn.functional.pad(codes, (0, G * 16 - N))
         # [P, G, 16] -> [G, P, 16]: plan-minor, sixteen ops per 16-byte word
@@ -127,12 +135,15 @@ class PlanEvaluator:
         except Exception:
             pass
 
-    def upload(self, batch: PlanBatch, validate: bool = True, ranges: Optional[np.ndarray] = None) -> DeviceBatch:
+    def upload(self, batch: PlanBatch, validate: bool = True, ranges: Optional[np.ndarray] = None,
+               staging=None) -> DeviceBatch:
+        """`validate` checks the encoding on the host first (a clear message instead of per-plan status
+        bytes; the kernel itself is safe for any byte content)."""
         if validate and ranges is None:
             msg = validate_batch(batch, self.tables)
             if msg:
                 raise ValueError(msg)
-        return DeviceBatch(batch, self.device, ranges)
+        return DeviceBatch(batch, self.device, ranges, staging)
 
     def _stream(self):
         return ctypes.c_void_p(self._torch.cuda.current_stream(self.device).cuda_stream)
@@ -193,9 +204,10 @@ class PlanEvaluator:
         return ms.value
 
     def score_stream(self, batches, k: int, memory_limit: Optional[float] = None, strict: bool = False):
-        """Score host-resident batches one after the other while the next one is uploaded: uploads run
-        on a second stream (same priority) into the buffers of the batch before last, scoring and the
-        per-batch top-k on the current stream.  Returns (global plan indices, times) of the k fastest
+        """Score host-resident batches one after the other while the next one is uploaded: uploads go
+        through two pinned staging buffers on a second stream (same priority), scoring and the
+        per-batch top-k run on the current stream.  Plans are not validated on the host: malformed or
+        unscorable ones come back infeasible.  Returns (global plan indices, times) of the k fastest
         feasible plans over all batches (ascending, ties -> lower global index) and the number of
         plans seen."""
         torch = self._torch
@@ -205,12 +217,19 @@ class PlanEvaluator:
         best_val = np.empty(0, dtype=np.float64)
         offset = 0
         it = iter(batches)
+        staging = [None, None]
+        turn = [0]
 
         def upload(b):
+            # buffer `turn` was last used two batches ago, and that batch has been scored and synchronised
+            need = b.n_plans * b.num_ops
+            if staging[turn[0]] is None or staging[turn[0]].numel() < need:
+                staging[turn[0]] = torch.empty(need, dtype=torch.uint8, pin_memory=True)
             with torch.cuda.stream(copy_stream):
-                d = self.upload(b)
+                d = self.upload(b, validate=False, staging=staging[turn[0]])
                 ev = torch.cuda.Event()
                 ev.record(copy_stream)
+            turn[0] ^= 1
             return d, ev
 
         nxt = next(it, None)

@@ -39,7 +39,8 @@ def _set_header(hdr_row, S, bidx, glogs, gpn):
 def make_neighbours(base: PlanBatch, tables: CompiledTables, n: int, rng: np.random.Generator,
                     max_move: int = 8) -> PlanBatch:
     """n single-move neighbours of base plan 0 (moves that would leave the profiled grid are replaced
-    by a copy of the base plan, so the batch always has n valid rows)."""
+    by a copy of the base plan, so the batch always has n valid rows).  All neighbours of one kind
+    are produced together: masks over a [neighbours, ops] byte matrix, no per-neighbour Python."""
     A = tables.db.n_algo
     N = tables.graph.num_ops
     gpn = tables.settings.num_gpus_per_node
@@ -47,100 +48,120 @@ def make_neighbours(base: PlanBatch, tables: CompiledTables, n: int, rng: np.ran
     S = int(hdr0[0] & 0xff)
     bidx = int(hdr0[0] >> 8) & 0xff
     gword = int(hdr0[1]) | (int(hdr0[2]) << 32)
-    glogs = np.array([(gword >> (4 * s)) & 15 for s in range(S)])
+    glogs = np.array([(gword >> (4 * s)) & 15 for s in range(S)], dtype=np.int64)
     starts, ends = _stage_bounds(row0)
     tunable = (tables.graph.flags[tables.graph.type_of_pos] & og.F_TUNABLE) != 0
     M = len(tables.db.mbs_list)
     codes = np.repeat(row0[None, :], n, axis=0)
     hdr = np.repeat(hdr0[None, :], n, axis=0)
     kinds = rng.integers(0, 6, size=n)
+    pos = np.arange(N)
+    tp0 = ((row0 & 7) // A).astype(np.int64)
+    stage_of_pos = np.cumsum((row0 >> 4) & 1) - 1
 
     def allowed(b, gl):
         return tables.allowed_tp_logs(b, gl)
 
-    def tp_logs(seg):
-        return (seg.astype(np.int64) & 7) // A
+    def ok_bits(b, gl):
+        return sum(1 << t for t in allowed(b, gl))
 
     def with_tp(seg, t):
         """The code bytes `seg` with their tp replaced by t (algo, recompute and stage bits kept)."""
-        return ((seg & 0xF8) | (np.asarray(t, dtype=np.int64) * A + (seg.astype(np.int64) & 7) % A).astype(np.uint8))
+        t8 = np.asarray(t).astype(np.uint8)
+        return (seg & np.uint8(0xF8)) | (t8 * np.uint8(A) + (seg & np.uint8(A - 1)))
 
-    for k in range(n):
-        kind = kinds[k]
-        row = codes[k]
-        if kind == 0 and S > 1:
-            # op migration: move a stage boundary by up to max_move ops; the ops that change stage
-            # take the tp of the op they now follow / precede in the receiving stage
-            j = int(rng.integers(1, S))
-            d = int(rng.integers(1, max_move + 1)) * (1 if rng.random() < 0.5 else -1)
-            cut = int(starts[j])
-            new_cut = cut + d
-            if new_cut <= starts[j - 1] or new_cut >= ends[j]:
+    # kind 0, op migration: move a stage boundary by up to max_move ops; the ops that change stage
+    # take the tp of the op they now follow / precede in the receiving stage
+    rows = np.flatnonzero(kinds == 0)
+    if S > 1 and len(rows):
+        j = rng.integers(1, S, size=len(rows))
+        d = rng.integers(1, max_move + 1, size=len(rows)) * np.where(rng.random(len(rows)) < 0.5, 1, -1)
+        cut = starts[j]
+        new_cut = cut + d
+        good = (new_cut > starts[j - 1]) & (new_cut < ends[j])
+        rows, cut, new_cut, d = rows[good], cut[good], new_cut[good], d[good]
+        ref = np.where(d > 0, tp0[cut - 1], tp0[cut])        # stage j-1 grows to the right / stage j to the left
+        moved = (pos[None, :] >= np.minimum(cut, new_cut)[:, None]) & (pos[None, :] < np.maximum(cut, new_cut)[:, None])
+        sub = codes[rows]
+        sub[np.arange(len(rows)), cut] &= 0xEF
+        sub = np.where(moved, with_tp(sub, ref[:, None]), sub)
+        sub[np.arange(len(rows)), new_cut] |= 16
+        codes[rows] = sub
+
+    # kind 1, tp <-> dp inside one stage: all ops one step up or down, if the stage allows it
+    rows = np.flatnonzero(kinds == 1)
+    if len(rows):
+        s = rng.integers(0, S, size=len(rows))
+        step = np.where(rng.random(len(rows)) < 0.5, 1, -1)
+        inside = (pos[None, :] >= starts[s][:, None]) & (pos[None, :] < ends[s][:, None])
+        # a stage's ops may sit on different tp: the move is legal iff every tp value present has a legal target
+        bits = np.array([ok_bits(bidx, int(g)) for g in glogs], dtype=np.int64)
+        present = np.array([sum(1 << int(v) for v in np.unique(tp0[starts[k]:ends[k]])) for k in range(S)], dtype=np.int64)
+        want = np.where(step > 0, present[s] << 1, present[s] >> 1)
+        lost = (step < 0) & ((present[s] & 1) == 1)                      # tp = 1 cannot go down
+        good = ((want & ~bits[s]) == 0) & ~lost
+        t8 = (tp0[None, :] + step[good][:, None]).clip(0, 7).astype(np.uint8)
+        sub = codes[rows[good]]
+        codes[rows[good]] = np.where(inside[good], with_tp(sub, t8), sub)
+
+    # kind 2, micro-batch size one step up or down, if every op stays on the profiled grid
+    rows = np.flatnonzero(kinds == 2)
+    if len(rows):
+        up = rng.random(len(rows)) < 0.5
+        for sign, sel in ((1, up), (-1, ~up)):
+            b2 = bidx + sign
+            if not 0 <= b2 < M or not sel.any():
                 continue
-            row[cut] &= 0xEF
-            if d > 0:      # stage j-1 grows: ops [cut, new_cut) join it with the tp of op cut-1
-                row[cut:new_cut] = with_tp(row[cut:new_cut], int(tp_logs(row[cut - 1:cut])[0]))
-            else:          # stage j grows to the left with the tp of its former first op
-                row[new_cut:cut] = with_tp(row[new_cut:cut], int(tp_logs(row[cut:cut + 1])[0]))
-            row[new_cut] |= 16
-        elif kind == 1:
-            # tp <-> dp inside one stage: all ops one step up or down, if the stage allows it
-            s = int(rng.integers(0, S))
-            step = 1 if rng.random() < 0.5 else -1
-            lo, hi = int(starts[s]), int(ends[s])
-            t = tp_logs(row[lo:hi]) + step
-            ok = allowed(bidx, int(glogs[s]))
-            if t.min() < 0 or not np.all(np.isin(t, ok)):
-                continue
-            row[lo:hi] = with_tp(row[lo:hi], t)
-        elif kind == 2:
-            # micro-batch size one step up or down, if every op stays on the profiled grid
-            b2 = bidx + (1 if rng.random() < 0.5 else -1)
-            if b2 < 0 or b2 >= M:
-                continue
-            good = True
-            for s in range(S):
-                t = tp_logs(row[starts[s]:ends[s]])
-                if not np.all(np.isin(t, allowed(b2, int(glogs[s])))):
-                    good = False
-                    break
-            if not good:
-                continue
-            hdr[k, 0] = S | (b2 << 8)
-        elif kind == 3:
-            # recompute: toggle a short run of ops
-            lo = int(rng.integers(0, N))
-            hi = min(N, lo + int(rng.integers(1, 14)))
-            row[lo:hi] ^= 8
-        elif kind == 4 and A == 2:
-            # partition algorithm of one tunable op
-            cand = np.flatnonzero(tunable)
-            i = int(cand[rng.integers(0, len(cand))])
-            row[i] ^= 1
-        elif kind == 5 and S > 1:
-            # move half of stage a's devices to a stage b that has exactly that many (sizes stay powers
-            # of two and the total is unchanged)
-            a, b = rng.choice(S, size=2, replace=False)
-            if glogs[a] - 1 != glogs[b]:
+            bits = np.array([ok_bits(b2, int(g)) for g in glogs], dtype=np.int64)[stage_of_pos]
+            if (((bits >> tp0) & 1) == 1).all():
+                hdr[rows[sel], 0] = S | (b2 << 8)
+
+    # kind 3, recompute: toggle a short run of ops
+    rows = np.flatnonzero(kinds == 3)
+    if len(rows):
+        lo = rng.integers(0, N, size=len(rows))
+        hi = np.minimum(N, lo + rng.integers(1, 14, size=len(rows)))
+        run = (pos[None, :] >= lo[:, None]) & (pos[None, :] < hi[:, None])
+        codes[rows] ^= (run * np.uint8(8)).astype(np.uint8)
+
+    # kind 4, partition algorithm of one tunable op
+    rows = np.flatnonzero(kinds == 4)
+    if A == 2 and len(rows):
+        cand = np.flatnonzero(tunable)
+        codes[rows, cand[rng.integers(0, len(cand), size=len(rows))]] ^= 1
+
+    # kind 5, move half of stage a's devices to a stage b that has exactly that many (sizes stay powers
+    # of two and the total is unchanged); few distinct (a, b) pairs, each built once
+    rows = np.flatnonzero(kinds == 5)
+    if S > 1 and len(rows):
+        a = rng.integers(0, S, size=len(rows))
+        b = (a + rng.integers(1, S, size=len(rows))) % S
+        for pa, pb in {(int(x), int(y)) for x, y in zip(a, b)}:
+            if glogs[pa] - 1 != glogs[pb]:
                 continue
             g2 = glogs.copy()
-            g2[a] -= 1
-            g2[b] += 1
-            if not allowed(bidx, int(g2[a])) or not allowed(bidx, int(g2[b])):
-                continue
+            g2[pa] -= 1
+            g2[pb] += 1
+            row = row0.copy()
             good = True
-            for s in (a, b):
-                ok = allowed(bidx, int(g2[s]))
-                lo, hi = int(starts[s]), int(ends[s])
-                t = np.clip(tp_logs(row[lo:hi]), min(ok), max(ok))
+            for st in (pa, pb):
+                ok = allowed(bidx, int(g2[st]))
+                if not ok:
+                    good = False
+                    break
+                lo, hi = int(starts[st]), int(ends[st])
+                t = np.clip(tp0[lo:hi], min(ok), max(ok))
                 if not np.all(np.isin(t, ok)):
                     good = False
                     break
                 row[lo:hi] = with_tp(row[lo:hi], t)
             if not good:
-                codes[k] = row0
                 continue
-            _set_header(hdr[k], S, bidx, g2, gpn)
+            sel = rows[(a == pa) & (b == pb)]
+            codes[sel] = row
+            h = hdr0.copy()
+            _set_header(h, S, bidx, g2, gpn)
+            hdr[sel] = h
     return PlanBatch(codes, hdr)
 
 

@@ -87,3 +87,15 @@ def test_hill_climb_improves_and_agrees_with_the_oracle():
     (t3,), (m3,), (f3,), _ = oracle_scores(orc, plan2, cm.tables)
     assert (f3 == 1 and t3 == t2 and m3 == m2) or t2 == float("inf")
     cm.close()
+
+
+@pytest.mark.gpu
+def test_stream_and_search_demo_runs(capsys):
+    """The end-to-end demo (streamed batches -> global top-k -> batched local search) at a small size."""
+    import json
+    from superscaler_amd import search_demo
+    search_demo.main(["--workload", "gpt3_1_3b", "--stream-plans", "10000", "--batch", "4096", "--steps", "4",
+                      "--neighbours", "512", "--greedy-recompute", "--workers", "2"])
+    out = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    assert out["streamed_plans"] == 10000 and out["batches"] == 3
+    assert out["search_best_ms"] <= out["search_start_ms"]

@@ -23,24 +23,35 @@ HBM_PEAK_GBPS = 8000.0
 MEASURED_TRAFFIC_BYTES_PER_PLAN = {("gpt3_13b", 523): 2109.0}
 
 
-def cpu_baseline(tables, batch, budget_s=15.0):
-    """The oracle (a loop-faithful Python port of the reference cost model) on one host core,
-    over as many plans of the same batch as fit the time budget."""
-    from tests.helpers import oracle_config, oracle_for
-    orc = oracle_for(tables)
-    cfgs = [oracle_config(batch, p, tables) for p in range(min(batch.n_plans, 16384))]
-    for c in cfgs[:8]:
-        orc.score(c)
+def cpu_baseline(tables, batch, threads):
+    """The oracle on the host's cores: its C restatement (one plan after the other per thread, the
+    reference's own order of operations) over the whole batch with `threads` threads, and on one
+    thread over a slice; the loop-faithful Python oracle on one core for scale."""
+    from tests.helpers import c_oracle_for, oracle_config, oracle_for, plan_arrays
+    co = c_oracle_for(tables)
+    arrays = plan_arrays(batch, tables)
+    P = batch.n_plans
+    co.score_arrays(*[a[:4096] for a in arrays], threads=threads)          # warm-up
     t0 = time.perf_counter()
-    n = 0
+    co.score_arrays(*arrays, threads=threads)
+    dt_all = time.perf_counter() - t0
+    n1 = min(P, 131072)
+    t0 = time.perf_counter()
+    co.score_arrays(*[a[:n1] for a in arrays], threads=1)
+    dt_one = time.perf_counter() - t0
+    orc = oracle_for(tables)
+    npy = min(P, 1024)
+    cfgs = [oracle_config(batch, p, tables) for p in range(npy)]
+    t0 = time.perf_counter()
     for c in cfgs:
         orc.score(c)
-        n += 1
-        if time.perf_counter() - t0 > budget_s:
-            break
-    dt = time.perf_counter() - t0
-    return {"value": n / dt, "unit": "plans/s", "cores": 1, "kind": "port",
-            "sample": f"first {n} plans of the same batch, {dt:.1f} s, pure-Python oracle, 1 process"}
+    dt_py = time.perf_counter() - t0
+    return {"value": P / dt_all, "unit": "plans/s", "cores": threads, "kind": "port",
+            "sample": f"all {P} plans of the same batch in {dt_all:.2f} s, C oracle (oracle/aceso_oracle.c), "
+                      f"{threads} OpenMP threads",
+            "single_core_value": n1 / dt_one, "single_core_sample": f"first {n1} plans, {dt_one:.2f} s, 1 thread",
+            "python_oracle_value": npy / dt_py,
+            "python_oracle_sample": f"first {npy} plans, {dt_py:.2f} s, pure-Python oracle, 1 process"}
 
 
 def main():
@@ -137,7 +148,7 @@ def main():
         torch.cuda.synchronize()
         out["config"]["calibration_copy_bytes"] = int(src.numel())
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(tables, batch)
+        out["cpu_baseline"] = cpu_baseline(tables, batch, threads=min(16, os.cpu_count() or 1))
     ev.close()
     print(json.dumps(out))
 

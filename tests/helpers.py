@@ -84,3 +84,40 @@ def emu_score(tables, batch, memory_limit=None, strict=False, breakdown=False, r
                            rec.ctypes.data_as(ctypes.c_void_p) if breakdown else None)
     assert rc == 0
     return it, pk, fe, st, rec
+
+
+def plan_arrays(batch, tables):
+    """A PlanBatch as the plain arrays the C oracle takes: (num_stages, micro_bs, stage_len[P,16],
+    tp_log, dp_log, algo, rc [P,N])."""
+    codes, hdr = batch.codes, batch.hdr
+    P, N = codes.shape
+    A = tables.db.n_algo
+    c = codes & 7
+    tp_log, algo, rc = (c // A).astype(np.uint8), (c % A).astype(np.uint8), ((codes >> 3) & 1).astype(np.uint8)
+    ns = ((codes >> 4) & 1).astype(np.int64)
+    stage = np.cumsum(ns, axis=1) - 1
+    S = (hdr[:, 0] & 0xff).astype(np.int32)
+    micro_bs = np.asarray(tables.db.mbs_list, dtype=np.int32)[(hdr[:, 0] >> 8) & 0xff]
+    gword = hdr[:, 1].astype(np.uint64) | (hdr[:, 2].astype(np.uint64) << np.uint64(32))
+    glog = ((gword[:, None] >> (4 * np.clip(stage, 0, 15)).astype(np.uint64)) & np.uint64(15)).astype(np.int64)
+    dp_log = (glog - tp_log).astype(np.uint8)
+    stage_len = np.zeros((P, 16), dtype=np.int32)
+    np.add.at(stage_len, (np.repeat(np.arange(P), N), np.clip(stage, 0, 15).ravel()), 1)
+    return S, micro_bs, stage_len, tp_log, dp_log, algo, rc
+
+
+_c_oracles = {}
+
+
+def c_oracle_for(tables):
+    """The C oracle loaded with exactly the data `tables` was compiled from (through the Python oracle)."""
+    from oracle.c_oracle import COracle
+    key = id(tables)
+    if key not in _c_oracles:
+        _c_oracles[key] = (COracle(oracle_for(tables), tables.graph.ops, tables.settings.global_batch_size), tables)
+    return _c_oracles[key][0]
+
+
+def c_oracle_scores(tables, batch, strict=False, threads=1, memory_limit=None, lists=False):
+    return c_oracle_for(tables).score_arrays(*plan_arrays(batch, tables), strict=strict, threads=threads,
+                                             memory_limit=memory_limit, lists=lists)

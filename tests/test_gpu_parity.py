@@ -12,7 +12,7 @@ from superscaler_amd.opgraph import OpGraph
 from superscaler_amd.plan import PlanBatch, get_config
 from superscaler_amd.profile_db import CostModelSettings, ProfileDB
 from superscaler_amd.tables import compile_tables
-from tests.helpers import emu_score, oracle_for, oracle_scores
+from tests.helpers import c_oracle_scores, emu_score, oracle_for, oracle_scores
 
 pytestmark = pytest.mark.gpu
 
@@ -154,6 +154,11 @@ def test_full_size_properties(torch_mod):
     oit, opk, ofe, _ = oracle_scores(oracle_for(tables), batch, tables, idx=sample)
     assert np.array_equal(t_it.cpu().numpy()[sample], oit) and np.array_equal(t_pk.cpu().numpy()[sample], opk)
     assert np.array_equal(t_fe.cpu().numpy()[sample], ofe)
+    # every one of the 1,048,576 plans against the C oracle, bit for bit
+    cit, cpk, cfe, cer = c_oracle_scores(tables, batch, threads=16)
+    assert not cer.any() and (t_st.cpu().numpy() == 0).all()
+    assert np.array_equal(t_it.cpu().numpy(), cit) and np.array_equal(t_pk.cpu().numpy(), cpk)
+    assert np.array_equal(t_fe.cpu().numpy(), cfe)
     # top-64 = the first 64 of a stable ascending sort of the feasible plans
     idx, val, cnt = ev.topk(t_it, t_fe, 64)
     h_it, h_fe = t_it.cpu().numpy(), t_fe.cpu().numpy()

@@ -188,6 +188,29 @@ def test_full_size_properties(torch_mod):
     ev.close()
 
 
+@pytest.mark.parametrize("name,n", [("gpt3_1_3b", 4096), ("t5_770m", 65536), ("wresnet_1b", 262144), ("gpt3_175b", 262144)])
+def test_configured_sizes_match_c_oracle(name, n, torch_mod):
+    """The other configurations at their full batch sizes (gpt3_175b: one of its 262,144-plan batches;
+    wresnet_1b runs the windowed kernel): every plan bit-identical to the C oracle, the top-64 equal
+    to a stable sort."""
+    from superscaler_amd.evaluator import PlanEvaluator
+    w = synth.WORKLOADS[name]
+    tables = synth.make_tables(w)
+    batch = synth.make_plans(w, tables, n_plans=n, seed_offset=13, workers=8)
+    ev = PlanEvaluator(tables)
+    it, pk, fe, st = ev.score_host(batch)
+    cit, cpk, cfe, cer = c_oracle_scores(tables, batch, threads=16)
+    assert not cer.any() and (st == 0).all()
+    assert np.array_equal(it, cit) and np.array_equal(pk, cpk) and np.array_equal(fe, cfe)
+    d = ev.upload(batch)
+    t_it, t_pk, t_fe, _ = ev.score(d)
+    idx, val, cnt = ev.topk(t_it, t_fe, 64)
+    feas = np.flatnonzero(cfe)
+    order = feas[np.argsort(cit[feas], kind="stable")][:64]
+    assert int(cnt.item()) == len(order) and np.array_equal(idx.cpu().numpy()[:len(order)], order)
+    ev.close()
+
+
 def test_known_answers_single_gpu_plans(golden_dir, torch_mod):
     """The reference tree's own single-GPU plans and published predictions
     (results/ref/perf_model_{time,mem}_large_{gpt,resnet}.csv), through the GPU path."""

@@ -25,7 +25,6 @@ Pinning status (what independently checks each function; see tests/test_oracle_*
 """
 import csv
 import math
-import os
 from dataclasses import dataclass, field
 from typing import List, Optional
 

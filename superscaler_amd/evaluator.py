@@ -5,7 +5,7 @@ score itself: if the HIP library is missing or no GPU is present it raises.
 """
 import ctypes
 import os
-from typing import Optional, Sequence, Tuple
+from typing import Optional
 
 import numpy as np
 

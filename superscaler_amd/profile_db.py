@@ -9,7 +9,6 @@ intra-node one.
 """
 import csv
 import math
-import os
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional
 

@@ -14,13 +14,13 @@ bytes.
 """
 import math
 from dataclasses import dataclass
-from typing import Dict, List, Optional, Sequence, Tuple
+from typing import Dict, List, Optional, Tuple
 
 import numpy as np
 
 from . import opgraph as og
 from .plan import PlanBatch
-from .profile_db import FIELDS, CostModelSettings, ProfileDB
+from .profile_db import CostModelSettings, ProfileDB
 from .tables import CompiledTables, compile_tables
 
 # saturating bandwidth curves, GB/s per size bucket 1 MB .. 1 GB (11 buckets, the shape of the

@@ -10,7 +10,7 @@ import os
 import pytest
 
 from oracle.aceso_oracle import (Oracle, Settings, config_from_json_dict, get_full_op_list,
-                                 get_op_spec, get_reshard_primitives, get_config, topk)
+                                 get_op_spec, get_reshard_primitives, topk)
 
 
 def single_gpu_case(golden_dir, model, size, plan, mbs_list, num_layers):

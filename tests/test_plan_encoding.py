@@ -7,7 +7,7 @@ import pytest
 
 from superscaler_amd import synth
 from superscaler_amd.plan import (PlanBatch, check_legality, config_from_json, config_to_json_dict,
-                                  cross_node_bits, get_config, validate_batch)
+                                  cross_node_bits, validate_batch)
 
 
 @pytest.fixture(scope="module")

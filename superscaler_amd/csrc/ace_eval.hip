@@ -314,7 +314,7 @@ __global__ __launch_bounds__(kTopBlock) void topk_ties_exact(const double *t, co
         __syncthreads();
         // inclusive scan (Hillis-Steele)
         for (int off = 1; off < kTopBlock; off <<= 1) {
-            unsigned int v = threadIdx.x >= off ? cnt[threadIdx.x - off] : 0u;
+            unsigned int v = (int)threadIdx.x >= off ? cnt[threadIdx.x - off] : 0u;
             __syncthreads();
             cnt[threadIdx.x] += v;
             __syncthreads();

@@ -113,7 +113,15 @@ __global__ __launch_bounds__(kBlock) void ace_score_kernel(const AceKernelArgs a
                                     i2.x, i2.y, i2.z, i2.w, i3.x, i3.y, i3.z, i3.w};
         ace_u4 nxt = ace_u4{0u, 0u, 0u, 0u};
         if (grp + 1 < g.G) nxt = a.codes[(size_t)(grp + 1) * g.P + pl];
-        const uint32_t words[5] = {cw.x, cw.y, cw.z, cw.w, nxt.x};
+        uint32_t words[5] = {cw.x, cw.y, cw.z, cw.w, nxt.x};
+        if (DEFER) {
+            // whatever the caller left in the bytes past the last op reads as zero
+#pragma unroll
+            for (int j = 0; j < 5; ++j) {
+                const int left = g.N - (base + 4 * j);          // code bytes of this word that belong to the plan
+                words[j] &= left >= 4 ? 0xffffffffu : (left <= 0 ? 0u : ((1u << (8 * left)) - 1u));
+            }
+        }
         // pair_bit() of the sixteen (op, next op) pairs, four at a time: bit 0 of each byte
         uint32_t pairs[4];
 #pragma unroll
@@ -132,7 +140,9 @@ __global__ __launch_bounds__(kBlock) void ace_score_kernel(const AceKernelArgs a
                 ++w;
                 next_win = a.win_pos[w];
             }
-            if (i < g.N) {
+            // DEFER: positions past the last op are processed too (zeroed code bytes, padded descriptors):
+            // the last stage was stashed at op N - 1, what follows lands in a stage nobody reads
+            if (DEFER || i < g.N) {
                 const uint32_t byte = (words[k >> 2] >> (8 * (k & 3))) & 0xffu;
                 // (past the last op the code bytes are zero padding)
                 const uint32_t nbyte = (words[(k + 1) >> 2] >> (8 * ((k + 1) & 3))) & 0xffu;

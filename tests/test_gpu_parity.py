@@ -271,6 +271,26 @@ def test_edge_shapes(layers, pp, n_plans, torch_mod):
     ev.close()
 
 
+def test_bytes_past_the_last_op_are_ignored(torch_mod):
+    """The 16-byte words of the last op group are padded; whatever sits in the padding must not matter."""
+    from superscaler_amd.evaluator import PlanEvaluator
+    w = synth.WORKLOADS["gpt3_13b"]                      # 523 ops: 11 real bytes + 5 of padding in the last word
+    tables = synth.make_tables(w)
+    batch = synth.make_plans(w, tables, n_plans=3000, seed_offset=4)
+    ev = PlanEvaluator(tables)
+    d = ev.upload(batch)
+    clean = [t.cpu().numpy() for t in ev.score(d)]
+    assert batch.num_ops % 16 != 0
+    d.codes[-1, :, batch.num_ops % 16:] = 0xFF
+    dirty = [t.cpu().numpy() for t in ev.score(d)]
+    _, _, _, _, rec_dirty = [t.cpu().numpy() for t in ev.score(d, breakdown=True)]
+    for a, b in zip(clean, dirty):
+        assert np.array_equal(a, b)
+    eit, epk, _, _, erec = emu_score(tables, batch.slice(0, 64), breakdown=True)
+    assert np.array_equal(rec_dirty[:64], erec) and (clean[3] == 0).all()
+    ev.close()
+
+
 def test_unscorable_and_malformed_plans_are_flagged(torch_mod):
     """A micro-batch / stage-size pair outside the profiled grid gives NaN + status 1 (the reference
     raises KeyError); inconsistent stage bits give status 3; neighbours in the batch are unaffected."""

@@ -114,7 +114,7 @@ struct AceGeom {
 ACE_HD uint32_t info_row(const AceGeom &g, uint32_t i) { return (i & 0xffu) * g.row_bytes; }
 ACE_HD uint32_t info_nextrow(const AceGeom &g, uint32_t i) { return ((i >> 8) & 0xffu) * g.row_bytes; }
 
-#define ACE_WS_REC 14          // doubles per deferred stage record (see PlanState::stash)
+#define ACE_WS_REC 10          // doubles per deferred stage record (see PlanState::stash)
 
 // BD: per-stage records for the caller.  RANGED: one stage over an op sub-range.  DEFER: stage
 // tails are not evaluated where the stage ends (where only the few lanes that cut at this op are
@@ -220,33 +220,44 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         }
     }
 
-    // DEFER: park the finished stage's accumulators in the plan's workspace slot `s`.
-    ACE_HD void stash(double *ws, uint32_t i_last, uint32_t c_last) {
+    // The reserved-memory term of a stage (get_reserved_memory :480-483 with max_collective = 0).
+    ACE_HD double reserved_term(const AceGeom &g) const {
+        if (g.flags & ACE_F_NO_RESERVED) return 0.0;
+        if (g.flags & ACE_F_RESERVED_MIN) return ace_max(ace_max(rfm, rbm), ace_max(W, 0.0));
+        return ace_max(rfm + rbm, W) + 0.0;
+    }
+
+    // DEFER: park the finished stage in the plan's workspace slot `s`: ten values in five 16-byte
+    // stores (a store from a lane or two costs as much as one from sixty-four, so what can be
+    // folded here without a table lookup is: fwd + bwd, the closed peak segment, the reserved term).
+    ACE_HD void stash(const AceGeom &g, double *ws, uint32_t i_last, uint32_t c_last) {
         if (ws == nullptr || s < 0 || s >= ACE_MAX_STAGES) return;
         ace_d2 *r = reinterpret_cast<ace_d2 *>(ws + (size_t)s * ACE_WS_REC);
-        uint64_t meta = (uint64_t)(first_meta | (c_last << 19) | ((uint32_t)lastclose << 22)) | ((uint64_t)i_last << 32);
+        uint64_t meta = (uint64_t)(first_meta | (c_last << 19)) | ((uint64_t)i_last << 32);
         double meta_d;
         __builtin_memcpy(&meta_d, &meta, 8);
-        r[0] = ace_d2{fwd, bwd}; r[1] = ace_d2{rcs, W}; r[2] = ace_d2{A, saved}; r[3] = ace_d2{run, peak};
-        r[4] = ace_d2{rfm, rbm}; r[5] = ace_d2{rs_f, rs_b}; r[6] = ace_d2{meta_d, 0.0};
+        const double fb = fwd + bwd;                                    // the first sum of :579
+        const double peakc = ace_max(peak, run * (lastclose ? 1.0 : 0.0));   // :439: max(peak, run) if the last pair closes
+        r[0] = ace_d2{fb, rcs}; r[1] = ace_d2{rs_f, rs_b}; r[2] = ace_d2{W, A}; r[3] = ace_d2{saved, peakc};
+        r[4] = ace_d2{reserved_term(g), meta_d};
     }
 
     // DEFER: evaluate stage `s2` from its stashed record (called for s2 = 0, 1, ... in order).
     ACE_HD void replay(const AceGeom &g, const AceLds &lds, const uint32_t *pos_info, const double *ws, int s2) {
         const ace_d2 *r = reinterpret_cast<const ace_d2 *>(ws + (size_t)s2 * ACE_WS_REC);
-        ace_d2 r0 = r[0], r1 = r[1], r2 = r[2], r3 = r[3], r4 = r[4], r5 = r[5], r6 = r[6];
+        ace_d2 r0 = r[0], r1 = r[1], r2 = r[2], r3 = r[3], r4 = r[4];
         s = s2 - 1;
         start_fast(g, lds, true);              // s = s2; per-stage offsets, mrow
         uint64_t meta;
-        __builtin_memcpy(&meta, &r6.x, 8);
+        __builtin_memcpy(&meta, &r4.y, 8);
         uint32_t lo32 = (uint32_t)meta, i_last = (uint32_t)(meta >> 32);
         uint32_t i_first = lo32 & 0xffffu, c_first = (lo32 >> 16) & 7u, c_last = (lo32 >> 19) & 7u;
         if (i_first >= (uint32_t)g.N) i_first = 0;     // garbage only if the plan was malformed
         if (i_last >= (uint32_t)g.N) i_last = 0;
         start_lookups(g, lds, info_row(g, pos_info[i_first]), c_first);
-        fwd = r0.x; bwd = r0.y; rcs = r1.x; W = r1.y; A = r2.x; saved = r2.y; run = r3.x; peak = r3.y;
-        rfm = r4.x; rbm = r4.y; rs_f = r5.x; rs_b = r5.y;
-        lastclose = (lo32 >> 22) & 1u;
+        // finish() recombines: (fb + 0) = fb; the peak is closed already; max(reserved + 0, W) = reserved
+        fwd = r0.x; bwd = 0.0; rcs = r0.y; rs_f = r1.x; rs_b = r1.y; W = r2.x; A = r2.y; saved = r3.x;
+        peak = r3.y; run = 0.0; lastclose = false; rfm = r4.x; rbm = 0.0;
         finish(g, lds, info_row(g, pos_info[i_last]), c_last, nullptr);
     }
 
@@ -266,10 +277,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         sum_t += t;
         max_t = ace_max(max_t, t);
         if (lastclose) peak = ace_max(peak, run);   // :439 "i + 1 == len(ops) - 1" closes the last segment
-        double reserved;
-        if (g.flags & ACE_F_NO_RESERVED) reserved = 0.0;
-        else if (g.flags & ACE_F_RESERVED_MIN) reserved = ace_max(ace_max(rfm, rbm), ace_max(W, 0.0));
-        else reserved = ace_max(rfm + rbm, W) + 0.0;                  // :481 (max_collective = 0)
+        const double reserved = reserved_term(g);
         double mp = W * g.main_params;
         double opt = W * g.optimizer;
         double x = (inputs + A) - saved;
@@ -346,7 +354,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         if (last) {
             // :439 "i + 1 == len(ops) - 1": the (previous, this) pair closes the last segment
             lastclose = pair_prev & (pinfo >> 25) & 1u;
-            if (DEFER) stash(rec, (uint32_t)i, c);
+            if (DEFER) stash(g, rec, (uint32_t)i, c);
             else finish(g, lds, row, c, rec);
             if (!RANGED) {
                 // (after the plan's last op this opens a stage that stays empty: s == S in the end)

@@ -344,8 +344,9 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
             // first op) adds 0.0, and the id past the last real table is all NaN (the reference raises there)
             const uint32_t r = r_next;
             const uint32_t pk = (info >> 16) & 0xffu;
-            r_next = lds.ld<uint8_t>((g.rk_lds_off + ace_mul24(pk, g.rk_kind_stride)) + (rk_v + ((c << 3) | nc)));
-            const uint32_t za = (row + g.z_off) + (z_v + c * 8u);
+            // (rk_v is a multiple of 64 and c * 8 + nc < 64: the sum is the [c][nc] entry of the stage-size block)
+            r_next = lds.ld<uint8_t>((g.rk_lds_off + ace_mul24(pk, g.rk_kind_stride)) + (ace_mad24(c, 8u, rk_v) + nc));
+            const uint32_t za = (row + g.z_off) + ace_mad24(c, 8u, z_v);
             rs_f += lds.ld<double>(za + ((r & 15u) << g.z_shift));
             rs_b += lds.ld<double>(za + ((r >> 4) << g.z_shift));
         }
@@ -374,11 +375,11 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         // are zero and pair is false: nothing happens.)
         const double pairf = (double)(int)pair;
         const double keepf = pairf * ace_scalar_01(!savez);       // 1.0 iff the pair continues the running segment
-        run = ace_fma(pairf, e1.y, run);                          // run += act             if pair
+        const double seg = ace_fma(pairf, e1.y, run);             // run + act              if pair
         saved = ace_fma(keepf, e1.y, saved);                      // saved += act           if pair and not savez
-        const double closed = run * (1.0 - keepf);                // run if the segment closes here, else 0.0
+        const double closed = ace_fma(-keepf, seg, seg);          // seg if the segment closes here, else seg - seg = 0.0
         peak = ace_max(peak, closed);                             // max(peak, 0.0) leaves peak (>= 0) alone
-        run = run - closed;                                       // 0.0 if closed, else run
+        run = seg * keepf;                                        // 0.0 if closed, else seg
         pair_prev = pair;
     }
 

@@ -53,7 +53,7 @@ struct AceKernelArgs {
     double *iter_ms, *peak_mb;
     uint8_t *feasible, *status;
     double *stage_out;
-    double *stage_ws;           // [ceil(P / kBlock) * kBlock][ACE_MAX_STAGES][ACE_WS_REC] for deferred stage tails
+    double *stage_ws;           // [ACE_MAX_STAGES][ceil(P / kBlock) * kBlock][ACE_WS_REC] for deferred stage tails
 };
 
 // Copy the rows window `w` needs from global memory into LDS (whole workgroup).
@@ -97,7 +97,11 @@ __global__ __launch_bounds__(kBlock) void ace_score_kernel(const AceKernelArgs a
     st.init(g, lds, h, range);
     const double nbm1 = a.nbm1[st.bidx];
     double *rec = (BD && a.stage_out && active) ? a.stage_out + (size_t)plan * (ACE_MAX_STAGES * ACE_STAGE_REC) : nullptr;
-    if (DEFER) rec = a.stage_ws + (size_t)plan * (ACE_MAX_STAGES * ACE_WS_REC);   // padded lanes own a slot too
+    if (DEFER) {
+        // stage-major: the records of one stage of consecutive plans are adjacent (padded lanes own a slot too)
+        rec = a.stage_ws + (size_t)plan * ACE_WS_REC;
+        st.ws_stride = gridDim.x * kBlock * (ACE_WS_REC / 2);
+    }
 
     int w = 1;
     int next_win = WIN ? a.win_pos[1] : 0x7fffffff;
@@ -600,6 +604,7 @@ static int ensure_stage_ws(ace_handle_t *h, AceKernelArgs *a) {
     a->stage_ws = nullptr;
     if (a->range || a->stage_out || h->n_windows > 1 || h->geom.N >= 65536) return ACE_OK;
     const size_t need = (((size_t)a->g.P + kBlock - 1) / kBlock) * kBlock;
+    if (need * ACE_MAX_STAGES * (ACE_WS_REC / 2) > 0xffffffffull) return ACE_OK;   // 32-bit record offsets: larger batches take the plain kernel
     if (need > h->stage_ws_plans) {
         if (h->d_stage_ws) ACE_HIP(hipFree(h->d_stage_ws));
         h->d_stage_ws = nullptr;

@@ -138,6 +138,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
     double id_fwd, id_bwd;
     bool lastclose;
     uint32_t first_meta;        // DEFER: first op of the current stage: position | code << 16
+    uint32_t ws_stride;         // DEFER: 16-byte units between two stages of one plan in the workspace
     uint64_t diags;             // the diag of every stage, 4 bits each, looked up once per plan
     uint32_t r_next;            // collective ids of the (previous op, this op) pair, fetched one op ahead
     uint32_t pair_prev;         // pair_bit of the (previous op, this op) pair
@@ -156,6 +157,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         sum_t = 0.0; max_t = 0.0; max_mem = 0.0;
         status = 0;
         lastclose = false; first_meta = 0; r_next = 0; pair_prev = 0;
+        ws_stride = ACE_WS_REC / 2;
         fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = rs_f = rs_b = 0.0;
         id_fwd = id_bwd = id_in = 0.0;
         in_comm = inputs = 0.0;
@@ -232,7 +234,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
     // folded here without a table lookup is: fwd + bwd, the closed peak segment, the reserved term).
     ACE_HD void stash(const AceGeom &g, double *ws, uint32_t i_last, uint32_t c_last) {
         if (ws == nullptr || s < 0 || s >= ACE_MAX_STAGES) return;
-        ace_d2 *r = reinterpret_cast<ace_d2 *>(ws + (size_t)s * ACE_WS_REC);
+        ace_d2 *r = reinterpret_cast<ace_d2 *>(ws) + (size_t)((uint32_t)s * ws_stride);
         uint64_t meta = (uint64_t)(first_meta | (c_last << 19)) | ((uint64_t)i_last << 32);
         double meta_d;
         __builtin_memcpy(&meta_d, &meta, 8);
@@ -244,7 +246,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
 
     // DEFER: evaluate stage `s2` from its stashed record (called for s2 = 0, 1, ... in order).
     ACE_HD void replay(const AceGeom &g, const AceLds &lds, const uint32_t *pos_info, const double *ws, int s2) {
-        const ace_d2 *r = reinterpret_cast<const ace_d2 *>(ws + (size_t)s2 * ACE_WS_REC);
+        const ace_d2 *r = reinterpret_cast<const ace_d2 *>(ws) + (size_t)((uint32_t)s2 * ws_stride);
         ace_d2 r0 = r[0], r1 = r[1], r2 = r[2], r3 = r[3], r4 = r[4];
         s = s2 - 1;
         start_fast(g, lds, true);              // s = s2; per-stage offsets, mrow

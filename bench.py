@@ -19,8 +19,8 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per plan of one scoring-kernel launch on the default workload, from two rocprofv3 --pmc
 # runs (FETCH_SIZE, then WRITE_SIZE) scaled by the readings of a plain 256 MiB copy in the same
-# runs (factors 2.000 and 1.000): 1,087 B read + 639 B written.  See profiles/.
-MEASURED_TRAFFIC_BYTES_PER_PLAN = {("gpt3_13b", 523): 1726.0}
+# runs (factors 2.000 and 1.000): 1,334 B read + 618 B written.  See profiles/.
+MEASURED_TRAFFIC_BYTES_PER_PLAN = {("gpt3_13b", 523): 1952.0}
 
 
 def cpu_baseline(tables, batch, threads):

@@ -46,7 +46,13 @@ def cpu_baseline(tables, batch, threads):
     for c in cfgs:
         orc.score(c)
     dt_py = time.perf_counter() - t0
-    return {"value": P / dt_all, "unit": "plans/s", "cores": threads, "kind": "port",
+    cpu_model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            cpu_model = next((ln.split(":", 1)[1].strip() for ln in f if ln.startswith("model name")), cpu_model)
+    except OSError:
+        pass
+    return {"value": P / dt_all, "unit": "plans/s", "cores": threads, "kind": "port", "cpu_model": cpu_model,
             "sample": f"all {P} plans of the same batch in {dt_all:.2f} s, C oracle (oracle/aceso_oracle.c), "
                       f"{threads} OpenMP threads",
             "single_core_value": n1 / dt_one, "single_core_sample": f"first {n1} plans, {dt_one:.2f} s, 1 thread",

@@ -129,7 +129,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
     int lo, hi;                 // RANGED: only ops lo <= i < hi belong to the plan (one stage)
     // stage state
     int s;
-    uint32_t hot_v, z_v, rk_v, mrow, dc_v;
+    uint32_t z_v, rk_v, mrow, dc_v;
     uint32_t t_first;
     bool out_cross;
     double in_comm, inputs, id_in;
@@ -161,7 +161,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = rs_f = rs_b = 0.0;
         id_fwd = id_bwd = id_in = 0.0;
         in_comm = inputs = 0.0;
-        hot_v = z_v = rk_v = mrow = t_first = dc_v = 0;
+        z_v = rk_v = mrow = t_first = dc_v = 0;
         out_cross = false;
         ideal_hot_v = ideal_start_v = 0;
         if (bidx >= (uint32_t)g.n_mbs) { status = ACE_PLAN_MALFORMED; bidx = 0; }
@@ -190,7 +190,6 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         const uint32_t sh = 4u * ((uint32_t)s & 15u);
         const uint32_t d = (uint32_t)(diags >> sh) & 15u;
         const uint32_t glog = (uint32_t)(glogs >> sh) & 15u;
-        hot_v = ace_mul24(d, (uint32_t)g.C * ACE_HOT_STRIDE);
         z_v = ace_mul24(d, (uint32_t)g.C * 8u);
         rk_v = (glog < (uint32_t)g.n_glog ? glog : 0u) << 6;   // (a stage size outside the tables is unscorable anyway)
         if (tail) {
@@ -326,7 +325,10 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         const uint32_t nc = nbyte & 7u;
         const bool rc = (byte >> 3) & 1u;
         const uint32_t row = info_row(g, info);
-        const uint32_t a = (row + g.hot_off) + ace_mad24(c, ACE_HOT_STRIDE, hot_v);
+        // entry index inside the diag's block, in 8-byte units: the hot entry is 48 bytes, the
+        // collective-cost entry 8 bytes, so one multiply-add serves both addresses
+        const uint32_t zc = ace_mad24(c, 8u, z_v);
+        const uint32_t a = ace_mad24(zc, ACE_HOT_STRIDE / 8u, row + g.hot_off);
         ace_d2 e0 = lds.ld<ace_d2>(a);         // fwd us, bwd us
         ace_d2 e1 = lds.ld<ace_d2>(a + 16);    // weights MB, activations MB (shared-buffer rule applied)
         ace_d2 e2 = lds.ld<ace_d2>(a + 32);    // fwd / bwd reserved MB
@@ -348,7 +350,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
             const uint32_t pk = (info >> 16) & 0xffu;
             // (rk_v is a multiple of 64 and c * 8 + nc < 64: the sum is the [c][nc] entry of the stage-size block)
             r_next = lds.ld<uint8_t>((g.rk_lds_off + ace_mul24(pk, g.rk_kind_stride)) + (ace_mad24(c, 8u, rk_v) + nc));
-            const uint32_t za = (row + g.z_off) + ace_mad24(c, 8u, z_v);
+            const uint32_t za = (row + g.z_off) + zc;
             rs_f += lds.ld<double>(za + ((r & 15u) << g.z_shift));
             rs_b += lds.ld<double>(za + ((r >> 4) << g.z_shift));
         }

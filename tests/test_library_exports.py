@@ -65,3 +65,23 @@ def test_no_gpu_means_no_scoring():
     tables = synth.make_tables(synth.WORKLOADS["gpt3_1_3b"])
     with pytest.raises(evaluator.AceError):
         evaluator.PlanEvaluator(tables)
+
+
+def test_header_is_plain_c_and_matches_the_library(tmp_path):
+    """include/ace_eval.h compiles as C99 on its own, and a C program that takes the address of every
+    declared function links against the library (the declarations and the exports agree)."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    hdr = os.path.join(root, "include", "ace_eval.h")
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic", "-fsyntax-only", "-x", "c", hdr], check=True)
+    src = tmp_path / "use.c"
+    src.write_text('#include "ace_eval.h"\n#include <stdio.h>\nint main(void) {\n'
+                   '  const void *f[] = {' + ", ".join(f"(const void *)&{n}" for n in evaluator.EXPORTS) + '};\n'
+                   '  printf("%d %d\\n", ace_abi_version(), (int)(sizeof f / sizeof f[0]));\n  return 0;\n}\n')
+    exe = tmp_path / "use"
+    libdir = os.path.join(root, "superscaler_amd")
+    subprocess.run(["gcc", "-std=c99", "-Wno-pedantic", "-I" + os.path.join(root, "include"), str(src), "-o", str(exe),
+                    "-L" + libdir, "-l:libace_eval.so", "-Wl,-rpath," + libdir], check=True)

@@ -137,7 +137,10 @@ void ace_destroy(ace_handle_t *h);
  * gen_megatron_plan.py:111).
  *  d_iter_ms, d_peak_mb: double[n_plans];  d_feasible, d_status: uint8[n_plans] (d_status may be NULL)
  *  d_stage_out: NULL, or double[n_plans][ACE_MAX_STAGES][ACE_STAGE_REC] receiving the per-stage
- *  quantities predict_time_breakdown / predict_stage_time / predict_stage_memory are made of. */
+ *  quantities predict_time_breakdown / predict_stage_time / predict_stage_memory are made of.
+ * Plain scoring (no d_stage_out, no d_range) uses a workspace owned by the handle (80 bytes per plan
+ * and stage, allocated on first use and grown when a larger batch arrives: that call allocates), so
+ * scoring calls on one handle must be stream-ordered with respect to each other. */
 int ace_score_batch(ace_handle_t *h, const ace_batch_t *batch, double memory_limit, int strict,
                     double *d_iter_ms, double *d_peak_mb, uint8_t *d_feasible, uint8_t *d_status,
                     double *d_stage_out, void *stream);

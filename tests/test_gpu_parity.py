@@ -211,6 +211,32 @@ def test_configured_sizes_match_c_oracle(name, n, torch_mod):
     ev.close()
 
 
+@pytest.mark.parametrize("name", list(synth.WORKLOADS))
+def test_stage_records_match_c_oracle_lists(name, torch_mod):
+    """The per-stage records (breakdown kernel; windowed for wresnet_1b) against the C oracle's
+    time_list / memory_list for a few thousand plans: memory per stage directly, time through
+    time_list[s] = t_s * (nb - 1) + sum(t)."""
+    from superscaler_amd.evaluator import PlanEvaluator
+    from superscaler_amd.tables import R_STAGE_MB, R_STAGE_MS
+    w = synth.WORKLOADS[name]
+    tables = synth.make_tables(w)
+    batch = synth.make_plans(w, tables, n_plans=4000, seed_offset=31, workers=4)
+    ev = PlanEvaluator(tables)
+    it, pk, fe, st, rec = ev.score_host(batch, breakdown=True)
+    ev.close()
+    cit, cpk, cfe, cer, tl, ml = c_oracle_scores(tables, batch, threads=8, lists=True)
+    assert not cer.any() and np.array_equal(it, cit) and np.array_equal(pk, cpk) and np.array_equal(fe, cfe)
+    S = (batch.hdr[:, 0] & 0xff).astype(int)
+    nbm1 = tables.nb_minus_1[(batch.hdr[:, 0] >> 8) & 0xff]
+    tsum = np.zeros(batch.n_plans)
+    for s in range(16):
+        tsum = np.where(S > s, tsum + rec[:, s, R_STAGE_MS], tsum)
+    for s in range(16):
+        m = S > s
+        assert np.array_equal(rec[m, s, R_STAGE_MB], ml[m, s])
+        assert np.array_equal((rec[:, s, R_STAGE_MS] * nbm1 + tsum)[m], tl[m, s])
+
+
 def test_known_answers_single_gpu_plans(golden_dir, torch_mod):
     """The reference tree's own single-GPU plans and published predictions
     (results/ref/perf_model_{time,mem}_large_{gpt,resnet}.csv), through the GPU path."""

@@ -73,12 +73,36 @@ def update_recompute_arrays(cm, batch: PlanBatch) -> PlanBatch:
         h[:, 0] = (q_nsb[qsel] + 1) | (q_bidx[qsel] << 8)
         h[:, 1] = q_glog[qsel]
         rg = np.stack([q_lo[qsel], q_hi[qsel]], axis=1).astype(np.uint32)
-        out = cm.evaluator.score_host(PlanBatch(codes[q_plan[qsel]], h), breakdown=True, ranges=rg)
-        cm._raise_for_status(out[3])
-        return out[4][:, 0, :]
+        batch = PlanBatch(codes[q_plan[qsel]], h)
+        ev = cm.evaluator
+        if hasattr(ev, "score"):
+            # a single-stage query fills stage record 0 only: bring back just that one
+            out = ev.score(ev.upload(batch, ranges=rg), breakdown=True)
+            status, rec0 = out[3].cpu().numpy(), out[4][:, 0, :].cpu().numpy()
+        else:
+            out = ev.score_host(batch, breakdown=True, ranges=rg)
+            status, rec0 = out[3], out[4][:, 0, :]
+        cm._raise_for_status(status)
+        return rec0
 
-    every = np.arange(Q)
-    mem = _stage_memory(cm, records(every), q_nsb.astype(np.float64)) + args.peak_mem_in_backward
+    def all_records():
+        """Stage records of every stage with all recompute bits cleared: one launch over the plans
+        themselves (a stage's memory terms do not depend on its neighbours)."""
+        ev = cm.evaluator
+        plans = PlanBatch(codes, hdr)
+        if hasattr(ev, "score"):
+            import torch
+            out = ev.score(ev.upload(plans), breakdown=True)
+            dev = out[4].device
+            pick = out[4][torch.from_numpy(q_plan).to(dev), torch.from_numpy(q_s).to(dev)]
+            status, rec = out[3].cpu().numpy(), pick.cpu().numpy()
+        else:
+            out = ev.score_host(plans, breakdown=True)
+            status, rec = out[3], out[4][q_plan, q_s]
+        cm._raise_for_status(status)
+        return rec
+
+    mem = _stage_memory(cm, all_records(), q_nsb.astype(np.float64)) + args.peak_mem_in_backward
     act = np.flatnonzero(mem - args.memory_limit > 0)
     if len(act) == 0:
         return PlanBatch(codes, hdr.copy())
@@ -89,7 +113,7 @@ def update_recompute_arrays(cm, batch: PlanBatch) -> PlanBatch:
     norec = (np.asarray(tables.graph.flags)[:n_types] & og.F_NO_RECOMPUTE) != 0
     lens = (q_hi - q_lo)[act]
     e_q = np.repeat(np.arange(len(act)), lens)                       # element -> active stage, in (stage, position) order
-    e_pos = np.concatenate([np.arange(lo, hi) for lo, hi in zip(q_lo[act], q_hi[act])])
+    e_pos = np.arange(int(lens.sum())) - np.repeat(np.cumsum(lens) - lens, lens) + np.repeat(q_lo[act], lens)
     e_type = type_of_pos[e_pos]
     e_code = (codes[q_plan[act][e_q], e_pos] & 7).astype(np.int64)
     e_tp, e_algo = e_code >> a_shift, e_code & (A - 1)
@@ -104,9 +128,11 @@ def update_recompute_arrays(cm, batch: PlanBatch) -> PlanBatch:
     first_pos = np.full((nA, n_types), N, dtype=np.int64)
     np.minimum.at(first_pos, (e_q, e_type), e_pos)
     # the members of every (stage, type) group, in position order
-    order = np.lexsort((e_pos, e_type, e_q))
+    # (elements are in (stage, position) order already: a stable sort by (stage, type) keeps positions ascending)
+    e_key = (e_q * n_types + e_type).astype(np.int32 if nA * n_types < 2 ** 31 else np.int64)
+    order = np.argsort(e_key, kind="stable")
     g_pos, g_size = e_pos[order], e_size[order]
-    g_key = e_q[order] * n_types + e_type[order]
+    g_key = e_key[order]
     g_start = np.full(nA * n_types, 0, dtype=np.int64)
     g_count = np.bincount(g_key, minlength=nA * n_types)
     g_start[1:] = np.cumsum(g_count)[:-1]

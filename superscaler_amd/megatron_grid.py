@@ -86,3 +86,53 @@ def best_uniform_plans(cm: CostModel, num_gpus: int, num_layers: Optional[int], 
         if t not in best or m < best[t][0]:
             best[t] = (m, i)
     return [(t, best[t][0], configs[best[t][1]]) for t in sorted(best)[:num_saved]]
+
+
+def main(argv=None) -> int:
+    """Command line with the arguments gen_megatron_plan.py reads (aceso_utils.py:359-531, the subset
+    this script uses): scores the whole uniform grid in one launch and writes the fastest feasible
+    plans as JSON files the runtime accepts, named like the reference's (:135)."""
+    import argparse
+    import time
+    from .plan import dump_config_to_json
+    from .profile_db import CostModelSettings
+    ap = argparse.ArgumentParser(description=main.__doc__)
+    ap.add_argument("--model-name", required=True, choices=["gpt", "t5", "resnet", "scale-layer"])
+    ap.add_argument("--model-size", required=True)
+    ap.add_argument("--num-layers", type=int, default=None)
+    ap.add_argument("--global-batch-size", type=int, default=1024)
+    ap.add_argument("--micro-batch-size", type=int, nargs="+", default=[1, 2, 4, 8])
+    ap.add_argument("--num-nodes", type=int, default=1)
+    ap.add_argument("--num-gpus-per-node", type=int, default=8)
+    ap.add_argument("--memory-limit", type=float, default=28000)
+    ap.add_argument("--max-tp", type=int, default=None)
+    ap.add_argument("--start-num-stages", type=int, default=1)
+    ap.add_argument("--end-num-stages", type=int, default=None)
+    ap.add_argument("--num-of-saved-configs", type=int, default=1)
+    ap.add_argument("--profiled-time-path", required=True, help="directory of the profiled CSV files, with the trailing /")
+    ap.add_argument("--config-save-path", default="./")
+    args = ap.parse_args(argv)
+    num_gpus = args.num_nodes * args.num_gpus_per_node
+    settings = CostModelSettings(model_name=args.model_name, micro_batch_size=list(args.micro_batch_size),
+                                 num_gpus_per_node=args.num_gpus_per_node, global_batch_size=args.global_batch_size,
+                                 memory_limit=args.memory_limit, max_tp=args.max_tp or args.num_gpus_per_node)
+    t0 = time.time()
+    cm = CostModel.from_directory(settings, args.model_name, args.model_size, args.profiled_time_path,
+                                  num_layers=args.num_layers)
+    try:
+        best = best_uniform_plans(cm, num_gpus, args.num_layers, args.num_of_saved_configs, args.start_num_stages,
+                                  args.end_num_stages)
+    finally:
+        cm.close()
+    if not best:
+        print("no feasible config")
+    for k, (t, m, cfg) in enumerate(best):
+        name = f"{args.config_save_path}{args.model_name}_{args.model_size}_{args.num_layers}layers_megatron_est_{int(t)}.json"
+        dump_config_to_json(cfg, name, args.model_name, args.model_size, args.num_layers)
+        print(f"best_{k}: {t:.2f} ms, {m:.2f} MB, {cfg.num_stages} stages, micro-batch {cfg.micro_bs} -> {name}")
+    print(f"[TOTAL TIME] {time.time() - t0} s.")
+    return 0
+
+
+if __name__ == "__main__":
+    raise SystemExit(main())

@@ -238,3 +238,34 @@ def test_recompute_arrays_gpu_equals_cpu_build():
         assert 0.1 < frac < 0.9
     finally:
         m.close()
+
+
+@pytest.mark.gpu
+def test_uniform_grid_command_line(golden_dir, tmp_path, capsys):
+    """`python -m superscaler_amd.megatron_grid` on the reference's GPT-1.3B database: writes plan JSON
+    files the loader reads back, best first, and the best one is what best_uniform_plans returns."""
+    from superscaler_amd import megatron_grid
+    from superscaler_amd.plan import config_from_json
+    with open(os.path.join(golden_dir, "gpt_1_3B.json")) as f:
+        g = json.load(f)
+    argv = ["--model-name", g["model_name"], "--model-size", g["model_size"], "--num-layers", str(g["num_layers"]),
+            "--global-batch-size", str(g["global_batch_size"]), "--micro-batch-size"] + [str(x) for x in g["micro_batch_size"]] + \
+           ["--num-nodes", "2", "--num-gpus-per-node", str(g["num_gpus_per_node"]), "--memory-limit", str(g["memory_limit"]),
+            "--profiled-time-path", os.path.join(golden_dir, "db_gpt_1_3B") + "/", "--config-save-path", str(tmp_path) + "/",
+            "--num-of-saved-configs", "3"]
+    assert megatron_grid.main(argv) == 0
+    out = capsys.readouterr().out
+    files = sorted(tmp_path.glob("*.json"))
+    assert 1 <= len(files) <= 3 and "best_0" in out
+    _, m = make_model(golden_dir, "gpt_1_3B", "gpu")
+    try:
+        want = megatron_grid.best_uniform_plans(m, 2 * g["num_gpus_per_node"], g["num_layers"], 3)
+        assert len(want) == len(files)
+        names = {f.name for f in files}
+        for t, mem, cfg in want:
+            assert f"gpt_{g['model_size']}_{g['num_layers']}layers_megatron_est_{int(t)}.json" in names
+        best = config_from_json(str(tmp_path / f"gpt_{g['model_size']}_{g['num_layers']}layers_megatron_est_{int(want[0][0])}.json"), m.graph.ops)
+        m.predict_time_breakdown(best)
+        assert max(best.time_list) == want[0][0] and max(best.memory_list) == want[0][1]
+    finally:
+        m.close()

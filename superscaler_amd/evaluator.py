@@ -250,6 +250,20 @@ class PlanEvaluator:
             del d
         return best_idx, best_val, offset
 
+    def stage_records_host(self, batch: PlanBatch, ranges: np.ndarray):
+        """Single-stage queries: (status, stage record 0 of every query) as numpy arrays."""
+        out = self.score(self.upload(batch, ranges=ranges), breakdown=True)
+        return out[3].cpu().numpy(), out[4][:, 0, :].cpu().numpy()
+
+    def picked_records_host(self, batch: PlanBatch, plan_idx: np.ndarray, stage_idx: np.ndarray):
+        """Whole plans: (status of every plan, the stage records [plan_idx[k], stage_idx[k]]) as numpy arrays
+        (picked on the device, so only those records cross the bus)."""
+        torch = self._torch
+        out = self.score(self.upload(batch), breakdown=True)
+        pick = out[4][torch.from_numpy(np.ascontiguousarray(plan_idx)).to(self.device),
+                      torch.from_numpy(np.ascontiguousarray(stage_idx)).to(self.device)]
+        return out[3].cpu().numpy(), pick.cpu().numpy()
+
     # convenience: host in, host out
     def score_host(self, batch: PlanBatch, memory_limit=None, strict=False, breakdown=False, ranges=None):
         d = self.upload(batch, ranges=ranges)

@@ -73,32 +73,14 @@ def update_recompute_arrays(cm, batch: PlanBatch) -> PlanBatch:
         h[:, 0] = (q_nsb[qsel] + 1) | (q_bidx[qsel] << 8)
         h[:, 1] = q_glog[qsel]
         rg = np.stack([q_lo[qsel], q_hi[qsel]], axis=1).astype(np.uint32)
-        batch = PlanBatch(codes[q_plan[qsel]], h)
-        ev = cm.evaluator
-        if hasattr(ev, "score"):
-            # a single-stage query fills stage record 0 only: bring back just that one
-            out = ev.score(ev.upload(batch, ranges=rg), breakdown=True)
-            status, rec0 = out[3].cpu().numpy(), out[4][:, 0, :].cpu().numpy()
-        else:
-            out = ev.score_host(batch, breakdown=True, ranges=rg)
-            status, rec0 = out[3], out[4][:, 0, :]
+        status, rec0 = cm.evaluator.stage_records_host(PlanBatch(codes[q_plan[qsel]], h), rg)
         cm._raise_for_status(status)
         return rec0
 
     def all_records():
         """Stage records of every stage with all recompute bits cleared: one launch over the plans
         themselves (a stage's memory terms do not depend on its neighbours)."""
-        ev = cm.evaluator
-        plans = PlanBatch(codes, hdr)
-        if hasattr(ev, "score"):
-            import torch
-            out = ev.score(ev.upload(plans), breakdown=True)
-            dev = out[4].device
-            pick = out[4][torch.from_numpy(q_plan).to(dev), torch.from_numpy(q_s).to(dev)]
-            status, rec = out[3].cpu().numpy(), pick.cpu().numpy()
-        else:
-            out = ev.score_host(plans, breakdown=True)
-            status, rec = out[3], out[4][q_plan, q_s]
+        status, rec = cm.evaluator.picked_records_host(PlanBatch(codes, hdr), q_plan, q_s)
         cm._raise_for_status(status)
         return rec
 

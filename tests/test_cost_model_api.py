@@ -29,6 +29,14 @@ class EmuEvaluator:
         it, pk, fe, st, rec = emu_score(self.tables, batch, memory_limit, strict, breakdown, ranges)
         return (it, pk, fe, st, rec) if (breakdown or ranges is not None) else (it, pk, fe, st)
 
+    def stage_records_host(self, batch, ranges):
+        out = emu_score(self.tables, batch, None, False, True, ranges)
+        return out[3], out[4][:, 0, :]
+
+    def picked_records_host(self, batch, plan_idx, stage_idx):
+        out = emu_score(self.tables, batch, None, False, True, None)
+        return out[3], out[4][plan_idx, stage_idx]
+
     def close(self):
         pass
 

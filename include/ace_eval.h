@@ -155,6 +155,24 @@ int ace_topk(ace_handle_t *h, const double *d_iter_ms, const uint8_t *d_feasible
              int64_t *d_idx, double *d_val, int32_t *d_count, void *d_workspace, size_t workspace_bytes,
              void *stream);
 
+/* Expand move descriptors into a batch of neighbour plans on the device, in the layout
+ * ace_score_batch reads.  Replaces the per-candidate object rebuilding of the reference's move
+ * primitives (search/aceso_prims.py:66-134 op migration, :357-375 tp / dp changes, :544-580
+ * micro-batch steps, recompute and algorithm fine-tuning) for candidates that differ from a
+ * template plan by one edit.
+ *  d_template_codes: uint8[n_templates][16 * ceil(num_ops / 16)], one byte per op as in ace_batch_t,
+ *                    plan-major (template 0 is normally the plan whose neighbours are wanted);
+ *  d_template_hdr:   uint32[n_templates][4];
+ *  d_moves:          uint32[n_moves][4] = template | op << 16, p0, p1, 0 with
+ *                    op 0 copy; 1 migrate ops across a stage boundary (p0 = cut | new cut << 16, p1 = log2 tp
+ *                    the moved ops take); 2 one tp step for the ops p0 = first | last + 1 << 16 (p1 = 1 up, 0 down);
+ *                    3 toggle the recompute bit of the ops p0 = first | last + 1 << 16; 4 toggle the algorithm of op p0;
+ *  d_codes_out:      uint8[ceil(num_ops / 16)][n_moves][16];  d_hdr_out: uint32[n_moves][4].
+ * The caller decides which moves are legal; the kernel only edits bytes. */
+int ace_apply_moves(const uint8_t *d_template_codes, const uint32_t *d_template_hdr, int n_templates,
+                    const uint32_t *d_moves, size_t n_moves, int num_ops, int n_algo, uint8_t *d_codes_out,
+                    uint32_t *d_hdr_out, void *stream);
+
 /* Average duration in milliseconds of the `reps` scoring-kernel launches of one
  * ace_score_batch-equivalent call sequence, measured with hipEvents on `stream`
  * (for bench.py's roofline figure; not part of the reference). */

@@ -413,6 +413,57 @@ struct ace_handle {
     size_t stage_ws_plans;     // capacity in plans
 };
 
+// ------------------------------------------------------------------------------------------
+// Move descriptors -> plans: one thread writes one 16-byte word (16 ops) of one neighbour.
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void apply_moves_kernel(const ace_u4 *tmpl_codes, const ace_u4 *tmpl_hdr, int n_templates,
+                                                          const ace_u4 *moves, unsigned long long n, int G, int a_shift,
+                                                          ace_u4 *codes_out, ace_u4 *hdr_out) {
+    const unsigned long long id = (unsigned long long)blockIdx.x * 256 + threadIdx.x;
+    if (id >= n * (unsigned long long)G) return;
+    const unsigned long long k = id % n;              // consecutive lanes: consecutive neighbours of one word
+    const int g = (int)(id / n);
+    const ace_u4 mv = moves[k];
+    uint32_t t = mv.x & 0xffffu;
+    if (t >= (uint32_t)n_templates) t = 0;
+    const uint32_t op = mv.x >> 16;
+    const ace_u4 src = tmpl_codes[(size_t)t * G + g];
+    if (g == 0) hdr_out[k] = tmpl_hdr[t];
+    uint32_t w[4] = {src.x, src.y, src.z, src.w};
+    const uint32_t lo16 = mv.y & 0xffffu, hi16 = mv.y >> 16;
+    const uint32_t amask = (1u << a_shift) - 1u;      // algo bits of a code
+    uint32_t lo = lo16, hi = hi16;                    // byte range [lo, hi) an edit covers
+    if (op == 1u) { lo = lo16 < hi16 ? lo16 : hi16; hi = lo16 < hi16 ? hi16 : lo16; }
+    if (op == 4u) { lo = lo16; hi = lo16 + 1u; }
+    const uint32_t base = (uint32_t)g * 16u;
+    const uint32_t hi_touch = op == 1u ? hi + 1u : hi;      // a migration also edits the byte at the far end
+    if (op != 0u && lo < base + 16u && hi_touch > base) {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const uint32_t p = base + (uint32_t)j;
+            uint32_t b = (w[j >> 2] >> (8 * (j & 3))) & 0xffu;
+            const bool in = p >= lo && p < hi;
+            if (op == 1u) {                            // migrate: cut = lo16, new cut = hi16, tp = mv.z
+                if (p == lo16) b &= 0xEFu;
+                if (in) b = ((b & 0xF8u) | ((mv.z << a_shift) + (b & amask))) & 0xffu;
+                if (p == hi16) b |= 0x10u;
+            } else if (op == 2u) {                     // every op of the stage one tp step up (mv.z = 1) or down
+                if (in) {
+                    int tp = (int)((b & 7u) >> a_shift) + (mv.z == 1u ? 1 : -1);
+                    tp = tp < 0 ? 0 : (tp > 7 ? 7 : tp);
+                    b = ((b & 0xF8u) | (((uint32_t)tp << a_shift) + (b & amask))) & 0xffu;
+                }
+            } else if (op == 3u) {                     // recompute toggle
+                if (in) b ^= 8u;
+            } else if (op == 4u) {                     // algorithm toggle
+                if (in) b ^= 1u;
+            }
+            w[j >> 2] = (w[j >> 2] & ~(0xffu << (8 * (j & 3)))) | (b << (8 * (j & 3)));
+        }
+    }
+    codes_out[(size_t)g * n + k] = ace_u4{w[0], w[1], w[2], w[3]};
+}
+
 extern "C" {
 
 int ace_abi_version(void) { return ACE_ABI_VERSION; }
@@ -690,6 +741,28 @@ int ace_topk(ace_handle_t *h, const double *d_iter_ms, const uint8_t *d_feasible
     // redo them exactly (lowest indices first).  Cheap single-workgroup scan that stops early.
     hipLaunchKernelGGL(topk_ties_exact, dim3(1), dim3(kTopBlock), 0, s, d_iter_ms, d_feasible, n, st, ties, cap);
     hipLaunchKernelGGL(topk_finish, dim3(1), dim3(1024), 0, s, st, less, ties, cap, k, buf, p2, (long long *)d_idx, d_val, d_count);
+    ACE_HIP(hipGetLastError());
+    return ACE_OK;
+}
+
+int ace_apply_moves(const uint8_t *d_template_codes, const uint32_t *d_template_hdr, int n_templates,
+                    const uint32_t *d_moves, size_t n_moves, int num_ops, int n_algo, uint8_t *d_codes_out,
+                    uint32_t *d_hdr_out, void *stream) {
+    if (!d_template_codes || !d_template_hdr || !d_moves || !d_codes_out || !d_hdr_out || n_templates <= 0 ||
+        n_templates > 65536 || n_moves == 0 || n_moves > 0x7fffffffull || num_ops <= 0 || num_ops >= 65536 ||
+        (n_algo != 1 && n_algo != 2))
+        return ACE_EINVAL;
+    if (((uintptr_t)d_template_codes & 15u) || ((uintptr_t)d_template_hdr & 15u) || ((uintptr_t)d_moves & 15u) ||
+        ((uintptr_t)d_codes_out & 15u) || ((uintptr_t)d_hdr_out & 15u))
+        return ACE_EINVAL;
+    const int G = (num_ops + 15) / 16;
+    const unsigned long long total = (unsigned long long)n_moves * (unsigned long long)G;
+    const unsigned long long blocks = (total + 255) / 256;
+    if (blocks > 0x7fffffffull) return ACE_ETOOBIG;
+    hipLaunchKernelGGL(apply_moves_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       reinterpret_cast<const ace_u4 *>(d_template_codes), reinterpret_cast<const ace_u4 *>(d_template_hdr),
+                       n_templates, reinterpret_cast<const ace_u4 *>(d_moves), (unsigned long long)n_moves, G,
+                       n_algo == 2 ? 1 : 0, reinterpret_cast<ace_u4 *>(d_codes_out), reinterpret_cast<ace_u4 *>(d_hdr_out));
     ACE_HIP(hipGetLastError());
     return ACE_OK;
 }

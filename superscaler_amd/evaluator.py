@@ -16,7 +16,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libace_eva
 _lib = None
 
 EXPORTS = ["ace_abi_version", "ace_strerror", "ace_last_hip_error", "ace_create", "ace_destroy",
-           "ace_score_batch", "ace_topk_workspace_bytes", "ace_topk", "ace_time_score_kernel"]
+           "ace_score_batch", "ace_topk_workspace_bytes", "ace_topk", "ace_time_score_kernel", "ace_apply_moves"]
 
 
 class AceBatchStruct(ctypes.Structure):
@@ -59,6 +59,9 @@ def load_library():
     lib.ace_time_score_kernel.argtypes = [ctypes.c_void_p, ctypes.POINTER(AceBatchStruct), ctypes.c_double,
                                           ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                           ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(ctypes.c_double)]
+    lib.ace_apply_moves.restype = ctypes.c_int
+    lib.ace_apply_moves.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t,
+                                    ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
     if lib.ace_abi_version() != ABI_VERSION:
         raise AceError("libace_eval.so has a different ABI version")
     _lib = lib
@@ -102,6 +105,15 @@ class DeviceBatch:
             self.ranges = torch.from_numpy(r.view(np.int32)).to(device)
         self.struct = AceBatchStruct(self.codes.data_ptr(), self.hdr.data_ptr(),
                                      self.ranges.data_ptr() if self.ranges is not None else None, P)
+
+    @classmethod
+    def from_device(cls, codes, hdr, num_ops: int):
+        """Wrap tensors that are already on the device in the kernel's layout: codes uint8 [G, P, 16], hdr int32 [P, 4]."""
+        self = cls.__new__(cls)
+        self.n_plans, self.num_ops = int(hdr.shape[0]), int(num_ops)
+        self.codes, self.hdr, self.ranges = codes, hdr, None
+        self.struct = AceBatchStruct(codes.data_ptr(), hdr.data_ptr(), None, self.n_plans)
+        return self
 
     @property
     def bytes_moved_per_plan(self):
@@ -249,6 +261,26 @@ class PlanEvaluator:
             offset += d.n_plans
             del d
         return best_idx, best_val, offset
+
+    def apply_moves(self, templates: PlanBatch, moves: np.ndarray) -> DeviceBatch:
+        """Expand move descriptors (neighbours.sample_moves) into a device-resident batch: only the
+        templates and 16 bytes per neighbour cross the bus."""
+        torch = self._torch
+        T, N = templates.codes.shape
+        G = (N + 15) // 16
+        n = int(moves.shape[0])
+        tc = np.zeros((T, G * 16), dtype=np.uint8)
+        tc[:, :N] = templates.codes
+        d_tc = torch.from_numpy(tc).to(self.device)
+        d_th = torch.from_numpy(np.ascontiguousarray(templates.hdr).view(np.int32)).to(self.device)
+        d_mv = torch.from_numpy(np.ascontiguousarray(moves, dtype=np.uint32).view(np.int32)).to(self.device)
+        codes = torch.empty((G, n, 16), dtype=torch.uint8, device=self.device)
+        hdr = torch.empty((n, 4), dtype=torch.int32, device=self.device)
+        with torch.cuda.device(self.device):
+            rc = self.lib.ace_apply_moves(d_tc.data_ptr(), d_th.data_ptr(), T, d_mv.data_ptr(), n, N,
+                                          self.tables.db.n_algo, codes.data_ptr(), hdr.data_ptr(), self._stream())
+        _check(self.lib, rc, "ace_apply_moves")
+        return DeviceBatch.from_device(codes, hdr, N)
 
     def stage_records_host(self, batch: PlanBatch, ranges: np.ndarray):
         """Single-stage queries: (status, stage record 0 of every query) as numpy arrays."""

@@ -36,13 +36,26 @@ def _set_header(hdr_row, S, bidx, glogs, gpn):
     hdr_row[3] = cross
 
 
-def make_neighbours(base: PlanBatch, tables: CompiledTables, n: int, rng: np.random.Generator,
-                    max_move: int = 8) -> PlanBatch:
-    """n single-move neighbours of base plan 0 (moves that would leave the profiled grid are replaced
-    by a copy of the base plan, so the batch always has n valid rows).  All neighbours of one kind
-    are produced together: masks over a [neighbours, ops] byte matrix, no per-neighbour Python."""
+# edit operations of a move descriptor (uint32[4]: template | op << 16, p0, p1, unused)
+OP_NONE, OP_MIGRATE, OP_TP_STEP, OP_RC_TOGGLE, OP_ALGO_TOGGLE = 0, 1, 2, 3, 4
+
+
+def sample_moves(base: PlanBatch, tables: CompiledTables, n: int, rng: np.random.Generator,
+                 max_move: int = 8) -> Tuple[PlanBatch, np.ndarray]:
+    """n single-move neighbours of base plan 0 as (templates, moves).  A neighbour is one template row
+    (0 = the base plan; the others carry a changed header: micro-batch steps and device moves between
+    stages) plus at most one edit of its code bytes, described by four words:
+        template | op << 16,  p0,  p1,  0
+        OP_MIGRATE      p0 = cut | new cut << 16, p1 = tp (log2) the moved ops take
+        OP_TP_STEP      p0 = first op | one past the last << 16, p1 = 1 (tp up) or 0 (tp down)
+        OP_RC_TOGGLE    p0 = first op | one past the last << 16
+        OP_ALGO_TOGGLE  p0 = op position
+    Moves that would leave the profiled grid become (template 0, OP_NONE): a copy of the base plan.
+    `apply_moves_host` (numpy) and the library's ace_apply_moves (on the device) expand them."""
     A = tables.db.n_algo
     N = tables.graph.num_ops
+    if N >= 65536:
+        raise ValueError("move descriptors hold 16-bit op positions")
     gpn = tables.settings.num_gpus_per_node
     row0, hdr0 = base.codes[0], base.hdr[0]
     S = int(hdr0[0] & 0xff)
@@ -52,23 +65,17 @@ def make_neighbours(base: PlanBatch, tables: CompiledTables, n: int, rng: np.ran
     starts, ends = _stage_bounds(row0)
     tunable = (tables.graph.flags[tables.graph.type_of_pos] & og.F_TUNABLE) != 0
     M = len(tables.db.mbs_list)
-    codes = np.repeat(row0[None, :], n, axis=0)
-    hdr = np.repeat(hdr0[None, :], n, axis=0)
-    kinds = rng.integers(0, 6, size=n)
-    pos = np.arange(N)
     tp0 = ((row0 & 7) // A).astype(np.int64)
     stage_of_pos = np.cumsum((row0 >> 4) & 1) - 1
+    kinds = rng.integers(0, 6, size=n)
+    moves = np.zeros((n, 4), dtype=np.uint32)
+    t_codes, t_hdr = [row0.copy()], [hdr0.copy()]
 
     def allowed(b, gl):
         return tables.allowed_tp_logs(b, gl)
 
     def ok_bits(b, gl):
         return sum(1 << t for t in allowed(b, gl))
-
-    def with_tp(seg, t):
-        """The code bytes `seg` with their tp replaced by t (algo, recompute and stage bits kept)."""
-        t8 = np.asarray(t).astype(np.uint8)
-        return (seg & np.uint8(0xF8)) | (t8 * np.uint8(A) + (seg & np.uint8(A - 1)))
 
     # kind 0, op migration: move a stage boundary by up to max_move ops; the ops that change stage
     # take the tp of the op they now follow / precede in the receiving stage
@@ -81,30 +88,27 @@ def make_neighbours(base: PlanBatch, tables: CompiledTables, n: int, rng: np.ran
         good = (new_cut > starts[j - 1]) & (new_cut < ends[j])
         rows, cut, new_cut, d = rows[good], cut[good], new_cut[good], d[good]
         ref = np.where(d > 0, tp0[cut - 1], tp0[cut])        # stage j-1 grows to the right / stage j to the left
-        moved = (pos[None, :] >= np.minimum(cut, new_cut)[:, None]) & (pos[None, :] < np.maximum(cut, new_cut)[:, None])
-        sub = codes[rows]
-        sub[np.arange(len(rows)), cut] &= 0xEF
-        sub = np.where(moved, with_tp(sub, ref[:, None]), sub)
-        sub[np.arange(len(rows)), new_cut] |= 16
-        codes[rows] = sub
+        moves[rows, 0] = OP_MIGRATE << 16
+        moves[rows, 1] = cut | (new_cut << 16)
+        moves[rows, 2] = ref
 
     # kind 1, tp <-> dp inside one stage: all ops one step up or down, if the stage allows it
     rows = np.flatnonzero(kinds == 1)
     if len(rows):
         s = rng.integers(0, S, size=len(rows))
         step = np.where(rng.random(len(rows)) < 0.5, 1, -1)
-        inside = (pos[None, :] >= starts[s][:, None]) & (pos[None, :] < ends[s][:, None])
         # a stage's ops may sit on different tp: the move is legal iff every tp value present has a legal target
         bits = np.array([ok_bits(bidx, int(g)) for g in glogs], dtype=np.int64)
         present = np.array([sum(1 << int(v) for v in np.unique(tp0[starts[k]:ends[k]])) for k in range(S)], dtype=np.int64)
         want = np.where(step > 0, present[s] << 1, present[s] >> 1)
         lost = (step < 0) & ((present[s] & 1) == 1)                      # tp = 1 cannot go down
         good = ((want & ~bits[s]) == 0) & ~lost
-        t8 = (tp0[None, :] + step[good][:, None]).clip(0, 7).astype(np.uint8)
-        sub = codes[rows[good]]
-        codes[rows[good]] = np.where(inside[good], with_tp(sub, t8), sub)
+        rows, s, step = rows[good], s[good], step[good]
+        moves[rows, 0] = OP_TP_STEP << 16
+        moves[rows, 1] = starts[s] | (ends[s] << 16)
+        moves[rows, 2] = (step > 0).astype(np.uint32)
 
-    # kind 2, micro-batch size one step up or down, if every op stays on the profiled grid
+    # kind 2, micro-batch size one step up or down, if every op stays on the profiled grid: a header-only template
     rows = np.flatnonzero(kinds == 2)
     if len(rows):
         up = rng.random(len(rows)) < 0.5
@@ -114,29 +118,34 @@ def make_neighbours(base: PlanBatch, tables: CompiledTables, n: int, rng: np.ran
                 continue
             bits = np.array([ok_bits(b2, int(g)) for g in glogs], dtype=np.int64)[stage_of_pos]
             if (((bits >> tp0) & 1) == 1).all():
-                hdr[rows[sel], 0] = S | (b2 << 8)
+                h = hdr0.copy()
+                h[0] = S | (b2 << 8)
+                t_codes.append(row0.copy())
+                t_hdr.append(h)
+                moves[rows[sel], 0] = len(t_codes) - 1
 
     # kind 3, recompute: toggle a short run of ops
     rows = np.flatnonzero(kinds == 3)
     if len(rows):
         lo = rng.integers(0, N, size=len(rows))
         hi = np.minimum(N, lo + rng.integers(1, 14, size=len(rows)))
-        run = (pos[None, :] >= lo[:, None]) & (pos[None, :] < hi[:, None])
-        codes[rows] ^= (run * np.uint8(8)).astype(np.uint8)
+        moves[rows, 0] = OP_RC_TOGGLE << 16
+        moves[rows, 1] = lo | (hi << 16)
 
     # kind 4, partition algorithm of one tunable op
     rows = np.flatnonzero(kinds == 4)
     if A == 2 and len(rows):
         cand = np.flatnonzero(tunable)
-        codes[rows, cand[rng.integers(0, len(cand), size=len(rows))]] ^= 1
+        moves[rows, 0] = OP_ALGO_TOGGLE << 16
+        moves[rows, 1] = cand[rng.integers(0, len(cand), size=len(rows))]
 
     # kind 5, move half of stage a's devices to a stage b that has exactly that many (sizes stay powers
-    # of two and the total is unchanged); few distinct (a, b) pairs, each built once
+    # of two and the total is unchanged); few distinct (a, b) pairs, each a template of its own
     rows = np.flatnonzero(kinds == 5)
     if S > 1 and len(rows):
         a = rng.integers(0, S, size=len(rows))
         b = (a + rng.integers(1, S, size=len(rows))) % S
-        for pa, pb in {(int(x), int(y)) for x, y in zip(a, b)}:
+        for pa, pb in sorted({(int(x), int(y)) for x, y in zip(a, b)}):
             if glogs[pa] - 1 != glogs[pb]:
                 continue
             g2 = glogs.copy()
@@ -154,15 +163,63 @@ def make_neighbours(base: PlanBatch, tables: CompiledTables, n: int, rng: np.ran
                 if not np.all(np.isin(t, ok)):
                     good = False
                     break
-                row[lo:hi] = with_tp(row[lo:hi], t)
+                row[lo:hi] = (row[lo:hi] & 0xF8) | (t * A + (row[lo:hi] & (A - 1))).astype(np.uint8)
             if not good:
                 continue
-            sel = rows[(a == pa) & (b == pb)]
-            codes[sel] = row
             h = hdr0.copy()
             _set_header(h, S, bidx, g2, gpn)
-            hdr[sel] = h
+            t_codes.append(row)
+            t_hdr.append(h)
+            moves[rows[(a == pa) & (b == pb)], 0] = len(t_codes) - 1
+    return PlanBatch(np.stack(t_codes), np.stack(t_hdr)), moves
+
+
+def apply_moves_host(templates: PlanBatch, moves: np.ndarray, n_algo: int) -> PlanBatch:
+    """Expand move descriptors into plans with numpy (masks over a [neighbours, ops] byte matrix)."""
+    A = np.uint8(n_algo)
+    tmpl = (moves[:, 0] & 0xffff).astype(np.int64)
+    op = (moves[:, 0] >> 16).astype(np.int64)
+    codes = templates.codes[tmpl]
+    hdr = templates.hdr[tmpl]
+    N = codes.shape[1]
+    pos = np.arange(N)
+    lo16, hi16 = (moves[:, 1] & 0xffff).astype(np.int64), (moves[:, 1] >> 16).astype(np.int64)
+
+    def with_tp(seg, t):
+        """The code bytes `seg` with their tp replaced by t (algo, recompute and stage bits kept)."""
+        return (seg & np.uint8(0xF8)) | (np.asarray(t).astype(np.uint8) * A + (seg & np.uint8(A - 1)))
+
+    rows = np.flatnonzero(op == OP_MIGRATE)
+    if len(rows):
+        cut, new_cut = lo16[rows], hi16[rows]
+        moved = (pos[None, :] >= np.minimum(cut, new_cut)[:, None]) & (pos[None, :] < np.maximum(cut, new_cut)[:, None])
+        sub = codes[rows]
+        sub[np.arange(len(rows)), cut] &= 0xEF
+        sub = np.where(moved, with_tp(sub, moves[rows, 2][:, None]), sub)
+        sub[np.arange(len(rows)), new_cut] |= 16
+        codes[rows] = sub
+    rows = np.flatnonzero(op == OP_TP_STEP)
+    if len(rows):
+        inside = (pos[None, :] >= lo16[rows][:, None]) & (pos[None, :] < hi16[rows][:, None])
+        sub = codes[rows]
+        t = ((sub & 7) // A).astype(np.int64) + np.where(moves[rows, 2] == 1, 1, -1)[:, None]
+        codes[rows] = np.where(inside, with_tp(sub, t.clip(0, 7)), sub)
+    rows = np.flatnonzero(op == OP_RC_TOGGLE)
+    if len(rows):
+        run = (pos[None, :] >= lo16[rows][:, None]) & (pos[None, :] < hi16[rows][:, None])
+        codes[rows] ^= (run * np.uint8(8)).astype(np.uint8)
+    rows = np.flatnonzero(op == OP_ALGO_TOGGLE)
+    if len(rows):
+        codes[rows, moves[rows, 1].astype(np.int64)] ^= 1
     return PlanBatch(codes, hdr)
+
+
+def make_neighbours(base: PlanBatch, tables: CompiledTables, n: int, rng: np.random.Generator,
+                    max_move: int = 8) -> PlanBatch:
+    """n single-move neighbours of base plan 0 (moves that would leave the profiled grid are replaced
+    by a copy of the base plan, so the batch always has n valid rows)."""
+    templates, moves = sample_moves(base, tables, n, rng, max_move)
+    return apply_moves_host(templates, moves, tables.db.n_algo)
 
 
 class VisitedPlans:
@@ -205,13 +262,19 @@ class VisitedPlans:
 
 
 def hill_climb(cm, start: PlanBatch, steps: int, n_neighbours: int, seed: int = 0, max_move: int = 8,
-               on_step=None, visited: VisitedPlans = None, greedy_recompute: bool = False) -> Tuple[PlanBatch, float, float]:
+               on_step=None, visited: VisitedPlans = None, greedy_recompute: bool = False,
+               device_moves: bool = False) -> Tuple[PlanBatch, float, float]:
     """Best-neighbour descent: at every step n_neighbours single-move neighbours of the current plan
     are scored in one launch and the fastest feasible one replaces it if it is faster.  With a
     `visited` set, neighbours seen in an earlier step (or twice in one step) are dropped before
     scoring, as aceso_search.py:47 does.  With `greedy_recompute` every neighbour's recompute bits are
     replaced by check_recompute's choice before it is scored, as the reference's primitives do
-    (aceso_prims.py:107-108).  Returns (plan, iteration ms, peak MB)."""
+    (aceso_prims.py:107-108).  With `device_moves` the neighbours never exist on the host: the move
+    descriptors (16 bytes each, duplicates within the step dropped) are expanded by the library on the
+    device and only the winner is rebuilt here; `visited` and `greedy_recompute`, which work on plan
+    bytes, do not apply then.  Returns (plan, iteration ms, peak MB)."""
+    if device_moves and (visited is not None or greedy_recompute):
+        raise ValueError("device_moves works on move descriptors: no visited set, no greedy recompute")
     rng = np.random.default_rng(seed)
     tables = cm.tables
     ev = cm.evaluator
@@ -222,6 +285,19 @@ def hill_climb(cm, start: PlanBatch, steps: int, n_neighbours: int, seed: int = 
     if visited is not None:
         visited.mark(cur)
     for step in range(steps):
+        if device_moves:
+            templates, moves = sample_moves(cur, tables, n_neighbours, rng, max_move)
+            moves = np.unique(moves, axis=0)
+            d = ev.apply_moves(templates, moves)
+            it, pk, fe, st = ev.score(d)
+            idx, val, cnt = ev.topk(it, fe, 1)
+            if int(cnt.item()) == 1 and float(val[0].item()) < cur_t:
+                best_i = int(idx[0].item())
+                cur = apply_moves_host(templates, moves[best_i:best_i + 1], tables.db.n_algo)
+                cur_t, cur_m = float(val[0].item()), float(pk[best_i].item())
+            if on_step is not None:
+                on_step(step, cur_t, cur_m)
+            continue
         nb = make_neighbours(cur, tables, n_neighbours, rng, max_move)
         if visited is not None:
             keep = np.flatnonzero(visited.unseen(nb))

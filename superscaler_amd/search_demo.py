@@ -26,6 +26,8 @@ def main(argv=None):
     ap.add_argument("--neighbours", type=int, default=16384)
     ap.add_argument("--topk", type=int, default=64)
     ap.add_argument("--greedy-recompute", action="store_true")
+    ap.add_argument("--device-moves", action="store_true",
+                    help="expand the move descriptors on the device (no visited set, no greedy recompute)")
     ap.add_argument("--workers", type=int, default=16)
     ap.add_argument("--distinct-batches", type=int, default=0,
                     help="generate only this many different batches and cycle through them (0 = all different); "
@@ -75,17 +77,18 @@ def main(argv=None):
             start = src.slice(r, r + 1)
         else:
             start = synth.make_plans(w, cm.tables, n_plans=1, seed_offset=1)
-        visited = VisitedPlans()
+        visited = None if args.device_moves else VisitedPlans()
         trace = []
         t0 = time.perf_counter()
         plan, t, m = hill_climb(cm, start, steps=args.steps, n_neighbours=args.neighbours, seed=7,
                                 on_step=lambda s, t_, m_: trace.append(t_), visited=visited,
-                                greedy_recompute=args.greedy_recompute)
+                                greedy_recompute=args.greedy_recompute, device_moves=args.device_moves)
         search_s = time.perf_counter() - t0
         out.update({"search_steps": args.steps, "neighbours_per_step": args.neighbours,
                     "search_wall_s": round(search_s, 3), "search_steps_per_s": args.steps / search_s,
                     "neighbours_generated_per_s": args.steps * args.neighbours / search_s,
-                    "distinct_plans_scored": len(visited), "greedy_recompute": bool(args.greedy_recompute),
+                    "distinct_plans_scored": len(visited) if visited is not None else None,
+                    "greedy_recompute": bool(args.greedy_recompute), "device_moves": bool(args.device_moves),
                     "search_start_ms": float(val[0]) if len(val) else None, "search_best_ms": t, "search_best_mb": m,
                     "improving_steps": int(np.sum(np.diff([trace[0]] + trace) < 0)) if trace else 0})
     cm.close()

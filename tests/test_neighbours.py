@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 from superscaler_amd import synth
-from superscaler_amd.neighbours import VisitedPlans, hill_climb, make_neighbours
+from superscaler_amd.neighbours import VisitedPlans, apply_moves_host, hill_climb, make_neighbours, sample_moves
 from superscaler_amd.plan import PlanBatch, config_details, is_visited, mark_visited, num_visited, validate_batch
 from tests.helpers import emu_score, oracle_for, oracle_scores
 
@@ -86,6 +86,10 @@ def test_hill_climb_improves_and_agrees_with_the_oracle():
     assert np.array_equal(cm.update_recompute_arrays(plan2).codes, plan2.codes) or t2 == (t0 if f0 else float("inf"))
     (t3,), (m3,), (f3,), _ = oracle_scores(orc, plan2, cm.tables)
     assert (f3 == 1 and t3 == t2 and m3 == m2) or t2 == float("inf")
+    # neighbours expanded on the device from move descriptors: the plan handed back scores as reported
+    plan4, t4, m4 = hill_climb(cm, start, steps=10, n_neighbours=2048, seed=3, device_moves=True)
+    (t5,), (m5,), (f5,), _ = oracle_scores(orc, plan4, cm.tables)
+    assert (f5 == 1 and t5 == t4 and m5 == m4 and t4 < t0) or not f0
     cm.close()
 
 
@@ -99,3 +103,31 @@ def test_stream_and_search_demo_runs(capsys):
     out = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
     assert out["streamed_plans"] == 10000 and out["batches"] == 3
     assert out["search_best_ms"] <= out["search_start_ms"]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["gpt3_1_3b", "gpt3_13b", "t5_770m", "wresnet_1b"])
+def test_moves_expand_on_the_device_like_on_the_host(name):
+    """ace_apply_moves writes byte for byte what apply_moves_host builds, in the kernel's layout,
+    and the batch scores the same either way."""
+    import torch
+    from superscaler_amd.evaluator import PlanEvaluator
+    w = synth.WORKLOADS[name]
+    tables = synth.make_tables(w)
+    ev = PlanEvaluator(tables)
+    rng = np.random.default_rng(11)
+    for p in range(3):
+        base = synth.make_plans(w, tables, n_plans=4, seed_offset=40 + p).slice(p, p + 1)
+        templates, moves = sample_moves(base, tables, 5000, rng)
+        host = apply_moves_host(templates, moves, tables.db.n_algo)
+        assert len(np.unique(moves[:, 0] >> 16)) >= 2
+        d = ev.apply_moves(templates, moves)
+        N, G = host.num_ops, (host.num_ops + 15) // 16
+        got = d.codes.permute(1, 0, 2).reshape(host.n_plans, G * 16).cpu().numpy()
+        assert np.array_equal(got[:, :N], host.codes) and not got[:, N:].any()
+        assert np.array_equal(d.hdr.cpu().numpy().view(np.uint32), host.hdr)
+        a = [t.cpu().numpy() for t in ev.score(d)]
+        b = ev.score_host(host)
+        for x, y in zip(a, b):
+            assert np.array_equal(x, y, equal_nan=True)
+    ev.close()

@@ -413,12 +413,24 @@ struct ace_handle {
     size_t stage_ws_plans;     // capacity in plans
 };
 
+// One 64-bit value per (16-byte word, word index): two rounds of the splitmix64 finaliser.
+__device__ __forceinline__ unsigned long long plan_key_word(uint32_t a, uint32_t b, uint32_t c, uint32_t d, uint32_t idx) {
+    unsigned long long x = ((unsigned long long)b << 32 | a) + 0x9E3779B97F4A7C15ull * (2ull * idx + 1ull);
+    unsigned long long y = ((unsigned long long)d << 32 | c) ^ (x >> 29);
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    x ^= x >> 31;
+    y = (y + x) * 0xBF58476D1CE4E5B9ull;
+    y = (y ^ (y >> 27)) * 0x94D049BB133111EBull;
+    return x ^ y ^ (y >> 31);
+}
+
 // ------------------------------------------------------------------------------------------
 // Move descriptors -> plans: one thread writes one 16-byte word (16 ops) of one neighbour.
 // ------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void apply_moves_kernel(const ace_u4 *tmpl_codes, const ace_u4 *tmpl_hdr, int n_templates,
                                                           const ace_u4 *moves, unsigned long long n, int G, int a_shift,
-                                                          ace_u4 *codes_out, ace_u4 *hdr_out) {
+                                                          ace_u4 *codes_out, ace_u4 *hdr_out, unsigned long long *key_out) {
     const unsigned long long id = (unsigned long long)blockIdx.x * 256 + threadIdx.x;
     if (id >= n * (unsigned long long)G) return;
     const unsigned long long k = id % n;              // consecutive lanes: consecutive neighbours of one word
@@ -462,6 +474,15 @@ __global__ __launch_bounds__(256) void apply_moves_kernel(const ace_u4 *tmpl_cod
         }
     }
     codes_out[(size_t)g * n + k] = ace_u4{w[0], w[1], w[2], w[3]};
+    if (key_out) {
+        // 64-bit key of the whole plan: XOR of one mixed value per 16-byte word (and one for the header)
+        unsigned long long hsh = plan_key_word(w[0], w[1], w[2], w[3], (uint32_t)g + 1u);
+        if (g == 0) {
+            const ace_u4 hh = tmpl_hdr[t];
+            hsh ^= plan_key_word(hh.x, hh.y, hh.z, 0u, 0u);      // (the fourth header word follows from the others)
+        }
+        atomicXor(&key_out[k], hsh);
+    }
 }
 
 extern "C" {
@@ -747,13 +768,13 @@ int ace_topk(ace_handle_t *h, const double *d_iter_ms, const uint8_t *d_feasible
 
 int ace_apply_moves(const uint8_t *d_template_codes, const uint32_t *d_template_hdr, int n_templates,
                     const uint32_t *d_moves, size_t n_moves, int num_ops, int n_algo, uint8_t *d_codes_out,
-                    uint32_t *d_hdr_out, void *stream) {
+                    uint32_t *d_hdr_out, uint64_t *d_keys_out, void *stream) {
     if (!d_template_codes || !d_template_hdr || !d_moves || !d_codes_out || !d_hdr_out || n_templates <= 0 ||
         n_templates > 65536 || n_moves == 0 || n_moves > 0x7fffffffull || num_ops <= 0 || num_ops >= 65536 ||
         (n_algo != 1 && n_algo != 2))
         return ACE_EINVAL;
     if (((uintptr_t)d_template_codes & 15u) || ((uintptr_t)d_template_hdr & 15u) || ((uintptr_t)d_moves & 15u) ||
-        ((uintptr_t)d_codes_out & 15u) || ((uintptr_t)d_hdr_out & 15u))
+        ((uintptr_t)d_codes_out & 15u) || ((uintptr_t)d_hdr_out & 15u) || ((uintptr_t)d_keys_out & 7u))
         return ACE_EINVAL;
     const int G = (num_ops + 15) / 16;
     const unsigned long long total = (unsigned long long)n_moves * (unsigned long long)G;
@@ -762,7 +783,8 @@ int ace_apply_moves(const uint8_t *d_template_codes, const uint32_t *d_template_
     hipLaunchKernelGGL(apply_moves_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
                        reinterpret_cast<const ace_u4 *>(d_template_codes), reinterpret_cast<const ace_u4 *>(d_template_hdr),
                        n_templates, reinterpret_cast<const ace_u4 *>(d_moves), (unsigned long long)n_moves, G,
-                       n_algo == 2 ? 1 : 0, reinterpret_cast<ace_u4 *>(d_codes_out), reinterpret_cast<ace_u4 *>(d_hdr_out));
+                       n_algo == 2 ? 1 : 0, reinterpret_cast<ace_u4 *>(d_codes_out), reinterpret_cast<ace_u4 *>(d_hdr_out),
+                       reinterpret_cast<unsigned long long *>(d_keys_out));
     ACE_HIP(hipGetLastError());
     return ACE_OK;
 }

@@ -61,7 +61,7 @@ def load_library():
                                           ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(ctypes.c_double)]
     lib.ace_apply_moves.restype = ctypes.c_int
     lib.ace_apply_moves.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t,
-                                    ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+                                    ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
     if lib.ace_abi_version() != ABI_VERSION:
         raise AceError("libace_eval.so has a different ABI version")
     _lib = lib
@@ -262,9 +262,11 @@ class PlanEvaluator:
             del d
         return best_idx, best_val, offset
 
-    def apply_moves(self, templates: PlanBatch, moves: np.ndarray) -> DeviceBatch:
+    def apply_moves(self, templates: PlanBatch, moves: np.ndarray, with_keys: bool = False):
         """Expand move descriptors (neighbours.sample_moves) into a device-resident batch: only the
-        templates and 16 bytes per neighbour cross the bus."""
+        templates and 16 bytes per neighbour cross the bus.  With `with_keys` also returns a device
+        tensor int64[n] holding a 64-bit key of every plan's bytes (neighbours.plan_keys_host computes
+        the same keys from a PlanBatch)."""
         torch = self._torch
         T, N = templates.codes.shape
         G = (N + 15) // 16
@@ -276,11 +278,19 @@ class PlanEvaluator:
         d_mv = torch.from_numpy(np.ascontiguousarray(moves, dtype=np.uint32).view(np.int32)).to(self.device)
         codes = torch.empty((G, n, 16), dtype=torch.uint8, device=self.device)
         hdr = torch.empty((n, 4), dtype=torch.int32, device=self.device)
+        keys = torch.zeros(n, dtype=torch.int64, device=self.device) if with_keys else None
         with torch.cuda.device(self.device):
             rc = self.lib.ace_apply_moves(d_tc.data_ptr(), d_th.data_ptr(), T, d_mv.data_ptr(), n, N,
-                                          self.tables.db.n_algo, codes.data_ptr(), hdr.data_ptr(), self._stream())
+                                          self.tables.db.n_algo, codes.data_ptr(), hdr.data_ptr(),
+                                          keys.data_ptr() if with_keys else None, self._stream())
         _check(self.lib, rc, "ace_apply_moves")
-        return DeviceBatch.from_device(codes, hdr, N)
+        d = DeviceBatch.from_device(codes, hdr, N)
+        return (d, keys) if with_keys else d
+
+    def select(self, d: DeviceBatch, index) -> DeviceBatch:
+        """The plans `index` (device int64 tensor) of a device-resident batch, as a new batch."""
+        return DeviceBatch.from_device(d.codes.index_select(1, index).contiguous(), d.hdr.index_select(0, index).contiguous(),
+                                       d.num_ops)
 
     def stage_records_host(self, batch: PlanBatch, ranges: np.ndarray):
         """Single-stage queries: (status, stage record 0 of every query) as numpy arrays."""

@@ -261,6 +261,75 @@ class VisitedPlans:
             self._seen.add(keys[int(p)].tobytes())
 
 
+_K0, _K1, _K2 = np.uint64(0x9E3779B97F4A7C15), np.uint64(0xBF58476D1CE4E5B9), np.uint64(0x94D049BB133111EB)
+
+
+def _key_word(a, b, c, d, idx):
+    """The library's per-word mixing (two rounds of the splitmix64 finaliser), on uint64 arrays."""
+    u = np.uint64
+    x = ((b << u(32)) | a) + _K0 * (u(2) * idx + u(1))
+    y = ((d << u(32)) | c) ^ (x >> u(29))
+    x = (x ^ (x >> u(30))) * _K1
+    x = (x ^ (x >> u(27))) * _K2
+    x = x ^ (x >> u(31))
+    y = (y + x) * _K1
+    y = (y ^ (y >> u(27))) * _K2
+    return x ^ y ^ (y >> u(31))
+
+
+def plan_keys_host(batch: PlanBatch) -> np.ndarray:
+    """The 64-bit plan keys ace_apply_moves writes, computed on the host (uint64[n_plans])."""
+    P, N = batch.codes.shape
+    G = (N + 15) // 16
+    padded = np.zeros((P, G * 16), dtype=np.uint8)
+    padded[:, :N] = batch.codes
+    w = padded.view(np.uint32).reshape(P, G, 4).astype(np.uint64)
+    idx = (np.arange(G, dtype=np.uint64) + np.uint64(1))[None, :]
+    with np.errstate(over="ignore"):
+        keys = np.bitwise_xor.reduce(_key_word(w[:, :, 0], w[:, :, 1], w[:, :, 2], w[:, :, 3], idx), axis=1)
+        h = batch.hdr.astype(np.uint64)
+        keys ^= _key_word(h[:, 0], h[:, 1], h[:, 2], np.zeros(P, dtype=np.uint64), np.uint64(0))
+    return keys
+
+
+class VisitedKeys:
+    """A visited set over 64-bit plan keys (for neighbours that only exist on the device): one sorted
+    array plus the keys marked since it was last merged."""
+
+    def __init__(self):
+        self._sorted = np.empty(0, dtype=np.uint64)
+        self._recent = []
+        self._n_recent = 0
+
+    def __len__(self):
+        self._merge()
+        return len(self._sorted)
+
+    def _merge(self):
+        if self._recent:
+            self._sorted = np.union1d(self._sorted, np.concatenate(self._recent))
+            self._recent, self._n_recent = [], 0
+
+    def unseen(self, keys: np.ndarray) -> np.ndarray:
+        """Mask of the keys not marked before that do not repeat an earlier entry of `keys`."""
+        if self._n_recent > 65536:
+            self._merge()
+        _, first = np.unique(keys, return_index=True)
+        mask = np.zeros(len(keys), dtype=bool)
+        mask[first] = True
+        if len(self._sorted):
+            pos = np.searchsorted(self._sorted, keys)
+            mask &= self._sorted[np.minimum(pos, len(self._sorted) - 1)] != keys
+        for r in self._recent:
+            mask &= ~np.isin(keys, r)
+        return mask
+
+    def mark(self, keys: np.ndarray) -> None:
+        k = np.unique(np.asarray(keys, dtype=np.uint64))
+        self._recent.append(k)
+        self._n_recent += len(k)
+
+
 def hill_climb(cm, start: PlanBatch, steps: int, n_neighbours: int, seed: int = 0, max_move: int = 8,
                on_step=None, visited: VisitedPlans = None, greedy_recompute: bool = False,
                device_moves: bool = False) -> Tuple[PlanBatch, float, float]:
@@ -270,11 +339,12 @@ def hill_climb(cm, start: PlanBatch, steps: int, n_neighbours: int, seed: int = 
     scoring, as aceso_search.py:47 does.  With `greedy_recompute` every neighbour's recompute bits are
     replaced by check_recompute's choice before it is scored, as the reference's primitives do
     (aceso_prims.py:107-108).  With `device_moves` the neighbours never exist on the host: the move
-    descriptors (16 bytes each, duplicates within the step dropped) are expanded by the library on the
-    device and only the winner is rebuilt here; `visited` and `greedy_recompute`, which work on plan
-    bytes, do not apply then.  Returns (plan, iteration ms, peak MB)."""
-    if device_moves and (visited is not None or greedy_recompute):
-        raise ValueError("device_moves works on move descriptors: no visited set, no greedy recompute")
+    descriptors (16 bytes each) are expanded by the library on the device and only the winner is
+    rebuilt here; `visited` is then a VisitedKeys (64-bit keys of the plan bytes, computed by the
+    same kernel) and `greedy_recompute`, which works on plan bytes on the host, does not apply.
+    Returns (plan, iteration ms, peak MB)."""
+    if device_moves and (greedy_recompute or isinstance(visited, VisitedPlans)):
+        raise ValueError("device_moves: use a VisitedKeys set; greedy recompute needs the plans on the host")
     rng = np.random.default_rng(seed)
     tables = cm.tables
     ev = cm.evaluator
@@ -283,12 +353,24 @@ def hill_climb(cm, start: PlanBatch, steps: int, n_neighbours: int, seed: int = 
     cur_t = float(it[0]) if fe[0] else float("inf")
     cur_m = float(pk[0])
     if visited is not None:
-        visited.mark(cur)
+        visited.mark(plan_keys_host(cur) if device_moves else cur)
     for step in range(steps):
         if device_moves:
             templates, moves = sample_moves(cur, tables, n_neighbours, rng, max_move)
             moves = np.unique(moves, axis=0)
-            d = ev.apply_moves(templates, moves)
+            if visited is None:
+                d = ev.apply_moves(templates, moves)
+            else:
+                d, keys = ev.apply_moves(templates, moves, with_keys=True)
+                keys = keys.cpu().numpy().view(np.uint64)
+                keep = np.flatnonzero(visited.unseen(keys))
+                if len(keep) == 0:
+                    if on_step is not None:
+                        on_step(step, cur_t, cur_m)
+                    continue
+                visited.mark(keys[keep])
+                moves = moves[keep]
+                d = ev.select(d, ev._torch.from_numpy(keep).to(d.hdr.device))
             it, pk, fe, st = ev.score(d)
             idx, val, cnt = ev.topk(it, fe, 1)
             if int(cnt.item()) == 1 and float(val[0].item()) < cur_t:

@@ -27,7 +27,7 @@ def main(argv=None):
     ap.add_argument("--topk", type=int, default=64)
     ap.add_argument("--greedy-recompute", action="store_true")
     ap.add_argument("--device-moves", action="store_true",
-                    help="expand the move descriptors on the device (no visited set, no greedy recompute)")
+                    help="expand the move descriptors on the device (visited set over 64-bit plan keys; no greedy recompute)")
     ap.add_argument("--workers", type=int, default=16)
     ap.add_argument("--distinct-batches", type=int, default=0,
                     help="generate only this many different batches and cycle through them (0 = all different); "
@@ -36,7 +36,7 @@ def main(argv=None):
 
     from . import synth
     from .aceso_cost_model import CostModel
-    from .neighbours import VisitedPlans, hill_climb
+    from .neighbours import VisitedKeys, VisitedPlans, hill_climb
 
     w = synth.WORKLOADS[args.workload]
     graph = synth.make_graph(w)
@@ -77,7 +77,7 @@ def main(argv=None):
             start = src.slice(r, r + 1)
         else:
             start = synth.make_plans(w, cm.tables, n_plans=1, seed_offset=1)
-        visited = None if args.device_moves else VisitedPlans()
+        visited = VisitedKeys() if args.device_moves else VisitedPlans()
         trace = []
         t0 = time.perf_counter()
         plan, t, m = hill_climb(cm, start, steps=args.steps, n_neighbours=args.neighbours, seed=7,

@@ -4,7 +4,8 @@ import numpy as np
 import pytest
 
 from superscaler_amd import synth
-from superscaler_amd.neighbours import VisitedPlans, apply_moves_host, hill_climb, make_neighbours, sample_moves
+from superscaler_amd.neighbours import (VisitedKeys, VisitedPlans, apply_moves_host, hill_climb, make_neighbours,
+                                        plan_keys_host, sample_moves)
 from superscaler_amd.plan import PlanBatch, config_details, is_visited, mark_visited, num_visited, validate_batch
 from tests.helpers import emu_score, oracle_for, oracle_scores
 
@@ -87,7 +88,9 @@ def test_hill_climb_improves_and_agrees_with_the_oracle():
     (t3,), (m3,), (f3,), _ = oracle_scores(orc, plan2, cm.tables)
     assert (f3 == 1 and t3 == t2 and m3 == m2) or t2 == float("inf")
     # neighbours expanded on the device from move descriptors: the plan handed back scores as reported
-    plan4, t4, m4 = hill_climb(cm, start, steps=10, n_neighbours=2048, seed=3, device_moves=True)
+    vkeys = VisitedKeys()
+    plan4, t4, m4 = hill_climb(cm, start, steps=10, n_neighbours=2048, seed=3, device_moves=True, visited=vkeys)
+    assert len(vkeys) > 100
     (t5,), (m5,), (f5,), _ = oracle_scores(orc, plan4, cm.tables)
     assert (f5 == 1 and t5 == t4 and m5 == m4 and t4 < t0) or not f0
     cm.close()
@@ -126,6 +129,16 @@ def test_moves_expand_on_the_device_like_on_the_host(name):
         got = d.codes.permute(1, 0, 2).reshape(host.n_plans, G * 16).cpu().numpy()
         assert np.array_equal(got[:, :N], host.codes) and not got[:, N:].any()
         assert np.array_equal(d.hdr.cpu().numpy().view(np.uint32), host.hdr)
+        # the plan keys of the kernel = the host's, and they separate exactly the distinct plans of the batch
+        d2, keys = ev.apply_moves(templates, moves, with_keys=True)
+        keys = keys.cpu().numpy().view(np.uint64)
+        assert np.array_equal(keys, plan_keys_host(host))
+        assert len(np.unique(keys)) == int(VisitedPlans().unseen(host).sum())
+        vk = VisitedKeys()
+        first = vk.unseen(keys)
+        assert np.array_equal(first, VisitedPlans().unseen(host))
+        vk.mark(keys[first][:7])
+        assert vk.unseen(keys).sum() == first.sum() - 7
         a = [t.cpu().numpy() for t in ev.score(d)]
         b = ev.score_host(host)
         for x, y in zip(a, b):

@@ -64,6 +64,28 @@ def test_visited_set_matches_the_reference_string_key():
     assert config_details(None) == ""
 
 
+def test_plan_keys_separate_distinct_plans_and_key_set_behaves():
+    w = synth.WORKLOADS["gpt3_13b"]
+    tables = synth.make_tables(w)
+    base = synth.make_plans(w, tables, n_plans=3, seed_offset=8)
+    nb = PlanBatch.concat([make_neighbours(base.slice(p, p + 1), tables, 4000, np.random.default_rng(p)) for p in range(3)])
+    keys = plan_keys_host(nb)
+    first = VisitedPlans().unseen(nb)
+    assert len(np.unique(keys)) == int(first.sum())            # no collision, no split
+    vk = VisitedKeys()
+    assert np.array_equal(vk.unseen(keys), first)
+    vk.mark(keys[:5000])
+    seen = set(keys[:5000].tolist())
+    want = first & ~np.array([k in seen for k in keys.tolist()])
+    assert np.array_equal(vk.unseen(keys), want)
+    vk._merge()
+    assert np.array_equal(vk.unseen(keys), want) and len(vk) == len(seen)
+    # a header-only change (another micro-batch size) changes the key
+    h = nb.hdr.copy()
+    h[:, 0] ^= 1 << 8
+    assert not np.any(plan_keys_host(PlanBatch(nb.codes, h)) == keys)
+
+
 @pytest.mark.gpu
 def test_hill_climb_improves_and_agrees_with_the_oracle():
     from superscaler_amd.aceso_cost_model import CostModel

@@ -357,8 +357,10 @@ def hill_climb(cm, start: PlanBatch, steps: int, n_neighbours: int, seed: int = 
     for step in range(steps):
         if device_moves:
             templates, moves = sample_moves(cur, tables, n_neighbours, rng, max_move)
-            moves = np.unique(moves, axis=0)
             if visited is None:
+                # equal descriptors are equal plans: keep one of each (template < 2^16, op < 2^8, p1 < 2^8)
+                packed = (moves[:, 0] | (moves[:, 2] << 24)).astype(np.uint64) | (moves[:, 1].astype(np.uint64) << np.uint64(32))
+                moves = moves[np.unique(packed, return_index=True)[1]]
                 d = ev.apply_moves(templates, moves)
             else:
                 d, keys = ev.apply_moves(templates, moves, with_keys=True)

@@ -175,6 +175,38 @@ int ace_apply_moves(const uint8_t *d_template_codes, const uint32_t *d_template_
                     const uint32_t *d_moves, size_t n_moves, int num_ops, int n_algo, uint8_t *d_codes_out,
                     uint32_t *d_hdr_out, uint64_t *d_keys_out, void *stream);
 
+/* The two steps of check_recompute's greedy loop (aceso_cost_model.py:822-872) that are not a stage
+ * evaluation, for many encoded stages at once (one stage = the ops [lo, hi) of one plan of the batch).
+ * The caller runs the loop: evaluate the stages (ace_score_batch with d_range), update their memory
+ * (:861-867), call ace_recompute_select for those still above the limit, repeat. */
+typedef struct ace_rc_tables {
+    const uint8_t *d_codes;          /* the batch, uint8[ceil(num_ops / 16)][n_plans][16] */
+    size_t n_plans;
+    const int32_t *d_type_of_pos;    /* int32[num_ops]: op type (table row) of every position */
+    const double *d_activations;     /* double[num_types][n_mbs][n_tp][n_algo]: the raw "activations" column
+                                        (get_activation_size, aceso_cost_model.py:487-491) */
+    const uint8_t *d_no_recompute;   /* uint8[num_types]: op names get_next_recompute_op_group never picks (:798) */
+    int32_t num_ops, num_types, n_mbs, n_tp, n_algo;
+} ace_rc_tables_t;
+
+/* Op groups of every stage (:835-843).  d_plan / d_lo / d_hi / d_nsb: int32[n_stages] (plan index, first op,
+ * one past the last op, num_stages_behind); d_mrow: uint32[n_stages], the micro-batch index of the stage per
+ * tp (4 bits each, as in ace_tables_t.stage_lut).  d_sum_size: double[n_stages][num_types] ZEROED by the
+ * caller; d_first_pos: int32[n_stages][num_types] FILLED WITH num_ops by the caller; d_bad: int32[n_stages]
+ * zeroed by the caller, set where an op sits outside the profiled grid (the reference raises KeyError). */
+int ace_recompute_groups(const ace_rc_tables_t *t, int n_stages, const int32_t *d_plan, const int32_t *d_lo,
+                         const int32_t *d_hi, const int32_t *d_nsb, const uint32_t *d_mrow, double *d_sum_size,
+                         int32_t *d_first_pos, int32_t *d_bad, void *stream);
+
+/* One greedy round for every stage with d_alive[k] != 0: get_next_recompute_op_group (:794-820) on the
+ * groups above and d_mem[k] - memory_limit, then the recompute bit of the chosen ops and of the op after each
+ * (:852-859) is set in d_codes_rw (normally the same buffer as t->d_codes).  d_recomputed:
+ * uint8[n_stages][num_types], zeroed before the first round; d_alive[k] is cleared where the loop ends. */
+int ace_recompute_select(const ace_rc_tables_t *t, uint8_t *d_codes_rw, int n_stages, const int32_t *d_plan,
+                         const int32_t *d_lo, const int32_t *d_hi, const int32_t *d_nsb, const uint32_t *d_mrow,
+                         const double *d_sum_size, const int32_t *d_first_pos, uint8_t *d_recomputed, const double *d_mem,
+                         double memory_limit, uint8_t *d_alive, void *stream);
+
 /* Average duration in milliseconds of the `reps` scoring-kernel launches of one
  * ace_score_batch-equivalent call sequence, measured with hipEvents on `stream`
  * (for bench.py's roofline figure; not part of the reference). */

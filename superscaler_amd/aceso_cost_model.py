@@ -489,6 +489,11 @@ class CostModel:
         from .recompute import update_recompute_arrays
         return update_recompute_arrays(self, batch)
 
+    def update_recompute_device(self, dbatch):
+        """update_recompute_arrays for a batch that lives on the device (evaluator.DeviceBatch in, a new one out)."""
+        from .recompute import update_recompute_device
+        return update_recompute_device(self, dbatch)
+
     def predict_value_after_move(self, config, bottleneck, partner, num_ops_moved, metric, inc_gpus=False,
                                  dec_gpus=False, dim=None):
         """aceso_cost_model.py:693-739."""

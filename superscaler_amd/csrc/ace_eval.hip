@@ -485,6 +485,96 @@ __global__ __launch_bounds__(256) void apply_moves_kernel(const ace_u4 *tmpl_cod
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// check_recompute for encoded stages (aceso_cost_model.py:794-872): the two steps of its greedy
+// loop that are not a stage evaluation.  One thread per stage; every sum runs over the stage's ops
+// in position order, as the reference's lists do.
+// ------------------------------------------------------------------------------------------
+struct RcTables {
+    const uint8_t *codes;          // [G][P][16], the batch being edited
+    unsigned long long P;
+    const int32_t *type_of_pos;    // [N]
+    const double *act;             // activations [n_types][n_mbs][n_tp][n_algo] (raw table entries, :487-491)
+    const uint8_t *norec;          // [n_types] never chosen for recomputation (:798)
+    int32_t N, n_types, n_mbs, n_tp, n_algo, a_shift;
+};
+
+__device__ __forceinline__ double rc_act_size(const RcTables &t, unsigned long long plan, int i, uint32_t mrow, int nsb,
+                                              int *type_out, int *bad) {
+    const uint32_t byte = t.codes[(((size_t)(i >> 4)) * t.P + plan) * 16 + (i & 15)];
+    const uint32_t c = byte & 7u, tp = c >> t.a_shift, al = c & (uint32_t)(t.n_algo - 1);
+    uint32_t m = (mrow >> (4u * tp)) & 15u;
+    if (tp >= (uint32_t)t.n_tp || m >= (uint32_t)t.n_mbs) { *bad = 1; m = 0; }
+    const int type = t.type_of_pos[i];
+    *type_out = type;
+    const uint32_t tpc = tp < (uint32_t)t.n_tp ? tp : 0u;
+    return t.act[(((size_t)type * t.n_mbs + m) * t.n_tp + tpc) * t.n_algo + al] * (double)(nsb + 1);   // :841
+}
+
+// op groups of a stage (:835-843): per op name the sum of the activation sizes and the first position
+__global__ void rc_groups_kernel(RcTables t, int n, const int32_t *q_plan, const int32_t *q_lo, const int32_t *q_hi,
+                                 const int32_t *q_nsb, const uint32_t *q_mrow, double *sum_size, int32_t *first_pos,
+                                 int32_t *bad) {
+    const int a = blockIdx.x * blockDim.x + threadIdx.x;
+    if (a >= n) return;
+    double *sum = sum_size + (size_t)a * t.n_types;
+    int32_t *first = first_pos + (size_t)a * t.n_types;
+    int flag = 0;
+    for (int i = q_lo[a]; i < q_hi[a]; ++i) {
+        int type;
+        const double sz = rc_act_size(t, (unsigned long long)q_plan[a], i, q_mrow[a], q_nsb[a], &type, &flag);
+        sum[type] += sz;
+        if (i < first[type]) first[type] = i;
+    }
+    if (flag) bad[a] = 1;
+}
+
+// one round of the greedy loop for every stage still above the limit: get_next_recompute_op_group
+// (:794-820) and the marking of the chosen ops and their successors (:852-859)
+__global__ void rc_select_kernel(RcTables t, uint8_t *codes_rw, int n, const int32_t *q_plan, const int32_t *q_lo,
+                                 const int32_t *q_hi, const int32_t *q_nsb, const uint32_t *q_mrow, const double *sum_size,
+                                 const int32_t *first_pos, uint8_t *recomputed, const double *mem, double memory_limit,
+                                 uint8_t *alive) {
+    const int a = blockIdx.x * blockDim.x + threadIdx.x;
+    if (a >= n || !alive[a]) return;
+    const double *sum = sum_size + (size_t)a * t.n_types;
+    const int32_t *first = first_pos + (size_t)a * t.n_types;
+    uint8_t *done = recomputed + (size_t)a * t.n_types;
+    // the largest group not yet taken; a tie goes to the op name that appears first in the stage (dict order)
+    double best = 0.0;
+    int T = -1, best_first = 0x7fffffff;
+    for (int ty = 0; ty < t.n_types; ++ty) {
+        const double s = sum[ty];
+        const int f = first[ty];
+        const bool open = !done[ty] && !t.norec[ty] && s > 0.0;
+        const bool better = open && (s > best || (s == best && f < best_first));
+        best = better ? s : best;
+        best_first = better ? f : best_first;
+        T = better ? ty : T;
+    }
+    if (T < 0) { alive[a] = 0; return; }                       // max_saved_size == 0
+    done[T] = 1;
+    const int lo = q_lo[a], hi = q_hi[a];
+    const int nxt = first[T] + 1;
+    if (nxt >= hi) { alive[a] = 0; return; }                    // :805-806
+    done[t.type_of_pos[nxt]] = 1;
+    const double exceed = mem[a] - memory_limit;
+    const bool all = best < exceed;                              // :809
+    const unsigned long long plan = (unsigned long long)q_plan[a];
+    double saved = 0.0;
+    int dummy = 0;
+    for (int i = lo; i < hi; ++i) {
+        if (t.type_of_pos[i] != T) continue;
+        if (!all) {
+            if (!(saved <= exceed)) break;                       // :814
+            int type;
+            saved += rc_act_size(t, plan, i, q_mrow[a], q_nsb[a], &type, &dummy);
+        }
+        codes_rw[(((size_t)(i >> 4)) * t.P + plan) * 16 + (i & 15)] |= 8u;
+        if (i + 1 < hi) codes_rw[(((size_t)((i + 1) >> 4)) * t.P + plan) * 16 + ((i + 1) & 15)] |= 8u;
+    }
+}
+
 extern "C" {
 
 int ace_abi_version(void) { return ACE_ABI_VERSION; }
@@ -785,6 +875,38 @@ int ace_apply_moves(const uint8_t *d_template_codes, const uint32_t *d_template_
                        n_templates, reinterpret_cast<const ace_u4 *>(d_moves), (unsigned long long)n_moves, G,
                        n_algo == 2 ? 1 : 0, reinterpret_cast<ace_u4 *>(d_codes_out), reinterpret_cast<ace_u4 *>(d_hdr_out),
                        reinterpret_cast<unsigned long long *>(d_keys_out));
+    ACE_HIP(hipGetLastError());
+    return ACE_OK;
+}
+
+int ace_recompute_groups(const ace_rc_tables_t *t, int n_stages, const int32_t *d_plan, const int32_t *d_lo,
+                         const int32_t *d_hi, const int32_t *d_nsb, const uint32_t *d_mrow, double *d_sum_size,
+                         int32_t *d_first_pos, int32_t *d_bad, void *stream) {
+    if (!t || n_stages <= 0 || !d_plan || !d_lo || !d_hi || !d_nsb || !d_mrow || !d_sum_size || !d_first_pos || !d_bad ||
+        !t->d_codes || !t->d_type_of_pos || !t->d_activations || !t->d_no_recompute || t->num_ops <= 0 || t->num_types <= 0 ||
+        t->n_tp <= 0 || t->n_tp > 4 || (t->n_algo != 1 && t->n_algo != 2) || t->n_mbs <= 0 || t->n_mbs > 15 || t->n_plans == 0)
+        return ACE_EINVAL;
+    RcTables k{t->d_codes, (unsigned long long)t->n_plans, t->d_type_of_pos, t->d_activations, t->d_no_recompute,
+               t->num_ops, t->num_types, t->n_mbs, t->n_tp, t->n_algo, t->n_algo == 2 ? 1 : 0};
+    hipLaunchKernelGGL(rc_groups_kernel, dim3((n_stages + 127) / 128), dim3(128), 0, (hipStream_t)stream, k, n_stages,
+                       d_plan, d_lo, d_hi, d_nsb, d_mrow, d_sum_size, d_first_pos, d_bad);
+    ACE_HIP(hipGetLastError());
+    return ACE_OK;
+}
+
+int ace_recompute_select(const ace_rc_tables_t *t, uint8_t *d_codes_rw, int n_stages, const int32_t *d_plan,
+                         const int32_t *d_lo, const int32_t *d_hi, const int32_t *d_nsb, const uint32_t *d_mrow,
+                         const double *d_sum_size, const int32_t *d_first_pos, uint8_t *d_recomputed, const double *d_mem,
+                         double memory_limit, uint8_t *d_alive, void *stream) {
+    if (!t || !d_codes_rw || n_stages <= 0 || !d_plan || !d_lo || !d_hi || !d_nsb || !d_mrow || !d_sum_size ||
+        !d_first_pos || !d_recomputed || !d_mem || !d_alive || !t->d_codes || !t->d_type_of_pos || !t->d_activations ||
+        !t->d_no_recompute || t->num_ops <= 0 || t->num_types <= 0 || t->n_plans == 0)
+        return ACE_EINVAL;
+    RcTables k{t->d_codes, (unsigned long long)t->n_plans, t->d_type_of_pos, t->d_activations, t->d_no_recompute,
+               t->num_ops, t->num_types, t->n_mbs, t->n_tp, t->n_algo, t->n_algo == 2 ? 1 : 0};
+    hipLaunchKernelGGL(rc_select_kernel, dim3((n_stages + 127) / 128), dim3(128), 0, (hipStream_t)stream, k, d_codes_rw,
+                       n_stages, d_plan, d_lo, d_hi, d_nsb, d_mrow, d_sum_size, d_first_pos, d_recomputed, d_mem,
+                       memory_limit, d_alive);
     ACE_HIP(hipGetLastError());
     return ACE_OK;
 }

@@ -16,12 +16,19 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libace_eva
 _lib = None
 
 EXPORTS = ["ace_abi_version", "ace_strerror", "ace_last_hip_error", "ace_create", "ace_destroy",
-           "ace_score_batch", "ace_topk_workspace_bytes", "ace_topk", "ace_time_score_kernel", "ace_apply_moves"]
+           "ace_score_batch", "ace_topk_workspace_bytes", "ace_topk", "ace_time_score_kernel", "ace_apply_moves",
+           "ace_recompute_groups", "ace_recompute_select"]
 
 
 class AceBatchStruct(ctypes.Structure):
     _fields_ = [("d_codes", ctypes.c_void_p), ("d_hdr", ctypes.c_void_p), ("d_range", ctypes.c_void_p),
                 ("n_plans", ctypes.c_size_t)]
+
+
+class AceRcTablesStruct(ctypes.Structure):
+    _fields_ = [("d_codes", ctypes.c_void_p), ("n_plans", ctypes.c_size_t), ("d_type_of_pos", ctypes.c_void_p),
+                ("d_activations", ctypes.c_void_p), ("d_no_recompute", ctypes.c_void_p), ("num_ops", ctypes.c_int32),
+                ("num_types", ctypes.c_int32), ("n_mbs", ctypes.c_int32), ("n_tp", ctypes.c_int32), ("n_algo", ctypes.c_int32)]
 
 
 class AceError(RuntimeError):
@@ -62,6 +69,11 @@ def load_library():
     lib.ace_apply_moves.restype = ctypes.c_int
     lib.ace_apply_moves.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t,
                                     ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    lib.ace_recompute_groups.restype = ctypes.c_int
+    lib.ace_recompute_groups.argtypes = [ctypes.POINTER(AceRcTablesStruct), ctypes.c_int] + [ctypes.c_void_p] * 9
+    lib.ace_recompute_select.restype = ctypes.c_int
+    lib.ace_recompute_select.argtypes = ([ctypes.POINTER(AceRcTablesStruct), ctypes.c_void_p, ctypes.c_int] +
+                                         [ctypes.c_void_p] * 9 + [ctypes.c_double, ctypes.c_void_p, ctypes.c_void_p])
     if lib.ace_abi_version() != ABI_VERSION:
         raise AceError("libace_eval.so has a different ABI version")
     _lib = lib
@@ -107,12 +119,14 @@ class DeviceBatch:
                                      self.ranges.data_ptr() if self.ranges is not None else None, P)
 
     @classmethod
-    def from_device(cls, codes, hdr, num_ops: int):
-        """Wrap tensors that are already on the device in the kernel's layout: codes uint8 [G, P, 16], hdr int32 [P, 4]."""
+    def from_device(cls, codes, hdr, num_ops: int, ranges=None):
+        """Wrap tensors that are already on the device in the kernel's layout: codes uint8 [G, P, 16], hdr int32
+        [P, 4], ranges (single-stage queries) int32 [P, 2] or None."""
         self = cls.__new__(cls)
         self.n_plans, self.num_ops = int(hdr.shape[0]), int(num_ops)
-        self.codes, self.hdr, self.ranges = codes, hdr, None
-        self.struct = AceBatchStruct(codes.data_ptr(), hdr.data_ptr(), None, self.n_plans)
+        self.codes, self.hdr, self.ranges = codes, hdr, ranges
+        self.struct = AceBatchStruct(codes.data_ptr(), hdr.data_ptr(), ranges.data_ptr() if ranges is not None else None,
+                                     self.n_plans)
         return self
 
     @property
@@ -291,6 +305,14 @@ class PlanEvaluator:
         """The plans `index` (device int64 tensor) of a device-resident batch, as a new batch."""
         return DeviceBatch.from_device(d.codes.index_select(1, index).contiguous(), d.hdr.index_select(0, index).contiguous(),
                                        d.num_ops)
+
+    def download(self, d: DeviceBatch, index=None) -> PlanBatch:
+        """A device-resident batch (or its plans `index`, a device int64 tensor) as a host PlanBatch."""
+        if index is not None:
+            d = self.select(d, index)
+        G, P, _ = d.codes.shape
+        codes = d.codes.permute(1, 0, 2).reshape(P, G * 16)[:, :d.num_ops].contiguous().cpu().numpy()
+        return PlanBatch(codes, d.hdr.cpu().numpy().view(np.uint32).copy())
 
     def stage_records_host(self, batch: PlanBatch, ranges: np.ndarray):
         """Single-stage queries: (status, stage record 0 of every query) as numpy arrays."""

@@ -341,10 +341,11 @@ def hill_climb(cm, start: PlanBatch, steps: int, n_neighbours: int, seed: int = 
     (aceso_prims.py:107-108).  With `device_moves` the neighbours never exist on the host: the move
     descriptors (16 bytes each) are expanded by the library on the device and only the winner is
     rebuilt here; `visited` is then a VisitedKeys (64-bit keys of the plan bytes, computed by the
-    same kernel) and `greedy_recompute`, which works on plan bytes on the host, does not apply.
+    same kernel, before any recompute bits are re-chosen) and `greedy_recompute` runs check_recompute's
+    loop on the device as well (CostModel.update_recompute_device).
     Returns (plan, iteration ms, peak MB)."""
-    if device_moves and (greedy_recompute or isinstance(visited, VisitedPlans)):
-        raise ValueError("device_moves: use a VisitedKeys set; greedy recompute needs the plans on the host")
+    if device_moves and isinstance(visited, VisitedPlans):
+        raise ValueError("device_moves: use a VisitedKeys set")
     rng = np.random.default_rng(seed)
     tables = cm.tables
     ev = cm.evaluator
@@ -373,11 +374,14 @@ def hill_climb(cm, start: PlanBatch, steps: int, n_neighbours: int, seed: int = 
                 visited.mark(keys[keep])
                 moves = moves[keep]
                 d = ev.select(d, ev._torch.from_numpy(keep).to(d.hdr.device))
+            if greedy_recompute:
+                d = cm.update_recompute_device(d)
             it, pk, fe, st = ev.score(d)
             idx, val, cnt = ev.topk(it, fe, 1)
             if int(cnt.item()) == 1 and float(val[0].item()) < cur_t:
                 best_i = int(idx[0].item())
-                cur = apply_moves_host(templates, moves[best_i:best_i + 1], tables.db.n_algo)
+                cur = ev.download(d, idx[:1]) if greedy_recompute else \
+                    apply_moves_host(templates, moves[best_i:best_i + 1], tables.db.n_algo)
                 cur_t, cur_m = float(val[0].item()), float(pk[best_i].item())
             if on_step is not None:
                 on_step(step, cur_t, cur_m)

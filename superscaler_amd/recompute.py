@@ -176,3 +176,117 @@ def update_recompute_arrays(cm, batch: PlanBatch) -> PlanBatch:
         a_peak[ids] = new_peak
         alive[ids[~(a_mem[ids] - args.memory_limit > 0)]] = False
     return PlanBatch(codes, hdr.copy())
+
+
+def update_recompute_device(cm, dbatch):
+    """update_recompute for every stage of every plan of a device-resident batch (evaluator.DeviceBatch),
+    without the plans ever visiting the host: the same greedy loop as `update_recompute_arrays`, with
+    the selection done by the library's ace_recompute_groups / ace_recompute_select kernels and the
+    memory bookkeeping by element-wise fp64 tensor operations (the reference's order of operations,
+    one rounding each).  Returns a new DeviceBatch; bit-identical to the host form."""
+    import ctypes
+    import torch
+    from .evaluator import AceRcTablesStruct, DeviceBatch, _check
+    args, tables, ev = cm.settings, cm.tables, cm.evaluator
+    dev = dbatch.hdr.device
+    N, P = dbatch.num_ops, dbatch.n_plans
+    G = (N + 15) // 16
+    codes = dbatch.codes.clone()
+    if not args.flex_recompute:
+        codes |= 8
+        if G * 16 != N:
+            codes.view(G, P, 16)[G - 1, :, N - (G - 1) * 16:] = 0
+        return DeviceBatch.from_device(codes, dbatch.hdr, N)
+    codes &= 0xF7
+    hdr = dbatch.hdr.to(torch.int64) & 0xFFFFFFFF
+    # ---- every stage of every plan: (plan, first op, one past the last op, stage index) ----------
+    rows = codes.permute(1, 0, 2).reshape(P, G * 16)[:, :N]
+    idx = ((rows & 16) != 0).nonzero()                      # sorted by plan, then by position
+    q_plan, q_lo = idx[:, 0].contiguous(), idx[:, 1].contiguous()
+    Q = int(q_plan.numel())
+    S = hdr[:, 0] & 0xff
+    if Q != int(S.sum().item()) or not bool(((rows[:, 0] & 16) != 0).all().item()):
+        raise ValueError("malformed encoding: stage bits do not match the stage counts")
+    same_next = torch.cat([q_plan[1:] == q_plan[:-1], torch.zeros(1, dtype=torch.bool, device=dev)])
+    q_hi = torch.where(same_next, torch.cat([q_lo[1:], q_lo.new_full((1,), N)]), q_lo.new_full((Q,), N))
+    first = torch.cat([torch.ones(1, dtype=torch.bool, device=dev), q_plan[1:] != q_plan[:-1]])
+    start_idx = first.nonzero().squeeze(1)
+    counts = torch.diff(torch.cat([start_idx, start_idx.new_full((1,), Q)]))
+    q_s = torch.arange(Q, device=dev) - torch.repeat_interleave(start_idx, counts)
+    q_nsb = S[q_plan] - 1 - q_s
+    q_bidx = (hdr[q_plan, 0] >> 8) & 0xff
+    gword = hdr[q_plan, 1] | (hdr[q_plan, 2] << 32)
+    q_glog = (gword >> (4 * q_s)) & 15
+
+    # ---- all stages with the recompute bits cleared: one launch over the plans themselves ---------
+    out = ev.score(DeviceBatch.from_device(codes, dbatch.hdr, N), breakdown=True)
+    cm._raise_for_status(out[3].cpu().numpy())
+    rec = out[4][q_plan, q_s]
+
+    def stage_memory(r, nsb):
+        w = r[:, R_WEIGHTS]
+        x = r[:, R_INPUTS] + r[:, R_ACT] - r[:, R_SAVED]
+        mr = r[:, R_RESERVED] if args.consider_reserved_space else torch.zeros_like(w)
+        return (w + w * args.memory_main_params) + w + w * args.memory_optimizer + x * nsb + (x + r[:, R_PEAK]) + mr
+
+    mem = stage_memory(rec, q_nsb.to(torch.float64)) + args.peak_mem_in_backward
+    act = (mem - args.memory_limit > 0).nonzero().squeeze(1)
+    nA = int(act.numel())
+    if nA == 0:
+        return DeviceBatch.from_device(codes, dbatch.hdr, N)
+
+    # ---- device tables of the selection kernels ----------------------------------------------------
+    n_types = len(tables.db.op_names)
+    act_tab = np.ascontiguousarray(tables.db.tables["activations"], dtype=np.float64)
+    d_act = torch.from_numpy(act_tab).to(dev)
+    d_types = torch.from_numpy(np.ascontiguousarray(tables.graph.type_of_pos, dtype=np.int32)).to(dev)
+    norec = ((np.asarray(tables.graph.flags)[:n_types] & og.F_NO_RECOMPUTE) != 0).astype(np.uint8)
+    d_norec = torch.from_numpy(norec).to(dev)
+    lut = torch.from_numpy(np.ascontiguousarray(tables.stage_lut).astype(np.int64)).to(dev)
+    t = AceRcTablesStruct(codes.data_ptr(), P, d_types.data_ptr(), d_act.data_ptr(), d_norec.data_ptr(), N, n_types,
+                          act_tab.shape[1], act_tab.shape[2], act_tab.shape[3])
+    a_plan = q_plan[act].to(torch.int32).contiguous()
+    a_lo, a_hi = q_lo[act].to(torch.int32).contiguous(), q_hi[act].to(torch.int32).contiguous()
+    a_nsb = q_nsb[act].to(torch.int32).contiguous()
+    a_mrow = (lut[q_bidx[act], q_glog[act]] >> 16).to(torch.int32).contiguous()      # (bit pattern of the uint32)
+    sum_size = torch.zeros((nA, n_types), dtype=torch.float64, device=dev)
+    first_pos = torch.full((nA, n_types), N, dtype=torch.int32, device=dev)
+    bad = torch.zeros(nA, dtype=torch.int32, device=dev)
+    stream = ev._stream()
+    with torch.cuda.device(dev):
+        _check(ev.lib, ev.lib.ace_recompute_groups(ctypes.byref(t), nA, a_plan.data_ptr(), a_lo.data_ptr(), a_hi.data_ptr(),
+                                                   a_nsb.data_ptr(), a_mrow.data_ptr(), sum_size.data_ptr(),
+                                                   first_pos.data_ptr(), bad.data_ptr(), stream), "ace_recompute_groups")
+    if bool(bad.any().item()):
+        raise KeyError("a stage's micro-batch size per replica is not in the profile database")
+    recomputed = torch.zeros((nA, n_types), dtype=torch.uint8, device=dev)
+    a_mem = mem[act].contiguous()
+    a_saved = torch.zeros(nA, dtype=torch.float64, device=dev)
+    a_peak = torch.zeros(nA, dtype=torch.float64, device=dev)     # get_peak_activations of an all-zero list is 0 (:421)
+    alive = torch.ones(nA, dtype=torch.uint8, device=dev)
+    q_hdr = torch.zeros((nA, 4), dtype=torch.int32, device=dev)
+    q_hdr[:, 0] = ((a_nsb.to(torch.int64) + 1) | (q_bidx[act] << 8)).to(torch.int32)
+    q_hdr[:, 1] = q_glog[act].to(torch.int32)
+    q_rng = torch.stack([a_lo, a_hi], dim=1).contiguous()
+    nsb1 = (a_nsb + 1).to(torch.float64)
+    while True:
+        with torch.cuda.device(dev):
+            _check(ev.lib, ev.lib.ace_recompute_select(ctypes.byref(t), codes.data_ptr(), nA, a_plan.data_ptr(), a_lo.data_ptr(),
+                                                       a_hi.data_ptr(), a_nsb.data_ptr(), a_mrow.data_ptr(), sum_size.data_ptr(),
+                                                       first_pos.data_ptr(), recomputed.data_ptr(), a_mem.data_ptr(),
+                                                       float(args.memory_limit), alive.data_ptr(), stream), "ace_recompute_select")
+        ids = alive.nonzero().squeeze(1)
+        if ids.numel() == 0:
+            break
+        # re-evaluate the stages that were changed: their plans' columns, as single-stage queries
+        sub = DeviceBatch.from_device(codes.index_select(1, a_plan[ids].to(torch.int64)).contiguous(), q_hdr[ids].contiguous(),
+                                      N, ranges=q_rng[ids].contiguous())
+        r = ev.score(sub, breakdown=True)[4][:, 0, :]
+        new_saved, new_peak = r[:, R_SAVED], r[:, R_PEAK]
+        m = a_mem[ids] - (new_saved - a_saved[ids]) * nsb1[ids]
+        a_saved[ids] = new_saved
+        m = m + (new_peak - a_peak[ids])
+        a_peak[ids] = new_peak
+        a_mem[ids] = m
+        alive[ids] = (m - args.memory_limit > 0).to(torch.uint8)
+    return DeviceBatch.from_device(codes, dbatch.hdr, N)

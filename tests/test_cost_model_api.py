@@ -277,3 +277,27 @@ def test_uniform_grid_command_line(golden_dir, tmp_path, capsys):
         assert max(best.time_list) == want[0][0] and max(best.memory_list) == want[0][1]
     finally:
         m.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,limit", [("gpt3_1_3b", 9000.0), ("gpt3_13b", 40000.0), ("t5_770m", 6000.0), ("wresnet_1b", 1500.0)])
+def test_recompute_on_the_device_equals_the_array_form(name, limit):
+    """The greedy loop with its selection on the device (ace_recompute_groups / ace_recompute_select)
+    sets exactly the bits the numpy form sets."""
+    import dataclasses
+    from superscaler_amd import synth
+    w = synth.WORKLOADS[name]
+    graph = synth.make_graph(w)
+    st = dataclasses.replace(synth.make_settings(w), memory_limit=limit)
+    m = acm.CostModel(st, synth.make_db(w, graph), graph)
+    try:
+        batch = synth.make_plans(w, m.tables, n_plans=1500, seed_offset=17)
+        want = m.update_recompute_arrays(batch)
+        d = m.update_recompute_device(m.evaluator.upload(batch))
+        N, G = batch.num_ops, (batch.num_ops + 15) // 16
+        got = d.codes.permute(1, 0, 2).reshape(batch.n_plans, G * 16).cpu().numpy()
+        assert np.array_equal(got[:, :N], want.codes) and not got[:, N:].any()
+        frac = (want.codes & 8).astype(bool).mean()
+        assert 0.02 < frac < 0.98
+    finally:
+        m.close()

@@ -115,6 +115,12 @@ def test_hill_climb_improves_and_agrees_with_the_oracle():
     assert len(vkeys) > 100
     (t5,), (m5,), (f5,), _ = oracle_scores(orc, plan4, cm.tables)
     assert (f5 == 1 and t5 == t4 and m5 == m4 and t4 < t0) or not f0
+    # the same with check_recompute's choice made on the device for every neighbour
+    plan6, t6, m6 = hill_climb(cm, start, steps=6, n_neighbours=1024, seed=4, device_moves=True, visited=VisitedKeys(),
+                               greedy_recompute=True)
+    assert np.array_equal(cm.update_recompute_arrays(plan6).codes, plan6.codes) or t6 == (t0 if f0 else float("inf"))
+    (t7,), (m7,), (f7,), _ = oracle_scores(orc, plan6, cm.tables)
+    assert (f7 == 1 and t7 == t6 and m7 == m6) or t6 == float("inf")
     cm.close()
 
 

@@ -193,7 +193,8 @@ typedef struct ace_rc_tables {
  * one past the last op, num_stages_behind); d_mrow: uint32[n_stages], the micro-batch index of the stage per
  * tp (4 bits each, as in ace_tables_t.stage_lut).  d_sum_size: double[n_stages][num_types] ZEROED by the
  * caller; d_first_pos: int32[n_stages][num_types] FILLED WITH num_ops by the caller; d_bad: int32[n_stages]
- * zeroed by the caller, set where an op sits outside the profiled grid (the reference raises KeyError). */
+ * zeroed by the caller, set where an op sits outside the profiled grid (the reference raises KeyError) or the
+ * stage does not lie inside the batch (such a stage is left alone by both calls). */
 int ace_recompute_groups(const ace_rc_tables_t *t, int n_stages, const int32_t *d_plan, const int32_t *d_lo,
                          const int32_t *d_hi, const int32_t *d_nsb, const uint32_t *d_mrow, double *d_sum_size,
                          int32_t *d_first_pos, int32_t *d_bad, void *stream);

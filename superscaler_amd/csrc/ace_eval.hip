@@ -136,8 +136,9 @@ __global__ __launch_bounds__(kBlock) void ace_score_kernel(const AceKernelArgs a
 #pragma unroll
         for (int k = 0; k < 16; ++k) {
             const int i = base + k;
-            if (WIN && (k & 3) == 0 && i == next_win) {
-                // every lane of the workgroup reaches this point together
+            if (WIN && (k & 3) == 0 && i == next_win && w < a.n_windows) {
+                // every lane of the workgroup reaches this point together (w < n_windows: the loop also
+                // walks the padding positions of the last group, which must never restage)
                 __syncthreads();
                 stage_window(a, lds_raw, w, tid);
                 __syncthreads();
@@ -505,7 +506,8 @@ __device__ __forceinline__ double rc_act_size(const RcTables &t, unsigned long l
     const uint32_t c = byte & 7u, tp = c >> t.a_shift, al = c & (uint32_t)(t.n_algo - 1);
     uint32_t m = (mrow >> (4u * tp)) & 15u;
     if (tp >= (uint32_t)t.n_tp || m >= (uint32_t)t.n_mbs) { *bad = 1; m = 0; }
-    const int type = t.type_of_pos[i];
+    int type = t.type_of_pos[i];
+    if (type < 0 || type >= t.n_types) { *bad = 1; type = 0; }
     *type_out = type;
     const uint32_t tpc = tp < (uint32_t)t.n_tp ? tp : 0u;
     return t.act[(((size_t)type * t.n_mbs + m) * t.n_tp + tpc) * t.n_algo + al] * (double)(nsb + 1);   // :841
@@ -520,7 +522,9 @@ __global__ void rc_groups_kernel(RcTables t, int n, const int32_t *q_plan, const
     double *sum = sum_size + (size_t)a * t.n_types;
     int32_t *first = first_pos + (size_t)a * t.n_types;
     int flag = 0;
-    for (int i = q_lo[a]; i < q_hi[a]; ++i) {
+    const int lo = q_lo[a], hi = q_hi[a];
+    if (lo < 0 || hi > t.N || lo >= hi || q_plan[a] < 0 || (unsigned long long)q_plan[a] >= t.P) { bad[a] = 1; return; }
+    for (int i = lo; i < hi; ++i) {
         int type;
         const double sz = rc_act_size(t, (unsigned long long)q_plan[a], i, q_mrow[a], q_nsb[a], &type, &flag);
         sum[type] += sz;
@@ -552,12 +556,15 @@ __global__ void rc_select_kernel(RcTables t, uint8_t *codes_rw, int n, const int
         best_first = better ? f : best_first;
         T = better ? ty : T;
     }
+    const int lo = q_lo[a], hi = q_hi[a];
+    // (a stage outside the plan: ace_recompute_groups has flagged it; nothing is touched)
+    if (lo < 0 || hi > t.N || lo >= hi || q_plan[a] < 0 || (unsigned long long)q_plan[a] >= t.P) { alive[a] = 0; return; }
     if (T < 0) { alive[a] = 0; return; }                       // max_saved_size == 0
     done[T] = 1;
-    const int lo = q_lo[a], hi = q_hi[a];
     const int nxt = first[T] + 1;
-    if (nxt >= hi) { alive[a] = 0; return; }                    // :805-806
-    done[t.type_of_pos[nxt]] = 1;
+    if (nxt >= hi || nxt < lo) { alive[a] = 0; return; }        // :805-806
+    const int tn = t.type_of_pos[nxt];
+    if (tn >= 0 && tn < t.n_types) done[tn] = 1;
     const double exceed = mem[a] - memory_limit;
     const bool all = best < exceed;                              // :809
     const unsigned long long plan = (unsigned long long)q_plan[a];

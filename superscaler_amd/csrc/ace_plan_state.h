@@ -139,6 +139,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
     bool lastclose;
     uint32_t first_meta;        // DEFER: first op of the current stage: position | code << 16
     uint32_t ws_stride;         // DEFER: 16-byte units between two stages of one plan in the workspace
+    uint32_t ws_off;            // DEFER: 16-byte units from the plan's first slot to the slot of the current stage (fits: see ensure_stage_ws)
     uint64_t diags;             // the diag of every stage, 4 bits each, looked up once per plan
     uint32_t r_next;            // collective ids of the (previous op, this op) pair, fetched one op ahead
     uint32_t pair_prev;         // pair_bit of the (previous op, this op) pair
@@ -158,6 +159,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         status = 0;
         lastclose = false; first_meta = 0; r_next = 0; pair_prev = 0;
         ws_stride = ACE_WS_REC / 2;
+        ws_off = 0;
         fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = rs_f = rs_b = 0.0;
         id_fwd = id_bwd = id_in = 0.0;
         in_comm = inputs = 0.0;
@@ -233,7 +235,10 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
     // folded here without a table lookup is: fwd + bwd, the closed peak segment, the reserved term).
     ACE_HD void stash(const AceGeom &g, double *ws, uint32_t i_last, uint32_t c_last) {
         if (ws == nullptr || s < 0 || s >= ACE_MAX_STAGES) return;
-        ace_d2 *r = reinterpret_cast<ace_d2 *>(ws) + (size_t)((uint32_t)s * ws_stride);
+        // stages are stashed in order, once each: slot s of this plan is ws_off further on (a running
+        // offset instead of s * ws_stride, which would be a slow 32-bit multiply per stage end)
+        ace_d2 *r = reinterpret_cast<ace_d2 *>(ws) + ws_off;
+        ws_off += ws_stride;
         uint64_t meta = (uint64_t)(first_meta | (c_last << 19)) | ((uint64_t)i_last << 32);
         double meta_d;
         __builtin_memcpy(&meta_d, &meta, 8);

@@ -381,7 +381,7 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
         win_row_begin.append(len(win_rows))
         win_pos.append(j)
         i = j
-    win_pos[-1] = max((win_pos[-1] + 3) // 4 * 4, N + 1)      # never reached: no restaging after the last window
+    win_pos[-1] = 0x7fffffff      # past every position the kernel walks (it walks 16 * ceil(N / 16)): no restaging after the last window
     lds_row_bytes = max(off for _, off in win_rows) + row_bytes
 
     # the (op k, op k + 1) pair, seen from position k

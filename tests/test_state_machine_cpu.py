@@ -66,3 +66,25 @@ def test_stage_records_bit_exact(case):
             assert r[R_STAGE_MB] == orc.predict_stage_memory(stg.ops, stg.recompute_ops, stg.tp_size, stg.dp_size,
                                                              oc.micro_bs, stg.num_stages_behind, stg.algo)
             assert r[R_STAGE_MS] == (f + b + ic + ocm + r[R_RECOMP]) / 1000
+
+
+@pytest.mark.parametrize("name", list(synth.WORKLOADS))
+def test_row_windows_never_restage_in_the_padding(name):
+    """The kernel walks 16 * ceil(N / 16) positions (the last group is padded) and restages rows where a
+    position equals the next window start: that may happen n_windows - 1 times, never in the padding
+    (for N = 134 a final entry of 136 would be met at padded position 136 and index past the window arrays)."""
+    t = synth.make_tables(synth.WORKLOADS[name])
+    N = t.graph.num_ops
+    walked = 16 * ((N + 15) // 16)
+    wp = [int(x) for x in t.win_pos]
+    assert wp[0] == 0 and len(wp) == t.n_windows + 1 and len(t.win_row_begin) == t.n_windows + 1
+    assert all(a < b and a % 4 == 0 and a < N for a, b in zip(wp[:-1], wp[1:]))
+    assert wp[-1] >= walked
+    w, next_win, restaged = 1, wp[1], 0
+    for i in range(walked):
+        if i % 4 == 0 and i == next_win:
+            assert w < t.n_windows
+            restaged += 1
+            w += 1
+            next_win = wp[w]
+    assert restaged == t.n_windows - 1

@@ -7,7 +7,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 LIB = os.path.join(HERE, "libace_eval.so")
 SOURCES = [os.path.join(HERE, "csrc", "ace_eval.hip")]
-HEADERS = [os.path.join(HERE, "csrc", "ace_plan_state.h"), os.path.join(ROOT, "include", "ace_eval.h")]
+HEADERS = [os.path.join(HERE, "csrc", "ace_plan_state.h"), os.path.join(HERE, "csrc", "ace_score_loop.h"),
+           os.path.join(ROOT, "include", "ace_eval.h")]
 
 # -ffp-contract=off: the scoring arithmetic must round exactly like the reference's Python floats,
 # so a*b+c may never be fused.  packed-fp32 ops are switched off for the whole translation unit.

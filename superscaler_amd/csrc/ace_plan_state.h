@@ -43,6 +43,7 @@ struct AceLds {
         return v;
     }
 };
+static inline AceLds ace_make_lds(const unsigned char *base, uint32_t size) { return AceLds{base, size}; }
 static inline double ace_max(double a, double b) { return a > b ? a : b; }
 #else
 #define ACE_HD __device__ __forceinline__
@@ -50,6 +51,7 @@ struct AceLds {
     const unsigned char *base;
     template <class T> ACE_HD T ld(uint32_t off) const { return *reinterpret_cast<const T *>(base + off); }
 };
+ACE_HD AceLds ace_make_lds(const unsigned char *base, uint32_t) { return AceLds{base}; }
 // One v_max_f64.  fmax() makes the compiler quiet both operands first (two more instructions);
 // table values are never signalling NaNs, and a NaN operand only occurs in plans that are
 // reported as unscorable anyway.

@@ -1,0 +1,156 @@
+// The scoring kernel's op loop, as a function of (workgroup, lane): the GPU kernel in ace_eval.hip
+// is a one-line wrapper around ace_score_body(), and a host build (ACE_HOST_EMU, one lane per
+// "workgroup") runs the very same loop on the CPU with every array behind guard pages, so that an
+// index error shows up as a host fault in the CPU test-suite instead of a memory fault on the GPU.
+#pragma once
+#include "ace_plan_state.h"
+
+#ifdef ACE_HOST_EMU
+#define ACE_SYNC() ((void)0)
+#define ACE_ANY(x) (x)
+#else
+#define ACE_SYNC() __syncthreads()
+#define ACE_ANY(x) __any(x)
+#endif
+
+struct AceKernelArgs {
+    AceGeom g;
+    const ace_u4 *codes;        // [G][P] 16 op bytes each
+    const ace_u4 *hdr;          // [P]
+    const ace_u2 *range;        // [P] (first op, one past the last op) or null
+    const double *rows;         // [n_types][row_doubles]
+    const uint32_t *pos_info;   // [N + 1], padded to 16 * G + 16 entries
+    const uint8_t *pair_kinds;  // -> LDS
+    const uint32_t *stage_lut;  // -> LDS
+    const double *nbm1;         // [n_mbs]
+    const int32_t *win_pos;     // [n_windows + 1], multiples of 4
+    const int32_t *win_row_begin;
+    const uint32_t *win_rows;   // pairs (type, lds byte offset)
+    int32_t n_windows, row_doubles, rk_bytes, stg_words;
+    double *iter_ms, *peak_mb;
+    uint8_t *feasible, *status;
+    double *stage_out;
+    double *stage_ws;           // [ACE_MAX_STAGES][plans rounded up to whole workgroups][ACE_WS_REC] for deferred stage tails
+};
+
+// Copy the rows window `w` needs from global memory into LDS (whole workgroup).
+template <int BLOCK> ACE_HD void stage_window(const AceKernelArgs &a, unsigned char *lds_raw, int w, int tid) {
+    const int rb = a.win_row_begin[w], re = a.win_row_begin[w + 1];
+    const int n16 = a.row_doubles / 2;
+    for (int r = rb; r < re; ++r) {
+        const uint32_t type = a.win_rows[2 * r], off = a.win_rows[2 * r + 1];
+        const ace_d2 *src = reinterpret_cast<const ace_d2 *>(a.rows + (size_t)type * a.row_doubles);
+        ace_d2 *dst = reinterpret_cast<ace_d2 *>(lds_raw + off);
+        for (int j = tid; j < n16; j += BLOCK) dst[j] = src[j];
+    }
+}
+
+// BD: also write per-stage records.  RANGED: each plan is one stage over an op sub-range.
+// WIN: the rows of all op types do not fit in LDS together; restage at window boundaries.
+// DEFER: stage tails are stashed in the workspace and evaluated after the op loop, when all lanes
+// are active again (needs every row resident, so never together with WIN).
+// `tid` lane of workgroup `block` of `n_blocks`, BLOCK lanes each; `lds_raw`: the workgroup's LDS (`lds_bytes` long).
+template <bool BD, bool RANGED, bool WIN, bool DEFER, int BLOCK>
+ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint32_t lds_bytes, int tid, long long block,
+                           uint32_t n_blocks) {
+    static_assert(!DEFER || (!BD && !RANGED && !WIN), "deferred stage tails: plain scoring only");
+    const AceGeom &g = a.g;
+    const long long plan = block * BLOCK + tid;
+    const bool active = plan < g.P;
+    const long long pl = active ? plan : (long long)g.P - 1;
+
+    // small tables: pair kinds and the (micro-batch, stage gpus) LUT; without windows, every row
+    for (int j = tid; j < a.rk_bytes; j += BLOCK) lds_raw[g.rk_lds_off + j] = a.pair_kinds[j];
+    for (int j = tid; j < a.stg_words; j += BLOCK)
+        reinterpret_cast<uint32_t *>(lds_raw + g.stg_lds_off)[j] = a.stage_lut[j];
+    stage_window<BLOCK>(a, lds_raw, 0, tid);        // every row, or the first window's
+    ACE_SYNC();
+
+    const AceLds lds = ace_make_lds(lds_raw, lds_bytes);
+    PlanState<BD, RANGED, DEFER> st;
+    const ace_u4 h = a.hdr[pl];
+    ace_u2 range{0u, 0u};
+    if (RANGED) range = a.range[pl];
+    st.init(g, lds, h, range);
+    const double nbm1 = a.nbm1[st.bidx];
+    double *rec = (BD && a.stage_out && active) ? a.stage_out + (size_t)plan * (ACE_MAX_STAGES * ACE_STAGE_REC) : nullptr;
+    if (DEFER) {
+        // stage-major: the records of one stage of consecutive plans are adjacent (padded lanes own a slot too)
+        rec = a.stage_ws + (size_t)plan * ACE_WS_REC;
+        st.ws_stride = n_blocks * (uint32_t)BLOCK * (ACE_WS_REC / 2);
+    }
+
+    int w = 1;
+    int next_win = WIN ? a.win_pos[1] : 0x7fffffff;
+    ace_u4 cw = a.codes[pl];                 // sixteen op bytes of this plan
+    if (!RANGED) st.begin(g, lds, 0, cw.x & 0xffu, a.pos_info[0]);
+    uint32_t pinfo = 0;                      // descriptor of the previous group's last position
+    for (int grp = 0; grp < g.G; ++grp) {
+        const int base = grp << 4;
+        // the sixteen position descriptors of this group: scalar loads (the array is padded)
+        const ace_u4 *ip = reinterpret_cast<const ace_u4 *>(a.pos_info + base);
+        const ace_u4 i0 = ip[0], i1 = ip[1], i2 = ip[2], i3 = ip[3];
+        const uint32_t infos[16] = {i0.x, i0.y, i0.z, i0.w, i1.x, i1.y, i1.z, i1.w,
+                                    i2.x, i2.y, i2.z, i2.w, i3.x, i3.y, i3.z, i3.w};
+        ace_u4 nxt = ace_u4{0u, 0u, 0u, 0u};
+        if (grp + 1 < g.G) nxt = a.codes[(size_t)(grp + 1) * g.P + pl];
+        uint32_t words[5] = {cw.x, cw.y, cw.z, cw.w, nxt.x};
+        if (DEFER) {
+            // whatever the caller left in the bytes past the last op reads as zero
+#pragma unroll
+            for (int j = 0; j < 5; ++j) {
+                const int left = g.N - (base + 4 * j);          // code bytes of this word that belong to the plan
+                words[j] &= left >= 4 ? 0xffffffffu : (left <= 0 ? 0u : ((1u << (8 * left)) - 1u));
+            }
+        }
+        // pair_bit() of the sixteen (op, next op) pairs, four at a time: bit 0 of each byte
+        uint32_t pairs[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t nw = (words[j] >> 8) | (words[j + 1] << 24);      // the next-op bytes of word j
+            pairs[j] = ((words[j] & nw) >> 3) & ~(nw >> 4) & 0x01010101u;
+        }
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            const int i = base + k;
+            if (WIN && (k & 3) == 0 && i == next_win && w < a.n_windows) {
+                // every lane of the workgroup reaches this point together (w < n_windows: the loop also
+                // walks the padding positions of the last group, which must never restage)
+                ACE_SYNC();
+                stage_window<BLOCK>(a, lds_raw, w, tid);
+                ACE_SYNC();
+                ++w;
+                next_win = a.win_pos[w];
+            }
+            // DEFER: positions past the last op are processed too (zeroed code bytes, padded descriptors):
+            // the last stage was stashed at op N - 1, what follows lands in a stage nobody reads
+            if (DEFER || i < g.N) {
+                const uint32_t byte = (words[k >> 2] >> (8 * (k & 3))) & 0xffu;
+                // (past the last op the code bytes are zero padding)
+                const uint32_t nbyte = (words[(k + 1) >> 2] >> (8 * ((k + 1) & 3))) & 0xffu;
+                const uint32_t pair = (pairs[k >> 2] >> (8 * (k & 3))) & 1u;
+                st.step(g, lds, i, byte, nbyte, pair, infos[k], k ? infos[k - 1] : pinfo, i + 1 == g.N, rec);
+            }
+        }
+        pinfo = infos[15];
+        cw = nxt;
+    }
+    if (DEFER) {
+        const int n_st = st.s;
+        for (int s2 = 0; s2 < ACE_MAX_STAGES; ++s2) {
+            const bool live = s2 < n_st;
+            if (!ACE_ANY(live)) break;
+            if (live) st.replay(g, lds, a.pos_info, rec, s2);
+        }
+        st.s = n_st;             // replay() walks s again; result() checks the count of the op loop
+    }
+    double iter, peak;
+    uint8_t feas, stat;
+    st.result(g, nbm1, iter, peak, feas, stat);
+    if (active) {
+        a.iter_ms[plan] = iter;
+        a.peak_mb[plan] = peak;
+        a.feasible[plan] = feas;
+        if (a.status) a.status[plan] = stat;
+    }
+}

@@ -4,7 +4,9 @@
 // access checked for range and alignment, before anything is launched on a GPU.  The product
 // library never links or loads this file.
 #define ACE_HOST_EMU 1
-#include "ace_plan_state.h"
+#include "ace_score_loop.h"
+
+#include <sys/mman.h>
 
 #include <vector>
 
@@ -87,5 +89,110 @@ extern "C" int ace_emu_score(const ace_tables_t *t, const uint8_t *codes /* [P][
         iter_ms[p] = iter; peak_mb[p] = peak; feasible[p] = feas;
         if (status) status[p] = st;
     }
+    return 0;
+}
+
+
+// ------------------------------------------------------------------------------------------
+// The kernel's own op loop (ace_score_loop.h) on the CPU, one lane per "workgroup", with every
+// array the kernel reads or writes placed flush against an inaccessible page: an index past an
+// array's end (or a page or more before its start) ends the process with SIGSEGV instead of
+// going unnoticed.  Callers run this in a child process.
+// ------------------------------------------------------------------------------------------
+namespace {
+
+struct GuardedPool {
+    struct Map { void *base; size_t len; };
+    std::vector<Map> maps;
+    // a writable copy of `bytes` bytes of `src` (zeros if null) whose end (rounded up to `align` bytes, the
+    // alignment the kernel's loads of that array need) touches a PROT_NONE page
+    void *place(const void *src, size_t bytes, size_t align = 16) {
+        const size_t pg = 4096, body = (bytes + pg - 1) / pg * pg + pg;
+        unsigned char *m = (unsigned char *)mmap(nullptr, body + 2 * pg, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS, -1, 0);
+        if (m == MAP_FAILED) { perror("mmap"); abort(); }
+        mprotect(m, pg, PROT_NONE);
+        mprotect(m + pg + body, pg, PROT_NONE);
+        maps.push_back({m, body + 2 * pg});
+        unsigned char *p = m + pg + body - ((bytes + align - 1) / align * align);
+        if (src) memcpy(p, src, bytes);
+        return p;
+    }
+    ~GuardedPool() { for (auto &m : maps) munmap(m.base, m.len); }
+};
+
+template <bool BD, bool RANGED, bool WIN, bool DEFER>
+void run_lanes(const AceKernelArgs &a, unsigned char *lds, uint32_t lds_bytes) {
+    for (long long p = 0; p < a.g.P; ++p) {
+        memset(lds, 0xff, lds_bytes);
+        ace_score_body<BD, RANGED, WIN, DEFER, 1>(a, lds, lds_bytes, 0, p, (uint32_t)a.g.P);
+    }
+}
+
+}  // namespace
+
+// codes: uint8 [G][P][16] (the kernel's layout).  Chooses the kernel variant as the library's launcher does.
+extern "C" int ace_emu_kernel(const ace_tables_t *t, const uint8_t *codes, const uint32_t *hdr, const uint32_t *range,
+                              long long P, double memory_limit, int strict, double *iter_ms, double *peak_mb,
+                              uint8_t *feasible, uint8_t *status, double *stage_out) {
+    if (range && !stage_out) return -1;
+    AceKernelArgs a;
+    memset(&a, 0, sizeof(a));
+    AceGeom &g = a.g;
+    const int C = t->n_tp * t->n_algo;
+    g.N = t->num_ops; g.P = (int32_t)P; g.G = (t->num_ops + 15) / 16;
+    g.C = C; g.A_shift = t->n_algo == 2 ? 1 : 0;
+    g.n_mbs = t->n_mbs; g.n_tp = t->n_tp; g.n_algo = t->n_algo; g.n_glog = t->n_glog; g.n_pair_kinds = t->n_pair_kinds;
+    g.hot_off = t->hot_off * 8u; g.start_off = t->start_off * 8u; g.out_off = t->out_off * 8u; g.z_off = t->z_off * 8u;
+    g.z_shift = 3;
+    while ((1 << (g.z_shift - 3)) < t->z_table_doubles) ++g.z_shift;
+    a.rk_bytes = t->n_pair_kinds * t->n_glog * 64;
+    g.rk_lds_off = (uint32_t)t->lds_row_bytes;
+    g.stg_lds_off = (g.rk_lds_off + (uint32_t)a.rk_bytes + 15u) & ~15u;
+    g.rk_kind_stride = (uint32_t)(t->n_glog * 64);
+    g.row_bytes = (uint32_t)t->row_doubles * 8u;
+    a.stg_words = t->n_mbs * 16;
+    const uint32_t lds_bytes = g.stg_lds_off + (uint32_t)a.stg_words * 4u;
+    g.flags = t->flags; g.main_params = t->main_params; g.optimizer = t->optimizer;
+    g.mem_limit = memory_limit; g.strict = strict ? 1 : 0;
+    a.n_windows = t->n_windows; a.row_doubles = t->row_doubles;
+
+    GuardedPool pool;
+    const size_t G = (size_t)g.G, n_win_rows = (size_t)t->win_row_begin[t->n_windows];
+    a.codes = (const ace_u4 *)pool.place(codes, G * (size_t)P * 16);
+    a.hdr = (const ace_u4 *)pool.place(hdr, (size_t)P * 16);
+    a.range = range ? (const ace_u2 *)pool.place(range, (size_t)P * 8, 8) : nullptr;
+    a.rows = (const double *)pool.place(t->rows, (size_t)t->num_types * t->row_doubles * 8);
+    // (the library uploads the num_ops + 1 descriptors into a zeroed array of 16 * G + 16)
+    uint32_t *pos = (uint32_t *)pool.place(nullptr, (G * 16 + 16) * 4);
+    memcpy(pos, t->pos_info, (size_t)(t->num_ops + 1) * 4);
+    a.pos_info = pos;
+    a.pair_kinds = (const uint8_t *)pool.place(t->pair_kinds, (size_t)a.rk_bytes, 1);
+    a.stage_lut = (const uint32_t *)pool.place(t->stage_lut, (size_t)a.stg_words * 4, 4);
+    a.nbm1 = (const double *)pool.place(t->nb_minus_1, (size_t)t->n_mbs * 8, 8);
+    a.win_pos = (const int32_t *)pool.place(t->win_pos, (size_t)(t->n_windows + 1) * 4, 4);
+    a.win_row_begin = (const int32_t *)pool.place(t->win_row_begin, (size_t)(t->n_windows + 1) * 4, 4);
+    a.win_rows = (const uint32_t *)pool.place(t->win_rows, n_win_rows * 8, 4);
+    a.iter_ms = (double *)pool.place(nullptr, (size_t)P * 8, 8);
+    a.peak_mb = (double *)pool.place(nullptr, (size_t)P * 8, 8);
+    a.feasible = (uint8_t *)pool.place(nullptr, (size_t)P, 1);
+    a.status = status ? (uint8_t *)pool.place(nullptr, (size_t)P, 1) : nullptr;
+    const size_t rec_bytes = (size_t)P * ACE_MAX_STAGES * ACE_STAGE_REC * 8;
+    a.stage_out = stage_out ? (double *)pool.place(stage_out, rec_bytes, 8) : nullptr;   // (records of unused stages stay as the caller left them)
+    unsigned char *lds = (unsigned char *)pool.place(nullptr, lds_bytes);
+    const bool win = t->n_windows > 1;
+    const bool defer = !range && !stage_out && !win && g.N < 65536;
+    if (defer) a.stage_ws = (double *)pool.place(nullptr, (size_t)P * ACE_MAX_STAGES * ACE_WS_REC * 8);
+
+    if (range) { if (win) run_lanes<true, true, true, false>(a, lds, lds_bytes); else run_lanes<true, true, false, false>(a, lds, lds_bytes); }
+    else if (stage_out) { if (win) run_lanes<true, false, true, false>(a, lds, lds_bytes); else run_lanes<true, false, false, false>(a, lds, lds_bytes); }
+    else if (defer) run_lanes<false, false, false, true>(a, lds, lds_bytes);
+    else if (win) run_lanes<false, false, true, false>(a, lds, lds_bytes);
+    else run_lanes<false, false, false, false>(a, lds, lds_bytes);
+
+    memcpy(iter_ms, a.iter_ms, (size_t)P * 8);
+    memcpy(peak_mb, a.peak_mb, (size_t)P * 8);
+    memcpy(feasible, a.feasible, (size_t)P);
+    if (status) memcpy(status, a.status, (size_t)P);
+    if (stage_out) memcpy(stage_out, a.stage_out, rec_bytes);
     return 0;
 }

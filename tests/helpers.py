@@ -54,13 +54,14 @@ def emu_lib():
     if _emu is None:
         so = os.path.join(ROOT, "tests", "emu", "libace_emu.so")
         src = os.path.join(ROOT, "tests", "emu", "ace_emu.cpp")
-        hdr = os.path.join(ROOT, "superscaler_amd", "csrc", "ace_plan_state.h")
-        if (not os.path.exists(so)) or os.path.getmtime(so) < max(os.path.getmtime(src), os.path.getmtime(hdr)):
+        hdrs = [os.path.join(ROOT, "superscaler_amd", "csrc", h) for h in ("ace_plan_state.h", "ace_score_loop.h")]
+        if (not os.path.exists(so)) or os.path.getmtime(so) < max(os.path.getmtime(f) for f in [src] + hdrs):
             subprocess.run(["g++", "-O2", "-std=c++17", "-ffp-contract=off", "-shared", "-fPIC",
                             "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(ROOT, "superscaler_amd", "csrc"),
                             src, "-o", so], check=True)
         _emu = ctypes.CDLL(so)
         _emu.ace_emu_score.restype = ctypes.c_int
+        _emu.ace_emu_kernel.restype = ctypes.c_int
     return _emu
 
 
@@ -82,6 +83,40 @@ def emu_score(tables, batch, memory_limit=None, strict=False, breakdown=False, r
                            it.ctypes.data_as(ctypes.c_void_p), pk.ctypes.data_as(ctypes.c_void_p),
                            fe.ctypes.data_as(ctypes.c_void_p), st.ctypes.data_as(ctypes.c_void_p),
                            rec.ctypes.data_as(ctypes.c_void_p) if breakdown else None)
+    assert rc == 0
+    return it, pk, fe, st, rec
+
+
+def kernel_layout(codes):
+    """uint8 [P][N] -> [ceil(N / 16)][P][16], zero padded: the layout the scoring kernel reads."""
+    P, N = codes.shape
+    G = (N + 15) // 16
+    out = np.zeros((P, G * 16), dtype=np.uint8)
+    out[:, :N] = codes
+    return np.ascontiguousarray(out.reshape(P, G, 16).transpose(1, 0, 2))
+
+
+def emu_kernel_score(tables, batch, memory_limit=None, strict=False, breakdown=False, ranges=None, raw_codes=None):
+    """The scoring kernel's own loop (csrc/ace_score_loop.h) on the CPU with guard pages behind every array:
+    an out-of-range index ends the process with SIGSEGV, so call this from a child process.
+    `raw_codes`: a [G][P][16] array to use as is (e.g. with junk in the padding bytes)."""
+    lib = emu_lib()
+    ts = tables.as_struct()
+    P = batch.n_plans
+    codes = kernel_layout(batch.codes) if raw_codes is None else np.ascontiguousarray(raw_codes)
+    hdr = np.ascontiguousarray(batch.hdr)
+    it = np.zeros(P); pk = np.zeros(P)
+    fe = np.zeros(P, dtype=np.uint8); st = np.zeros(P, dtype=np.uint8)
+    if ranges is not None:
+        ranges = np.ascontiguousarray(ranges, dtype=np.uint32)
+        breakdown = True
+    rec = np.zeros((P, 16, 18)) if breakdown else None
+    limit = tables.settings.memory_limit if memory_limit is None else memory_limit
+    vp = ctypes.c_void_p
+    rc = lib.ace_emu_kernel(ctypes.byref(ts), codes.ctypes.data_as(vp), hdr.ctypes.data_as(vp),
+                            ranges.ctypes.data_as(vp) if ranges is not None else None, ctypes.c_longlong(P),
+                            ctypes.c_double(limit), ctypes.c_int(int(strict)), it.ctypes.data_as(vp), pk.ctypes.data_as(vp),
+                            fe.ctypes.data_as(vp), st.ctypes.data_as(vp), rec.ctypes.data_as(vp) if breakdown else None)
     assert rc == 0
     return it, pk, fe, st, rec
 

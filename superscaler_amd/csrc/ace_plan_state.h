@@ -44,14 +44,38 @@ struct AceLds {
     }
 };
 static inline AceLds ace_make_lds(const unsigned char *base, uint32_t size) { return AceLds{base, size}; }
+static inline uint32_t ace_lds_base(const unsigned char *) { return 0u; }   // host: offsets from `base`
 static inline double ace_max(double a, double b) { return a > b ? a : b; }
 #else
 #define ACE_HD __device__ __forceinline__
+// LDS reads take the absolute LDS byte address.  The address of the workgroup's LDS array is a
+// link-time constant (zero when the kernel has no other LDS variables) that the compiler cannot fold
+// while it compiles; left inside per-lane address arithmetic it costs two or three vector
+// instructions per op.  ace_lds_base() exposes it as a number, and the caller adds it to the
+// wave-uniform region offsets once (scalar arithmetic), so per-lane address math never sees it.
 struct AceLds {
-    const unsigned char *base;
-    template <class T> ACE_HD T ld(uint32_t off) const { return *reinterpret_cast<const T *>(base + off); }
+    template <class T> ACE_HD T ld(uint32_t addr) const {
+#if defined(__HIP_DEVICE_COMPILE__)
+        typedef const unsigned char __attribute__((address_space(3))) *lptr;
+        T v;
+        __builtin_memcpy(&v, (lptr)(uintptr_t)addr, sizeof(T));
+        return v;
+#else
+        (void)addr;
+        return T{};             // (the host pass of the GPU build never runs this)
+#endif
+    }
 };
-ACE_HD AceLds ace_make_lds(const unsigned char *base, uint32_t) { return AceLds{base}; }
+ACE_HD AceLds ace_make_lds(const unsigned char *, uint32_t) { return AceLds{}; }
+ACE_HD uint32_t ace_lds_base(const unsigned char *lds) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef const unsigned char __attribute__((address_space(3))) *lptr;
+    return (uint32_t)(uintptr_t)(lptr)lds;
+#else
+    (void)lds;
+    return 0u;
+#endif
+}
 // One v_max_f64.  fmax() makes the compiler quiet both operands first (two more instructions);
 // table values are never signalling NaNs, and a NaN operand only occurs in plans that are
 // reported as unscorable anyway.

@@ -54,15 +54,20 @@ template <bool BD, bool RANGED, bool WIN, bool DEFER, int BLOCK>
 ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint32_t lds_bytes, int tid, long long block,
                            uint32_t n_blocks) {
     static_assert(!DEFER || (!BD && !RANGED && !WIN), "deferred stage tails: plain scoring only");
-    const AceGeom &g = a.g;
+    // region offsets as absolute LDS addresses for the reads (see AceLds); the staging loops below
+    // write through `lds_raw` with the plain offsets of a.g
+    AceGeom g = a.g;
+    const uint32_t lds_base = ace_lds_base(lds_raw);
+    g.hot_off += lds_base; g.start_off += lds_base; g.out_off += lds_base; g.z_off += lds_base;
+    g.rk_lds_off += lds_base; g.stg_lds_off += lds_base;
     const long long plan = block * BLOCK + tid;
     const bool active = plan < g.P;
     const long long pl = active ? plan : (long long)g.P - 1;
 
     // small tables: pair kinds and the (micro-batch, stage gpus) LUT; without windows, every row
-    for (int j = tid; j < a.rk_bytes; j += BLOCK) lds_raw[g.rk_lds_off + j] = a.pair_kinds[j];
+    for (int j = tid; j < a.rk_bytes; j += BLOCK) lds_raw[a.g.rk_lds_off + j] = a.pair_kinds[j];
     for (int j = tid; j < a.stg_words; j += BLOCK)
-        reinterpret_cast<uint32_t *>(lds_raw + g.stg_lds_off)[j] = a.stage_lut[j];
+        reinterpret_cast<uint32_t *>(lds_raw + a.g.stg_lds_off)[j] = a.stage_lut[j];
     stage_window<BLOCK>(a, lds_raw, 0, tid);        // every row, or the first window's
     ACE_SYNC();
 

@@ -8,6 +8,7 @@ ROOT = os.path.dirname(HERE)
 LIB = os.path.join(HERE, "libace_eval.so")
 SOURCES = [os.path.join(HERE, "csrc", "ace_eval.hip")]
 HEADERS = [os.path.join(HERE, "csrc", "ace_plan_state.h"), os.path.join(HERE, "csrc", "ace_score_loop.h"),
+           os.path.join(HERE, "csrc", "ace_edit_kernels.h"),
            os.path.join(ROOT, "include", "ace_eval.h")]
 
 # -ffp-contract=off: the scoring arithmetic must round exactly like the reference's Python floats,

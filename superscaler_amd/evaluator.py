@@ -171,6 +171,10 @@ class PlanEvaluator:
                 raise ValueError(msg)
         return DeviceBatch(batch, self.device, ranges, staging)
 
+    def device_context(self):
+        """Context manager that makes this evaluator's GPU the current one (for raw library calls)."""
+        return self._torch.cuda.device(self.device)
+
     def _stream(self):
         return ctypes.c_void_p(self._torch.cuda.current_stream(self.device).cuda_stream)
 

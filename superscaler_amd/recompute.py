@@ -253,7 +253,7 @@ def update_recompute_device(cm, dbatch):
     first_pos = torch.full((nA, n_types), N, dtype=torch.int32, device=dev)
     bad = torch.zeros(nA, dtype=torch.int32, device=dev)
     stream = ev._stream()
-    with torch.cuda.device(dev):
+    with ev.device_context():
         _check(ev.lib, ev.lib.ace_recompute_groups(ctypes.byref(t), nA, a_plan.data_ptr(), a_lo.data_ptr(), a_hi.data_ptr(),
                                                    a_nsb.data_ptr(), a_mrow.data_ptr(), sum_size.data_ptr(),
                                                    first_pos.data_ptr(), bad.data_ptr(), stream), "ace_recompute_groups")
@@ -270,7 +270,7 @@ def update_recompute_device(cm, dbatch):
     q_rng = torch.stack([a_lo, a_hi], dim=1).contiguous()
     nsb1 = (a_nsb + 1).to(torch.float64)
     while True:
-        with torch.cuda.device(dev):
+        with ev.device_context():
             _check(ev.lib, ev.lib.ace_recompute_select(ctypes.byref(t), codes.data_ptr(), nA, a_plan.data_ptr(), a_lo.data_ptr(),
                                                        a_hi.data_ptr(), a_nsb.data_ptr(), a_mrow.data_ptr(), sum_size.data_ptr(),
                                                        first_pos.data_ptr(), recomputed.data_ptr(), a_mem.data_ptr(),

@@ -4,6 +4,7 @@
 // access checked for range and alignment, before anything is launched on a GPU.  The product
 // library never links or loads this file.
 #define ACE_HOST_EMU 1
+#include "ace_edit_kernels.h"
 #include "ace_score_loop.h"
 
 #include <sys/mman.h>
@@ -194,5 +195,97 @@ extern "C" int ace_emu_kernel(const ace_tables_t *t, const uint8_t *codes, const
     memcpy(feasible, a.feasible, (size_t)P);
     if (status) memcpy(status, a.status, (size_t)P);
     if (stage_out) memcpy(stage_out, a.stage_out, rec_bytes);
+    return 0;
+}
+
+
+// ------------------------------------------------------------------------------------------
+// The plan-editing kernels (ace_edit_kernels.h) on the CPU, one call per work item, arrays behind
+// guard pages as above.  Sizes follow the C ABI's documentation of ace_apply_moves /
+// ace_recompute_groups / ace_recompute_select.
+// ------------------------------------------------------------------------------------------
+extern "C" int ace_emu_apply_moves(const uint8_t *tmpl_codes, const uint32_t *tmpl_hdr, int n_templates, const uint32_t *moves,
+                                   long long n, int num_ops, int n_algo, uint8_t *codes_out, uint32_t *hdr_out,
+                                   unsigned long long *keys_out) {
+    GuardedPool pool;
+    const int G = (num_ops + 15) / 16;
+    const size_t cb = (size_t)G * 16;
+    const ace_u4 *tc = (const ace_u4 *)pool.place(tmpl_codes, (size_t)n_templates * cb);
+    const ace_u4 *th = (const ace_u4 *)pool.place(tmpl_hdr, (size_t)n_templates * 16);
+    const ace_u4 *mv = (const ace_u4 *)pool.place(moves, (size_t)n * 16);
+    ace_u4 *co = (ace_u4 *)pool.place(nullptr, (size_t)n * cb);
+    ace_u4 *ho = (ace_u4 *)pool.place(nullptr, (size_t)n * 16);
+    unsigned long long *ko = keys_out ? (unsigned long long *)pool.place(keys_out, (size_t)n * 8, 8) : nullptr;
+    // (the library launches whole workgroups of 256: ids past n * G must fall out at the first test)
+    const unsigned long long total = ((unsigned long long)n * G + 255) / 256 * 256;
+    for (unsigned long long id = 0; id < total; ++id)
+        apply_moves_body(id, tc, th, n_templates, mv, (unsigned long long)n, G, n_algo == 2 ? 1 : 0, co, ho, ko);
+    memcpy(codes_out, co, (size_t)n * cb);
+    memcpy(hdr_out, ho, (size_t)n * 16);
+    if (keys_out) memcpy(keys_out, ko, (size_t)n * 8);
+    return 0;
+}
+
+namespace {
+struct RcHost {
+    GuardedPool pool;
+    RcTables k;
+    uint8_t *codes;
+    size_t code_bytes;
+    const int32_t *plan, *lo, *hi, *nsb;
+    const uint32_t *mrow;
+    RcHost(const ace_rc_tables_t *t, int n, const int32_t *q_plan, const int32_t *q_lo, const int32_t *q_hi, const int32_t *q_nsb,
+           const uint32_t *q_mrow) {
+        code_bytes = (size_t)((t->num_ops + 15) / 16) * t->n_plans * 16;
+        codes = (uint8_t *)pool.place(t->d_codes, code_bytes);
+        k = RcTables{codes, (unsigned long long)t->n_plans,
+                     (const int32_t *)pool.place(t->d_type_of_pos, (size_t)t->num_ops * 4, 4),
+                     (const double *)pool.place(t->d_activations, (size_t)t->num_types * t->n_mbs * t->n_tp * t->n_algo * 8, 8),
+                     (const uint8_t *)pool.place(t->d_no_recompute, (size_t)t->num_types, 1),
+                     t->num_ops, t->num_types, t->n_mbs, t->n_tp, t->n_algo, t->n_algo == 2 ? 1 : 0};
+        plan = (const int32_t *)pool.place(q_plan, (size_t)n * 4, 4);
+        lo = (const int32_t *)pool.place(q_lo, (size_t)n * 4, 4);
+        hi = (const int32_t *)pool.place(q_hi, (size_t)n * 4, 4);
+        nsb = (const int32_t *)pool.place(q_nsb, (size_t)n * 4, 4);
+        mrow = (const uint32_t *)pool.place(q_mrow, (size_t)n * 4, 4);
+    }
+};
+}  // namespace
+
+// (same parameter lists as ace_recompute_groups / ace_recompute_select, so a test double can stand in for the library)
+extern "C" int ace_emu_rc_groups(const ace_rc_tables_t *t, int n, const int32_t *q_plan, const int32_t *q_lo, const int32_t *q_hi,
+                                 const int32_t *q_nsb, const uint32_t *q_mrow, double *sum_size, int32_t *first_pos, int32_t *bad,
+                                 void * /*stream*/) {
+    RcHost h(t, n, q_plan, q_lo, q_hi, q_nsb, q_mrow);
+    const size_t nt = (size_t)n * t->num_types;
+    double *sum = (double *)h.pool.place(sum_size, nt * 8, 8);
+    int32_t *first = (int32_t *)h.pool.place(first_pos, nt * 4, 4);
+    int32_t *b = (int32_t *)h.pool.place(bad, (size_t)n * 4, 4);
+    for (int a = 0; a < (n + 127) / 128 * 128; ++a)
+        rc_groups_body(a, h.k, n, h.plan, h.lo, h.hi, h.nsb, h.mrow, sum, first, b);
+    memcpy(sum_size, sum, nt * 8);
+    memcpy(first_pos, first, nt * 4);
+    memcpy(bad, b, (size_t)n * 4);
+    return 0;
+}
+
+// (codes_rw must be t->d_codes, the usual call: the batch is edited in place)
+extern "C" int ace_emu_rc_select(const ace_rc_tables_t *t, uint8_t *codes_rw, int n, const int32_t *q_plan, const int32_t *q_lo,
+                                 const int32_t *q_hi, const int32_t *q_nsb, const uint32_t *q_mrow, const double *sum_size,
+                                 const int32_t *first_pos, uint8_t *recomputed, const double *mem, double memory_limit,
+                                 uint8_t *alive, void * /*stream*/) {
+    if (codes_rw != t->d_codes) return -1;
+    RcHost h(t, n, q_plan, q_lo, q_hi, q_nsb, q_mrow);
+    const size_t nt = (size_t)n * t->num_types;
+    const double *sum = (const double *)h.pool.place(sum_size, nt * 8, 8);
+    const int32_t *first = (const int32_t *)h.pool.place(first_pos, nt * 4, 4);
+    uint8_t *done = (uint8_t *)h.pool.place(recomputed, nt, 1);
+    const double *m = (const double *)h.pool.place(mem, (size_t)n * 8, 8);
+    uint8_t *al = (uint8_t *)h.pool.place(alive, (size_t)n, 1);
+    for (int a = 0; a < (n + 127) / 128 * 128; ++a)
+        rc_select_body(a, h.k, h.codes, n, h.plan, h.lo, h.hi, h.nsb, h.mrow, sum, first, done, m, memory_limit, al);
+    memcpy(codes_rw, h.codes, h.code_bytes);
+    memcpy(recomputed, done, nt);
+    memcpy(alive, al, (size_t)n);
     return 0;
 }

@@ -4,7 +4,10 @@ when every output equals the state-machine emulation's (NaNs included); an out-o
 loop ends this process with SIGSEGV instead.
 
 MODE: plain | breakdown | ranged | junk (random bytes for codes, headers and padding: results are not
-compared, the loop only has to stay inside its arrays) | golden_resnet (the reference's ResNet plans)."""
+compared, the loop only has to stay inside its arrays) | golden_resnet (the reference's ResNet plans) |
+moves (csrc/ace_edit_kernels.h: move descriptors -> plans and keys, against the numpy forms; then random
+descriptors) | recompute (check_recompute's loop for device-resident batches, run on CPU tensors with
+the host build of the selection kernels, against the array form; then random stage tables)."""
 import json
 import os
 import sys
@@ -91,6 +94,80 @@ def main(workload, mode, n):
             emu_kernel_score(tables, junk, raw_codes=raw, ranges=rg)
             if trial == 1:
                 assert same(out, emu_score(tables, batch))
+    elif mode == "moves":
+        import ctypes
+        from superscaler_amd.neighbours import apply_moves_host, plan_keys_host, sample_moves
+        from tests.helpers import emu_lib
+        lib = emu_lib()
+        vp = ctypes.c_void_p
+        lib.ace_emu_apply_moves.restype = ctypes.c_int
+        lib.ace_emu_apply_moves.argtypes = [vp, vp, ctypes.c_int, vp, ctypes.c_longlong, ctypes.c_int, ctypes.c_int, vp, vp, vp]
+        rng = np.random.default_rng(9)
+        N = tables.graph.num_ops
+        G = (N + 15) // 16
+
+        def expand(templates, moves, keys):
+            T, m = templates.n_plans, len(moves)
+            tc = np.zeros((T, G * 16), dtype=np.uint8)
+            tc[:, :N] = templates.codes
+            th = np.ascontiguousarray(templates.hdr)
+            mv = np.ascontiguousarray(moves, dtype=np.uint32)
+            co = np.zeros((G, m, 16), dtype=np.uint8)
+            ho = np.zeros((m, 4), dtype=np.uint32)
+            ko = np.zeros(m, dtype=np.uint64) if keys else None
+            assert lib.ace_emu_apply_moves(tc.ctypes.data, th.ctypes.data, T, mv.ctypes.data, m, N, tables.db.n_algo,
+                                           co.ctypes.data, ho.ctypes.data, ko.ctypes.data if keys else None) == 0
+            return co, ho, ko
+
+        for p in range(min(n, 4)):
+            templates, moves = sample_moves(batch.slice(p, p + 1), tables, 700, rng)
+            want = apply_moves_host(templates, moves, tables.db.n_algo)
+            co, ho, ko = expand(templates, moves, True)
+            assert np.array_equal(co, kernel_layout(want.codes)) and np.array_equal(ho, want.hdr)
+            assert np.array_equal(ko, plan_keys_host(want))
+            junk = rng.integers(0, 2 ** 32, size=(512, 4), dtype=np.uint64).astype(np.uint32)
+            junk[::2, 0] &= 0x0007ffff                 # half of them with a known op and a small template index
+            expand(templates, junk, True)
+            expand(templates, junk, False)
+    elif mode == "recompute":
+        import dataclasses
+        from superscaler_amd import aceso_cost_model as acm
+        from tests.helpers import EmuDeviceEvaluator
+        limit = {"gpt3_1_3b": 9000.0, "gpt3_13b": 40000.0, "t5_770m": 6000.0, "wresnet_1b": 1500.0, "gpt3_175b": 60000.0}[workload]
+        graph = synth.make_graph(w)
+        st = dataclasses.replace(synth.make_settings(w), memory_limit=limit)
+        cm = acm.CostModel(st, synth.make_db(w, graph), graph)
+        cm._evaluator = EmuDeviceEvaluator(cm.tables)
+        want = cm.update_recompute_arrays(batch)
+        d = cm.update_recompute_device(cm.evaluator.upload(batch))
+        N = batch.num_ops
+        got = d.codes.permute(1, 0, 2).reshape(batch.n_plans, -1).numpy()
+        assert np.array_equal(got[:, :N], want.codes) and not got[:, N:].any()
+        assert (want.codes & 8).any() and not (want.codes & 8).all()      # the greedy loop had work to do
+        # random stage tables: the kernels flag or ignore what lies outside the batch
+        import ctypes
+        import torch
+        from superscaler_amd.evaluator import AceRcTablesStruct
+        rng = np.random.default_rng(4)
+        ev = cm.evaluator
+        nq, nt = 300, len(cm.tables.db.op_names)
+        act = np.ascontiguousarray(cm.tables.db.tables["activations"], dtype=np.float64)
+        types = np.ascontiguousarray(cm.tables.graph.type_of_pos, dtype=np.int32)
+        norec = np.zeros(nt, dtype=np.uint8)
+        codes = d.codes.clone()
+        t = AceRcTablesStruct(codes.data_ptr(), batch.n_plans, types.ctypes.data, act.ctypes.data, norec.ctypes.data, N, nt,
+                              act.shape[1], act.shape[2], act.shape[3])
+        q = [np.ascontiguousarray(rng.integers(-5, m, size=nq), dtype=np.int32) for m in (batch.n_plans + 5, N + 5, N + 5, 20)]
+        mrow = rng.integers(0, 2 ** 32, size=nq, dtype=np.uint64).astype(np.uint32)
+        sums, first, bad = np.zeros((nq, nt)), np.full((nq, nt), N, dtype=np.int32), np.zeros(nq, dtype=np.int32)
+        assert ev.lib.ace_recompute_groups(ctypes.byref(t), nq, *[a.ctypes.data for a in q], mrow.ctypes.data, sums.ctypes.data,
+                                           first.ctypes.data, bad.ctypes.data, None) == 0
+        first = rng.integers(-3, N + 3, size=(nq, nt)).astype(np.int32)     # even with garbage group tables
+        done, alive = np.zeros((nq, nt), dtype=np.uint8), np.ones(nq, dtype=np.uint8)
+        mem = rng.uniform(0, 2 * limit, size=nq)
+        assert ev.lib.ace_recompute_select(ctypes.byref(t), codes.data_ptr(), nq, *[a.ctypes.data for a in q], mrow.ctypes.data,
+                                           sums.ctypes.data, first.ctypes.data, done.ctypes.data, mem.ctypes.data, float(limit),
+                                           alive.ctypes.data, None) == 0
     else:
         raise SystemExit(f"unknown mode {mode}")
     print("ok")

@@ -156,3 +156,68 @@ def c_oracle_for(tables):
 def c_oracle_scores(tables, batch, strict=False, threads=1, memory_limit=None, lists=False):
     return c_oracle_for(tables).score_arrays(*plan_arrays(batch, tables), strict=strict, threads=threads,
                                              memory_limit=memory_limit, lists=lists)
+
+
+class EmuEvaluator:
+    """Test double with PlanEvaluator.score_host's signature, backed by tests/emu."""
+
+    def __init__(self, tables):
+        self.tables = tables
+
+    def score_host(self, batch, memory_limit=None, strict=False, breakdown=False, ranges=None):
+        it, pk, fe, st, rec = emu_score(self.tables, batch, memory_limit, strict, breakdown, ranges)
+        return (it, pk, fe, st, rec) if (breakdown or ranges is not None) else (it, pk, fe, st)
+
+    def stage_records_host(self, batch, ranges):
+        out = emu_score(self.tables, batch, None, False, True, ranges)
+        return out[3], out[4][:, 0, :]
+
+    def picked_records_host(self, batch, plan_idx, stage_idx):
+        out = emu_score(self.tables, batch, None, False, True, None)
+        return out[3], out[4][plan_idx, stage_idx]
+
+    def close(self):
+        pass
+
+
+class EmuDeviceEvaluator(EmuEvaluator):
+    """Test double for the device-resident calls of PlanEvaluator, on CPU tensors: `score` runs the kernel's
+    own loop behind guard pages (tests/emu), `lib` offers ace_recompute_groups / ace_recompute_select from
+    the host build of csrc/ace_edit_kernels.h.  A wrong index ends the process: use it in a child process."""
+
+    def __init__(self, tables):
+        import contextlib
+        import types
+        import torch
+        super().__init__(tables)
+        self._torch = torch
+        self.device = torch.device("cpu")
+        emu = emu_lib()
+        vp = ctypes.c_void_p
+        emu.ace_emu_rc_groups.restype = ctypes.c_int
+        emu.ace_emu_rc_groups.argtypes = [vp, ctypes.c_int] + [vp] * 9
+        emu.ace_emu_rc_select.restype = ctypes.c_int
+        emu.ace_emu_rc_select.argtypes = [vp, vp, ctypes.c_int] + [vp] * 9 + [ctypes.c_double, vp, vp]
+        self.lib = types.SimpleNamespace(ace_recompute_groups=lambda t, *a: emu.ace_emu_rc_groups(ctypes.cast(t, vp), *a),
+                                         ace_recompute_select=lambda t, *a: emu.ace_emu_rc_select(ctypes.cast(t, vp), *a),
+                                         ace_strerror=lambda code: b"emulation error")
+        self.device_context = contextlib.nullcontext
+
+    def _stream(self):
+        return None
+
+    def upload(self, batch, validate=True, ranges=None, staging=None):
+        from superscaler_amd.evaluator import DeviceBatch
+        return DeviceBatch(batch, "cpu", ranges)
+
+    def score(self, dbatch, memory_limit=None, strict=False, breakdown=False, out=None):
+        torch = self._torch
+        from superscaler_amd.plan import PlanBatch
+        P, N = dbatch.n_plans, dbatch.num_ops
+        stub = PlanBatch(np.zeros((P, N), dtype=np.uint8), dbatch.hdr.numpy().view(np.uint32).copy())
+        rg = dbatch.ranges.numpy().view(np.uint32) if dbatch.ranges is not None else None
+        it, pk, fe, st, rec = emu_kernel_score(self.tables, stub, memory_limit, strict, breakdown, rg,
+                                               raw_codes=dbatch.codes.contiguous().numpy())
+        return (torch.from_numpy(it), torch.from_numpy(pk), torch.from_numpy(fe), torch.from_numpy(st),
+                torch.from_numpy(rec) if rec is not None else None)
+

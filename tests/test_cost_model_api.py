@@ -14,31 +14,9 @@ import pytest
 from superscaler_amd import aceso_cost_model as acm
 from superscaler_amd.plan import get_config
 from superscaler_amd.profile_db import CostModelSettings
-from tests.helpers import emu_score
+from tests.helpers import EmuEvaluator, emu_score
 
 CASES = ["gpt_1_3B", "resnet_500M", "t5_770M"]
-
-
-class EmuEvaluator:
-    """Test double with PlanEvaluator.score_host's signature, backed by tests/emu."""
-
-    def __init__(self, tables):
-        self.tables = tables
-
-    def score_host(self, batch, memory_limit=None, strict=False, breakdown=False, ranges=None):
-        it, pk, fe, st, rec = emu_score(self.tables, batch, memory_limit, strict, breakdown, ranges)
-        return (it, pk, fe, st, rec) if (breakdown or ranges is not None) else (it, pk, fe, st)
-
-    def stage_records_host(self, batch, ranges):
-        out = emu_score(self.tables, batch, None, False, True, ranges)
-        return out[3], out[4][:, 0, :]
-
-    def picked_records_host(self, batch, plan_idx, stage_idx):
-        out = emu_score(self.tables, batch, None, False, True, None)
-        return out[3], out[4][plan_idx, stage_idx]
-
-    def close(self):
-        pass
 
 
 def make_model(golden_dir, case, backend):

@@ -293,41 +293,43 @@ def plan_keys_host(batch: PlanBatch) -> np.ndarray:
 
 
 class VisitedKeys:
-    """A visited set over 64-bit plan keys (for neighbours that only exist on the device): one sorted
-    array plus the keys marked since it was last merged."""
+    """A visited set over 64-bit plan keys (for neighbours that only exist on the device): two sorted
+    arrays, a large one and a small one that takes the new keys and is folded into the large one
+    when it has grown (so marking costs a merge of the small array only)."""
+
+    SMALL_LIMIT = 65536
 
     def __init__(self):
         self._sorted = np.empty(0, dtype=np.uint64)
-        self._recent = []
-        self._n_recent = 0
+        self._small = np.empty(0, dtype=np.uint64)
 
     def __len__(self):
-        self._merge()
-        return len(self._sorted)
+        return len(self._sorted) + len(self._small)
 
-    def _merge(self):
-        if self._recent:
-            self._sorted = np.union1d(self._sorted, np.concatenate(self._recent))
-            self._recent, self._n_recent = [], 0
+    @staticmethod
+    def _absent(sorted_keys: np.ndarray, keys: np.ndarray) -> np.ndarray:
+        if len(sorted_keys) == 0:
+            return np.ones(len(keys), dtype=bool)
+        pos = np.searchsorted(sorted_keys, keys)
+        return sorted_keys[np.minimum(pos, len(sorted_keys) - 1)] != keys
 
     def unseen(self, keys: np.ndarray) -> np.ndarray:
         """Mask of the keys not marked before that do not repeat an earlier entry of `keys`."""
-        if self._n_recent > 65536:
-            self._merge()
         _, first = np.unique(keys, return_index=True)
         mask = np.zeros(len(keys), dtype=bool)
         mask[first] = True
-        if len(self._sorted):
-            pos = np.searchsorted(self._sorted, keys)
-            mask &= self._sorted[np.minimum(pos, len(self._sorted) - 1)] != keys
-        for r in self._recent:
-            mask &= ~np.isin(keys, r)
+        cand = np.flatnonzero(mask)
+        ok = self._absent(self._sorted, keys[cand]) & self._absent(self._small, keys[cand])
+        mask[cand[~ok]] = False
         return mask
 
     def mark(self, keys: np.ndarray) -> None:
         k = np.unique(np.asarray(keys, dtype=np.uint64))
-        self._recent.append(k)
-        self._n_recent += len(k)
+        k = k[self._absent(self._sorted, k)]              # (the two arrays stay disjoint: __len__ is their sum)
+        self._small = np.union1d(self._small, k)
+        if len(self._small) > self.SMALL_LIMIT:
+            self._sorted = np.union1d(self._sorted, self._small)
+            self._small = np.empty(0, dtype=np.uint64)
 
 
 def hill_climb(cm, start: PlanBatch, steps: int, n_neighbours: int, seed: int = 0, max_move: int = 8,

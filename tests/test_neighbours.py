@@ -78,8 +78,15 @@ def test_plan_keys_separate_distinct_plans_and_key_set_behaves():
     seen = set(keys[:5000].tolist())
     want = first & ~np.array([k in seen for k in keys.tolist()])
     assert np.array_equal(vk.unseen(keys), want)
-    vk._merge()
-    assert np.array_equal(vk.unseen(keys), want) and len(vk) == len(seen)
+    assert len(vk) == len(seen)
+    # the same after the small array has been folded into the large one, and with keys marked twice
+    vk.SMALL_LIMIT = 100
+    vk.mark(keys[4000:5000])
+    assert len(vk._small) == 0 and len(vk) == len(seen) and np.array_equal(vk.unseen(keys), want)
+    vk.mark(keys[4500:5500])
+    seen |= set(keys[5000:5500].tolist())
+    want = first & ~np.array([k in seen for k in keys.tolist()])
+    assert len(vk) == len(seen) and np.array_equal(vk.unseen(keys), want)
     # a header-only change (another micro-batch size) changes the key
     h = nb.hdr.copy()
     h[:, 0] ^= 1 << 8

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define ACE_ABI_VERSION 3
+#define ACE_ABI_VERSION 4
 #define ACE_MAX_STAGES 16      /* aceso_utils.py:502: end_num_stages = min(num_gpus, 16) */
 #define ACE_STAGE_REC 18       /* doubles per stage record, see ACE_R_* */
 
@@ -121,6 +121,14 @@ typedef struct ace_batch {
                                   predict_stage_time / predict_stage_memory (aceso_cost_model.py:493-539);
                                   results are read from stage record 0, so d_stage_out is required. */
     size_t n_plans;
+    const uint32_t *d_order;   /* NULL, or uint32[n_plans]: slot i of d_codes / d_hdr / d_range holds the caller's plan
+                                  d_order[i], and every result of that plan (d_iter_ms, d_peak_mb, d_feasible,
+                                  d_status, d_stage_out) is written at index d_order[i].  Lets the caller store the
+                                  plans in the order that suits the kernel -- lanes of a wavefront that close their
+                                  stages at the same ops do not wait for each other, so grouping plans by pipeline
+                                  depth (deepest first) and first stage boundary is worth about a tenth of the
+                                  kernel time on mixed batches -- and still get results in its own order.  Must be
+                                  a permutation of 0 .. n_plans - 1 (entries >= n_plans are skipped). */
 } ace_batch_t;
 
 int ace_abi_version(void);

@@ -451,7 +451,8 @@ static int fill_args(ace_handle_t *h, const ace_batch_t *b, double memory_limit,
                      double *d_peak_mb, uint8_t *d_feasible, uint8_t *d_status, double *d_stage_out, AceKernelArgs *a) {
     if (!h || !b || !b->d_codes || !b->d_hdr || !d_iter_ms || !d_peak_mb || !d_feasible) return ACE_EINVAL;
     if (b->n_plans == 0 || b->n_plans > 0x7fffffffull) return ACE_EINVAL;
-    if (((uintptr_t)b->d_codes & 15u) || ((uintptr_t)b->d_hdr & 15u) || ((uintptr_t)b->d_range & 7u)) return ACE_EINVAL;
+    if (((uintptr_t)b->d_codes & 15u) || ((uintptr_t)b->d_hdr & 15u) || ((uintptr_t)b->d_range & 7u) || ((uintptr_t)b->d_order & 3u))
+        return ACE_EINVAL;
     if (b->d_range && !d_stage_out) return ACE_EINVAL;   // single-stage queries are read from their stage record
     a->g = h->geom;
     a->g.P = (int32_t)b->n_plans;
@@ -460,6 +461,7 @@ static int fill_args(ace_handle_t *h, const ace_batch_t *b, double memory_limit,
     a->codes = reinterpret_cast<const ace_u4 *>(b->d_codes);
     a->hdr = reinterpret_cast<const ace_u4 *>(b->d_hdr);
     a->range = reinterpret_cast<const ace_u2 *>(b->d_range);
+    a->order = b->d_order;
     a->rows = h->d_rows; a->pos_info = h->d_pos_info; a->pair_kinds = h->d_pair_kinds; a->stage_lut = h->d_stage_lut;
     a->nbm1 = h->d_nbm1; a->win_pos = h->d_win_pos; a->win_row_begin = h->d_win_row_begin; a->win_rows = h->d_win_rows;
     a->n_windows = h->n_windows; a->row_doubles = h->row_doubles; a->rk_bytes = h->rk_bytes; a->stg_words = h->stg_words;

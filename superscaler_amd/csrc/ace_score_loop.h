@@ -18,6 +18,7 @@ struct AceKernelArgs {
     const ace_u4 *codes;        // [G][P] 16 op bytes each
     const ace_u4 *hdr;          // [P]
     const ace_u2 *range;        // [P] (first op, one past the last op) or null
+    const uint32_t *order;      // [P] result index of the plan in each slot, or null (slot i -> result i)
     const double *rows;         // [n_types][row_doubles]
     const uint32_t *pos_info;   // [N + 1], padded to 16 * G + 16 entries
     const uint8_t *pair_kinds;  // -> LDS
@@ -61,8 +62,11 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     g.hot_off += lds_base; g.start_off += lds_base; g.out_off += lds_base; g.z_off += lds_base;
     g.rk_lds_off += lds_base; g.stg_lds_off += lds_base;
     const long long plan = block * BLOCK + tid;
-    const bool active = plan < g.P;
-    const long long pl = active ? plan : (long long)g.P - 1;
+    const bool in_batch = plan < g.P;
+    const long long pl = in_batch ? plan : (long long)g.P - 1;      // slot this lane reads
+    // where this lane's results go; a slot whose entry is not a valid index computes but writes nothing
+    const long long out = a.order ? (long long)a.order[pl] : plan;
+    const bool active = in_batch && out < g.P;
 
     // small tables: pair kinds and the (micro-batch, stage gpus) LUT; without windows, every row
     for (int j = tid; j < a.rk_bytes; j += BLOCK) lds_raw[a.g.rk_lds_off + j] = a.pair_kinds[j];
@@ -78,7 +82,7 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     if (RANGED) range = a.range[pl];
     st.init(g, lds, h, range);
     const double nbm1 = a.nbm1[st.bidx];
-    double *rec = (BD && a.stage_out && active) ? a.stage_out + (size_t)plan * (ACE_MAX_STAGES * ACE_STAGE_REC) : nullptr;
+    double *rec = (BD && a.stage_out && active) ? a.stage_out + (size_t)out * (ACE_MAX_STAGES * ACE_STAGE_REC) : nullptr;
     if (DEFER) {
         // stage-major: the records of one stage of consecutive plans are adjacent (padded lanes own a slot too)
         rec = a.stage_ws + (size_t)plan * ACE_WS_REC;
@@ -153,9 +157,9 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     uint8_t feas, stat;
     st.result(g, nbm1, iter, peak, feas, stat);
     if (active) {
-        a.iter_ms[plan] = iter;
-        a.peak_mb[plan] = peak;
-        a.feasible[plan] = feas;
-        if (a.status) a.status[plan] = stat;
+        a.iter_ms[out] = iter;
+        a.peak_mb[out] = peak;
+        a.feasible[out] = feas;
+        if (a.status) a.status[out] = stat;
     }
 }

@@ -22,7 +22,7 @@ EXPORTS = ["ace_abi_version", "ace_strerror", "ace_last_hip_error", "ace_create"
 
 class AceBatchStruct(ctypes.Structure):
     _fields_ = [("d_codes", ctypes.c_void_p), ("d_hdr", ctypes.c_void_p), ("d_range", ctypes.c_void_p),
-                ("n_plans", ctypes.c_size_t)]
+                ("n_plans", ctypes.c_size_t), ("d_order", ctypes.c_void_p)]
 
 
 class AceRcTablesStruct(ctypes.Structure):
@@ -87,51 +87,73 @@ def _check(lib, rc, what):
         raise AceError(f"{what}: {msg}" + (f" ({hip})" if hip and rc == -3 else ""))
 
 
+def depth_order(batch: PlanBatch) -> np.ndarray:
+    """Permutation that sorts the plans by pipeline depth (deepest first: the long jobs start first),
+    then by the position of their first stage boundary (stable)."""
+    S = (batch.hdr[:, 0] & 0xff).astype(np.int64)
+    first_cut = ((batch.codes[:, 1:] & 16) != 0).argmax(axis=1) if batch.codes.shape[1] > 1 else np.zeros(len(S), dtype=np.int64)
+    return np.lexsort((first_cut, -S))
+
+
 class DeviceBatch:
     """A PlanBatch resident in HBM in the layout the kernel streams."""
 
-    def __init__(self, batch: PlanBatch, device="cuda:0", ranges: Optional[np.ndarray] = None, staging=None):
+    def __init__(self, batch: PlanBatch, device="cuda:0", ranges: Optional[np.ndarray] = None, staging=None,
+                 group_by_depth: bool = False):
         """`staging`: a pinned uint8 host tensor of at least P * N bytes; the plan bytes then go through
         it and the copy to the device does not block the host (the caller must not reuse the tensor
-        before that copy has completed)."""
+        before that copy has completed).
+        `group_by_depth`: store the plans sorted by pipeline depth (deepest first) and position of the
+        first stage boundary, with the permutation alongside (`order`), so that the lanes of a
+        wavefront close their stages together; results still come back in the caller's order."""
         import torch
         self.n_plans = batch.n_plans
         self.num_ops = batch.num_ops
         P, N = batch.codes.shape
         G = (N + 15) // 16
+        host_codes, host_hdr = batch.codes, batch.hdr
+        self.order = None
+        if group_by_depth and P > 1:
+            perm = depth_order(batch)
+            host_codes, host_hdr = host_codes[perm], host_hdr[perm]
+            if ranges is not None:
+                ranges = np.asarray(ranges)[perm]
+            self.order = torch.from_numpy(perm.astype(np.int32)).to(device)
         if staging is not None:
             stage = staging[:P * N].view(P, N)
-            stage.copy_(torch.from_numpy(np.ascontiguousarray(batch.codes)))
+            stage.copy_(torch.from_numpy(np.ascontiguousarray(host_codes)))
             codes = stage.to(device, non_blocking=True)
         else:
-            codes = torch.from_numpy(np.ascontiguousarray(batch.codes)).to(device)
+            codes = torch.from_numpy(np.ascontiguousarray(host_codes)).to(device)
         if G * 16 != N:
             codes = torch.nn.functional.pad(codes, (0, G * 16 - N))
         # [P, G, 16] -> [G, P, 16]: plan-minor, sixteen ops per 16-byte word
         self.codes = codes.view(P, G, 16).permute(1, 0, 2).contiguous()
-        self.hdr = torch.from_numpy(np.ascontiguousarray(batch.hdr).view(np.int32)).to(device)
+        self.hdr = torch.from_numpy(np.ascontiguousarray(host_hdr).view(np.int32)).to(device)
         self.ranges = None
         if ranges is not None:
             r = np.ascontiguousarray(ranges, dtype=np.uint32)
             assert r.shape == (P, 2)
             self.ranges = torch.from_numpy(r.view(np.int32)).to(device)
         self.struct = AceBatchStruct(self.codes.data_ptr(), self.hdr.data_ptr(),
-                                     self.ranges.data_ptr() if self.ranges is not None else None, P)
+                                     self.ranges.data_ptr() if self.ranges is not None else None, P,
+                                     self.order.data_ptr() if self.order is not None else None)
 
     @classmethod
-    def from_device(cls, codes, hdr, num_ops: int, ranges=None):
+    def from_device(cls, codes, hdr, num_ops: int, ranges=None, order=None):
         """Wrap tensors that are already on the device in the kernel's layout: codes uint8 [G, P, 16], hdr int32
-        [P, 4], ranges (single-stage queries) int32 [P, 2] or None."""
+        [P, 4], ranges (single-stage queries) int32 [P, 2] or None, order int32 [P] (result index of the plan in
+        each slot) or None."""
         self = cls.__new__(cls)
         self.n_plans, self.num_ops = int(hdr.shape[0]), int(num_ops)
-        self.codes, self.hdr, self.ranges = codes, hdr, ranges
+        self.codes, self.hdr, self.ranges, self.order = codes, hdr, ranges, order
         self.struct = AceBatchStruct(codes.data_ptr(), hdr.data_ptr(), ranges.data_ptr() if ranges is not None else None,
-                                     self.n_plans)
+                                     self.n_plans, order.data_ptr() if order is not None else None)
         return self
 
     @property
     def bytes_moved_per_plan(self):
-        return self.codes.shape[0] * 16 + 16
+        return self.codes.shape[0] * 16 + 16 + (4 if self.order is not None else 0)
 
 
 class PlanEvaluator:
@@ -162,14 +184,14 @@ class PlanEvaluator:
             pass
 
     def upload(self, batch: PlanBatch, validate: bool = True, ranges: Optional[np.ndarray] = None,
-               staging=None) -> DeviceBatch:
+               staging=None, group_by_depth: bool = False) -> DeviceBatch:
         """`validate` checks the encoding on the host first (a clear message instead of per-plan status
-        bytes; the kernel itself is safe for any byte content)."""
+        bytes; the kernel itself is safe for any byte content).  `group_by_depth`: see DeviceBatch."""
         if validate and ranges is None:
             msg = validate_batch(batch, self.tables)
             if msg:
                 raise ValueError(msg)
-        return DeviceBatch(batch, self.device, ranges, staging)
+        return DeviceBatch(batch, self.device, ranges, staging, group_by_depth)
 
     def device_context(self):
         """Context manager that makes this evaluator's GPU the current one (for raw library calls)."""
@@ -307,6 +329,8 @@ class PlanEvaluator:
 
     def select(self, d: DeviceBatch, index) -> DeviceBatch:
         """The plans `index` (device int64 tensor) of a device-resident batch, as a new batch."""
+        if d.order is not None:
+            raise ValueError("select: the batch is stored in grouped order (group_by_depth)")
         return DeviceBatch.from_device(d.codes.index_select(1, index).contiguous(), d.hdr.index_select(0, index).contiguous(),
                                        d.num_ops)
 
@@ -314,6 +338,8 @@ class PlanEvaluator:
         """A device-resident batch (or its plans `index`, a device int64 tensor) as a host PlanBatch."""
         if index is not None:
             d = self.select(d, index)
+        if d.order is not None:
+            raise ValueError("download: the batch is stored in grouped order (group_by_depth)")
         G, P, _ = d.codes.shape
         codes = d.codes.permute(1, 0, 2).reshape(P, G * 16)[:, :d.num_ops].contiguous().cpu().numpy()
         return PlanBatch(codes, d.hdr.cpu().numpy().view(np.uint32).copy())
@@ -333,8 +359,9 @@ class PlanEvaluator:
         return out[3].cpu().numpy(), pick.cpu().numpy()
 
     # convenience: host in, host out
-    def score_host(self, batch: PlanBatch, memory_limit=None, strict=False, breakdown=False, ranges=None):
-        d = self.upload(batch, ranges=ranges)
+    def score_host(self, batch: PlanBatch, memory_limit=None, strict=False, breakdown=False, ranges=None,
+                   group_by_depth: bool = False):
+        d = self.upload(batch, ranges=ranges, group_by_depth=group_by_depth)
         out = self.score(d, memory_limit, strict, breakdown)
         self._torch.cuda.synchronize(self.device)
         return tuple(None if t is None else t.cpu().numpy() for t in out)

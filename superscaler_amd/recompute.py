@@ -188,6 +188,8 @@ def update_recompute_device(cm, dbatch):
     import torch
     from .evaluator import AceRcTablesStruct, DeviceBatch, _check
     args, tables, ev = cm.settings, cm.tables, cm.evaluator
+    if getattr(dbatch, "order", None) is not None:
+        raise ValueError("update_recompute_device: the batch is stored in grouped order (group_by_depth)")
     dev = dbatch.hdr.device
     N, P = dbatch.num_ops, dbatch.n_plans
     G = (N + 15) // 16

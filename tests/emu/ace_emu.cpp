@@ -133,8 +133,8 @@ void run_lanes(const AceKernelArgs &a, unsigned char *lds, uint32_t lds_bytes) {
 
 // codes: uint8 [G][P][16] (the kernel's layout).  Chooses the kernel variant as the library's launcher does.
 extern "C" int ace_emu_kernel(const ace_tables_t *t, const uint8_t *codes, const uint32_t *hdr, const uint32_t *range,
-                              long long P, double memory_limit, int strict, double *iter_ms, double *peak_mb,
-                              uint8_t *feasible, uint8_t *status, double *stage_out) {
+                              const uint32_t *order /* nullable [P] */, long long P, double memory_limit, int strict,
+                              double *iter_ms, double *peak_mb, uint8_t *feasible, uint8_t *status, double *stage_out) {
     if (range && !stage_out) return -1;
     AceKernelArgs a;
     memset(&a, 0, sizeof(a));
@@ -162,6 +162,7 @@ extern "C" int ace_emu_kernel(const ace_tables_t *t, const uint8_t *codes, const
     a.codes = (const ace_u4 *)pool.place(codes, G * (size_t)P * 16);
     a.hdr = (const ace_u4 *)pool.place(hdr, (size_t)P * 16);
     a.range = range ? (const ace_u2 *)pool.place(range, (size_t)P * 8, 8) : nullptr;
+    a.order = order ? (const uint32_t *)pool.place(order, (size_t)P * 4, 4) : nullptr;
     a.rows = (const double *)pool.place(t->rows, (size_t)t->num_types * t->row_doubles * 8);
     // (the library uploads the num_ops + 1 descriptors into a zeroed array of 16 * G + 16)
     uint32_t *pos = (uint32_t *)pool.place(nullptr, (G * 16 + 16) * 4);
@@ -173,10 +174,10 @@ extern "C" int ace_emu_kernel(const ace_tables_t *t, const uint8_t *codes, const
     a.win_pos = (const int32_t *)pool.place(t->win_pos, (size_t)(t->n_windows + 1) * 4, 4);
     a.win_row_begin = (const int32_t *)pool.place(t->win_row_begin, (size_t)(t->n_windows + 1) * 4, 4);
     a.win_rows = (const uint32_t *)pool.place(t->win_rows, n_win_rows * 8, 4);
-    a.iter_ms = (double *)pool.place(nullptr, (size_t)P * 8, 8);
-    a.peak_mb = (double *)pool.place(nullptr, (size_t)P * 8, 8);
-    a.feasible = (uint8_t *)pool.place(nullptr, (size_t)P, 1);
-    a.status = status ? (uint8_t *)pool.place(nullptr, (size_t)P, 1) : nullptr;
+    a.iter_ms = (double *)pool.place(iter_ms, (size_t)P * 8, 8);
+    a.peak_mb = (double *)pool.place(peak_mb, (size_t)P * 8, 8);
+    a.feasible = (uint8_t *)pool.place(feasible, (size_t)P, 1);
+    a.status = status ? (uint8_t *)pool.place(status, (size_t)P, 1) : nullptr;
     const size_t rec_bytes = (size_t)P * ACE_MAX_STAGES * ACE_STAGE_REC * 8;
     a.stage_out = stage_out ? (double *)pool.place(stage_out, rec_bytes, 8) : nullptr;   // (records of unused stages stay as the caller left them)
     unsigned char *lds = (unsigned char *)pool.place(nullptr, lds_bytes);

@@ -64,6 +64,21 @@ def main(workload, mode, n):
     if mode == "plain":
         assert same(emu_kernel_score(tables, batch), emu_score(tables, batch))
         assert same(emu_kernel_score(tables, batch, strict=True, memory_limit=1.0), emu_score(tables, batch, strict=True, memory_limit=1.0))
+        # plans stored in another order, results in the caller's order (ace_batch_t.d_order)
+        from superscaler_amd.evaluator import depth_order
+        perm = depth_order(batch)
+        assert sorted(perm.tolist()) == list(range(batch.n_plans)) and not np.array_equal(perm, np.arange(batch.n_plans))
+        stored = PlanBatch(np.ascontiguousarray(batch.codes[perm]), np.ascontiguousarray(batch.hdr[perm]))
+        assert same(emu_kernel_score(tables, stored, order=perm), emu_score(tables, batch))
+        assert same(emu_kernel_score(tables, stored, order=perm, breakdown=True), emu_score(tables, batch, breakdown=True))
+        # entries that are no index of the batch: nothing is written for those slots
+        wild = perm.astype(np.uint32).copy()
+        wild[::5] = np.random.default_rng(1).integers(batch.n_plans, 2 ** 32, size=len(wild[::5]), dtype=np.uint64).astype(np.uint32)
+        got, ref = emu_kernel_score(tables, stored, order=wild, breakdown=True), emu_score(tables, batch, breakdown=True)
+        keep = np.ones(batch.n_plans, dtype=bool)
+        keep[perm[::5]] = False
+        assert all(np.array_equal(g[keep], r[keep], equal_nan=True) for g, r in zip(got, ref))
+        assert all(not np.any(g[~keep]) for g in got)
     elif mode == "breakdown":
         assert same(emu_kernel_score(tables, batch, breakdown=True), emu_score(tables, batch, breakdown=True))
     elif mode == "ranged":

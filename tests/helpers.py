@@ -96,7 +96,7 @@ def kernel_layout(codes):
     return np.ascontiguousarray(out.reshape(P, G, 16).transpose(1, 0, 2))
 
 
-def emu_kernel_score(tables, batch, memory_limit=None, strict=False, breakdown=False, ranges=None, raw_codes=None):
+def emu_kernel_score(tables, batch, memory_limit=None, strict=False, breakdown=False, ranges=None, raw_codes=None, order=None):
     """The scoring kernel's own loop (csrc/ace_score_loop.h) on the CPU with guard pages behind every array:
     an out-of-range index ends the process with SIGSEGV, so call this from a child process.
     `raw_codes`: a [G][P][16] array to use as is (e.g. with junk in the padding bytes)."""
@@ -113,8 +113,11 @@ def emu_kernel_score(tables, batch, memory_limit=None, strict=False, breakdown=F
     rec = np.zeros((P, 16, 18)) if breakdown else None
     limit = tables.settings.memory_limit if memory_limit is None else memory_limit
     vp = ctypes.c_void_p
+    if order is not None:
+        order = np.ascontiguousarray(order, dtype=np.uint32)
     rc = lib.ace_emu_kernel(ctypes.byref(ts), codes.ctypes.data_as(vp), hdr.ctypes.data_as(vp),
-                            ranges.ctypes.data_as(vp) if ranges is not None else None, ctypes.c_longlong(P),
+                            ranges.ctypes.data_as(vp) if ranges is not None else None,
+                            order.ctypes.data_as(vp) if order is not None else None, ctypes.c_longlong(P),
                             ctypes.c_double(limit), ctypes.c_int(int(strict)), it.ctypes.data_as(vp), pk.ctypes.data_as(vp),
                             fe.ctypes.data_as(vp), st.ctypes.data_as(vp), rec.ctypes.data_as(vp) if breakdown else None)
     assert rc == 0
@@ -216,8 +219,9 @@ class EmuDeviceEvaluator(EmuEvaluator):
         P, N = dbatch.n_plans, dbatch.num_ops
         stub = PlanBatch(np.zeros((P, N), dtype=np.uint8), dbatch.hdr.numpy().view(np.uint32).copy())
         rg = dbatch.ranges.numpy().view(np.uint32) if dbatch.ranges is not None else None
+        order = dbatch.order.numpy().view(np.uint32) if getattr(dbatch, "order", None) is not None else None
         it, pk, fe, st, rec = emu_kernel_score(self.tables, stub, memory_limit, strict, breakdown, rg,
-                                               raw_codes=dbatch.codes.contiguous().numpy())
+                                               raw_codes=dbatch.codes.contiguous().numpy(), order=order)
         return (torch.from_numpy(it), torch.from_numpy(pk), torch.from_numpy(fe), torch.from_numpy(st),
                 torch.from_numpy(rec) if rec is not None else None)
 

@@ -137,6 +137,31 @@ def test_reference_golden_vectors(name, golden_dir, torch_mod):
     ev.close()
 
 
+def test_grouped_storage_returns_results_in_the_callers_order(torch_mod):
+    """ace_batch_t.d_order: plans stored sorted by depth and first cut score exactly as in their own order,
+    stage records included."""
+    from superscaler_amd.evaluator import PlanEvaluator, depth_order
+    for name, n in (("gpt3_13b", 20000), ("wresnet_1b", 5000), ("t5_770m", 3000)):
+        w = synth.WORKLOADS[name]
+        tables = synth.make_tables(w)
+        batch = synth.make_plans(w, tables, n_plans=n, seed_offset=21)
+        ev = PlanEvaluator(tables)
+        plain = ev.score_host(batch)
+        grouped = ev.score_host(batch, group_by_depth=True)
+        assert all(np.array_equal(a, b, equal_nan=True) for a, b in zip(plain, grouped))
+        small = batch.slice(0, 512)
+        plain = ev.score_host(small, breakdown=True)
+        grouped = ev.score_host(small, breakdown=True, group_by_depth=True)
+        S = small.hdr[:, 0] & 0xff
+        used = np.arange(16)[None, :] < S[:, None]
+        assert all(np.array_equal(a, b, equal_nan=True) for a, b in zip(plain[:4], grouped[:4]))
+        assert np.array_equal(plain[4][used], grouped[4][used], equal_nan=True)
+        d = ev.upload(batch, group_by_depth=True)
+        perm = depth_order(batch)
+        assert np.array_equal(d.order.cpu().numpy(), perm) and not np.array_equal(perm, np.arange(n))
+        ev.close()
+
+
 def test_full_size_properties(torch_mod):
     """GPT-3 13B at the benchmark's full size (1,048,576 plans), which the oracle cannot cover:
     size-independent properties, an oracle spot check and the top-k against a stable sort."""

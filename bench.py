@@ -74,7 +74,7 @@ def main():
                     help="restrict the pipeline depths the plans are drawn from (profiling aid)")
     ap.add_argument("--caller-order", action="store_true",
                     help="keep the plans in the generator's order in HBM instead of grouping them by pipeline "
-                         "depth and first stage boundary at upload (results are in the generator's order either way)")
+                         "depth and first stage boundaries at upload (results are in the generator's order either way)")
     ap.add_argument("--no-layout-comparison", action="store_true",
                     help="do not also time the kernel on the plans in the generator's order (keeps a profiler's "
                          "per-kernel average to the benchmark's own layout)")
@@ -149,7 +149,7 @@ def main():
                                f"memory cap {w.memory_limit:.0f} MB, global batch {w.global_batch}, top-{args.topk}",
                    "step": "score kernel + device-wide top-k, inputs resident in HBM",
                    "layout": ("plans in the generator's order" if args.caller_order else
-                              "plans stored grouped by pipeline depth (deepest first) and first stage boundary, "
+                              "plans stored grouped by pipeline depth (deepest first) and first two stage boundaries, "
                               "grouped once at upload; results and top-k indices in the generator's order"),
                    "feasible_plans": n_feasible, "best_iter_ms": best, "plan_generation_s": round(gen_s, 1)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",

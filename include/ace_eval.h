@@ -126,7 +126,7 @@ typedef struct ace_batch {
                                   d_status, d_stage_out) is written at index d_order[i].  Lets the caller store the
                                   plans in the order that suits the kernel -- lanes of a wavefront that close their
                                   stages at the same ops do not wait for each other, so grouping plans by pipeline
-                                  depth (deepest first) and first stage boundary is worth about a tenth of the
+                                  depth (deepest first) and first stage boundaries is worth about a seventh of the
                                   kernel time on mixed batches -- and still get results in its own order.  Must be
                                   a permutation of 0 .. n_plans - 1 (entries >= n_plans are skipped). */
 } ace_batch_t;

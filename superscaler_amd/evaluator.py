@@ -89,10 +89,16 @@ def _check(lib, rc, what):
 
 def depth_order(batch: PlanBatch) -> np.ndarray:
     """Permutation that sorts the plans by pipeline depth (deepest first: the long jobs start first),
-    then by the position of their first stage boundary (stable)."""
+    then by the positions of their first and second stage boundary (stable)."""
     S = (batch.hdr[:, 0] & 0xff).astype(np.int64)
-    first_cut = ((batch.codes[:, 1:] & 16) != 0).argmax(axis=1) if batch.codes.shape[1] > 1 else np.zeros(len(S), dtype=np.int64)
-    return np.lexsort((first_cut, -S))
+    P, N = batch.codes.shape
+    if N < 2:
+        return np.argsort(-S, kind="stable")
+    cuts = (batch.codes[:, 1:] & 16) != 0
+    c1 = cuts.argmax(axis=1)
+    cuts[np.arange(P), c1] = False
+    c2 = cuts.argmax(axis=1)
+    return np.lexsort((c2, c1, -S))
 
 
 class DeviceBatch:
@@ -104,7 +110,7 @@ class DeviceBatch:
         it and the copy to the device does not block the host (the caller must not reuse the tensor
         before that copy has completed).
         `group_by_depth`: store the plans sorted by pipeline depth (deepest first) and position of the
-        first stage boundary, with the permutation alongside (`order`), so that the lanes of a
+        first two stage boundaries, with the permutation alongside (`order`), so that the lanes of a
         wavefront close their stages together; results still come back in the caller's order."""
         import torch
         self.n_plans = batch.n_plans

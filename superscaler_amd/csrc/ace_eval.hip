@@ -24,6 +24,8 @@ namespace {
 #define ACE_BLOCK 1024
 #endif
 constexpr int kBlock = ACE_BLOCK;        // lanes (= plans) per workgroup: 16 wavefronts, 4 per SIMD
+constexpr int kSmallBlock = 256;         // ... for small batches: 4 wavefronts, 1 per SIMD
+constexpr int kSmallBatchBlocks = 128;   // batches of fewer than this many kBlock workgroups use kSmallBlock
 constexpr uint32_t kMaxLds = 160 * 1024;  // CDNA4 LDS per workgroup
 
 thread_local char g_hip_err[256] = "";
@@ -38,10 +40,14 @@ thread_local char g_hip_err[256] = "";
     } while (0)
 
 // BD / RANGED / WIN / DEFER: see ace_score_body (ace_score_loop.h), which holds the whole kernel.
-template <bool BD, bool RANGED, bool WIN, bool DEFER>
-__global__ __launch_bounds__(kBlock) void ace_score_kernel(const AceKernelArgs a) {
+// BLOCK: kBlock lanes for large batches; kSmallBlock for batches that would otherwise occupy only a
+// few CUs (a workgroup keeps a CU to itself either way: the tables fill its LDS): the walk over the
+// op sequence is sequential per wavefront, so a small batch finishes soonest with one wavefront per
+// SIMD on as many CUs as it can reach.
+template <bool BD, bool RANGED, bool WIN, bool DEFER, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void ace_score_kernel(const AceKernelArgs a) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
-    ace_score_body<BD, RANGED, WIN, DEFER, kBlock>(a, lds_raw, 0u, (int)threadIdx.x, (long long)blockIdx.x, gridDim.x);
+    ace_score_body<BD, RANGED, WIN, DEFER, BLOCK>(a, lds_raw, 0u, (int)threadIdx.x, (long long)blockIdx.x, gridDim.x);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -333,7 +339,9 @@ static int upload(void **dst, const void *src, size_t bytes, size_t alloc_bytes 
 }  // extern "C"
 
 template <bool BD, bool RANGED, bool WIN, bool DEFER> static int allow_big_lds() {
-    ACE_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&ace_score_kernel<BD, RANGED, WIN, DEFER>),
+    ACE_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&ace_score_kernel<BD, RANGED, WIN, DEFER, kBlock>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
+    ACE_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&ace_score_kernel<BD, RANGED, WIN, DEFER, kSmallBlock>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
     return ACE_OK;
 }
@@ -472,21 +480,28 @@ static int fill_args(ace_handle_t *h, const ace_batch_t *b, double memory_limit,
 
 }  // extern "C"
 
-template <bool BD, bool RANGED>
-static void launch_score_w(const ace_handle_t *h, const AceKernelArgs &a, hipStream_t s, unsigned blocks) {
-    if (h->n_windows > 1)
-        hipLaunchKernelGGL((ace_score_kernel<BD, RANGED, true, false>), dim3(blocks), dim3(kBlock), h->lds_bytes, s, a);
+template <bool BD, bool RANGED, bool WIN, bool DEFER>
+static void launch_score_b(const ace_handle_t *h, const AceKernelArgs &a, hipStream_t s) {
+    const size_t P = (size_t)a.g.P;
+    if ((P + kBlock - 1) / kBlock < (size_t)kSmallBatchBlocks)
+        hipLaunchKernelGGL((ace_score_kernel<BD, RANGED, WIN, DEFER, kSmallBlock>), dim3((unsigned)((P + kSmallBlock - 1) / kSmallBlock)),
+                           dim3(kSmallBlock), h->lds_bytes, s, a);
     else
-        hipLaunchKernelGGL((ace_score_kernel<BD, RANGED, false, false>), dim3(blocks), dim3(kBlock), h->lds_bytes, s, a);
+        hipLaunchKernelGGL((ace_score_kernel<BD, RANGED, WIN, DEFER, kBlock>), dim3((unsigned)((P + kBlock - 1) / kBlock)),
+                           dim3(kBlock), h->lds_bytes, s, a);
+}
+
+template <bool BD, bool RANGED>
+static void launch_score_w(const ace_handle_t *h, const AceKernelArgs &a, hipStream_t s) {
+    if (h->n_windows > 1) launch_score_b<BD, RANGED, true, false>(h, a, s);
+    else launch_score_b<BD, RANGED, false, false>(h, a, s);
 }
 
 static void launch_score(const ace_handle_t *h, const AceKernelArgs &a, hipStream_t s) {
-    const unsigned blocks = (unsigned)(((size_t)a.g.P + kBlock - 1) / kBlock);
-    if (a.range) launch_score_w<true, true>(h, a, s, blocks);
-    else if (a.stage_out) launch_score_w<true, false>(h, a, s, blocks);
-    else if (a.stage_ws)
-        hipLaunchKernelGGL((ace_score_kernel<false, false, false, true>), dim3(blocks), dim3(kBlock), h->lds_bytes, s, a);
-    else launch_score_w<false, false>(h, a, s, blocks);
+    if (a.range) launch_score_w<true, true>(h, a, s);
+    else if (a.stage_out) launch_score_w<true, false>(h, a, s);
+    else if (a.stage_ws) launch_score_b<false, false, false, true>(h, a, s);
+    else launch_score_w<false, false>(h, a, s);
 }
 
 // Plain scoring with every row resident uses the deferred-stage-tail kernel, which needs a

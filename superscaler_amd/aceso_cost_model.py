@@ -367,51 +367,31 @@ class CostModel:
 
     def check_recompute(self, ops, base_batch_size, tp_size, dp_size, num_stages_behind, algo_list):
         """Greedy choice of recomputed ops until the stage fits the memory limit
-        (aceso_cost_model.py:822-872).  The loop runs here; stage memory and the saved / peak
-        activations of each trial come from the GPU."""
-        args = self.settings
-        num_ops = len(ops)
-        if not args.flex_recompute:
-            return [1 for _ in range(num_ops)]
-        recompute_ops = [0 for _ in range(num_ops)]
-        stage_memory = self.predict_stage_memory_helper(None, None, ops, recompute_ops, tp_size, dp_size,
-                                                        base_batch_size, num_stages_behind, algo_list)
-        stage_memory += args.peak_mem_in_backward
-        if stage_memory - args.memory_limit <= 0:
-            return recompute_ops
-        op_groups = {}
-        for index in range(num_ops):
-            g = op_groups.setdefault(ops[index], {"index": [], "activation_size": [], "recomputed": False, "sum_size": 0})
-            g["index"].append(index)
-            sz = self.get_activation_size(ops[index], base_batch_size // dp_size[index], tp_size[index],
-                                          algo_list[index]) * (num_stages_behind + 1)
-            g["activation_size"].append(sz)
-            g["sum_size"] += sz
-        initial_saved = 0
-        current_peak = 0        # get_peak_activations of an all-zero recompute list is 0 (:421)
-        while stage_memory - args.memory_limit > 0:
-            idx_group, _ = self._next_recompute_op_group(ops, op_groups, stage_memory - args.memory_limit)
-            if idx_group is None:
+        (aceso_cost_model.py:822-872): check_recompute_batch for one stage."""
+        return self.check_recompute_batch([(ops, base_batch_size, tp_size, dp_size, num_stages_behind, algo_list)])[0]
+
+    @staticmethod
+    def _mark_recompute(rc, idx_group):
+        """aceso_cost_model.py:852-859: the chosen ops and the op after each."""
+        for si in idx_group:
+            if si < 0:
                 break
-            for si in idx_group:
-                if si < 0:
-                    break
-                recompute_ops[si] = 1
-                if si < num_ops - 1:
-                    recompute_ops[si + 1] = 1
-            r = self._stage_records([(ops, recompute_ops, tp_size, dp_size, base_batch_size, num_stages_behind, algo_list)])[0]
-            new_saved, new_peak = float(r[R_SAVED]), float(r[R_PEAK])
-            stage_memory -= (new_saved - initial_saved) * (num_stages_behind + 1)
-            initial_saved = new_saved
-            stage_memory += (new_peak - current_peak)
-            current_peak = new_peak
-        return recompute_ops
+            rc[si] = 1
+            if si < len(rc) - 1:
+                rc[si + 1] = 1
 
     def check_recompute_batch(self, queries):
-        """check_recompute for many stages at once: the greedy passes advance in lockstep and every
-        round costs ONE launch for all stages still above the limit.
-        queries: [(ops, micro_bs, tp_size, dp_size, num_stages_behind, algo_list)]; returns the
-        recompute lists in the same order, identical to check_recompute called one by one."""
+        """check_recompute for many stages at once, identical to calling it one by one.
+        queries: [(ops, micro_bs, tp_size, dp_size, num_stages_behind, algo_list)]; returns the recompute lists.
+
+        Which op group a greedy round takes (:794-806) depends only on the group sums and on which
+        groups earlier rounds took, not on the memory figures; those only decide whether the round
+        takes the whole group or a prefix of it (:809-820) and when the loop stops.  So instead of one
+        launch per round, the states "after the next 1, 2, ... whole groups" of every stage still above
+        the limit are evaluated together in one launch and the reference's bookkeeping (:861-867) is
+        replayed over the records in order; only a round that takes a prefix leaves that chain and
+        asks for another launch.  Three launches are typical where the reference's loop makes a dozen
+        stage evaluations."""
         args = self.settings
         n = len(queries)
         if not args.flex_recompute:
@@ -419,13 +399,20 @@ class CostModel:
         rcs = [[0] * len(q[0]) for q in queries]
         if n == 0:
             return rcs
-        rec = self._stage_records([(q[0], rcs[k], q[2], q[3], q[1], q[4], q[5]) for k, q in enumerate(queries)])
-        state = []
+        limit = args.memory_limit
+
+        def query(k, rc):
+            q = queries[k]
+            return (q[0], rc, q[2], q[3], q[1], q[4], q[5])
+
+        rec = self._stage_records([query(k, rcs[k]) for k in range(n)])
+        state, pending = [], []
         for k, (ops, micro_bs, tp_size, dp_size, nsb, algo_list) in enumerate(queries):
             mw, mg, mo, ma, mp, mr = self._memory_breakdown([float(x) for x in rec[k]], nsb)
             stage_memory = (mw + mg + mo + ma + mp + mr) + args.peak_mem_in_backward
-            st = {"mem": stage_memory, "saved": 0, "peak": 0, "groups": None, "active": stage_memory - args.memory_limit > 0}
-            if st["active"]:
+            # get_peak_activations of an all-zero recompute list is 0 (:421)
+            st = {"mem": stage_memory, "saved": 0, "peak": 0, "groups": None, "stale": False}
+            if stage_memory - limit > 0:
                 groups = {}
                 for index in range(len(ops)):
                     g = groups.setdefault(ops[index], {"index": [], "activation_size": [], "recomputed": False, "sum_size": 0})
@@ -435,43 +422,81 @@ class CostModel:
                     g["activation_size"].append(sz)
                     g["sum_size"] += sz
                 st["groups"] = groups
+                pending.append(k)
             state.append(st)
-        while True:
-            todo = []
-            for k, st in enumerate(state):
-                if not st["active"]:
-                    continue
-                ops = queries[k][0]
-                idx_group, _ = self._next_recompute_op_group(ops, st["groups"], st["mem"] - args.memory_limit)
-                if idx_group is None:
-                    st["active"] = False
-                    continue
-                for si in idx_group:
-                    if si < 0:
+
+        def account(st, r, nsb):
+            new_saved, new_peak = float(r[R_SAVED]), float(r[R_PEAK])
+            st["mem"] -= (new_saved - st["saved"]) * (nsb + 1)
+            st["saved"] = new_saved
+            st["mem"] += (new_peak - st["peak"])
+            st["peak"] = new_peak
+
+        while pending:
+            launch, plan = [], {}
+            for k in pending:
+                st, ops = state[k], queries[k][0]
+                states = [list(rcs[k])] if st["stale"] else []       # a prefix round: its own state is not evaluated yet
+                # the whole-group rounds that would follow, on a copy of the "taken" marks
+                trial = {name: dict(g) for name, g in st["groups"].items()}
+                cur, chain, gain = list(rcs[k]), [], 0.0
+                want = st["mem"] - limit
+                while True:
+                    idx, sizes = self._next_recompute_op_group(ops, trial, math.inf)
+                    if idx is None:
                         break
-                    rcs[k][si] = 1
-                    if si < len(ops) - 1:
-                        rcs[k][si + 1] = 1
-                todo.append(k)
-            if not todo:
-                return rcs
-            rec = self._stage_records([(queries[k][0], rcs[k], queries[k][2], queries[k][3], queries[k][1],
-                                        queries[k][4], queries[k][5]) for k in todo])
-            for j, k in enumerate(todo):
-                st, nsb = state[k], queries[k][4]
-                new_saved, new_peak = float(rec[j, R_SAVED]), float(rec[j, R_PEAK])
-                st["mem"] -= (new_saved - st["saved"]) * (nsb + 1)
-                st["saved"] = new_saved
-                st["mem"] += (new_peak - st["peak"])
-                st["peak"] = new_peak
-                st["active"] = st["mem"] - args.memory_limit > 0
+                    cur = list(cur)
+                    self._mark_recompute(cur, idx)
+                    chain.append(len(idx))
+                    states.append(cur)
+                    gain += sum(sizes)
+                    # enough groups to get below the limit by their own sizes; after a prefix round (whose
+                    # effect is not known yet) the loop mostly ends, so one group ahead; a later launch continues if needed
+                    if st["stale"] or gain > want or len(chain) >= 16:
+                        break
+                plan[k] = (len(launch), chain, int(st["stale"]))
+                launch.extend(query(k, rc) for rc in states)
+            rec = self._stage_records(launch) if launch else np.zeros((0, STAGE_REC))
+            again = []
+            for k in pending:
+                st, ops, nsb = state[k], queries[k][0], queries[k][4]
+                base, chain, off = plan[k]
+                if st["stale"]:
+                    account(st, rec[base], nsb)
+                    st["stale"] = False
+                j = 0
+                while st["mem"] - limit > 0:
+                    if j >= len(chain):
+                        again.append(k)          # the evaluated chain is used up (or there was none): next launch
+                        break
+                    idx_group, _ = self._next_recompute_op_group(ops, st["groups"], st["mem"] - limit)
+                    if idx_group is None:
+                        break
+                    self._mark_recompute(rcs[k], idx_group)
+                    if len(idx_group) == chain[j]:
+                        account(st, rec[base + off + j], nsb)
+                        j += 1
+                    else:
+                        st["stale"] = True           # a prefix of the group: a state no launch has seen
+                        again.append(k)
+                        break
+            # a stage whose chain was empty has no group left: _next_recompute_op_group returned None above
+            pending = [k for k in again if state[k]["stale"] or self._has_open_group(queries[k][0], state[k]["groups"])]
+        return rcs
+
+    def _has_open_group(self, ops, groups) -> bool:
+        """Whether _next_recompute_op_group would still return a group."""
+        trial = {name: dict(g) for name, g in groups.items()}
+        return self._next_recompute_op_group(ops, trial, math.inf)[0] is not None
 
     def update_recompute(self, config, stage_idx=None):
-        """aceso_cost_model.py:874-883."""
-        for k in ([stage_idx] if stage_idx is not None else range(config.num_stages)):
-            st = config.stages[k]
-            st.recompute_ops = self.check_recompute(st.ops, config.micro_bs, st.tp_size, st.dp_size,
-                                                    st.num_stages_behind, st.algo)
+        """aceso_cost_model.py:874-883 (the stages are independent: all of them go through one
+        check_recompute_batch)."""
+        stages = [config.stages[k] for k in ([stage_idx] if stage_idx is not None else range(config.num_stages))]
+        rcs = self.check_recompute_batch([(st.ops, config.micro_bs, st.tp_size, st.dp_size, st.num_stages_behind, st.algo)
+                                          for st in stages])
+        for st, rc in zip(stages, rcs):
+            st.recompute_ops = rc
 
     def update_recompute_batch(self, configs) -> None:
         """update_recompute(config) for every stage of every plan, in lockstep on the GPU."""

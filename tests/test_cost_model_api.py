@@ -126,6 +126,41 @@ def test_recompute_arrays_match_the_staged_loop(name, limit):
     assert rounds > 10, "the limit should force partial recomputation in many stages"
 
 
+@pytest.mark.parametrize("name,limits", [("gpt3_1_3b", (20000.0, 9000.0, 3000.0)), ("wresnet_1b", (4000.0, 1500.0, 600.0)),
+                                         ("gpt3_13b", (60000.0, 30000.0))])
+def test_check_recompute_equals_the_oracles_loop(name, limits):
+    """check_recompute evaluates several greedy rounds ahead in one launch and replays the reference's
+    bookkeeping over the records; the oracle runs the reference's loop round by round.  Limits from
+    mild (few whole groups) to harsh (every group, prefixes, stages that cannot be brought under it)."""
+    import dataclasses
+    from superscaler_amd import synth
+    from tests.helpers import oracle_for
+    w = synth.WORKLOADS[name]
+    graph = synth.make_graph(w)
+    launches = 0
+    for limit in limits:
+        st = dataclasses.replace(synth.make_settings(w), memory_limit=limit)
+        m = acm.CostModel(st, synth.make_db(w, graph), graph)
+        ev = EmuEvaluator(m.tables)
+        calls = []
+        score = ev.score_host
+        ev.score_host = lambda *a, **k: (calls.append(1), score(*a, **k))[1]
+        m._evaluator = ev
+        orc = oracle_for(m.tables)
+        batch = synth.make_plans(w, m.tables, n_plans=6, seed_offset=31)
+        kinds = set()
+        for k in range(batch.n_plans):
+            c = batch.to_config(k, m.tables)
+            qs = [(s.ops, c.micro_bs, s.tp_size, s.dp_size, s.num_stages_behind, s.algo) for s in c.stages]
+            want = [orc.check_recompute(*q) for q in qs]
+            assert m.check_recompute_batch(qs) == want
+            assert [m.check_recompute(*q) for q in qs[:2]] == want[:2]
+            kinds |= {"none" if not any(r) else "all" if all(r) else "some" for r in want}
+        launches += len(calls)
+        assert "some" in kinds or "all" in kinds
+    assert launches > 0
+
+
 @pytest.mark.parametrize("case", CASES)
 def test_api_matches_reference_emu(golden_dir, case):
     g, m = make_model(golden_dir, case, "emu")

@@ -87,18 +87,41 @@ def _check(lib, rc, what):
         raise AceError(f"{what}: {msg}" + (f" ({hip})" if hip and rc == -3 else ""))
 
 
+WAVE = 64            # lanes of a wavefront
+WAVES_PER_GROUP = 16  # wavefronts of the scoring kernel's large workgroup
+
+
 def depth_order(batch: PlanBatch) -> np.ndarray:
-    """Permutation that sorts the plans by pipeline depth (deepest first: the long jobs start first),
-    then by the positions of their first and second stage boundary (stable)."""
+    """Storage order for a batch: perm[i] = the caller's index of the plan stored in slot i.
+    The plans are sorted by pipeline depth and by the positions of their first two stage boundaries
+    (plans that close their stages at the same ops sit in one wavefront), cut into wavefronts of 64,
+    and the wavefronts are dealt round-robin to the workgroups, so that every workgroup (every CU)
+    gets the same mix of deep and shallow wavefronts."""
     S = (batch.hdr[:, 0] & 0xff).astype(np.int64)
     P, N = batch.codes.shape
     if N < 2:
-        return np.argsort(-S, kind="stable")
-    cuts = (batch.codes[:, 1:] & 16) != 0
-    c1 = cuts.argmax(axis=1)
-    cuts[np.arange(P), c1] = False
-    c2 = cuts.argmax(axis=1)
-    return np.lexsort((c2, c1, -S))
+        perm = np.argsort(-S, kind="stable")
+    else:
+        cuts = (batch.codes[:, 1:] & 16) != 0
+        c1 = cuts.argmax(axis=1)
+        cuts[np.arange(P), c1] = False
+        c2 = cuts.argmax(axis=1)
+        perm = np.lexsort((c2, c1, -S))
+    full = P // WAVE
+    groups = (full + WAVES_PER_GROUP - 1) // WAVES_PER_GROUP
+    if groups > 1:
+        # workgroup b takes the sorted wavefronts b, b + groups, b + 2 * groups, ...
+        chunk = np.arange(full)
+        snake = np.array([0, 1, 2, 3, 7, 6, 5, 4, 8, 9, 10, 11, 15, 14, 13, 12])
+        dealt = []
+        for b in range(groups):
+            mine = chunk[b::groups]                       # deepest ... shallowest of this workgroup
+            # wavefront w of a workgroup runs on SIMD w % 4: boustrophedon, so the four SIMDs get equal shares too
+            dealt.append(mine[snake[snake < len(mine)]] if len(mine) == WAVES_PER_GROUP else mine)
+        dealt = np.concatenate(dealt)
+        head = perm[:full * WAVE].reshape(full, WAVE)[dealt].reshape(-1)
+        perm = np.concatenate([head, perm[full * WAVE:]])
+    return perm
 
 
 class DeviceBatch:

@@ -183,6 +183,20 @@ int ace_apply_moves(const uint8_t *d_template_codes, const uint32_t *d_template_
                     const uint32_t *d_moves, size_t n_moves, int num_ops, int n_algo, uint8_t *d_codes_out,
                     uint32_t *d_hdr_out, uint64_t *d_keys_out, void *stream);
 
+/* Sort keys for grouped storage (ace_batch_t.d_order) of a batch that is already on the device: d_keys[i]
+ * (uint64[n_plans]) orders the plans by pipeline depth, deepest first, then by the positions of their first two
+ * stage boundaries.  The caller sorts the keys (stably), deals the sorted wavefronts of 64 to the workgroups and
+ * gathers d_codes / d_hdr into that order (superscaler_amd/evaluator.py: PlanEvaluator.group shows how).
+ * d_codes: uint8[ceil(num_ops / 16)][n_plans][16], d_hdr: uint32[n_plans][4] as in ace_batch_t.
+ * No counterpart in the reference, which scores one plan at a time. */
+int ace_group_keys(const uint8_t *d_codes, const uint32_t *d_hdr, size_t n_plans, int num_ops, uint64_t *d_keys, void *stream);
+
+/* Reorder a device-resident batch: slot i of the output holds plan d_perm[i] (uint32[n_plans]) of the input; the
+ * same d_perm is then the d_order of the output batch.  Input and output must not overlap.
+ * No counterpart in the reference. */
+int ace_gather_plans(const uint8_t *d_codes_in, const uint32_t *d_hdr_in, const uint32_t *d_perm, size_t n_plans, int num_ops,
+                     uint8_t *d_codes_out, uint32_t *d_hdr_out, void *stream);
+
 /* The two steps of check_recompute's greedy loop (aceso_cost_model.py:822-872) that are not a stage
  * evaluation, for many encoded stages at once (one stage = the ops [lo, hi) of one plan of the batch).
  * The caller runs the loop: evaluate the stages (ace_score_batch with d_range), update their memory

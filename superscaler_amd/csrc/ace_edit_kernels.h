@@ -175,3 +175,39 @@ ACE_HD void rc_select_body(int a, RcTables t, uint8_t *codes_rw, int n, const in
         if (i + 1 < hi) codes_rw[(((size_t)((i + 1) >> 4)) * t.P + plan) * 16 + ((i + 1) & 15)] |= 8u;
     }
 }
+
+// ------------------------------------------------------------------------------------------
+// Sort key of a plan for grouped storage (ace_batch_t.d_order): pipeline depth (deepest first),
+// then the positions of its first two stage boundaries.  One work item per plan.
+// ------------------------------------------------------------------------------------------
+ACE_HD void group_keys_body(unsigned long long p, const ace_u4 *codes, const ace_u4 *hdr, unsigned long long n, int G, int N,
+                            unsigned long long *keys) {
+    if (p >= n) return;
+    const uint32_t S = hdr[p].x & 0xffu;
+    uint32_t cut[2] = {0u, 0u};
+    int found = 0;
+    for (int g = 0; g < G && found < 2; ++g) {
+        const ace_u4 w = codes[(size_t)g * n + p];
+        const uint32_t words[4] = {w.x, w.y, w.z, w.w};
+        for (int k = 0; k < 16 && found < 2; ++k) {
+            const int i = g * 16 + k;
+            if (i == 0 || i >= N) continue;                 // (the first op opens stage 0; padding bytes do not count)
+            if ((words[k >> 2] >> (8 * (k & 3))) & 0x10u) cut[found++] = (uint32_t)i;
+        }
+    }
+    // (positions are below 2^20: move descriptors and the kernels' range checks keep N under 65536 * 16)
+    keys[p] = ((unsigned long long)(255u - S) << 40) | ((unsigned long long)(cut[0] & 0xfffffu) << 20) | (cut[1] & 0xfffffu);
+}
+
+// Reorder a batch: slot i of the output holds plan perm[i] of the input.  One work item per 16-byte
+// word (16 ops of one plan); consecutive items write consecutive words.
+ACE_HD void gather_plans_body(unsigned long long id, const ace_u4 *codes_in, const ace_u4 *hdr_in, const uint32_t *perm,
+                              unsigned long long n, int G, ace_u4 *codes_out, ace_u4 *hdr_out) {
+    if (id >= n * (unsigned long long)G) return;
+    const unsigned long long i = id % n;
+    const int g = (int)(id / n);
+    unsigned long long src = perm[i];
+    if (src >= n) src = i;                        // (not a permutation entry: the plan stays where it is)
+    codes_out[(size_t)g * n + i] = codes_in[(size_t)g * n + src];
+    if (g == 0) hdr_out[i] = hdr_in[src];
+}

@@ -294,6 +294,16 @@ __global__ __launch_bounds__(256) void apply_moves_kernel(const ace_u4 *tmpl_cod
                      codes_out, hdr_out, key_out);
 }
 
+__global__ __launch_bounds__(256) void group_keys_kernel(const ace_u4 *codes, const ace_u4 *hdr, unsigned long long n, int G, int N,
+                                                         unsigned long long *keys) {
+    group_keys_body((unsigned long long)blockIdx.x * 256 + threadIdx.x, codes, hdr, n, G, N, keys);
+}
+
+__global__ __launch_bounds__(256) void gather_plans_kernel(const ace_u4 *codes_in, const ace_u4 *hdr_in, const uint32_t *perm,
+                                                           unsigned long long n, int G, ace_u4 *codes_out, ace_u4 *hdr_out) {
+    gather_plans_body((unsigned long long)blockIdx.x * 256 + threadIdx.x, codes_in, hdr_in, perm, n, G, codes_out, hdr_out);
+}
+
 __global__ void rc_groups_kernel(RcTables t, int n, const int32_t *q_plan, const int32_t *q_lo, const int32_t *q_hi,
                                  const int32_t *q_nsb, const uint32_t *q_mrow, double *sum_size, int32_t *first_pos,
                                  int32_t *bad) {
@@ -619,6 +629,35 @@ int ace_apply_moves(const uint8_t *d_template_codes, const uint32_t *d_template_
                        n_templates, reinterpret_cast<const ace_u4 *>(d_moves), (unsigned long long)n_moves, G,
                        n_algo == 2 ? 1 : 0, reinterpret_cast<ace_u4 *>(d_codes_out), reinterpret_cast<ace_u4 *>(d_hdr_out),
                        reinterpret_cast<unsigned long long *>(d_keys_out));
+    ACE_HIP(hipGetLastError());
+    return ACE_OK;
+}
+
+int ace_group_keys(const uint8_t *d_codes, const uint32_t *d_hdr, size_t n_plans, int num_ops, uint64_t *d_keys, void *stream) {
+    if (!d_codes || !d_hdr || !d_keys || n_plans == 0 || n_plans > 0x7fffffffull || num_ops <= 0 || num_ops >= (1 << 20)) return ACE_EINVAL;
+    if (((uintptr_t)d_codes & 15u) || ((uintptr_t)d_hdr & 15u) || ((uintptr_t)d_keys & 7u)) return ACE_EINVAL;
+    const int G = (num_ops + 15) / 16;
+    hipLaunchKernelGGL(group_keys_kernel, dim3((unsigned)((n_plans + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       reinterpret_cast<const ace_u4 *>(d_codes), reinterpret_cast<const ace_u4 *>(d_hdr),
+                       (unsigned long long)n_plans, G, num_ops, reinterpret_cast<unsigned long long *>(d_keys));
+    ACE_HIP(hipGetLastError());
+    return ACE_OK;
+}
+
+int ace_gather_plans(const uint8_t *d_codes_in, const uint32_t *d_hdr_in, const uint32_t *d_perm, size_t n_plans, int num_ops,
+                     uint8_t *d_codes_out, uint32_t *d_hdr_out, void *stream) {
+    if (!d_codes_in || !d_hdr_in || !d_perm || !d_codes_out || !d_hdr_out || n_plans == 0 || n_plans > 0x7fffffffull ||
+        num_ops <= 0 || num_ops >= (1 << 20) || d_codes_in == d_codes_out || d_hdr_in == d_hdr_out)
+        return ACE_EINVAL;
+    if (((uintptr_t)d_codes_in & 15u) || ((uintptr_t)d_hdr_in & 15u) || ((uintptr_t)d_codes_out & 15u) ||
+        ((uintptr_t)d_hdr_out & 15u) || ((uintptr_t)d_perm & 3u))
+        return ACE_EINVAL;
+    const int G = (num_ops + 15) / 16;
+    const unsigned long long blocks = ((unsigned long long)n_plans * G + 255) / 256;
+    if (blocks > 0x7fffffffull) return ACE_ETOOBIG;
+    hipLaunchKernelGGL(gather_plans_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       reinterpret_cast<const ace_u4 *>(d_codes_in), reinterpret_cast<const ace_u4 *>(d_hdr_in), d_perm,
+                       (unsigned long long)n_plans, G, reinterpret_cast<ace_u4 *>(d_codes_out), reinterpret_cast<ace_u4 *>(d_hdr_out));
     ACE_HIP(hipGetLastError());
     return ACE_OK;
 }

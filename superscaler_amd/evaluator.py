@@ -17,7 +17,7 @@ _lib = None
 
 EXPORTS = ["ace_abi_version", "ace_strerror", "ace_last_hip_error", "ace_create", "ace_destroy",
            "ace_score_batch", "ace_topk_workspace_bytes", "ace_topk", "ace_time_score_kernel", "ace_apply_moves",
-           "ace_recompute_groups", "ace_recompute_select"]
+           "ace_recompute_groups", "ace_recompute_select", "ace_group_keys", "ace_gather_plans"]
 
 
 class AceBatchStruct(ctypes.Structure):
@@ -69,6 +69,10 @@ def load_library():
     lib.ace_apply_moves.restype = ctypes.c_int
     lib.ace_apply_moves.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t,
                                     ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    lib.ace_group_keys.restype = ctypes.c_int
+    lib.ace_group_keys.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    lib.ace_gather_plans.restype = ctypes.c_int
+    lib.ace_gather_plans.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_size_t, ctypes.c_int] + [ctypes.c_void_p] * 3
     lib.ace_recompute_groups.restype = ctypes.c_int
     lib.ace_recompute_groups.argtypes = [ctypes.POINTER(AceRcTablesStruct), ctypes.c_int] + [ctypes.c_void_p] * 9
     lib.ace_recompute_select.restype = ctypes.c_int
@@ -89,39 +93,46 @@ def _check(lib, rc, what):
 
 WAVE = 64            # lanes of a wavefront
 WAVES_PER_GROUP = 16  # wavefronts of the scoring kernel's large workgroup
+_SNAKE = np.array([0, 1, 2, 3, 7, 6, 5, 4, 8, 9, 10, 11, 15, 14, 13, 12])
+
+
+def deal_slots(n_plans: int) -> np.ndarray:
+    """For a batch sorted from deep to shallow: which sorted position goes into each storage slot.
+    The sorted plans are cut into wavefronts of 64 and the wavefronts are dealt round-robin to the
+    workgroups of 16, so that every workgroup (every CU) gets the same mix of deep and shallow
+    wavefronts; inside a workgroup they are laid out boustrophedon, because wavefront w runs on SIMD
+    w % 4 and the four SIMDs should get equal shares too.  The last n_plans % 64 plans keep their place."""
+    full = n_plans // WAVE
+    groups = (full + WAVES_PER_GROUP - 1) // WAVES_PER_GROUP
+    chunk = np.arange(full)
+    if groups > 1:
+        dealt = []
+        for b in range(groups):
+            mine = chunk[b::groups]                       # deepest ... shallowest wavefront of this workgroup
+            dealt.append(mine[_SNAKE] if len(mine) == WAVES_PER_GROUP else mine)
+        chunk = np.concatenate(dealt)
+    slots = (chunk[:, None] * WAVE + np.arange(WAVE)[None, :]).reshape(-1)
+    return np.concatenate([slots, np.arange(full * WAVE, n_plans)])
 
 
 def depth_order(batch: PlanBatch) -> np.ndarray:
-    """Storage order for a batch: perm[i] = the caller's index of the plan stored in slot i.
-    The plans are sorted by pipeline depth and by the positions of their first two stage boundaries
-    (plans that close their stages at the same ops sit in one wavefront), cut into wavefronts of 64,
-    and the wavefronts are dealt round-robin to the workgroups, so that every workgroup (every CU)
-    gets the same mix of deep and shallow wavefronts."""
+    """Storage order for a batch: perm[i] = the caller's index of the plan stored in slot i.  The plans
+    are sorted (stably) by pipeline depth, deepest first, and by the positions of their first two
+    stage boundaries, so that plans that close their stages at the same ops share a wavefront; the
+    wavefronts are then dealt to the workgroups (deal_slots)."""
     S = (batch.hdr[:, 0] & 0xff).astype(np.int64)
     P, N = batch.codes.shape
     if N < 2:
         perm = np.argsort(-S, kind="stable")
     else:
         cuts = (batch.codes[:, 1:] & 16) != 0
-        c1 = cuts.argmax(axis=1)
-        cuts[np.arange(P), c1] = False
-        c2 = cuts.argmax(axis=1)
+        c1 = cuts.argmax(axis=1) + 1
+        c1[~cuts.any(axis=1)] = 0
+        cuts[np.arange(P), c1 - 1] &= (c1 == 0)
+        c2 = cuts.argmax(axis=1) + 1
+        c2[~cuts.any(axis=1)] = 0
         perm = np.lexsort((c2, c1, -S))
-    full = P // WAVE
-    groups = (full + WAVES_PER_GROUP - 1) // WAVES_PER_GROUP
-    if groups > 1:
-        # workgroup b takes the sorted wavefronts b, b + groups, b + 2 * groups, ...
-        chunk = np.arange(full)
-        snake = np.array([0, 1, 2, 3, 7, 6, 5, 4, 8, 9, 10, 11, 15, 14, 13, 12])
-        dealt = []
-        for b in range(groups):
-            mine = chunk[b::groups]                       # deepest ... shallowest of this workgroup
-            # wavefront w of a workgroup runs on SIMD w % 4: boustrophedon, so the four SIMDs get equal shares too
-            dealt.append(mine[snake[snake < len(mine)]] if len(mine) == WAVES_PER_GROUP else mine)
-        dealt = np.concatenate(dealt)
-        head = perm[:full * WAVE].reshape(full, WAVE)[dealt].reshape(-1)
-        perm = np.concatenate([head, perm[full * WAVE:]])
-    return perm
+    return perm[deal_slots(P)]
 
 
 class DeviceBatch:
@@ -199,6 +210,7 @@ class PlanEvaluator:
             h = ctypes.c_void_p()
             _check(self.lib, self.lib.ace_create(ctypes.byref(ts), ctypes.byref(h)), "ace_create")
         self.handle = h
+        self._deal_cache = {}
         self._topk_ws = None
 
     def close(self):
@@ -372,6 +384,31 @@ class PlanEvaluator:
         G, P, _ = d.codes.shape
         codes = d.codes.permute(1, 0, 2).reshape(P, G * 16)[:, :d.num_ops].contiguous().cpu().numpy()
         return PlanBatch(codes, d.hdr.cpu().numpy().view(np.uint32).copy())
+
+    def group(self, d: DeviceBatch) -> DeviceBatch:
+        """A copy of a device-resident batch in grouped storage order (see DeviceBatch), made on the
+        device: sort keys from the library (ace_group_keys), a stable sort, one gather of the plan
+        bytes.  Worth it for a batch that is scored more than once; results of the copy come back in the
+        order of `d`.  Equal to upload(batch, group_by_depth=True) of the same plans."""
+        torch = self._torch
+        if d.order is not None or d.ranges is not None:
+            raise ValueError("group: a plain batch in its own order is expected")
+        P = d.n_plans
+        keys = torch.empty(P, dtype=torch.int64, device=self.device)
+        with self.device_context():
+            _check(self.lib, self.lib.ace_group_keys(d.codes.data_ptr(), d.hdr.data_ptr(), P, d.num_ops, keys.data_ptr(),
+                                                     self._stream()), "ace_group_keys")
+        by_key = torch.sort(keys, stable=True).indices       # (keys are below 2^48: signed order = unsigned order)
+        slots = self._deal_cache.get(P)
+        if slots is None:
+            slots = torch.from_numpy(deal_slots(P)).to(self.device)
+            self._deal_cache = {P: slots}
+        perm = by_key.index_select(0, slots).to(torch.int32)
+        codes, hdr = torch.empty_like(d.codes), torch.empty_like(d.hdr)
+        with self.device_context():
+            _check(self.lib, self.lib.ace_gather_plans(d.codes.data_ptr(), d.hdr.data_ptr(), perm.data_ptr(), P, d.num_ops,
+                                                       codes.data_ptr(), hdr.data_ptr(), self._stream()), "ace_gather_plans")
+        return DeviceBatch.from_device(codes, hdr, d.num_ops, order=perm)
 
     def stage_records_host(self, batch: PlanBatch, ranges: np.ndarray):
         """Single-stage queries: (status, stage record 0 of every query) as numpy arrays."""

@@ -290,3 +290,33 @@ extern "C" int ace_emu_rc_select(const ace_rc_tables_t *t, uint8_t *codes_rw, in
     memcpy(alive, al, (size_t)n);
     return 0;
 }
+
+extern "C" int ace_emu_group_keys(const uint8_t *codes /* [G][P][16] */, const uint32_t *hdr, long long n, int num_ops,
+                                  unsigned long long *keys) {
+    GuardedPool pool;
+    const int G = (num_ops + 15) / 16;
+    const ace_u4 *c = (const ace_u4 *)pool.place(codes, (size_t)G * n * 16);
+    const ace_u4 *h = (const ace_u4 *)pool.place(hdr, (size_t)n * 16);
+    unsigned long long *k = (unsigned long long *)pool.place(nullptr, (size_t)n * 8, 8);
+    for (unsigned long long p = 0; p < ((unsigned long long)n + 255) / 256 * 256; ++p)
+        group_keys_body(p, c, h, (unsigned long long)n, G, num_ops, k);
+    memcpy(keys, k, (size_t)n * 8);
+    return 0;
+}
+
+extern "C" int ace_emu_gather_plans(const uint8_t *codes_in, const uint32_t *hdr_in, const uint32_t *perm, long long n, int num_ops,
+                                    uint8_t *codes_out, uint32_t *hdr_out) {
+    GuardedPool pool;
+    const int G = (num_ops + 15) / 16;
+    const ace_u4 *ci = (const ace_u4 *)pool.place(codes_in, (size_t)G * n * 16);
+    const ace_u4 *hi = (const ace_u4 *)pool.place(hdr_in, (size_t)n * 16);
+    const uint32_t *pm = (const uint32_t *)pool.place(perm, (size_t)n * 4, 4);
+    ace_u4 *co = (ace_u4 *)pool.place(nullptr, (size_t)G * n * 16);
+    ace_u4 *ho = (ace_u4 *)pool.place(nullptr, (size_t)n * 16);
+    const unsigned long long total = ((unsigned long long)n * G + 255) / 256 * 256;
+    for (unsigned long long id = 0; id < total; ++id) gather_plans_body(id, ci, hi, pm, (unsigned long long)n, G, co, ho);
+    memcpy(codes_out, co, (size_t)G * n * 16);
+    memcpy(hdr_out, ho, (size_t)n * 16);
+    return 0;
+}
+

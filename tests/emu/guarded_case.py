@@ -71,6 +71,30 @@ def main(workload, mode, n):
         stored = PlanBatch(np.ascontiguousarray(batch.codes[perm]), np.ascontiguousarray(batch.hdr[perm]))
         assert same(emu_kernel_score(tables, stored, order=perm), emu_score(tables, batch))
         assert same(emu_kernel_score(tables, stored, order=perm, breakdown=True), emu_score(tables, batch, breakdown=True))
+        # the device's sort keys (ace_group_keys) give the same order
+        import ctypes
+        from superscaler_amd.evaluator import deal_slots
+        from tests.helpers import emu_lib
+        keys = np.zeros(batch.n_plans, dtype=np.uint64)
+        raw = kernel_layout(batch.codes)
+        hdr32 = np.ascontiguousarray(batch.hdr)
+        assert emu_lib().ace_emu_group_keys(ctypes.c_void_p(raw.ctypes.data), ctypes.c_void_p(hdr32.ctypes.data),
+                                            ctypes.c_longlong(batch.n_plans), ctypes.c_int(batch.num_ops),
+                                            ctypes.c_void_p(keys.ctypes.data)) == 0
+        assert np.array_equal(np.argsort(keys, kind="stable")[deal_slots(batch.n_plans)], perm)
+        # ... and the gather puts the plans into that order (entries that are no index: the plan stays)
+        co, ho = np.zeros_like(raw), np.zeros_like(hdr32)
+        p32 = perm.astype(np.uint32)
+        vp = ctypes.c_void_p
+        assert emu_lib().ace_emu_gather_plans(vp(raw.ctypes.data), vp(hdr32.ctypes.data), vp(p32.ctypes.data),
+                                              ctypes.c_longlong(batch.n_plans), ctypes.c_int(batch.num_ops),
+                                              vp(co.ctypes.data), vp(ho.ctypes.data)) == 0
+        assert np.array_equal(co, kernel_layout(stored.codes)) and np.array_equal(ho, stored.hdr)
+        p32[::7] = 0xfffffff0
+        assert emu_lib().ace_emu_gather_plans(vp(raw.ctypes.data), vp(hdr32.ctypes.data), vp(p32.ctypes.data),
+                                              ctypes.c_longlong(batch.n_plans), ctypes.c_int(batch.num_ops),
+                                              vp(co.ctypes.data), vp(ho.ctypes.data)) == 0
+        assert np.array_equal(ho[::7], hdr32[::7])
         # entries that are no index of the batch: nothing is written for those slots
         wild = perm.astype(np.uint32).copy()
         wild[::5] = np.random.default_rng(1).integers(batch.n_plans, 2 ** 32, size=len(wild[::5]), dtype=np.uint64).astype(np.uint32)

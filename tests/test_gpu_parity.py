@@ -159,6 +159,12 @@ def test_grouped_storage_returns_results_in_the_callers_order(torch_mod):
         d = ev.upload(batch, group_by_depth=True)
         perm = depth_order(batch)
         assert np.array_equal(d.order.cpu().numpy(), perm) and not np.array_equal(perm, np.arange(n))
+        # the same grouping made on the device from a plain upload
+        g = ev.group(ev.upload(batch))
+        assert np.array_equal(g.order.cpu().numpy(), perm)
+        assert torch_mod.equal(g.codes, d.codes) and torch_mod.equal(g.hdr, d.hdr)
+        it, pk, fe, st = ev.score(g)
+        assert all(np.array_equal(a, b.cpu().numpy(), equal_nan=True) for a, b in zip(ev.score_host(batch), (it, pk, fe, st)))
         ev.close()
 
 

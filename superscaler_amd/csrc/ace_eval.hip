@@ -683,7 +683,8 @@ int ace_recompute_select(const ace_rc_tables_t *t, uint8_t *d_codes_rw, int n_st
                          double memory_limit, uint8_t *d_alive, void *stream) {
     if (!t || !d_codes_rw || n_stages <= 0 || !d_plan || !d_lo || !d_hi || !d_nsb || !d_mrow || !d_sum_size ||
         !d_first_pos || !d_recomputed || !d_mem || !d_alive || !t->d_codes || !t->d_type_of_pos || !t->d_activations ||
-        !t->d_no_recompute || t->num_ops <= 0 || t->num_types <= 0 || t->n_plans == 0)
+        !t->d_no_recompute || t->num_ops <= 0 || t->num_types <= 0 || t->n_tp <= 0 || t->n_tp > 4 ||
+        (t->n_algo != 1 && t->n_algo != 2) || t->n_mbs <= 0 || t->n_mbs > 15 || t->n_plans == 0)
         return ACE_EINVAL;
     RcTables k{t->d_codes, (unsigned long long)t->n_plans, t->d_type_of_pos, t->d_activations, t->d_no_recompute,
                t->num_ops, t->num_types, t->n_mbs, t->n_tp, t->n_algo, t->n_algo == 2 ? 1 : 0};

@@ -164,6 +164,8 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
     double id_fwd, id_bwd;
     bool lastclose;
     uint32_t first_meta;        // DEFER: first op of the current stage: position | code << 16
+    uint64_t rk_all;            // per stage (4 bits each): the stage size as the pair-kind tables index it
+    uint64_t diag_next, rk_next;   // diags / rk_all shifted down by the stages handed out so far
     uint32_t ws_stride;         // DEFER: 16-byte units between two stages of one plan in the workspace
     uint32_t ws_off;            // DEFER: 16-byte units from the plan's first slot to the slot of the current stage (fits: see ensure_stage_ws)
     uint64_t diags;             // the diag of every stage, 4 bits each, looked up once per plan
@@ -196,11 +198,15 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         if (RANGED && (lo < 0 || hi > g.N || lo >= hi)) { status = ACE_PLAN_MALFORMED; lo = 0; hi = 1; }
         // one LUT read per possible stage now, none where a stage begins (where few lanes are active)
         diags = 0;
+        uint64_t rks = 0;
         for (uint32_t k = 0; k < ACE_MAX_STAGES; ++k) {
             uint32_t glog = (uint32_t)(glogs >> (4u * k)) & 15u;
             uint32_t w = lds.ld<uint32_t>(g.stg_lds_off + (bidx * 16u + glog) * 4u);
             diags |= (uint64_t)(w & 15u) << (4u * k);
+            // the stage size as the pair-kind tables index it (a size outside the tables is unscorable anyway: block 0)
+            rks |= (uint64_t)(glog < (uint32_t)g.n_glog ? glog : 0u) << (4u * k);
         }
+        rewind(rks);
         if (BD) {
             // the "ideal" pass uses tp = dp = 1 and micro-batch = micro_bs (aceso_cost_model.py:588-590):
             // the diag of (micro_bs, 1 gpu)
@@ -210,17 +216,27 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         }
     }
 
+    // Start handing out the per-stage nibbles from stage 0 again (init; before the replay of stashed stages).
+    ACE_HD void rewind(uint64_t rks) {
+        rk_all = rks;
+        diag_next = diags;
+        rk_next = rks;
+    }
+
     // Stage head, part 1: the per-stage offsets the op loop needs, accumulators back to zero.
     // `tail`: also what only finish() uses (one LDS read).
     ACE_HD void start_fast(const AceGeom &g, const AceLds &lds, bool tail) {
         ++s;
-        // (a plan with more than 16 stage bits is caught by result())
-        const uint32_t sh = 4u * ((uint32_t)s & 15u);
-        const uint32_t d = (uint32_t)(diags >> sh) & 15u;
-        const uint32_t glog = (uint32_t)(glogs >> sh) & 15u;
+        // the next stage's nibbles sit at the bottom of diag_next / rk_next (stages come in order; past
+        // the sixteenth they read zero, and such a plan is caught by result())
+        const uint32_t d = (uint32_t)diag_next & 15u;
+        const uint32_t rk = (uint32_t)rk_next & 15u;
+        diag_next >>= 4;
+        rk_next >>= 4;
         z_v = ace_mul24(d, (uint32_t)g.C * 8u);
-        rk_v = (glog < (uint32_t)g.n_glog ? glog : 0u) << 6;   // (a stage size outside the tables is unscorable anyway)
+        rk_v = rk << 6;
         if (tail) {
+            const uint32_t glog = (uint32_t)(glogs >> (4u * ((uint32_t)s & 15u))) & 15u;
             dc_v = ace_mul24(d, (uint32_t)g.C);
             mrow = lds.ld<uint32_t>(g.stg_lds_off + (bidx * 16u + glog) * 4u) >> 16;
         }
@@ -259,7 +275,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
     // DEFER: park the finished stage in the plan's workspace slot `s`: ten values in five 16-byte
     // stores (a store from a lane or two costs as much as one from sixty-four, so what can be
     // folded here without a table lookup is: fwd + bwd, the closed peak segment, the reserved term).
-    ACE_HD void stash(const AceGeom &g, double *ws, uint32_t i_last, uint32_t c_last) {
+    ACE_HD void stash(const AceGeom &g, double *ws, uint32_t i_last, uint32_t c_last, bool prev_ordinary) {
         if (ws == nullptr || s < 0 || s >= ACE_MAX_STAGES) return;
         // stages are stashed in order, once each: slot s of this plan is ws_off further on (a running
         // offset instead of s * ws_stride, which would be a slow 32-bit multiply per stage end)
@@ -269,7 +285,10 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         double meta_d;
         __builtin_memcpy(&meta_d, &meta, 8);
         const double fb = fwd + bwd;                                    // the first sum of :579
-        const double peakc = ace_max(peak, run * (lastclose ? 1.0 : 0.0));   // :439: max(peak, run) if the last pair closes
+        // :439: max(peak, run) if the (previous op, last op) pair closes the last segment, i.e. if that pair is a
+        // recompute pair and the previous op an ordinary one.  `run` is 0.0 unless that pair is a recompute pair
+        // that continued the segment, so the wave-uniform half of the condition is all that has to be applied.
+        const double peakc = ace_max(peak, run * ace_scalar_01(prev_ordinary));
         r[0] = ace_d2{fb, rcs}; r[1] = ace_d2{rs_f, rs_b}; r[2] = ace_d2{W, A}; r[3] = ace_d2{saved, peakc};
         r[4] = ace_d2{reserved_term(g), meta_d};
     }
@@ -278,8 +297,9 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
     ACE_HD void replay(const AceGeom &g, const AceLds &lds, const uint32_t *pos_info, const double *ws, int s2) {
         const ace_d2 *r = reinterpret_cast<const ace_d2 *>(ws) + (size_t)((uint32_t)s2 * ws_stride);
         ace_d2 r0 = r[0], r1 = r[1], r2 = r[2], r3 = r[3], r4 = r[4];
+        if (s2 == 0) rewind(rk_all);
         s = s2 - 1;
-        start_fast(g, lds, true);              // s = s2; per-stage offsets, mrow
+        start_fast(g, lds, true);              // s = s2; per-stage offsets, mrow (called for s2 = 0, 1, ... in order)
         uint64_t meta;
         __builtin_memcpy(&meta, &r4.y, 8);
         uint32_t lo32 = (uint32_t)meta, i_last = (uint32_t)(meta >> 32);
@@ -385,24 +405,29 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
             rs_f += lds.ld<double>(za + ((r & 15u) << g.z_shift));
             rs_b += lds.ld<double>(za + ((r >> 4) << g.z_shift));
         }
+        double rf_new = ace_max(rfm, e2.x), rb_new = ace_max(rbm, e2.y);
         // the stage ends with this op
         const bool last = RANGED ? (i + 1 == hi) : (((nbyte >> 4) & 1u) || plan_end);
         if (last) {
             // :439 "i + 1 == len(ops) - 1": the (previous, this) pair closes the last segment
-            lastclose = pair_prev & (pinfo >> 25) & 1u;
-            if (DEFER) stash(g, rec, (uint32_t)i, c);
-            else finish(g, lds, row, c, rec);
+            if (DEFER) stash(g, rec, (uint32_t)i, c, (pinfo >> 25) & 1u);
+            else {
+                lastclose = pair_prev & (pinfo >> 25) & 1u;
+                finish(g, lds, row, c, rec);
+            }
             if (!RANGED) {
                 // (after the plan's last op this opens a stage that stays empty: s == S in the end)
                 start_fast(g, lds, !DEFER);
                 if (DEFER) first_meta = (uint32_t)(i + 1) | (nc << 16);
                 else if (i + 1 < g.N) start_lookups(g, lds, info_nextrow(g, info), nc);
             }
-            // the reserved maxima run over every op but the stage's last (get_reserved_memory :453-460)
-            e2 = ace_d2{0.0, 0.0};
+            // the reserved maxima run over every op but the stage's last (get_reserved_memory :453-460):
+            // the stage that ended took them as they were before this op, the new one starts from zero
+            rf_new = 0.0;
+            rb_new = 0.0;
         }
-        rfm = ace_max(rfm, e2.x);
-        rbm = ace_max(rbm, e2.y);
+        rfm = rf_new;
+        rbm = rb_new;
         // pair: (this op, next op) both recomputed and in one stage
         const bool savez = (info >> 24) & 1u;     // this is an ordinary op followed by a layer start
         // All of this is arithmetic on 0.0 / 1.0 factors instead of selects: x*1.0 and x+0.0 are exact,

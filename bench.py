@@ -20,8 +20,8 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per plan of one scoring-kernel launch on the default workload, from two rocprofv3 --pmc
 # runs (FETCH_SIZE, then WRITE_SIZE) scaled by the readings of a plain 256 MiB copy in the same
 # runs (factors 2.000 and 1.000), keyed by (workload, ops, plans grouped at upload):
-# 1,049 B read + 683 B written with the grouped layout, 1,334 + 618 in the generator's order.
-MEASURED_TRAFFIC_BYTES_PER_PLAN = {("gpt3_13b", 523, True): 1732.0, ("gpt3_13b", 523, False): 1952.0}
+# 1,049 B read + 681 B written with the grouped layout, 1,334 + 618 in the generator's order.
+MEASURED_TRAFFIC_BYTES_PER_PLAN = {("gpt3_13b", 523, True): 1731.0, ("gpt3_13b", 523, False): 1952.0}
 
 
 def cpu_baseline(tables, batch, threads):

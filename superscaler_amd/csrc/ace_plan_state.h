@@ -155,7 +155,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
     int lo, hi;                 // RANGED: only ops lo <= i < hi belong to the plan (one stage)
     // stage state
     int s;
-    uint32_t z_v, rk_v, mrow, dc_v;
+    uint32_t z_v, rk_v, mrow, dc_v;     // rk_v: pair-kind block offset of the stage MINUS z_v (see start_fast)
     uint32_t t_first;
     bool out_cross;
     double in_comm, inputs, id_in;
@@ -234,7 +234,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         diag_next >>= 4;
         rk_next >>= 4;
         z_v = ace_mul24(d, (uint32_t)g.C * 8u);
-        rk_v = rk << 6;
+        rk_v = (rk << 6) - z_v;      // relative to z_v, so that the op loop adds the same `zc` to both bases
         if (tail) {
             const uint32_t glog = (uint32_t)(glogs >> (4u * ((uint32_t)s & 15u))) & 15u;
             dc_v = ace_mul24(d, (uint32_t)g.C);
@@ -399,8 +399,8 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
             // first op) adds 0.0, and the id past the last real table is all NaN (the reference raises there)
             const uint32_t r = r_next;
             const uint32_t pk = (info >> 16) & 0xffu;
-            // (rk_v is a multiple of 64 and c * 8 + nc < 64: the sum is the [c][nc] entry of the stage-size block)
-            r_next = lds.ld<uint8_t>((g.rk_lds_off + ace_mul24(pk, g.rk_kind_stride)) + (ace_mad24(c, 8u, rk_v) + nc));
+            // (rk_v + zc = stage-size block * 64 + c * 8, and c * 8 + nc < 64: the [c][nc] entry of that block)
+            r_next = lds.ld<uint8_t>((g.rk_lds_off + ace_mul24(pk, g.rk_kind_stride)) + ((rk_v + zc) + nc));
             const uint32_t za = (row + g.z_off) + zc;
             rs_f += lds.ld<double>(za + ((r & 15u) << g.z_shift));
             rs_b += lds.ld<double>(za + ((r >> 4) << g.z_shift));

@@ -88,3 +88,42 @@ def test_row_windows_never_restage_in_the_padding(name):
             w += 1
             next_win = wp[w]
     assert restaged == t.n_windows - 1
+
+
+def settings_matrix():
+    """Every combination of the switches that change what the model returns (aceso_utils.py:359-531)."""
+    import itertools
+    for pred, shared, reserved, resh, pmb in itertools.product(("MAX", "MIN"), (True, False), (True, False), (True, False), (0, 1500)):
+        yield dict(memory_pred_type=pred, consider_shared_space=shared, consider_reserved_space=reserved,
+                   resharding=resh, peak_mem_in_backward=pmb)
+
+
+@pytest.mark.parametrize("name", ["gpt3_1_3b", "wresnet_1b"])
+def test_every_settings_combination_matches_the_oracle(name):
+    """MAX / MIN memory prediction, shared-buffer rule, reserved space, resharding on and off (peak_mem_in_backward
+    only enters check_recompute): kernel source on the CPU (stage tails in place and deferred, stage records) and
+    the C restatement against the Python oracle, bit for bit."""
+    import dataclasses
+    from superscaler_amd.tables import compile_tables
+    from tests.helpers import c_oracle_scores
+    w = synth.WORKLOADS[name]
+    graph = synth.make_graph(w)
+    db = synth.make_db(w, graph)
+    base = synth.make_tables(w)
+    batch = synth.make_plans(w, base, n_plans=24, seed_offset=77)
+    seen = set()
+    for kw in settings_matrix():
+        st = dataclasses.replace(synth.make_settings(w), **kw)
+        tables = compile_tables(graph, db, st)
+        orc = oracle_for(tables)
+        oit, opk, ofe, cfgs = oracle_scores(orc, batch, tables)
+        for defer in (False, True):
+            it, pk, fe, status, _ = emu_score(tables, batch, defer=defer)
+            assert (status == 0).all() and np.array_equal(it, oit) and np.array_equal(pk, opk) and np.array_equal(fe, ofe), kw
+        cit, cpk, cfe, cer = c_oracle_scores(tables, batch)
+        assert not cer.any() and np.array_equal(cit, oit) and np.array_equal(cpk, opk) and np.array_equal(cfe, ofe), kw
+        _, _, _, _, rec = emu_score(tables, batch, breakdown=True)
+        for p, c in enumerate(cfgs):
+            assert [rec[p, s, R_STAGE_MB] for s in range(c.num_stages)] == list(c.memory_list), kw
+        seen.add((tuple(opk.tolist()), tuple(oit.tolist())))
+    assert len(seen) >= 8          # the switches do change the answers

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define ACE_ABI_VERSION 4
+#define ACE_ABI_VERSION 5
 #define ACE_MAX_STAGES 16      /* aceso_utils.py:502: end_num_stages = min(num_gpus, 16) */
 #define ACE_STAGE_REC 18       /* doubles per stage record, see ACE_R_* */
 
@@ -100,6 +100,9 @@ typedef struct ace_tables {
 #define ACE_F_RESHARDING 1      /* args.resharding (aceso_utils.py:523-526) */
 #define ACE_F_RESERVED_MIN 2    /* memory_pred_type == "MIN" (aceso_cost_model.py:482) */
 #define ACE_F_NO_RESERVED 4     /* not consider_reserved_space (aceso_cost_model.py:525-528) */
+#define ACE_F_COLLECTIVE_MEM 8   /* consider_collective_memory (aceso_cost_model.py:462-478): n_z more tables follow the
+                                   n_z cost tables in every row, holding the MB each collective occupies
+                                   (get_reshard_memory, :262-273) */
 
 typedef struct ace_handle ace_handle_t;
 

@@ -36,8 +36,6 @@ from .tables import (MAX_STAGES, R_ACT, R_BWD, R_FWD, R_IDEAL_BWD, R_IDEAL_FWD, 
 
 def settings_from_args(args) -> CostModelSettings:
     """The reference's argparse namespace (aceso_utils.py:455-531) -> CostModelSettings."""
-    if getattr(args, "consider_collective_memory", False):
-        raise NotImplementedError("--consider-collective-memory (aceso_cost_model.py:463-478) is not supported")
     gpn = args.num_gpus_per_node
     return CostModelSettings(
         model_name=args.model_name, micro_batch_size=list(args.micro_batch_size), num_gpus_per_node=gpn,
@@ -48,7 +46,8 @@ def settings_from_args(args) -> CostModelSettings:
         flex_recompute=getattr(args, "flex_recompute", True),
         peak_mem_in_backward=getattr(args, "peak_mem_in_backward", 0),
         memory_pred_type=getattr(args, "memory_pred_type", "MAX"),
-        resharding=getattr(args, "resharding", None))
+        resharding=getattr(args, "resharding", None),
+        consider_collective_memory=bool(getattr(args, "consider_collective_memory", False)))
 
 
 class CostModel:

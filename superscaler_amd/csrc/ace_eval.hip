@@ -44,10 +44,11 @@ thread_local char g_hip_err[256] = "";
 // few CUs (a workgroup keeps a CU to itself either way: the tables fill its LDS): the walk over the
 // op sequence is sequential per wavefront, so a small batch finishes soonest with one wavefront per
 // SIMD on as many CUs as it can reach.
-template <bool BD, bool RANGED, bool WIN, bool DEFER, int BLOCK>
+// COLL: tables compiled with consider_collective_memory (large workgroups only: a switch few callers set).
+template <bool BD, bool RANGED, bool WIN, bool DEFER, int BLOCK, bool COLL = false>
 __global__ __launch_bounds__(BLOCK) void ace_score_kernel(const AceKernelArgs a) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
-    ace_score_body<BD, RANGED, WIN, DEFER, BLOCK>(a, lds_raw, 0u, (int)threadIdx.x, (long long)blockIdx.x, gridDim.x);
+    ace_score_body<BD, RANGED, WIN, DEFER, BLOCK, COLL>(a, lds_raw, 0u, (int)threadIdx.x, (long long)blockIdx.x, gridDim.x);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -353,6 +354,9 @@ template <bool BD, bool RANGED, bool WIN, bool DEFER> static int allow_big_lds()
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
     ACE_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&ace_score_kernel<BD, RANGED, WIN, DEFER, kSmallBlock>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
+    if (!DEFER)
+        ACE_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&ace_score_kernel<BD, RANGED, WIN, false, kBlock, true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
     return ACE_OK;
 }
 
@@ -374,7 +378,8 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     const int64_t hot_end = (int64_t)t->hot_off + (int64_t)(t->n_diag + 1) * C * 6;
     const int64_t start_end = (int64_t)t->start_off + (int64_t)t->n_diag * C * 4;
     const int64_t out_end = (int64_t)t->out_off + (int64_t)t->n_mbs * t->n_tp * t->n_algo * 2;
-    const int64_t z_end = (int64_t)t->z_off + (int64_t)t->n_z * t->z_table_doubles;
+    if ((t->flags & ACE_F_COLLECTIVE_MEM) && !(t->flags & ACE_F_RESHARDING)) return ACE_EINVAL;
+    const int64_t z_end = (int64_t)t->z_off + (int64_t)t->n_z * t->z_table_doubles * ((t->flags & ACE_F_COLLECTIVE_MEM) ? 2 : 1);
     if (t->z_table_doubles < t->n_diag * C) return ACE_EINVAL;
     if ((t->hot_off & 1) || (t->start_off & 1) || (t->out_off & 1) || (t->z_off & 1) || t->hot_off < 0 ||
         t->start_off < 0 || t->out_off < 0 || t->z_off < 0 ||
@@ -427,6 +432,7 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     g.out_off = (uint32_t)t->out_off * 8u; g.z_off = (uint32_t)t->z_off * 8u;
     g.z_shift = 3;
     while ((1 << (g.z_shift - 3)) < t->z_table_doubles) ++g.z_shift;
+    g.zm_delta = (uint32_t)t->n_z << g.z_shift;
     g.rk_lds_off = rk_off; g.stg_lds_off = stg_off;
     g.rk_kind_stride = (uint32_t)(t->n_glog * 64);
     g.row_bytes = (uint32_t)row_bytes;
@@ -493,7 +499,11 @@ static int fill_args(ace_handle_t *h, const ace_batch_t *b, double memory_limit,
 template <bool BD, bool RANGED, bool WIN, bool DEFER>
 static void launch_score_b(const ace_handle_t *h, const AceKernelArgs &a, hipStream_t s) {
     const size_t P = (size_t)a.g.P;
-    if ((P + kBlock - 1) / kBlock < (size_t)kSmallBatchBlocks)
+    if (a.g.flags & ACE_F_COLLECTIVE_MEM) {
+        if (!DEFER)         // (ensure_stage_ws never hands such tables to the deferred kernel)
+            hipLaunchKernelGGL((ace_score_kernel<BD, RANGED, WIN, false, kBlock, true>), dim3((unsigned)((P + kBlock - 1) / kBlock)),
+                               dim3(kBlock), h->lds_bytes, s, a);
+    } else if ((P + kBlock - 1) / kBlock < (size_t)kSmallBatchBlocks)
         hipLaunchKernelGGL((ace_score_kernel<BD, RANGED, WIN, DEFER, kSmallBlock>), dim3((unsigned)((P + kSmallBlock - 1) / kSmallBlock)),
                            dim3(kSmallBlock), h->lds_bytes, s, a);
     else
@@ -518,7 +528,7 @@ static void launch_score(const ace_handle_t *h, const AceKernelArgs &a, hipStrea
 // per-plan workspace; the handle keeps one and grows it on demand.
 static int ensure_stage_ws(ace_handle_t *h, AceKernelArgs *a) {
     a->stage_ws = nullptr;
-    if (a->range || a->stage_out || h->n_windows > 1 || h->geom.N >= 65536) return ACE_OK;
+    if (a->range || a->stage_out || h->n_windows > 1 || h->geom.N >= 65536 || (h->geom.flags & ACE_F_COLLECTIVE_MEM)) return ACE_OK;
     const size_t need = (((size_t)a->g.P + kBlock - 1) / kBlock) * kBlock;
     if (need * ACE_MAX_STAGES * (ACE_WS_REC / 2) > 0xffffffffull) return ACE_OK;   // 32-bit record offsets: larger batches take the plain kernel
     if (need > h->stage_ws_plans) {

@@ -126,6 +126,7 @@ struct AceGeom {
     int32_t n_mbs, n_tp, n_algo, n_glog, n_pair_kinds;
     uint32_t hot_off, start_off, out_off, z_off;   // bytes inside a row
     uint32_t z_shift;           // log2(bytes of one resharding-cost table inside a row)
+    uint32_t zm_delta;          // bytes from a cost table to the memory table of the same collective (ACE_F_COLLECTIVE_MEM)
     uint32_t rk_lds_off, stg_lds_off;              // LDS byte offsets of the pair-kind and stage LUT regions
     uint32_t rk_kind_stride;    // bytes of one pair kind (n_glog * 64)
     uint32_t row_bytes;         // bytes of one op type's row
@@ -142,10 +143,11 @@ ACE_HD uint32_t info_nextrow(const AceGeom &g, uint32_t i) { return ((i >> 8) & 
 
 #define ACE_WS_REC 10          // doubles per deferred stage record (see PlanState::stash)
 
+// COLL: consider_collective_memory (the tables carry ACE_F_COLLECTIVE_MEM).
 // BD: per-stage records for the caller.  RANGED: one stage over an op sub-range.  DEFER: stage
 // tails are not evaluated where the stage ends (where only the few lanes that cut at this op are
 // active) but stashed to a per-plan workspace and replayed after the op loop with every lane busy.
-template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
+template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false> struct PlanState {
     // plan constants
     int S;
     uint32_t bidx;
@@ -160,7 +162,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
     bool out_cross;
     double in_comm, inputs, id_in;
     // per-op accumulators (reset at every stage head)
-    double fwd, bwd, rcs, W, A, saved, run, peak, rfm, rbm, rs_f, rs_b;
+    double fwd, bwd, rcs, W, A, saved, run, peak, rfm, rbm, rs_f, rs_b, mc;
     double id_fwd, id_bwd;
     bool lastclose;
     uint32_t first_meta;        // DEFER: first op of the current stage: position | code << 16
@@ -188,7 +190,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
         lastclose = false; first_meta = 0; r_next = 0; pair_prev = 0;
         ws_stride = ACE_WS_REC / 2;
         ws_off = 0;
-        fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = rs_f = rs_b = 0.0;
+        fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = rs_f = rs_b = mc = 0.0;
         id_fwd = id_bwd = id_in = 0.0;
         in_comm = inputs = 0.0;
         z_v = rk_v = mrow = t_first = dc_v = 0;
@@ -240,7 +242,7 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
             dc_v = ace_mul24(d, (uint32_t)g.C);
             mrow = lds.ld<uint32_t>(g.stg_lds_off + (bidx * 16u + glog) * 4u) >> 16;
         }
-        fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = rs_f = rs_b = 0.0;
+        fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = rs_f = rs_b = mc = 0.0;
         lastclose = false;
         r_next = 0;             // a stage's first op pays no resharding
     }
@@ -267,9 +269,11 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
 
     // The reserved-memory term of a stage (get_reserved_memory :480-483 with max_collective = 0).
     ACE_HD double reserved_term(const AceGeom &g) const {
+        // (mc: the largest collective buffer, :480-483; without COLL the reference adds its integer 0)
+        const double coll = COLL ? mc : 0.0;
         if (g.flags & ACE_F_NO_RESERVED) return 0.0;
-        if (g.flags & ACE_F_RESERVED_MIN) return ace_max(ace_max(rfm, rbm), ace_max(W, 0.0));
-        return ace_max(rfm + rbm, W) + 0.0;
+        if (g.flags & ACE_F_RESERVED_MIN) return ace_max(ace_max(rfm, rbm), ace_max(W, coll));
+        return ace_max(rfm + rbm, W) + coll;
     }
 
     // DEFER: park the finished stage in the plan's workspace slot `s`: ten values in five 16-byte
@@ -402,8 +406,14 @@ template <bool BD, bool RANGED, bool DEFER = false> struct PlanState {
             // (rk_v + zc = stage-size block * 64 + c * 8, and c * 8 + nc < 64: the [c][nc] entry of that block)
             r_next = lds.ld<uint8_t>((g.rk_lds_off + ace_mul24(pk, g.rk_kind_stride)) + ((rk_v + zc) + nc));
             const uint32_t za = (row + g.z_off) + zc;
-            rs_f += lds.ld<double>(za + ((r & 15u) << g.z_shift));
-            rs_b += lds.ld<double>(za + ((r >> 4) << g.z_shift));
+            const uint32_t af = za + ((r & 15u) << g.z_shift), ab = za + ((r >> 4) << g.z_shift);
+            rs_f += lds.ld<double>(af);
+            rs_b += lds.ld<double>(ab);
+            if (COLL) {
+                // max_collective of get_reserved_memory (:462-478): the same pairs, the collectives' buffers
+                mc = ace_max(mc, lds.ld<double>(af + g.zm_delta));
+                mc = ace_max(mc, lds.ld<double>(ab + g.zm_delta));
+            }
         }
         double rf_new = ace_max(rfm, e2.x), rb_new = ace_max(rbm, e2.y);
         // the stage ends with this op

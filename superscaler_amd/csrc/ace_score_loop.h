@@ -51,10 +51,10 @@ template <int BLOCK> ACE_HD void stage_window(const AceKernelArgs &a, unsigned c
 // DEFER: stage tails are stashed in the workspace and evaluated after the op loop, when all lanes
 // are active again (needs every row resident, so never together with WIN).
 // `tid` lane of workgroup `block` of `n_blocks`, BLOCK lanes each; `lds_raw`: the workgroup's LDS (`lds_bytes` long).
-template <bool BD, bool RANGED, bool WIN, bool DEFER, int BLOCK>
+template <bool BD, bool RANGED, bool WIN, bool DEFER, int BLOCK, bool COLL = false>
 ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint32_t lds_bytes, int tid, long long block,
                            uint32_t n_blocks) {
-    static_assert(!DEFER || (!BD && !RANGED && !WIN), "deferred stage tails: plain scoring only");
+    static_assert(!DEFER || (!BD && !RANGED && !WIN && !COLL), "deferred stage tails: plain scoring only");
     // region offsets as absolute LDS addresses for the reads (see AceLds); the staging loops below
     // write through `lds_raw` with the plain offsets of a.g
     AceGeom g = a.g;
@@ -76,7 +76,7 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     ACE_SYNC();
 
     const AceLds lds = ace_make_lds(lds_raw, lds_bytes);
-    PlanState<BD, RANGED, DEFER> st;
+    PlanState<BD, RANGED, DEFER, COLL> st;
     const ace_u4 h = a.hdr[pl];
     ace_u2 range{0u, 0u};
     if (RANGED) range = a.range[pl];

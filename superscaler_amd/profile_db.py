@@ -38,6 +38,7 @@ class CostModelSettings:
     peak_mem_in_backward: int = 0
     memory_pred_type: str = "MAX"
     resharding: Optional[bool] = None
+    consider_collective_memory: bool = False     # aceso_utils.py:448, aceso_cost_model.py:462-478
 
     def __post_init__(self):
         if self.max_tp is None:

@@ -38,11 +38,11 @@ import numpy as np
 from . import opgraph as og
 from .profile_db import CostModelSettings, ProfileDB
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 MAX_STAGES = 16
 STAGE_REC = 18
 LDS_BYTES = 160 * 1024
-F_RESHARDING, F_RESERVED_MIN, F_NO_RESERVED = 1, 2, 4
+F_RESHARDING, F_RESERVED_MIN, F_NO_RESERVED, F_COLLECTIVE_MEM = 1, 2, 4, 8
 
 (R_FWD, R_BWD, R_IN_COMM, R_OUT_COMM, R_RECOMP, R_WEIGHTS, R_INPUTS, R_ACT, R_SAVED, R_PEAK,
  R_RESERVED, R_IDEAL_FWD, R_IDEAL_BWD, R_IDEAL_IN, R_IDEAL_OUT, R_STAGE_MS, R_STAGE_MB, R_RESHARD) = range(18)
@@ -195,11 +195,15 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
 
     ERR = 15   # placeholder while the number of real tables is still growing
 
+    coll_mem = bool(getattr(settings, "consider_collective_memory", False) and settings.resharding
+                    and settings.consider_reserved_space)
+
     def z_id(prim, n):
-        if prim in (og.P_NONE, og.P_SPLIT):
+        if prim == og.P_NONE or (prim == og.P_SPLIT and not coll_mem):
             return 0          # nothing to pay: split is free (aceso_cost_model.py:257-258)
         name = og.PRIM_NAMES[prim]
-        if name not in db.collectives or n not in db.collectives[name]:
+        # (split costs no time but occupies memory, :262-266: with collective memory it gets a table of its own)
+        if prim != og.P_SPLIT and (name not in db.collectives or n not in db.collectives[name]):
             return ERR        # KeyError in the reference (:251)
         if (prim, n) not in z_keys:
             if len(z_keys) >= 13:
@@ -275,7 +279,8 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
     z_table_doubles = 1
     while z_table_doubles < ND * C:
         z_table_doubles *= 2          # one collective's table, padded so its index is a shift
-    row_doubles = z_off + NZ * z_table_doubles
+    # with collective memory a second set of tables follows: MB a collective occupies (get_reshard_memory :262-273)
+    row_doubles = z_off + NZ * z_table_doubles * (2 if coll_mem else 1)
     row_doubles += row_doubles & 1
     if ND > 14:
         raise ValueError("more than 14 distinct micro-batch maps: a plan packs one 4-bit diag per stage")
@@ -297,6 +302,8 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
         start = np.full((ND, C, 4), nan)
         z = np.full((max(NZ, 1), ND, C), nan)
         z[0] = 0.0
+        zm = np.full((max(NZ, 1), ND, C), nan)
+        zm[0] = 0.0
         for d, tup in enumerate(diag_tuples):
             for t in range(T):
                 m = tup[t]
@@ -317,6 +324,8 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
                     start[d, c] = (insz, db.p2p_time(insz, db.intra_band), db.p2p_time(insz, db.inter_band), 0.0)
                     for k, (prim, n) in enumerate(z_keys):
                         z[k + 1, d, c] = db.reshard_time(og.PRIM_NAMES[prim], n, insz)
+                        # get_reshard_memory: the data itself, times the group size for the gathering collectives
+                        zm[k + 1, d, c] = insz * n if og.PRIM_NAMES[prim] in ("all_gather", "all_to_all") else insz
         out = np.zeros((M, T, A, 2))
         for m in range(M):
             for t in range(T):
@@ -329,6 +338,10 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
         for k in range(NZ):
             rows[ty, z_off + k * z_table_doubles:z_off + (k + 1) * z_table_doubles] = nan if k == NZ - 1 else 0.0
             rows[ty, z_off + k * z_table_doubles:z_off + k * z_table_doubles + ND * C] = z[k].ravel()
+            if coll_mem:
+                o = z_off + (NZ + k) * z_table_doubles
+                rows[ty, o:o + z_table_doubles] = nan if k == NZ - 1 else 0.0
+                rows[ty, o:o + ND * C] = zm[k].ravel()
 
     # ---- LDS residency: one window if every row fits, else windows over op positions ----------
     row_bytes = row_doubles * 8
@@ -402,6 +415,8 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
         flags |= F_NO_RESERVED
     elif settings.memory_pred_type == "MIN":
         flags |= F_RESERVED_MIN
+    if coll_mem and (flags & F_RESHARDING):
+        flags |= F_COLLECTIVE_MEM
     nbm1 = np.array([float(settings.global_batch_size // mb - 1) for mb in db.mbs_list], dtype=np.float64)
     return CompiledTables(
         graph=graph, db=db, settings=settings, n_diag=ND, n_glog=n_glog, n_z=NZ,

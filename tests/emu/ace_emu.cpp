@@ -13,14 +13,14 @@
 
 namespace {
 
-template <bool BD, bool RANGED, bool DEFER = false>
+template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false>
 void score_one(const ace_tables_t *t, const AceGeom &g, std::vector<unsigned char> &lds, uint32_t lds_bytes,
                const uint8_t *codes, ace_u4 h, ace_u2 range, double *rec, double &iter, double &peak, uint8_t &feas,
                uint8_t &st) {
     const size_t row_bytes = (size_t)t->row_doubles * 8;
     const uint32_t *pos = t->pos_info;
     AceLds view{lds.data(), lds_bytes};
-    PlanState<BD, RANGED, DEFER> s;
+    PlanState<BD, RANGED, DEFER, COLL> s;
     std::vector<double> ws(ACE_MAX_STAGES * ACE_WS_REC, __builtin_nan(""));
     if (DEFER) rec = ws.data();
     s.init(g, view, h, range);
@@ -60,6 +60,7 @@ extern "C" int ace_emu_score(const ace_tables_t *t, const uint8_t *codes /* [P][
     g.hot_off = t->hot_off * 8u; g.start_off = t->start_off * 8u; g.out_off = t->out_off * 8u; g.z_off = t->z_off * 8u;
     g.z_shift = 3;
     while ((1 << (g.z_shift - 3)) < t->z_table_doubles) ++g.z_shift;
+    g.zm_delta = (uint32_t)t->n_z << g.z_shift;
     const int32_t rk_bytes = t->n_pair_kinds * t->n_glog * 64;
     g.rk_lds_off = (uint32_t)t->lds_row_bytes;
     g.stg_lds_off = (g.rk_lds_off + (uint32_t)rk_bytes + 15u) & ~15u;
@@ -83,7 +84,13 @@ extern "C" int ace_emu_score(const ace_tables_t *t, const uint8_t *codes /* [P][
         const uint8_t *c = codes + (size_t)p * g.N;
         double iter, peak;
         uint8_t feas, st;
-        if (range) score_one<true, true>(t, g, lds, lds_bytes, c, h, rg, rec, iter, peak, feas, st);
+        const bool coll = (t->flags & ACE_F_COLLECTIVE_MEM) != 0;
+        if (coll) {
+            if (range) score_one<true, true, false, true>(t, g, lds, lds_bytes, c, h, rg, rec, iter, peak, feas, st);
+            else if (stage_out) score_one<true, false, false, true>(t, g, lds, lds_bytes, c, h, rg, rec, iter, peak, feas, st);
+            else score_one<false, false, false, true>(t, g, lds, lds_bytes, c, h, rg, rec, iter, peak, feas, st);
+        }
+        else if (range) score_one<true, true>(t, g, lds, lds_bytes, c, h, rg, rec, iter, peak, feas, st);
         else if (stage_out) score_one<true, false>(t, g, lds, lds_bytes, c, h, rg, rec, iter, peak, feas, st);
         else if (defer && t->n_windows == 1) score_one<false, false, true>(t, g, lds, lds_bytes, c, h, rg, rec, iter, peak, feas, st);
         else score_one<false, false>(t, g, lds, lds_bytes, c, h, rg, rec, iter, peak, feas, st);
@@ -121,11 +128,11 @@ struct GuardedPool {
     ~GuardedPool() { for (auto &m : maps) munmap(m.base, m.len); }
 };
 
-template <bool BD, bool RANGED, bool WIN, bool DEFER>
+template <bool BD, bool RANGED, bool WIN, bool DEFER, bool COLL = false>
 void run_lanes(const AceKernelArgs &a, unsigned char *lds, uint32_t lds_bytes) {
     for (long long p = 0; p < a.g.P; ++p) {
         memset(lds, 0xff, lds_bytes);
-        ace_score_body<BD, RANGED, WIN, DEFER, 1>(a, lds, lds_bytes, 0, p, (uint32_t)a.g.P);
+        ace_score_body<BD, RANGED, WIN, DEFER, 1, COLL>(a, lds, lds_bytes, 0, p, (uint32_t)a.g.P);
     }
 }
 
@@ -146,6 +153,7 @@ extern "C" int ace_emu_kernel(const ace_tables_t *t, const uint8_t *codes, const
     g.hot_off = t->hot_off * 8u; g.start_off = t->start_off * 8u; g.out_off = t->out_off * 8u; g.z_off = t->z_off * 8u;
     g.z_shift = 3;
     while ((1 << (g.z_shift - 3)) < t->z_table_doubles) ++g.z_shift;
+    g.zm_delta = (uint32_t)t->n_z << g.z_shift;
     a.rk_bytes = t->n_pair_kinds * t->n_glog * 64;
     g.rk_lds_off = (uint32_t)t->lds_row_bytes;
     g.stg_lds_off = (g.rk_lds_off + (uint32_t)a.rk_bytes + 15u) & ~15u;
@@ -182,10 +190,17 @@ extern "C" int ace_emu_kernel(const ace_tables_t *t, const uint8_t *codes, const
     a.stage_out = stage_out ? (double *)pool.place(stage_out, rec_bytes, 8) : nullptr;   // (records of unused stages stay as the caller left them)
     unsigned char *lds = (unsigned char *)pool.place(nullptr, lds_bytes);
     const bool win = t->n_windows > 1;
-    const bool defer = !range && !stage_out && !win && g.N < 65536;
+    const bool coll = (t->flags & ACE_F_COLLECTIVE_MEM) != 0;
+    const bool defer = !range && !stage_out && !win && g.N < 65536 && !coll;
     if (defer) a.stage_ws = (double *)pool.place(nullptr, (size_t)P * ACE_MAX_STAGES * ACE_WS_REC * 8);
 
-    if (range) { if (win) run_lanes<true, true, true, false>(a, lds, lds_bytes); else run_lanes<true, true, false, false>(a, lds, lds_bytes); }
+    if (coll) {
+        if (range) { if (win) run_lanes<true, true, true, false, true>(a, lds, lds_bytes); else run_lanes<true, true, false, false, true>(a, lds, lds_bytes); }
+        else if (stage_out) { if (win) run_lanes<true, false, true, false, true>(a, lds, lds_bytes); else run_lanes<true, false, false, false, true>(a, lds, lds_bytes); }
+        else if (win) run_lanes<false, false, true, false, true>(a, lds, lds_bytes);
+        else run_lanes<false, false, false, false, true>(a, lds, lds_bytes);
+    }
+    else if (range) { if (win) run_lanes<true, true, true, false>(a, lds, lds_bytes); else run_lanes<true, true, false, false>(a, lds, lds_bytes); }
     else if (stage_out) { if (win) run_lanes<true, false, true, false>(a, lds, lds_bytes); else run_lanes<true, false, false, false>(a, lds, lds_bytes); }
     else if (defer) run_lanes<false, false, false, true>(a, lds, lds_bytes);
     else if (win) run_lanes<false, false, true, false>(a, lds, lds_bytes);

@@ -3,7 +3,7 @@ WORKLOAD MODE N_PLANS`): the scoring kernel's own loop on the CPU behind guard p
 when every output equals the state-machine emulation's (NaNs included); an out-of-range index in the
 loop ends this process with SIGSEGV instead.
 
-MODE: plain | breakdown | ranged | junk (random bytes for codes, headers and padding: results are not
+MODE: plain | collective (plain with consider_collective_memory) | breakdown | ranged | junk (random bytes for codes, headers and padding: results are not
 compared, the loop only has to stay inside its arrays) | golden_resnet (the reference's ResNet plans) |
 moves (csrc/ace_edit_kernels.h: move descriptors -> plans and keys, against the numpy forms; then random
 descriptors) | recompute (check_recompute's loop for device-resident batches, run on CPU tensors with
@@ -61,6 +61,15 @@ def main(workload, mode, n):
     w = synth.WORKLOADS[workload]
     tables = synth.make_tables(w)
     batch = synth.make_plans(w, tables, n_plans=n, seed_offset=5)
+    if mode == "collective":
+        # consider_collective_memory: longer rows (memory tables after the cost tables), hence more row windows
+        import dataclasses
+        from superscaler_amd.tables import compile_tables
+        graph = synth.make_graph(w)
+        tables = compile_tables(graph, synth.make_db(w, graph),
+                                dataclasses.replace(synth.make_settings(w), consider_collective_memory=True))
+        assert tables.flags & 8
+        mode = "plain"
     if mode == "plain":
         assert same(emu_kernel_score(tables, batch), emu_score(tables, batch))
         assert same(emu_kernel_score(tables, batch, strict=True, memory_limit=1.0), emu_score(tables, batch, strict=True, memory_limit=1.0))

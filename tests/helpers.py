@@ -22,7 +22,8 @@ def oracle_for(tables):
                  num_gpus_per_node=st.num_gpus_per_node, memory_limit=st.memory_limit, max_tp=st.max_tp,
                  consider_shared_space=st.consider_shared_space,
                  consider_reserved_space=st.consider_reserved_space, flex_recompute=st.flex_recompute,
-                 peak_mem_in_backward=st.peak_mem_in_backward, memory_pred_type=st.memory_pred_type)
+                 peak_mem_in_backward=st.peak_mem_in_backward, memory_pred_type=st.memory_pred_type,
+                 consider_collective_memory=bool(getattr(st, "consider_collective_memory", False)))
     s.resharding = st.resharding
     orc = Oracle(s)
     orc.load_dense(db.op_names, {ORACLE_FIELD[k]: v.tolist() for k, v in db.tables.items()},

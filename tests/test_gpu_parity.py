@@ -198,6 +198,34 @@ def test_every_settings_combination_matches_the_c_oracle(name, torch_mod):
     assert len(answers) >= 8
 
 
+@pytest.mark.parametrize("name", ["gpt3_1_3b", "wresnet_1b"])
+def test_collective_memory_switch_matches_the_oracle(name, torch_mod):
+    """consider_collective_memory (aceso_cost_model.py:462-483): the buffers of the resharding collectives enter the
+    reserved memory; the rows grow by the memory tables, so these runs also use the windowed kernel."""
+    import dataclasses
+    from superscaler_amd.evaluator import PlanEvaluator
+    w = synth.WORKLOADS[name]
+    graph = synth.make_graph(w)
+    db = synth.make_db(w, graph)
+    batch = synth.make_plans(w, synth.make_tables(w), n_plans=192, seed_offset=79)
+    changed = 0
+    for pred in ("MAX", "MIN"):
+        st = dataclasses.replace(synth.make_settings(w), memory_pred_type=pred, consider_collective_memory=True)
+        tables = compile_tables(graph, db, st)
+        ev = PlanEvaluator(tables)
+        it, pk, fe, status, rec = ev.score_host(batch, breakdown=True)
+        it2, pk2, fe2, status2 = ev.score_host(batch)
+        ev.close()
+        oit, opk, ofe, cfgs = oracle_scores(oracle_for(tables), batch, tables)
+        assert (status == 0).all() and np.array_equal(it, oit) and np.array_equal(pk, opk) and np.array_equal(fe, ofe)
+        assert np.array_equal(it2, oit) and np.array_equal(pk2, opk) and np.array_equal(fe2, ofe)
+        for p, c in enumerate(cfgs):
+            assert [rec[p, s, 16] for s in range(c.num_stages)] == list(c.memory_list)
+        off = compile_tables(graph, db, dataclasses.replace(st, consider_collective_memory=False))
+        changed += int((oracle_scores(oracle_for(off), batch, off)[1] != opk).sum())
+    assert changed > 0
+
+
 def test_full_size_properties(torch_mod):
     """GPT-3 13B at the benchmark's full size (1,048,576 plans), which the oracle cannot cover:
     size-independent properties, an oracle spot check and the top-k against a stable sort."""

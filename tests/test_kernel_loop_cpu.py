@@ -15,7 +15,9 @@ from superscaler_amd import synth
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 CASES = [(name, mode, 96 if name != "gpt3_175b" else 24) for name in synth.WORKLOADS
-         for mode in ("plain", "breakdown", "ranged", "junk", "moves", "recompute")] + [("-", "golden_resnet", 0)]
+         for mode in ("plain", "breakdown", "ranged", "junk", "moves", "recompute")] + [("-", "golden_resnet", 0),
+                                                                                       ("gpt3_1_3b", "collective", 96),
+                                                                                       ("wresnet_1b", "collective", 96)]
 
 
 @pytest.mark.parametrize("workload,mode,n", CASES, ids=[f"{c[0]}-{c[1]}" for c in CASES])

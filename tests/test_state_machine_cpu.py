@@ -96,6 +96,9 @@ def settings_matrix():
     for pred, shared, reserved, resh, pmb in itertools.product(("MAX", "MIN"), (True, False), (True, False), (True, False), (0, 1500)):
         yield dict(memory_pred_type=pred, consider_shared_space=shared, consider_reserved_space=reserved,
                    resharding=resh, peak_mem_in_backward=pmb)
+        if resh and reserved and pmb == 0:      # where the collectives' buffers can enter the reserved memory (:462-483)
+            yield dict(memory_pred_type=pred, consider_shared_space=shared, consider_reserved_space=reserved,
+                       resharding=resh, peak_mem_in_backward=pmb, consider_collective_memory=True)
 
 
 @pytest.mark.parametrize("name", ["gpt3_1_3b", "wresnet_1b"])
@@ -120,10 +123,11 @@ def test_every_settings_combination_matches_the_oracle(name):
         for defer in (False, True):
             it, pk, fe, status, _ = emu_score(tables, batch, defer=defer)
             assert (status == 0).all() and np.array_equal(it, oit) and np.array_equal(pk, opk) and np.array_equal(fe, ofe), kw
-        cit, cpk, cfe, cer = c_oracle_scores(tables, batch)
-        assert not cer.any() and np.array_equal(cit, oit) and np.array_equal(cpk, opk) and np.array_equal(cfe, ofe), kw
+        if not kw.get("consider_collective_memory"):          # (the C restatement leaves that switch out)
+            cit, cpk, cfe, cer = c_oracle_scores(tables, batch)
+            assert not cer.any() and np.array_equal(cit, oit) and np.array_equal(cpk, opk) and np.array_equal(cfe, ofe), kw
         _, _, _, _, rec = emu_score(tables, batch, breakdown=True)
         for p, c in enumerate(cfgs):
             assert [rec[p, s, R_STAGE_MB] for s in range(c.num_stages)] == list(c.memory_list), kw
         seen.add((tuple(opk.tolist()), tuple(oit.tolist())))
-    assert len(seen) >= 8          # the switches do change the answers
+    assert len(seen) >= 10         # the switches do change the answers

@@ -47,6 +47,7 @@ typedef struct orc_db {
     int32_t resharding, shared_space, reserved_space, pred_min;
     int32_t gpus_per_node, global_bs;
     double main_params, optimizer, memory_limit;
+    int32_t collective_memory;            /* args.consider_collective_memory (:462) */
 } orc_db;
 
 typedef struct orc_plans {
@@ -278,7 +279,7 @@ static double get_peak_activations(const stage_t *s, int *err) {   /* :419-447 *
     return best;
 }
 
-static double get_reserved_memory(const stage_t *s, double memory_weights, int *err) {   /* :449-485, no collective memory */
+static double get_reserved_memory(const stage_t *s, double memory_weights, int *err) {   /* :449-485 */
     const orc_db *db = s->db;
     double cur_f = 0, cur_b = 0;
     for (int i = 0; i < s->n - 1; ++i) {
@@ -287,6 +288,22 @@ static double get_reserved_memory(const stage_t *s, double memory_weights, int *
         if (db->field[F_RB][e] > cur_b) cur_b = db->field[F_RB][e];
     }
     double max_collective = 0;
+    if (db->collective_memory && db->resharding) {           /* :462-478, get_reshard_memory :262-273 */
+        for (int i = 1; i < s->n; ++i) {
+            int tp_p = 1 << s->tp_log[i - 1], dp_p = 1 << s->dp_log[i - 1], tp_c = 1 << s->tp_log[i], dp_c = 1 << s->dp_log[i];
+            spec_t prev = make_spec(db->spec_kind[((size_t)s->types[i - 1] * db->n_algo + s->algo[i - 1]) * 2 + 0], tp_p, dp_p);
+            spec_t cur = make_spec(db->spec_kind[((size_t)s->types[i] * db->n_algo + s->algo[i]) * 2 + 1], tp_c, dp_c);
+            int fp, bp, nd;
+            if (!reshard_primitives(&prev, &cur, &fp, &bp, &nd)) { *err = ORC_TYPE_ERROR; continue; }
+            double sz = db->field[F_IN][entry(db, s->types[i], op_m(s, i, err), s->tp_log[i], s->algo[i])];
+            int prims[2] = {fp, bp};
+            for (int k = 0; k < 2; ++k) {
+                if (prims[k] == PRIM_NONE) continue;
+                double c = (prims[k] == PRIM_ALL_GATHER || prims[k] == PRIM_ALL_TO_ALL) ? sz * nd : sz;
+                if (c > max_collective) max_collective = c;
+            }
+        }
+    }
     if (!db->pred_min) {
         double a = cur_f + cur_b;
         return (a >= memory_weights ? a : memory_weights) + max_collective;   /* max(a, w): first wins ties */

@@ -45,7 +45,8 @@ class _Db(ctypes.Structure):
                 ("n_intra", ctypes.c_int32), ("n_inter", ctypes.c_int32),
                 ("resharding", ctypes.c_int32), ("shared_space", ctypes.c_int32), ("reserved_space", ctypes.c_int32),
                 ("pred_min", ctypes.c_int32), ("gpus_per_node", ctypes.c_int32), ("global_bs", ctypes.c_int32),
-                ("main_params", ctypes.c_double), ("optimizer", ctypes.c_double), ("memory_limit", ctypes.c_double)]
+                ("main_params", ctypes.c_double), ("optimizer", ctypes.c_double), ("memory_limit", ctypes.c_double),
+                ("collective_memory", ctypes.c_int32)]
 
 
 class _Plans(ctypes.Structure):
@@ -82,8 +83,8 @@ class COracle:
         self.lib.orc_score.restype = ctypes.c_int
         self.lib.orc_score.argtypes = [ctypes.POINTER(_Db), ctypes.POINTER(_Plans), ctypes.c_int] + [ctypes.c_void_p] * 6 + [ctypes.c_int]
         args = orc.args
-        if args.consider_collective_memory or args.support_comm_predict:
-            raise NotImplementedError("the C oracle covers the default flags only")
+        if args.support_comm_predict:
+            raise NotImplementedError("support_comm_predict only changes a printed column: not restated in C")
         names = list(orc.op_list)
         self.type_index = {n: k for k, n in enumerate(names)}
         self.full_op_list = list(full_op_list)
@@ -147,6 +148,7 @@ class COracle:
         db.global_bs = int(global_batch_size)
         db.main_params, db.optimizer = float(args.memory_main_params), float(args.memory_optimizer)
         db.memory_limit = float(args.memory_limit)
+        db.collective_memory = int(bool(args.consider_collective_memory))
         self.db = db
 
     def score_arrays(self, num_stages, micro_bs, stage_len, tp_log, dp_log, algo, rc, strict=False, lists=False,

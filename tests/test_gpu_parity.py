@@ -180,9 +180,11 @@ def test_every_settings_combination_matches_the_c_oracle(name, torch_mod):
     db = synth.make_db(w, graph)
     batch = synth.make_plans(w, synth.make_tables(w), n_plans=3000, seed_offset=78)
     answers = set()
-    for pred, shared, reserved, resh in itertools.product(("MAX", "MIN"), (True, False), (True, False), (True, False)):
+    combos = [c + (False,) for c in itertools.product(("MAX", "MIN"), (True, False), (True, False), (True, False))]
+    combos += [(pred, shared, True, True, True) for pred in ("MAX", "MIN") for shared in (True, False)]   # collective memory
+    for pred, shared, reserved, resh, coll in combos:
         st = dataclasses.replace(synth.make_settings(w), memory_pred_type=pred, consider_shared_space=shared,
-                                 consider_reserved_space=reserved, resharding=resh)
+                                 consider_reserved_space=reserved, resharding=resh, consider_collective_memory=coll)
         tables = compile_tables(graph, db, st)
         ev = PlanEvaluator(tables)
         it, pk, fe, status = ev.score_host(batch, group_by_depth=shared)
@@ -190,12 +192,12 @@ def test_every_settings_combination_matches_the_c_oracle(name, torch_mod):
         ev.close()
         cit, cpk, cfe, cer, tl, ml = c_oracle_scores(tables, batch, threads=8, lists=True)
         assert not cer.any() and (status == 0).all()
-        assert np.array_equal(it, cit) and np.array_equal(pk, cpk) and np.array_equal(fe, cfe), (pred, shared, reserved, resh)
+        assert np.array_equal(it, cit) and np.array_equal(pk, cpk) and np.array_equal(fe, cfe), (pred, shared, reserved, resh, coll)
         S = batch.hdr[:256, 0] & 0xff
         used = np.arange(16)[None, :] < S[:, None]
         assert np.array_equal(rec[:, :, 16][used], ml[:256][used])
         answers.add((float(pk.sum()), float(it.sum())))
-    assert len(answers) >= 8
+    assert len(answers) >= 10
 
 
 @pytest.mark.parametrize("name", ["gpt3_1_3b", "wresnet_1b"])

@@ -123,9 +123,8 @@ def test_every_settings_combination_matches_the_oracle(name):
         for defer in (False, True):
             it, pk, fe, status, _ = emu_score(tables, batch, defer=defer)
             assert (status == 0).all() and np.array_equal(it, oit) and np.array_equal(pk, opk) and np.array_equal(fe, ofe), kw
-        if not kw.get("consider_collective_memory"):          # (the C restatement leaves that switch out)
-            cit, cpk, cfe, cer = c_oracle_scores(tables, batch)
-            assert not cer.any() and np.array_equal(cit, oit) and np.array_equal(cpk, opk) and np.array_equal(cfe, ofe), kw
+        cit, cpk, cfe, cer = c_oracle_scores(tables, batch)
+        assert not cer.any() and np.array_equal(cit, oit) and np.array_equal(cpk, opk) and np.array_equal(cfe, ofe), kw
         _, _, _, _, rec = emu_score(tables, batch, breakdown=True)
         for p, c in enumerate(cfgs):
             assert [rec[p, s, R_STAGE_MB] for s in range(c.num_stages)] == list(c.memory_list), kw

@@ -226,3 +226,25 @@ class EmuDeviceEvaluator(EmuEvaluator):
         return (torch.from_numpy(it), torch.from_numpy(pk), torch.from_numpy(fe), torch.from_numpy(st),
                 torch.from_numpy(rec) if rec is not None else None)
 
+
+
+def odd_workloads():
+    """Small workloads at the corners of the table geometry: one tp, one micro-batch size, 16 ops (one full
+    group, no padding), six micro-batch sizes with deep pipelines (rows in windows), stages wider than a node,
+    short ResNets with one row per op."""
+    from superscaler_amd.synth import Workload
+    return [
+        Workload("gpt_1tp_1mbs", "gpt", 1, 256, 128, 0, [1], 1, 1, 8, 2000.0, [1], 32, 0.5, seed=1),
+        Workload("gpt_16ops", "gpt", 1, 256, 128, 0, [1, 2], 2, 2, 8, 200.0, [1, 2], 64, 0.5, seed=2),
+        Workload("gpt_wide_stages", "gpt", 2, 512, 256, 0, [2, 4], 8, 2, 64, 500.0, [1, 2, 4, 8], 64, 0.4, seed=3),
+        Workload("gpt_6mbs_64gpus", "gpt", 1, 256, 128, 0, [1, 2, 4, 8, 16, 32], 64, 8, 128, 100.0, [1, 2, 4, 8, 16], 64, 0.6, seed=4),
+        Workload("gpt_3tp", "gpt", 3, 256, 128, 0, [4], 4, 4, 16, 300.0, [1, 2, 4], 64, 0.2, seed=5),
+        Workload("t5_1layer", "t5", 1, 256, 64, 32, [1, 2], 4, 4, 16, 300.0, [1, 2, 4], 64, 0.5, seed=6),
+        Workload("t5_1tp", "t5", 2, 256, 64, 32, [8], 2, 1, 16, 300.0, [1, 2], 64, 0.5, seed=7),
+        Workload("resnet_1111", "resnet", None, 32, 64, 0, [1, 2, 4], 4, 4, 32, 300.0, [1, 2, 4], 64, 0.5, conv=True,
+                 resnet_blocks=(1, 1, 1, 1), seed=8),
+        Workload("resnet_16gpus", "resnet", None, 32, 64, 0, [2], 16, 8, 32, 100.0, [1, 4, 16], 64, 0.5, conv=True,
+                 resnet_blocks=(2, 1, 1, 2), seed=9),
+        Workload("resnet_2tp", "resnet", None, 64, 64, 0, [1, 2, 4, 8], 8, 2, 64, 100.0, [1, 8], 64, 0.9, conv=True,
+                 resnet_blocks=(1, 2, 3, 1), seed=10),
+    ]

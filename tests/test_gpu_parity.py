@@ -328,6 +328,36 @@ def test_stage_records_match_c_oracle_lists(name, torch_mod):
         assert np.array_equal((rec[:, s, R_STAGE_MS] * nbm1 + tsum)[m], tl[m, s])
 
 
+def test_odd_table_geometries(torch_mod):
+    """Corners of the table geometry (helpers.odd_workloads: one tp, one micro-batch size, exactly 16 ops, six
+    micro-batch sizes, stages wider than a node, short ResNets) with 3,000 plans each: scores, flags and the
+    per-stage memory against the C oracle, in plain and in grouped storage, and the top 32."""
+    from superscaler_amd.evaluator import PlanEvaluator
+    from superscaler_amd.tables import R_STAGE_MB
+    from tests.helpers import odd_workloads
+    for w in odd_workloads():
+        tables = synth.make_tables(w)
+        batch = synth.make_plans(w, tables, n_plans=3000, seed_offset=5, workers=2)
+        print(f"[case] {w.name} ops={tables.graph.num_ops} windows={tables.n_windows}", flush=True)
+        cit, cpk, cfe, cer, tl, ml = c_oracle_scores(tables, batch, threads=8, lists=True)
+        assert not cer.any()
+        ev = PlanEvaluator(tables)
+        for grouped in (False, True):
+            it, pk, fe, st = ev.score_host(batch, group_by_depth=grouped)
+            assert (st == 0).all() and np.array_equal(it, cit) and np.array_equal(pk, cpk) and np.array_equal(fe, cfe), (w.name, grouped)
+        _, _, _, _, rec = ev.score_host(batch, breakdown=True)
+        S = (batch.hdr[:, 0] & 0xff).astype(int)
+        for s in range(16):
+            assert np.array_equal(rec[S > s, s, R_STAGE_MB], ml[S > s, s]), w.name
+        d = ev.upload(batch)
+        dit, _, dfe, _ = ev.score(d)[:4]
+        idx, val, cnt = ev.topk(dit, dfe, 32)
+        feas = np.flatnonzero(cfe)
+        order = feas[np.argsort(cit[feas], kind="stable")][:32]
+        assert int(cnt.item()) == len(order) and np.array_equal(idx.cpu().numpy()[:len(order)], order), w.name
+        ev.close()
+
+
 def test_known_answers_single_gpu_plans(golden_dir, torch_mod):
     """The reference tree's own single-GPU plans and published predictions
     (results/ref/perf_model_{time,mem}_large_{gpt,resnet}.csv), through the GPU path."""

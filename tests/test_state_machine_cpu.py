@@ -130,3 +130,24 @@ def test_every_settings_combination_matches_the_oracle(name):
             assert [rec[p, s, R_STAGE_MB] for s in range(c.num_stages)] == list(c.memory_list), kw
         seen.add((tuple(opk.tolist()), tuple(oit.tolist())))
     assert len(seen) >= 10         # the switches do change the answers
+
+
+def test_odd_table_geometries():
+    """Corners of the table geometry (see helpers.odd_workloads): state machine, the kernel's own loop and the C
+    restatement against the Python oracle, bit for bit."""
+    from tests.helpers import c_oracle_scores, emu_kernel_score, odd_workloads
+    shapes = set()
+    for w in odd_workloads():
+        tables = synth.make_tables(w)
+        batch = synth.make_plans(w, tables, n_plans=w.n_plans)
+        orc = oracle_for(tables)
+        oit, opk, ofe, _ = oracle_scores(orc, batch, tables)
+        for defer in (False, True):
+            it, pk, fe, st, _ = emu_score(tables, batch, defer=defer)
+            assert (st == 0).all() and np.array_equal(it, oit) and np.array_equal(pk, opk) and np.array_equal(fe, ofe), w.name
+        out = emu_kernel_score(tables, batch)
+        assert np.array_equal(out[0], oit) and np.array_equal(out[1], opk) and np.array_equal(out[2], ofe), w.name
+        cit, cpk, cfe, cer = c_oracle_scores(tables, batch)
+        assert not cer.any() and np.array_equal(cit, oit) and np.array_equal(cpk, opk) and np.array_equal(cfe, ofe), w.name
+        shapes.add((tables.graph.num_ops, len(tables.db.tp_list), len(tables.db.mbs_list), tables.n_windows))
+    assert len(shapes) == 10

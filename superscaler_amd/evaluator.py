@@ -212,6 +212,7 @@ class PlanEvaluator:
         self.handle = h
         self._deal_cache = {}
         self._topk_ws = None
+        self._small = None
 
     def close(self):
         if getattr(self, "handle", None):
@@ -424,9 +425,79 @@ class PlanEvaluator:
                       torch.from_numpy(np.ascontiguousarray(stage_idx)).to(self.device)]
         return out[3].cpu().numpy(), pick.cpu().numpy()
 
+    # ---- small host-in / host-out calls ------------------------------------------------------------
+    # The reference's search calls the cost model for one plan or one stage at a time, so the time of such
+    # a call is what a host-side search sees.  Small batches therefore go through one pinned buffer each
+    # way: the plans are laid out for the kernel on the host, one copy takes codes, headers and ranges to
+    # the device, one copy brings every output back.
+    SMALL_IO_BYTES = 1 << 20
+
+    def _small_io(self):
+        if self._small is None:
+            torch = self._torch
+            n = self.SMALL_IO_BYTES
+            h_in = torch.empty(n, dtype=torch.uint8, pin_memory=True)
+            h_out = torch.empty(n, dtype=torch.uint8, pin_memory=True)
+            self._small = (h_in, h_in.numpy(), torch.empty(n, dtype=torch.uint8, device=self.device),
+                           h_out, h_out.numpy(), torch.empty(n, dtype=torch.uint8, device=self.device))
+        return self._small
+
+    def _score_small(self, batch: PlanBatch, limit: float, strict: bool, breakdown: bool, ranges):
+        """score_host for a batch whose inputs and outputs fit SMALL_IO_BYTES; None if they do not."""
+        P, N = batch.codes.shape
+        G = (N + 15) // 16
+        breakdown = breakdown or ranges is not None
+        off_hdr = G * P * 16
+        off_rng = off_hdr + P * 16
+        n_in = off_rng + (P * 8 if ranges is not None else 0)
+        rec_bytes = P * MAX_STAGES * STAGE_REC * 8 if breakdown else 0
+        off_fe = 16 * P + rec_bytes
+        n_out = off_fe + 2 * P
+        if n_in > self.SMALL_IO_BYTES or n_out > self.SMALL_IO_BYTES:
+            return None
+        h_in, np_in, d_in, h_out, np_out, d_out = self._small_io()
+        lay = np_in[:off_hdr].reshape(G, P, 16)
+        if G * 16 == N:
+            lay[...] = batch.codes.reshape(P, G, 16).transpose(1, 0, 2)
+        else:
+            full = N // 16
+            if full:
+                lay[:full] = batch.codes[:, :full * 16].reshape(P, full, 16).transpose(1, 0, 2)
+            lay[full, :, :N - full * 16] = batch.codes[:, full * 16:]
+            lay[full, :, N - full * 16:] = 0
+        np_in[off_hdr:off_rng].view(np.uint32).reshape(P, 4)[...] = batch.hdr
+        if ranges is not None:
+            np_in[off_rng:n_in].view(np.uint32).reshape(P, 2)[...] = ranges
+        d_in[:n_in].copy_(h_in[:n_in], non_blocking=True)
+        if breakdown:
+            d_out[16 * P:off_fe].zero_()
+        base_in, base_out = d_in.data_ptr(), d_out.data_ptr()
+        struct = AceBatchStruct(base_in, base_in + off_hdr, base_in + off_rng if ranges is not None else None, P, None)
+        with self._torch.cuda.device(self.device):
+            rc = self.lib.ace_score_batch(self.handle, ctypes.byref(struct), limit, int(strict), base_out, base_out + 8 * P,
+                                          base_out + off_fe, base_out + off_fe + P,
+                                          base_out + 16 * P if breakdown else None, self._stream())
+        _check(self.lib, rc, "ace_score_batch")
+        h_out[:n_out].copy_(d_out[:n_out], non_blocking=True)
+        self._torch.cuda.current_stream(self.device).synchronize()
+        f64 = np_out[:off_fe].view(np.float64)
+        out = (f64[:P].copy(), f64[P:2 * P].copy(), np_out[off_fe:off_fe + P].copy(), np_out[off_fe + P:n_out].copy())
+        if breakdown:
+            out += (f64[2 * P:].reshape(P, MAX_STAGES, STAGE_REC).copy(),)
+        return out
+
     # convenience: host in, host out
     def score_host(self, batch: PlanBatch, memory_limit=None, strict=False, breakdown=False, ranges=None,
                    group_by_depth: bool = False):
+        if not group_by_depth and batch.n_plans <= 4096:
+            if ranges is None:
+                msg = validate_batch(batch, self.tables)
+                if msg:
+                    raise ValueError(msg)
+            limit = float(self.tables.settings.memory_limit if memory_limit is None else memory_limit)
+            out = self._score_small(batch, limit, strict, breakdown, ranges)
+            if out is not None:
+                return out
         d = self.upload(batch, ranges=ranges, group_by_depth=group_by_depth)
         out = self.score(d, memory_limit, strict, breakdown)
         self._torch.cuda.synchronize(self.device)

@@ -358,6 +358,34 @@ def test_odd_table_geometries(torch_mod):
         ev.close()
 
 
+def test_small_calls_take_the_same_answers_through_the_pinned_buffers(torch_mod):
+    """score_host sends small batches through one pinned buffer each way (layout done on the host); the
+    results must be the bytes of the general path (upload + score), for whole plans, stage records and
+    single-stage queries, with the last 16-op group full (16 ops) and partly filled (523, 134 ops)."""
+    from superscaler_amd.evaluator import PlanEvaluator
+    from tests.helpers import odd_workloads
+    for w in [synth.WORKLOADS["gpt3_13b"], synth.WORKLOADS["wresnet_1b"], odd_workloads()[1]]:
+        tables = synth.make_tables(w)
+        N = tables.graph.num_ops
+        ev = PlanEvaluator(tables)
+        for n in (1, 7, 300):
+            batch = synth.make_plans(w, tables, n_plans=n, seed_offset=n)
+            for breakdown in (False, True):
+                small = ev._score_small(batch, float(w.memory_limit), False, breakdown, None)
+                assert small is not None
+                big = ev.score(ev.upload(batch), breakdown=breakdown)
+                for a, b in zip(small, big):
+                    assert np.array_equal(a, b.cpu().numpy()), (w.name, n, breakdown)
+            # every plan's first stage as a single-stage query
+            cut = np.where((batch.codes[:, 1:] & 16) != 0, np.arange(1, N)[None, :], N).min(axis=1)
+            ranges = np.stack([np.zeros(n, dtype=np.uint32), cut.astype(np.uint32)], axis=1)
+            small = ev._score_small(batch, float(w.memory_limit), False, True, ranges)
+            big = ev.score(ev.upload(batch, ranges=ranges), breakdown=True)
+            assert np.array_equal(small[3], big[3].cpu().numpy())
+            assert np.array_equal(small[4][:, 0], big[4][:, 0].cpu().numpy()), (w.name, n)
+        ev.close()
+
+
 def test_known_answers_single_gpu_plans(golden_dir, torch_mod):
     """The reference tree's own single-GPU plans and published predictions
     (results/ref/perf_model_{time,mem}_large_{gpt,resnet}.csv), through the GPU path."""

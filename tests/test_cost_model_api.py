@@ -194,6 +194,48 @@ def test_errors_match_reference_behaviour(golden_dir):
         m.predict_stage_time(["enc-MLP-gelu", "encoder-embedding"], [0, 0], [1, 1], [1, 1], 1, [0, 0])
 
 
+@pytest.mark.gpu
+def test_module_level_calls_as_the_reference_makes_them(golden_dir):
+    """The way aceso_search.py / aceso_prims.py use the module (aceso_search.py:4, aceso_prims.py:7): an argparse
+    namespace, read_profiled_time(), then the functions by name -- against the reference's own vectors."""
+    import argparse
+    with open(os.path.join(golden_dir, "gpt_1_3B.json")) as f:
+        g = json.load(f)
+    ns = argparse.Namespace(model_name=g["model_name"], model_size=g["model_size"], micro_batch_size=g["micro_batch_size"],
+                            num_gpus_per_node=g["num_gpus_per_node"], num_nodes=g["num_nodes"],
+                            global_batch_size=g["global_batch_size"], memory_limit=g["memory_limit"], max_tp=None,
+                            num_layers=g["num_layers"], consider_shared_space=True, consider_reserved_space=True,
+                            flex_recompute=True, peak_mem_in_backward=0, memory_pred_type="MAX", resharding=None,
+                            consider_collective_memory=False, support_comm_predict=False)
+    acm.configure(ns)
+    try:
+        n_types = acm.read_profiled_time(g["model_name"], g["model_size"], os.path.join(golden_dir, "db_gpt_1_3B") + "/")
+        assert isinstance(n_types, int) and n_types == len(acm._m().db.op_names) > 0
+        for p in g["plans"][:6]:
+            c = cfg_of(g, acm._m(), p)
+            assert acm.predict_time_breakdown(c) is None
+            assert c.time_list == p["time_list"] and c.memory_list == p["memory_list"]
+            assert acm.get_reserved_memory_list(c) == p["reserved_memory_list"]
+            mbs = p["micro_batch_size"]
+            for s, st in enumerate(c.stages):
+                assert acm.predict_stage_time(st.ops, st.recompute_ops, st.tp_size, st.dp_size, mbs, st.algo) == p["stage_time"][s]
+                assert acm.predict_stage_memory(st.ops, st.recompute_ops, st.tp_size, st.dp_size, mbs, st.num_stages_behind,
+                                                st.algo) == p["stage_memory"][s]
+                assert acm.check_recompute(st.ops, mbs, st.tp_size, st.dp_size, st.num_stages_behind, st.algo) == p["check_recompute"][s]
+            for b, partner, k, metric, v, r in p["value_after_move"]:
+                gv, gr = acm.predict_value_after_move(c, b, partner, k, metric)
+                assert gv == v and list(gr) == r
+            for b, partner, k, dec, v in p["delta_time"]:
+                assert acm.wrap_predict_delta_time(c, b, partner, k, decrease=dec) == v
+            acm.update_recompute(c)
+            assert [st.recompute_ops for st in c.stages] == p["check_recompute"]
+    finally:
+        if acm._model is not None:
+            acm._model.close()
+        acm._model = None
+        acm.args = None
+
+
 def test_module_level_api_requires_configuration():
     acm._model = None
     with pytest.raises(RuntimeError):

@@ -68,18 +68,44 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     const long long out = a.order ? (long long)a.order[pl] : plan;
     const bool active = in_batch && out < g.P;
 
+    // RANGED: the workgroup walks only the 16-op groups that hold an op of one of its queries (a single-stage
+    // query covers a fraction of the sequence, and the walk is what such a call waits for)
+    ace_u2 range{0u, 0u};
+    int grp_begin = 0, grp_end = g.G;
+    if (RANGED) {
+        range = a.range[pl];
+        // (what PlanState::init() makes of a malformed range)
+        const bool ok = range.x < range.y && range.y <= (uint32_t)g.N;
+        uint32_t lo = ok ? range.x : 0u, hi = ok ? range.y : 1u;
+#ifndef ACE_HOST_EMU
+        unsigned int *red = reinterpret_cast<unsigned int *>(lds_raw);     // two words, before anything is staged there
+        if (tid == 0) { red[0] = 0xffffffffu; red[1] = 0u; }
+        ACE_SYNC();
+        atomicMin(&red[0], lo);
+        atomicMax(&red[1], hi);
+        ACE_SYNC();
+        lo = red[0];
+        hi = red[1];
+        ACE_SYNC();
+#endif
+        grp_begin = (int)(lo >> 4);
+        grp_end = (int)((hi + 15u) >> 4);
+    }
+    // the window that holds the first position walked
+    int w0 = 0;
+    if (RANGED && WIN)
+        while (w0 + 1 < a.n_windows && a.win_pos[w0 + 1] <= (grp_begin << 4)) ++w0;
+
     // small tables: pair kinds and the (micro-batch, stage gpus) LUT; without windows, every row
     for (int j = tid; j < a.rk_bytes; j += BLOCK) lds_raw[a.g.rk_lds_off + j] = a.pair_kinds[j];
     for (int j = tid; j < a.stg_words; j += BLOCK)
         reinterpret_cast<uint32_t *>(lds_raw + a.g.stg_lds_off)[j] = a.stage_lut[j];
-    stage_window<BLOCK>(a, lds_raw, 0, tid);        // every row, or the first window's
+    stage_window<BLOCK>(a, lds_raw, w0, tid);       // every row, or the first window's
     ACE_SYNC();
 
     const AceLds lds = ace_make_lds(lds_raw, lds_bytes);
     PlanState<BD, RANGED, DEFER, COLL> st;
     const ace_u4 h = a.hdr[pl];
-    ace_u2 range{0u, 0u};
-    if (RANGED) range = a.range[pl];
     st.init(g, lds, h, range);
     const double nbm1 = a.nbm1[st.bidx];
     double *rec = (BD && a.stage_out && active) ? a.stage_out + (size_t)out * (ACE_MAX_STAGES * ACE_STAGE_REC) : nullptr;
@@ -89,12 +115,12 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
         st.ws_stride = n_blocks * (uint32_t)BLOCK * (ACE_WS_REC / 2);
     }
 
-    int w = 1;
-    int next_win = WIN ? a.win_pos[1] : 0x7fffffff;
-    ace_u4 cw = a.codes[pl];                 // sixteen op bytes of this plan
+    int w = w0 + 1;
+    int next_win = WIN ? a.win_pos[w] : 0x7fffffff;
+    ace_u4 cw = a.codes[(size_t)grp_begin * g.P + pl];     // sixteen op bytes of this plan
     if (!RANGED) st.begin(g, lds, 0, cw.x & 0xffu, a.pos_info[0]);
-    uint32_t pinfo = 0;                      // descriptor of the previous group's last position
-    for (int grp = 0; grp < g.G; ++grp) {
+    uint32_t pinfo = grp_begin ? a.pos_info[(grp_begin << 4) - 1] : 0u;    // descriptor of the previous group's last position
+    for (int grp = grp_begin; grp < grp_end; ++grp) {
         const int base = grp << 4;
         // the sixteen position descriptors of this group: scalar loads (the array is padded)
         const ace_u4 *ip = reinterpret_cast<const ace_u4 *>(a.pos_info + base);

@@ -292,7 +292,8 @@ def test_recompute_arrays_gpu_equals_cpu_build():
     m = acm.CostModel(st, synth.make_db(w, graph), graph)
     try:
         batch = synth.make_plans(w, m.tables, n_plans=2048, seed_offset=9)
-        on_gpu = m.update_recompute_arrays(batch)
+        on_gpu = m.update_recompute_arrays(batch, on_device=False)
+        assert np.array_equal(on_gpu.codes, m.update_recompute_arrays(batch).codes)      # selection on the device
         real, m._evaluator = m._evaluator, EmuEvaluator(m.tables)
         on_cpu = m.update_recompute_arrays(batch)
         m._evaluator = real
@@ -347,7 +348,7 @@ def test_recompute_on_the_device_equals_the_array_form(name, limit):
     m = acm.CostModel(st, synth.make_db(w, graph), graph)
     try:
         batch = synth.make_plans(w, m.tables, n_plans=1500, seed_offset=17)
-        want = m.update_recompute_arrays(batch)
+        want = m.update_recompute_arrays(batch, on_device=False)
         d = m.update_recompute_device(m.evaluator.upload(batch))
         N, G = batch.num_ops, (batch.num_ops + 15) // 16
         got = d.codes.permute(1, 0, 2).reshape(batch.n_plans, G * 16).cpu().numpy()

@@ -386,6 +386,36 @@ def test_small_calls_take_the_same_answers_through_the_pinned_buffers(torch_mod)
         ev.close()
 
 
+def test_handles_coexist_and_release_their_memory(torch_mod):
+    """Two handles with different tables alive at once (interleaved launches, one of them with windowed rows)
+    keep to their own tables and workspaces; creating and destroying handles leaves no device memory behind."""
+    from superscaler_amd.evaluator import PlanEvaluator
+    torch = torch_mod
+    ta, tb = synth.make_tables(synth.WORKLOADS["gpt3_1_3b"]), synth.make_tables(synth.WORKLOADS["wresnet_1b"])
+    ba = synth.make_plans(synth.WORKLOADS["gpt3_1_3b"], ta, n_plans=5000, seed_offset=3)
+    bb = synth.make_plans(synth.WORKLOADS["wresnet_1b"], tb, n_plans=5000, seed_offset=3)
+    want_a, want_b = c_oracle_scores(ta, ba, threads=8), c_oracle_scores(tb, bb, threads=8)
+    ea, eb = PlanEvaluator(ta), PlanEvaluator(tb)
+    da, db = ea.upload(ba), eb.upload(bb)
+    for _ in range(3):
+        oa, ob = ea.score(da), eb.score(db)
+        oa2 = ea.score(da, breakdown=True)
+        for got, want in ((oa, want_a), (ob, want_b), (oa2, want_a)):
+            assert all(np.array_equal(g.cpu().numpy(), w) for g, w in zip(got[:3], want[:3]))
+    ea.close()
+    eb.close()
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    free0 = torch.cuda.mem_get_info()[0]
+    for k in range(40):
+        ev = PlanEvaluator(ta if k % 2 else tb)
+        ev.score_host(ba.slice(0, 2000) if k % 2 else bb.slice(0, 2000))        # allocates the handle's workspace too
+        ev.close()
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    assert free0 - torch.cuda.mem_get_info()[0] < (8 << 20)
+
+
 def test_known_answers_single_gpu_plans(golden_dir, torch_mod):
     """The reference tree's own single-GPU plans and published predictions
     (results/ref/perf_model_{time,mem}_large_{gpt,resnet}.csv), through the GPU path."""

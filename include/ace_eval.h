@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define ACE_ABI_VERSION 5
+#define ACE_ABI_VERSION 6
 #define ACE_MAX_STAGES 16      /* aceso_utils.py:502: end_num_stages = min(num_gpus, 16) */
 #define ACE_STAGE_REC 18       /* doubles per stage record, see ACE_R_* */
 
@@ -148,7 +148,8 @@ void ace_destroy(ace_handle_t *h);
  * gen_megatron_plan.py:111).
  *  d_iter_ms, d_peak_mb: double[n_plans];  d_feasible, d_status: uint8[n_plans] (d_status may be NULL)
  *  d_stage_out: NULL, or double[n_plans][ACE_MAX_STAGES][ACE_STAGE_REC] receiving the per-stage
- *  quantities predict_time_breakdown / predict_stage_time / predict_stage_memory are made of.
+ *  quantities predict_time_breakdown / predict_stage_time / predict_stage_memory are made of; for a
+ *  batch of single-stage queries (batch->d_range) one record each: double[n_plans][ACE_STAGE_REC].
  * Plain scoring (no d_stage_out, no d_range) uses a workspace owned by the handle (80 bytes per plan
  * and stage, allocated on first use and grown when a larger batch arrives: that call allocates), so
  * scoring calls on one handle must be stream-ordered with respect to each other. */

@@ -30,7 +30,7 @@ struct AceKernelArgs {
     int32_t n_windows, row_doubles, rk_bytes, stg_words;
     double *iter_ms, *peak_mb;
     uint8_t *feasible, *status;
-    double *stage_out;
+    double *stage_out;          // [P][ACE_MAX_STAGES][ACE_STAGE_REC], single-stage queries [P][ACE_STAGE_REC]
     double *stage_ws;           // [ACE_MAX_STAGES][plans rounded up to whole workgroups][ACE_WS_REC] for deferred stage tails
 };
 
@@ -108,7 +108,9 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     const ace_u4 h = a.hdr[pl];
     st.init(g, lds, h, range);
     const double nbm1 = a.nbm1[st.bidx];
-    double *rec = (BD && a.stage_out && active) ? a.stage_out + (size_t)out * (ACE_MAX_STAGES * ACE_STAGE_REC) : nullptr;
+    // (a single-stage query has one record, a whole plan one per possible stage)
+    const size_t rec_doubles = RANGED ? (size_t)ACE_STAGE_REC : (size_t)(ACE_MAX_STAGES * ACE_STAGE_REC);
+    double *rec = (BD && a.stage_out && active) ? a.stage_out + (size_t)out * rec_doubles : nullptr;
     if (DEFER) {
         // stage-major: the records of one stage of consecutive plans are adjacent (padded lanes own a slot too)
         rec = a.stage_ws + (size_t)plan * ACE_WS_REC;

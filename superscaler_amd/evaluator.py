@@ -244,7 +244,8 @@ class PlanEvaluator:
 
     def score(self, dbatch: DeviceBatch, memory_limit: Optional[float] = None, strict: bool = False,
               breakdown: bool = False, out=None):
-        """Launch the scoring kernel; returns device tensors (iter_ms, peak_mb, feasible, status[, stage records])."""
+        """Launch the scoring kernel; returns device tensors (iter_ms, peak_mb, feasible, status[, stage records
+        [P, 16, STAGE_REC]; [P, 1, STAGE_REC] for single-stage queries])."""
         torch = self._torch
         P = dbatch.n_plans
         limit = float(self.tables.settings.memory_limit if memory_limit is None else memory_limit)
@@ -256,7 +257,9 @@ class PlanEvaluator:
         else:
             it, pk, fe, st = out
         breakdown = breakdown or dbatch.ranges is not None
-        rec = torch.zeros((P, MAX_STAGES, STAGE_REC), dtype=torch.float64, device=self.device) if breakdown else None
+        # (a single-stage query has one record)
+        n_rec = 1 if dbatch.ranges is not None else MAX_STAGES
+        rec = torch.zeros((P, n_rec, STAGE_REC), dtype=torch.float64, device=self.device) if breakdown else None
         with torch.cuda.device(self.device):
             rc = self.lib.ace_score_batch(self.handle, ctypes.byref(dbatch.struct), limit, int(strict),
                                           it.data_ptr(), pk.data_ptr(), fe.data_ptr(), st.data_ptr(),
@@ -450,7 +453,8 @@ class PlanEvaluator:
         off_hdr = G * P * 16
         off_rng = off_hdr + P * 16
         n_in = off_rng + (P * 8 if ranges is not None else 0)
-        rec_bytes = P * MAX_STAGES * STAGE_REC * 8 if breakdown else 0
+        n_rec = 1 if ranges is not None else MAX_STAGES          # a single-stage query has one record
+        rec_bytes = P * n_rec * STAGE_REC * 8 if breakdown else 0
         off_fe = 16 * P + rec_bytes
         n_out = off_fe + 2 * P
         if n_in > self.SMALL_IO_BYTES or n_out > self.SMALL_IO_BYTES:
@@ -483,7 +487,7 @@ class PlanEvaluator:
         f64 = np_out[:off_fe].view(np.float64)
         out = (f64[:P].copy(), f64[P:2 * P].copy(), np_out[off_fe:off_fe + P].copy(), np_out[off_fe + P:n_out].copy())
         if breakdown:
-            out += (f64[2 * P:].reshape(P, MAX_STAGES, STAGE_REC).copy(),)
+            out += (f64[2 * P:].reshape(P, n_rec, STAGE_REC).copy(),)
         return out
 
     # convenience: host in, host out

@@ -50,7 +50,7 @@ void score_one(const ace_tables_t *t, const AceGeom &g, std::vector<unsigned cha
 extern "C" int ace_emu_score(const ace_tables_t *t, const uint8_t *codes /* [P][N] plan-major */,
                              const uint32_t *hdr /* [P][4] */, const uint32_t *range /* nullable [P][2] */,
                              long long P, double memory_limit, int strict, int defer, double *iter_ms, double *peak_mb,
-                             uint8_t *feasible, uint8_t *status, double *stage_out /* nullable [P][16][18] */) {
+                             uint8_t *feasible, uint8_t *status, double *stage_out /* nullable [P][16][18]; with ranges [P][18] */) {
     const int C = t->n_tp * t->n_algo;
     AceGeom g;
     memset(&g, 0, sizeof(g));
@@ -80,7 +80,7 @@ extern "C" int ace_emu_score(const ace_tables_t *t, const uint8_t *codes /* [P][
         memcpy(&h, hdr + 4 * p, 16);
         ace_u2 rg{0u, 0u};
         if (range) memcpy(&rg, range + 2 * p, 8);
-        double *rec = stage_out ? stage_out + (size_t)p * ACE_MAX_STAGES * ACE_STAGE_REC : nullptr;
+        double *rec = stage_out ? stage_out + (size_t)p * (range ? 1 : ACE_MAX_STAGES) * ACE_STAGE_REC : nullptr;
         const uint8_t *c = codes + (size_t)p * g.N;
         double iter, peak;
         uint8_t feas, st;
@@ -186,7 +186,7 @@ extern "C" int ace_emu_kernel(const ace_tables_t *t, const uint8_t *codes, const
     a.peak_mb = (double *)pool.place(peak_mb, (size_t)P * 8, 8);
     a.feasible = (uint8_t *)pool.place(feasible, (size_t)P, 1);
     a.status = status ? (uint8_t *)pool.place(status, (size_t)P, 1) : nullptr;
-    const size_t rec_bytes = (size_t)P * ACE_MAX_STAGES * ACE_STAGE_REC * 8;
+    const size_t rec_bytes = (size_t)P * (range ? 1 : ACE_MAX_STAGES) * ACE_STAGE_REC * 8;
     a.stage_out = stage_out ? (double *)pool.place(stage_out, rec_bytes, 8) : nullptr;   // (records of unused stages stay as the caller left them)
     unsigned char *lds = (unsigned char *)pool.place(nullptr, lds_bytes);
     const bool win = t->n_windows > 1;

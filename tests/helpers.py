@@ -74,7 +74,7 @@ def emu_score(tables, batch, memory_limit=None, strict=False, breakdown=False, r
     hdr = np.ascontiguousarray(batch.hdr)
     it = np.zeros(P); pk = np.zeros(P)
     fe = np.zeros(P, dtype=np.uint8); st = np.zeros(P, dtype=np.uint8)
-    rec = np.zeros((P, 16, 18)) if (breakdown or ranges is not None) else None
+    rec = np.zeros((P, 1 if ranges is not None else 16, 18)) if (breakdown or ranges is not None) else None
     limit = tables.settings.memory_limit if memory_limit is None else memory_limit
     if ranges is not None:
         ranges = np.ascontiguousarray(ranges, dtype=np.uint32)
@@ -111,7 +111,7 @@ def emu_kernel_score(tables, batch, memory_limit=None, strict=False, breakdown=F
     if ranges is not None:
         ranges = np.ascontiguousarray(ranges, dtype=np.uint32)
         breakdown = True
-    rec = np.zeros((P, 16, 18)) if breakdown else None
+    rec = np.zeros((P, 1 if ranges is not None else 16, 18)) if breakdown else None
     limit = tables.settings.memory_limit if memory_limit is None else memory_limit
     vp = ctypes.c_void_p
     if order is not None:

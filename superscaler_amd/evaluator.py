@@ -135,6 +135,27 @@ def depth_order(batch: PlanBatch) -> np.ndarray:
     return perm[deal_slots(P)]
 
 
+def pack_small_inputs(buf: np.ndarray, batch: PlanBatch, ranges) -> int:
+    """Lay a small batch out for the kernel in `buf` (uint8): codes [ceil(N/16)][P][16] (zero padded), then the
+    headers uint32 [P][4], then the ranges uint32 [P][2] if given.  Returns the number of bytes used."""
+    P, N = batch.codes.shape
+    G = (N + 15) // 16
+    off_hdr = G * P * 16
+    off_rng = off_hdr + P * 16
+    n_in = off_rng + (P * 8 if ranges is not None else 0)
+    lay = buf[:off_hdr].reshape(G, P, 16)
+    full = N // 16
+    if full:
+        lay[:full] = batch.codes[:, :full * 16].reshape(P, full, 16).transpose(1, 0, 2)
+    if full < G:
+        lay[full, :, :N - full * 16] = batch.codes[:, full * 16:]
+        lay[full, :, N - full * 16:] = 0
+    buf[off_hdr:off_rng].view(np.uint32).reshape(P, 4)[...] = batch.hdr
+    if ranges is not None:
+        buf[off_rng:n_in].view(np.uint32).reshape(P, 2)[...] = ranges
+    return n_in
+
+
 class DeviceBatch:
     """A PlanBatch resident in HBM in the layout the kernel streams."""
 
@@ -460,18 +481,7 @@ class PlanEvaluator:
         if n_in > self.SMALL_IO_BYTES or n_out > self.SMALL_IO_BYTES:
             return None
         h_in, np_in, d_in, h_out, np_out, d_out = self._small_io()
-        lay = np_in[:off_hdr].reshape(G, P, 16)
-        if G * 16 == N:
-            lay[...] = batch.codes.reshape(P, G, 16).transpose(1, 0, 2)
-        else:
-            full = N // 16
-            if full:
-                lay[:full] = batch.codes[:, :full * 16].reshape(P, full, 16).transpose(1, 0, 2)
-            lay[full, :, :N - full * 16] = batch.codes[:, full * 16:]
-            lay[full, :, N - full * 16:] = 0
-        np_in[off_hdr:off_rng].view(np.uint32).reshape(P, 4)[...] = batch.hdr
-        if ranges is not None:
-            np_in[off_rng:n_in].view(np.uint32).reshape(P, 2)[...] = ranges
+        pack_small_inputs(np_in, batch, ranges)
         d_in[:n_in].copy_(h_in[:n_in], non_blocking=True)
         if breakdown:
             d_out[16 * P:off_fe].zero_()

@@ -85,3 +85,27 @@ def test_json_form_and_legality(golden_dir, small):
     assert check_legality(cfg, 1, 1, 1)
     assert check_legality(c, w.num_gpus, w.gpus_per_node, 1) == all(s.num_gpus in (1, 2, 4, 8) for s in c.stages)
     assert not check_legality(c, w.num_gpus + 1, w.gpus_per_node, 1)
+
+
+def test_small_call_packing_is_the_kernel_layout():
+    """evaluator.pack_small_inputs (one pinned buffer for codes, headers and ranges of a small host call) against
+    the plan-minor layout built the plain way, with the last 16-op group full, partly filled and the only one."""
+    import numpy as np
+    from superscaler_amd.evaluator import pack_small_inputs
+    from superscaler_amd.plan import PlanBatch
+    from tests.helpers import kernel_layout
+    rng = np.random.default_rng(5)
+    for P, N in ((1, 523), (7, 16), (33, 134), (5, 9), (64, 1251), (3, 32)):
+        codes = rng.integers(0, 32, size=(P, N), dtype=np.uint8)
+        hdr = rng.integers(0, 2 ** 32, size=(P, 4), dtype=np.uint64).astype(np.uint32)
+        ranges = rng.integers(0, N, size=(P, 2), dtype=np.uint64).astype(np.uint32)
+        G = (N + 15) // 16
+        for rg in (None, ranges):
+            buf = np.full(G * P * 16 + P * 16 + P * 8 + 64, 0xAB, dtype=np.uint8)
+            n = pack_small_inputs(buf, PlanBatch(codes, hdr), rg)
+            assert n == G * P * 16 + P * 16 + (P * 8 if rg is not None else 0)
+            assert np.array_equal(buf[:G * P * 16].reshape(G, P, 16), kernel_layout(codes))
+            assert np.array_equal(buf[G * P * 16:G * P * 16 + P * 16].view(np.uint32).reshape(P, 4), hdr)
+            if rg is not None:
+                assert np.array_equal(buf[G * P * 16 + P * 16:n].view(np.uint32).reshape(P, 2), rg)
+            assert (buf[n:] == 0xAB).all()

@@ -503,16 +503,16 @@ class PlanEvaluator:
     # convenience: host in, host out
     def score_host(self, batch: PlanBatch, memory_limit=None, strict=False, breakdown=False, ranges=None,
                    group_by_depth: bool = False):
+        if ranges is None:
+            msg = validate_batch(batch, self.tables)
+            if msg:
+                raise ValueError(msg)
         if not group_by_depth and batch.n_plans <= 4096:
-            if ranges is None:
-                msg = validate_batch(batch, self.tables)
-                if msg:
-                    raise ValueError(msg)
             limit = float(self.tables.settings.memory_limit if memory_limit is None else memory_limit)
             out = self._score_small(batch, limit, strict, breakdown, ranges)
             if out is not None:
                 return out
-        d = self.upload(batch, ranges=ranges, group_by_depth=group_by_depth)
+        d = self.upload(batch, validate=False, ranges=ranges, group_by_depth=group_by_depth)
         out = self.score(d, memory_limit, strict, breakdown)
         self._torch.cuda.synchronize(self.device)
         return tuple(None if t is None else t.cpu().numpy() for t in out)

@@ -234,6 +234,8 @@ class PlanEvaluator:
         self._deal_cache = {}
         self._topk_ws = None
         self._small = None
+        self._ws_slots = 0          # plans the handle's workspace of deferred stage tails holds (as the library sizes it)
+        self._graphs_alive = 0
 
     def close(self):
         if getattr(self, "handle", None):
@@ -278,6 +280,14 @@ class PlanEvaluator:
         else:
             it, pk, fe, st = out
         breakdown = breakdown or dbatch.ranges is not None
+        if not breakdown:
+            # plain scoring uses the handle's workspace, which grows (is reallocated) for a larger batch:
+            # a captured step holds its address
+            slots = -(-P // 1024) * 1024
+            if self._graphs_alive and slots > self._ws_slots:
+                raise AceError("this batch would reallocate the workspace that a captured step of this evaluator uses: "
+                               "capture after the largest batch has been scored, or use another evaluator")
+            self._ws_slots = max(self._ws_slots, slots)
         # (a single-stage query has one record)
         n_rec = 1 if dbatch.ranges is not None else MAX_STAGES
         rec = torch.zeros((P, n_rec, STAGE_REC), dtype=torch.float64, device=self.device) if breakdown else None
@@ -304,6 +314,14 @@ class PlanEvaluator:
                                    self._stream())
         _check(self.lib, rc, "ace_topk")
         return idx, val, cnt
+
+    def capture_step(self, dbatch: DeviceBatch, k: int, memory_limit: Optional[float] = None, strict: bool = False):
+        """Score + top-k of a resident batch recorded once in a HIP graph (the library's launches record into a
+        capturing stream as they are; nothing in them clears memory with a memset node).  Returns a StepGraph:
+        `replay()` runs the recorded launches again on the batch's current bytes and returns the same output
+        tensors ((iter_ms, peak_mb, feasible, status), (indices, times, count)).  For a batch that is scored
+        again and again after edits in place; the seventeen launches of a step then cost one submission."""
+        return StepGraph(self, dbatch, k, memory_limit, strict)
 
     def time_score_kernel(self, dbatch: DeviceBatch, reps: int, memory_limit: Optional[float] = None) -> float:
         """Average scoring-kernel duration in ms over `reps` back-to-back launches (hipEvents on the
@@ -516,3 +534,48 @@ class PlanEvaluator:
         out = self.score(d, memory_limit, strict, breakdown)
         self._torch.cuda.synchronize(self.device)
         return tuple(None if t is None else t.cpu().numpy() for t in out)
+
+
+class StepGraph:
+    """See PlanEvaluator.capture_step."""
+
+    def __init__(self, ev: PlanEvaluator, dbatch: DeviceBatch, k: int, memory_limit=None, strict=False):
+        torch = ev._torch
+        self.batch = dbatch                       # the graph holds its addresses
+        P = dbatch.n_plans
+        self.scores = (torch.empty(P, dtype=torch.float64, device=ev.device), torch.empty(P, dtype=torch.float64, device=ev.device),
+                       torch.empty(P, dtype=torch.uint8, device=ev.device), torch.empty(P, dtype=torch.uint8, device=ev.device))
+        # one eager step on a side stream first: the handle's workspace and the top-k workspace are allocated
+        # there, never inside the capture
+        side = torch.cuda.Stream(device=ev.device)
+        side.wait_stream(torch.cuda.current_stream(ev.device))
+        with torch.cuda.stream(side):
+            ev.score(dbatch, memory_limit, strict, out=self.scores)
+            ev.topk(self.scores[0], self.scores[2], k)
+        torch.cuda.current_stream(ev.device).wait_stream(side)
+        torch.cuda.synchronize(ev.device)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            ev.score(dbatch, memory_limit, strict, out=self.scores)
+            self.top = ev.topk(self.scores[0], self.scores[2], k)
+        self._ev = ev
+        ev._graphs_alive += 1
+
+    def replay(self):
+        if self._ev is None or not self._ev.handle:
+            raise AceError("the captured step was released, or its evaluator closed")
+        self.graph.replay()
+        return self.scores, self.top
+
+    def release(self):
+        """Forget the recorded launches (the evaluator may then score larger batches again)."""
+        if self._ev is not None:
+            self._ev._graphs_alive -= 1
+            self._ev = None
+            self.graph = None
+
+    def __del__(self):
+        try:
+            self.release()
+        except Exception:
+            pass

@@ -416,6 +416,53 @@ def test_handles_coexist_and_release_their_memory(torch_mod):
     assert free0 - torch.cuda.mem_get_info()[0] < (8 << 20)
 
 
+def test_captured_step_replays_to_the_eager_results(torch_mod):
+    """score + top-k recorded in a HIP graph: four replays, with eager launches and synchronisations between
+    them and the outputs cleared before each, give the eager step's bytes; after an edit of the resident
+    plans in place the replay gives the edited batch's results."""
+    from superscaler_amd.evaluator import PlanEvaluator
+    torch = torch_mod
+    w = synth.WORKLOADS["gpt3_13b"]
+    tables = synth.make_tables(w)
+    batch = synth.make_plans(w, tables, n_plans=200000, seed_offset=12, workers=4)
+    ev = PlanEvaluator(tables)
+    d = ev.upload(batch)
+    eager = ev.score(d)
+    etop = ev.topk(eager[0], eager[2], 64)
+    torch.cuda.synchronize()
+    want = [t.clone() for t in eager] + [t.clone() for t in etop]
+    g = ev.capture_step(d, 64)
+    for r in range(4):
+        for t in g.scores:
+            t.zero_()
+        (scores, top) = g.replay()
+        torch.cuda.synchronize()
+        assert all(torch.equal(a, b) for a, b in zip(list(scores) + list(top), want)), r
+        other = ev.score(ev.upload(batch.slice(0, 5000)))          # eager work between the replays
+        ev.topk(other[0], other[2], 8)
+        torch.cuda.synchronize()
+    # edit in place: clear every recompute bit of the resident plans, replay, compare with a fresh eager step
+    d.codes &= 0xF7
+    (scores, top) = g.replay()
+    torch.cuda.synchronize()
+    fresh = ev.score(d)
+    ftop = ev.topk(fresh[0], fresh[2], 64)
+    torch.cuda.synchronize()
+    assert all(torch.equal(a, b) for a, b in zip(list(scores) + list(top), list(fresh) + list(ftop)))
+    assert not torch.equal(scores[1], want[1])
+    # a larger batch would make the library reallocate the workspace whose address the graph holds
+    from superscaler_amd.evaluator import AceError
+    bigger = ev.upload(synth.make_plans(w, tables, n_plans=201000, seed_offset=13, workers=4))
+    with pytest.raises(AceError):
+        ev.score(bigger)
+    g.release()
+    ev.score(bigger)
+    with pytest.raises(AceError):
+        g.replay()
+    torch.cuda.synchronize()
+    ev.close()
+
+
 def test_known_answers_single_gpu_plans(golden_dir, torch_mod):
     """The reference tree's own single-GPU plans and published predictions
     (results/ref/perf_model_{time,mem}_large_{gpt,resnet}.csv), through the GPU path."""

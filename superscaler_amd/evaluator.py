@@ -280,8 +280,8 @@ class PlanEvaluator:
         else:
             it, pk, fe, st = out
         breakdown = breakdown or dbatch.ranges is not None
-        if not breakdown:
-            # plain scoring uses the handle's workspace, which grows (is reallocated) for a larger batch:
+        if not breakdown and self.tables.n_windows == 1:
+            # plain scoring with every row resident uses the handle's workspace, which grows (is reallocated) for a larger batch:
             # a captured step holds its address
             slots = -(-P // 1024) * 1024
             if self._graphs_alive and slots > self._ws_slots:

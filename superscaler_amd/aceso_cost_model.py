@@ -140,7 +140,7 @@ class CostModel:
         ideal_per_gpu, eff_loss_list, recomp_list = [], [], []
         time_strings, memory_strings = [], []
         for i in range(config.num_stages):
-            r = [float(x) for x in rec[i]]
+            r = rec[i].tolist()
             num_gpus = config.stages[i].num_gpus
             fwd, bwd, in_comm, out_comm, recomp = r[R_FWD], r[R_BWD], r[R_IN_COMM], r[R_OUT_COMM], r[R_RECOMP]
             sum_time = (fwd + bwd + in_comm + out_comm + recomp) / 1000
@@ -277,7 +277,7 @@ class CostModel:
         """aceso_cost_model.py:493-512 (ms; cross-node bandwidth never used here)."""
         if len(ops) == 0:
             return 0 / 1000
-        r = [float(x) for x in self._stage_records([(ops, recompute_ops, tp_size, dp_size, base_batch_size, 0, algo_list)])[0]]
+        r = self._stage_records([(ops, recompute_ops, tp_size, dp_size, base_batch_size, 0, algo_list)])[0].tolist()
         fwd_comp, bwd_comp, in_comm, out_comm, recomp_time = r[R_FWD], r[R_BWD], r[R_IN_COMM], r[R_OUT_COMM], r[R_RECOMP]
         if not delta:
             sum_time = fwd_comp + bwd_comp + in_comm + out_comm + recomp_time
@@ -290,8 +290,7 @@ class CostModel:
     def predict_stage_memory(self, ops, recompute_ops, tp_size, dp_size, base_batch_size, num_stages_behind,
                              algo_list, breakdown=False):
         """aceso_cost_model.py:514-539 (MB)."""
-        r = [float(x) for x in self._stage_records([(ops, recompute_ops, tp_size, dp_size, base_batch_size,
-                                                      num_stages_behind, algo_list)])[0]]
+        r = self._stage_records([(ops, recompute_ops, tp_size, dp_size, base_batch_size, num_stages_behind, algo_list)])[0].tolist()
         mw, mg, mo, ma, mp, mr = self._memory_breakdown(r, num_stages_behind)
         if breakdown:
             return mw, mg, mo, ma, mp, mr
@@ -407,7 +406,7 @@ class CostModel:
         rec = self._stage_records([query(k, rcs[k]) for k in range(n)])
         state, pending = [], []
         for k, (ops, micro_bs, tp_size, dp_size, nsb, algo_list) in enumerate(queries):
-            mw, mg, mo, ma, mp, mr = self._memory_breakdown([float(x) for x in rec[k]], nsb)
+            mw, mg, mo, ma, mp, mr = self._memory_breakdown(rec[k].tolist(), nsb)
             stage_memory = (mw + mg + mo + ma + mp + mr) + args.peak_mem_in_backward
             # get_peak_activations of an all-zero recompute list is 0 (:421)
             st = {"mem": stage_memory, "saved": 0, "peak": 0, "groups": None, "stale": False}

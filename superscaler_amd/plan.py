@@ -11,6 +11,7 @@ plus four 32-bit words per plan --
     [1..2] log2(stage gpus), 4 bits per stage
     [3] in-cross-node bit per stage | out-cross-node bits << 16   (aceso_cost_model.py:572-574)
 """
+import itertools
 import json
 from dataclasses import dataclass, field
 from typing import List, Optional, Sequence
@@ -153,48 +154,56 @@ class PlanBatch:
         N = tables.graph.num_ops
         A = db.n_algo
         mbs_index = {m: k for k, m in enumerate(db.mbs_list)}
-        tp_index = {t: k for k, t in enumerate(db.tp_list)}
+        # tp size -> index in the profile database (0xff: not profiled), as a lookup table
+        tp_lut = np.full(max(db.tp_list) + 2, 0xff, dtype=np.uint8)
+        tp_lut[np.asarray(db.tp_list)] = np.arange(len(db.tp_list), dtype=np.uint8)
         P = len(configs)
         codes = np.zeros((P, N), dtype=np.uint8)
         hdr = np.zeros((P, 4), dtype=np.uint32)
         gpn = tables.settings.num_gpus_per_node
+        chain = itertools.chain.from_iterable
         for p, cfg in enumerate(configs):
             S = cfg.num_stages
             if S < 1 or S > MAX_STAGES:
                 raise ValueError(f"plan {p}: {S} stages (1..{MAX_STAGES} supported)")
             bidx = mbs_index[cfg.micro_bs]
-            pos = 0
+            stages = cfg.stages
+            lens = [len(st.ops) for st in stages]
             glogs = 0
             gl = []
-            for s, st in enumerate(cfg.stages):
-                n = len(st.ops)
-                if n == 0:
+            for s, st in enumerate(stages):
+                if lens[s] == 0:
                     raise ValueError(f"plan {p}: stage {s} is empty")
                 g = st.tp_size[0] * st.dp_size[0]
                 if g & (g - 1) or g.bit_length() - 1 > 15:
                     raise ValueError(f"plan {p}: stage {s} has {g} devices (power of two expected)")
                 gl.append(g)
                 glogs |= (g.bit_length() - 1) << (4 * s)
-                tp = np.asarray(st.tp_size, dtype=np.int64)
-                dp = np.asarray(st.dp_size, dtype=np.int64)
-                if np.any(tp * dp != g):
-                    raise ValueError(f"plan {p}: stage {s} mixes tp*dp products")
                 for d in set(st.dp_size):
                     if cfg.micro_bs // d not in mbs_index:
                         raise KeyError(cfg.micro_bs // d)
-                try:
-                    t = np.array([tp_index[x] for x in st.tp_size], dtype=np.uint8)
-                except KeyError as e:
-                    raise ValueError(f"plan {p}: tp size {e} is not in the profile database") from None
-                al = np.asarray(st.algo, dtype=np.uint8)
-                if np.any(al >= A):
-                    raise ValueError(f"plan {p}: algo index outside the profile database")
-                rc = (np.asarray(st.recompute_ops) == 1).astype(np.uint8)
-                codes[p, pos:pos + n] = (t * A + al) | (rc << 3)
-                codes[p, pos] |= 1 << 4
-                pos += n
-            if pos != N:
-                raise ValueError(f"plan {p} has {pos} ops, the op graph {N}")
+            total = sum(lens)
+            if total != N:
+                raise ValueError(f"plan {p} has {total} ops, the op graph {N}")
+            # the per-op lists of all stages, flattened once each
+            tp = np.fromiter(chain(st.tp_size for st in stages), dtype=np.int64, count=N)
+            dp = np.fromiter(chain(st.dp_size for st in stages), dtype=np.int64, count=N)
+            al = np.fromiter(chain(st.algo for st in stages), dtype=np.int64, count=N)
+            rc = np.fromiter(chain(st.recompute_ops for st in stages), dtype=np.int64, count=N)
+            g_of_op = np.repeat(np.asarray(gl, dtype=np.int64), lens)
+            bad = np.flatnonzero(tp * dp != g_of_op)
+            if len(bad):
+                s = int(np.searchsorted(np.cumsum(lens), bad[0], side="right"))
+                raise ValueError(f"plan {p}: stage {s} mixes tp*dp products")
+            t = tp_lut[np.clip(tp, 0, len(tp_lut) - 1)]
+            if (t == 0xff).any():
+                raise ValueError(f"plan {p}: tp size {int(tp[np.flatnonzero(t == 0xff)[0]])} is not in the profile database")
+            if ((al < 0) | (al >= A)).any():
+                raise ValueError(f"plan {p}: algo index outside the profile database")
+            row = (t * A + al.astype(np.uint8)) | ((rc == 1).astype(np.uint8) << 3)
+            starts = np.cumsum([0] + lens[:-1])
+            row[starts] |= 1 << 4
+            codes[p] = row
             hdr[p, 0] = S | (bidx << 8)
             hdr[p, 1] = glogs & 0xFFFFFFFF
             hdr[p, 2] = glogs >> 32

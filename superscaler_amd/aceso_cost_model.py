@@ -31,7 +31,7 @@ from .plan import AcesoConfig, AcesoStageInfo, PlanBatch, get_config  # noqa: F4
 from .profile_db import CostModelSettings, ProfileDB
 from .tables import (MAX_STAGES, R_ACT, R_BWD, R_FWD, R_IDEAL_BWD, R_IDEAL_FWD, R_IDEAL_IN, R_IDEAL_OUT, R_IN_COMM,
                      R_INPUTS, R_OUT_COMM, R_PEAK, R_RECOMP, R_RESERVED, R_SAVED, R_RESHARD, R_STAGE_MB, R_STAGE_MS,
-                     R_WEIGHTS, CompiledTables, compile_tables)
+                     R_WEIGHTS, STAGE_REC, CompiledTables, compile_tables)
 
 
 def settings_from_args(args) -> CostModelSettings:

@@ -357,3 +357,70 @@ def test_recompute_on_the_device_equals_the_array_form(name, limit):
         assert 0.02 < frac < 0.98
     finally:
         m.close()
+
+
+# ---- check_recompute on stages the greedy pass cannot help -------------------------------------
+def _no_group_stages(m):
+    """Stages with nothing to recompute (one op, ops the pass never picks) and ordinary ones, each under
+    limits from "below the weights alone" to "fits anyway"."""
+    ops = m.graph.ops
+    N = len(ops)
+    flags = m.graph.flags
+    norc = [i for i in range(N) if int(flags[m._type_index[ops[i]]]) & acm.og.F_NO_RECOMPUTE]
+    slices = [(0, 1), (0, 2), (N - 1, N), (N - 2, N), (1, 2), (1, 14), (0, 30)]
+    for i in norc[:3]:
+        slices.append((i, i + 1))
+    # maximal runs of never-picked ops
+    run_lo = None
+    for i in range(N + 1):
+        is_norc = i < N and i in set(norc)
+        if is_norc and run_lo is None:
+            run_lo = i
+        if not is_norc and run_lo is not None:
+            slices.append((run_lo, i))
+            run_lo = None
+    return sorted(set(slices))
+
+
+def _check_no_group(name, backend):
+    import dataclasses
+    from superscaler_amd import synth
+    from tests.helpers import oracle_for
+    w = synth.WORKLOADS[name]
+    graph = synth.make_graph(w)
+    mbs = w.mbs_list[-1]
+    for limit in (1.0, 200.0, 1e9):
+        st = dataclasses.replace(synth.make_settings(w), memory_limit=limit)
+        m = acm.CostModel(st, synth.make_db(w, graph), graph)
+        if backend == "emu":
+            m._evaluator = EmuEvaluator(m.tables)
+        try:
+            orc = oracle_for(m.tables)
+            qs = []
+            for lo, hi in _no_group_stages(m):
+                n = hi - lo
+                for nsb in (0, 3):
+                    qs.append((graph.ops[lo:hi], mbs, [1] * n, [1] * n, nsb, [0] * n))
+            want = [orc.check_recompute(*q) for q in qs]
+            assert any(not any(r) for r in want)
+            assert m.check_recompute_batch(qs) == want
+            assert [m.check_recompute(*q) for q in qs[:6]] == want[:6]
+            # the callers of the same path
+            cfg = get_config([1, len(graph.ops) - 1], [1] * len(graph.ops), [1] * len(graph.ops), [0] * len(graph.ops),
+                             mbs, w.global_batch, graph.ops, [0] * len(graph.ops))
+            m.update_recompute(cfg, 0)
+            assert cfg.stages[0].recompute_ops == orc.check_recompute(graph.ops[:1], mbs, [1], [1], 1, [0])
+        finally:
+            m.close()
+
+
+@pytest.mark.parametrize("name", ["gpt3_1_3b", "wresnet_1b", "t5_770m"])
+def test_check_recompute_without_a_recomputable_group_emu(name):
+    """aceso_cost_model.py:822-872 returns the zero list for a stage above the limit in which no op group can be
+    recomputed (a one-op stage, embedding / post-process ops only); so must every form of the call here."""
+    _check_no_group(name, "emu")
+
+
+@pytest.mark.gpu
+def test_check_recompute_without_a_recomputable_group_gpu():
+    _check_no_group("gpt3_1_3b", "gpu")

@@ -14,8 +14,19 @@ plans and records what the reference returns for them into tests/golden/<case>.j
 The functions covered are the ones no reference-held output pins: multi-stage / mixed-tp /
 resharding-active predict_time_breakdown (all lists it writes), predict_stage_time and its
 delta variants, predict_stage_memory (breakdown), get_reserved_memory_list, check_recompute,
-predict_value_after_move, wrap_predict_delta_time.  Floats are stored via repr and
-round-trip exactly through JSON.
+predict_value_after_move (also with inc_gpus / dec_gpus), wrap_predict_delta_time.  Floats are
+stored via repr and round-trip exactly through JSON.
+
+Further children of the same kind write
+  variants/<case>__<variant>.json  the same plans under the reference's non-default switches
+                                   (VARIANTS: --memory-pred-type MIN, --consider-collective-memory,
+                                   --do-not-consider-shared-tensor-space, --do-not-consider-reserved-space,
+                                   --do-not-use-flex-recompute, --peak-mem-in-backward);
+  moves_<case>.json                what the reference's move primitives (search/aceso_prims.py:
+                                   action_move_once, prim_mig_op, prim_tp_dp, prim_mbs,
+                                   prim_tp_dp_exchange) make of seeded legal plans;
+  megatron_grid_<case>.json        the plan files search/gen_megatron_plan.py itself writes (run as
+                                   the script it is, in a scratch directory).
 """
 import json
 import os
@@ -33,6 +44,18 @@ CASES = {
     "resnet_500M": ("resnet", "500M", "profiler/profiled-time-miniset", [32, 64], 1, 4, 768, 12000, None),
     "t5_770M": ("t5", "770M", "profiler/profiled-time-miniset", [1, 2, 4, 8], 1, 4, 512, 9000, 24),
 }
+
+# non-default switches of the cost model (aceso_utils.py:405, 423-430, 448)
+VARIANTS = {
+    "min": ["--memory-pred-type", "MIN"],
+    "collmem": ["--consider-collective-memory"],
+    "min_collmem": ["--memory-pred-type", "MIN", "--consider-collective-memory"],
+    "noshared": ["--do-not-consider-shared-tensor-space"],
+    "noreserved": ["--do-not-consider-reserved-space"],
+    "noflex": ["--do-not-use-flex-recompute"],
+    "peakbwd": ["--peak-mem-in-backward", "700"],
+}
+MOVE_CASES = ["gpt_1_3B", "resnet_500M"]
 
 
 def copy_db(case):
@@ -97,13 +120,39 @@ def rand_plan(rng, full_ops, tunable, num_gpus, mbs_list, max_stages, max_tp, un
         return nops, tp, dp, rc, algo, rng.choice(ok_mbs)
 
 
+def reference_argv(case, extra=()):
+    model, size, db, mbs_list, nodes, gpn, gbs, limit, num_layers = CASES[case]
+    dbdir = os.path.join(HERE, f"db_{case}") + "/"
+    return ["golden", "--model-name", model, "--model-size", size,
+            "--num-nodes", str(nodes), "--num-gpus-per-node", str(gpn),
+            "--global-batch-size", str(gbs), "--memory-limit", str(limit),
+            "--profiled-time-path", dbdir, "--micro-batch-size"] + [str(m) for m in mbs_list] + list(extra)
+
+
+def gpu_moves(cm, config, mbs_list, max_tp):
+    """predict_value_after_move with inc_gpus / dec_gpus (aceso_cost_model.py:715-728), for every stage and
+    dimension the tables can answer (aceso_prims.py:290-323 make the same checks before they ask)."""
+    out = []
+    for b, st in enumerate(config.stages):
+        for dim in ("tp", "dp"):
+            for inc in (True, False):
+                if dim == "tp":
+                    ok = max(st.tp_size) * 2 <= max_tp if inc else min(st.tp_size) > 1
+                else:
+                    new_dp = [d * 2 for d in st.dp_size] if inc else [d // 2 for d in st.dp_size]
+                    ok = (inc or min(st.dp_size) > 1) and all(config.micro_bs // d in mbs_list for d in new_dp)
+                if not ok:
+                    continue
+                for metric in ("time", "memory"):
+                    v, r = cm.predict_value_after_move(config, b, None, 0, metric, inc_gpus=inc, dec_gpus=not inc, dim=dim)
+                    out.append([b, dim, inc, metric, v, list(r)])
+    return out
+
+
 def child(case):
     model, size, db, mbs_list, nodes, gpn, gbs, limit, num_layers = CASES[case]
     dbdir = os.path.join(HERE, f"db_{case}") + "/"
-    sys.argv = ["golden", "--model-name", model, "--model-size", size,
-                "--num-nodes", str(nodes), "--num-gpus-per-node", str(gpn),
-                "--global-batch-size", str(gbs), "--memory-limit", str(limit),
-                "--profiled-time-path", dbdir, "--micro-batch-size"] + [str(m) for m in mbs_list]
+    sys.argv = reference_argv(case)
     sys.path.insert(0, os.path.join(REF, "search"))
     import aceso_cost_model as cm          # noqa: the reference, imported to record its outputs
     from aceso_utils import get_config
@@ -154,19 +203,170 @@ def child(case):
                     for dec in (True, False):
                         rec["delta_time"].append([b, partner, k, dec,
                                                   cm.wrap_predict_delta_time(config, b, partner, k, decrease=dec)])
+        rec["value_after_gpu_move"] = gpu_moves(cm, config, mbs_list, min(gpn, 8)) if p < 8 else []
         out["plans"].append(rec)
     with open(os.path.join(HERE, f"{case}.json"), "w") as f:
         json.dump(out, f)
     print(f"[golden] {case}: {len(out['plans'])} plans written")
 
 
+def child_variant(case, variant):
+    """Seeded plans (the base case's generator and seed) under one of VARIANTS."""
+    model, size, db, mbs_list, nodes, gpn, gbs, limit, num_layers = CASES[case]
+    dbdir = os.path.join(HERE, f"db_{case}") + "/"
+    sys.argv = reference_argv(case, VARIANTS[variant])
+    sys.path.insert(0, os.path.join(REF, "search"))
+    import aceso_cost_model as cm          # noqa: the reference, imported to record its outputs
+    from aceso_utils import get_config
+    from model_ops_info import get_full_op_list, get_tunable_op_list
+    args = cm.args
+    cm.read_profiled_time(model, size, dbdir)
+    full_ops = get_full_op_list(args)
+    tunable = [] if model == "t5" else get_tunable_op_list(args)
+    rng = random.Random(0xACE50 + sum(map(ord, case)))
+    num_gpus = nodes * gpn
+    out = {"case": case, "variant": variant, "flags": VARIANTS[variant], "model_name": model, "model_size": size,
+           "micro_batch_size": mbs_list, "num_nodes": nodes, "num_gpus_per_node": gpn, "global_batch_size": gbs,
+           "memory_limit": limit, "num_layers": num_layers, "num_ops": len(full_ops), "plans": []}
+    for p in range(16 if model == "gpt" else 8):
+        nops, tp, dp, rc, algo, mbs = rand_plan(rng, full_ops, tunable, num_gpus, mbs_list, 4, min(gpn, 8),
+                                                uniform_stage=(p % 4 == 3))
+        if p % 3 == 2:                    # (keeps the files small)
+            continue
+        config = get_config(nops, tp, dp, rc, mbs, gbs, full_ops, algo)
+        cm.predict_time_breakdown(config)
+        rec = {"num_ops_in_each_stage": nops, "tp": tp, "dp": dp, "recompute_ops": rc, "algo": algo,
+               "micro_batch_size": mbs, "time_list": config.time_list, "memory_list": config.memory_list,
+               "efficient_time_list": config.efficient_time_list,
+               "reserved_memory_list": cm.get_reserved_memory_list(config),
+               "stage_memory_breakdown": [], "check_recompute": [], "value_after_move": []}
+        for st in config.stages:
+            rec["stage_memory_breakdown"].append(list(cm.predict_stage_memory(st.ops, st.recompute_ops, st.tp_size, st.dp_size, mbs, st.num_stages_behind, st.algo, breakdown=True)))
+            rec["check_recompute"].append(cm.check_recompute(st.ops, mbs, st.tp_size, st.dp_size, st.num_stages_behind, st.algo))
+        S = config.num_stages
+        for b in range(S):
+            partner = b + 1 if b + 1 < S else b - 1
+            if 0 <= partner < S and len(config.stages[b].ops) > 3:
+                for metric in ("time", "memory"):
+                    v, r = cm.predict_value_after_move(config, b, partner, 2, metric)
+                    rec["value_after_move"].append([b, partner, 2, metric, v, list(r)])
+        out["plans"].append(rec)
+    os.makedirs(os.path.join(HERE, "variants"), exist_ok=True)
+    with open(os.path.join(HERE, "variants", f"{case}__{variant}.json"), "w") as f:
+        json.dump(out, f)
+    print(f"[golden] {case} / {variant}: {len(out['plans'])} plans written")
+
+
+def pack_plan(config):
+    """A plan as the reference's config_details lists (aceso_utils.py:116-135), flattened over the stages;
+    small integers as digit strings."""
+    flat = lambda key: [x for st in config.stages for x in getattr(st, key)]
+    digits = lambda xs: "".join(str(int(x).bit_length() - 1) for x in xs)
+    return {"num_ops_in_each_stage": [len(st.ops) for st in config.stages], "tp_log2": digits(flat("tp_size")),
+            "dp_log2": digits(flat("dp_size")), "recompute_ops": "".join(str(int(x)) for x in flat("recompute_ops")),
+            "algo": "".join(str(int(x)) for x in flat("algo")), "micro_batch_size": config.micro_bs,
+            "num_gpus": [st.num_gpus for st in config.stages]}
+
+
+def child_moves(case):
+    """What the reference's move primitives return for seeded legal plans whose recompute lists are
+    check_recompute's own (as initialize_search leaves them, aceso_search.py:26-27)."""
+    import copy
+    model, size, db, mbs_list, nodes, gpn, gbs, limit, num_layers = CASES[case]
+    dbdir = os.path.join(HERE, f"db_{case}") + "/"
+    sys.argv = reference_argv(case, ["--add-action-tp-dp-exchange", "--time-budget-total", "1000000", "--max-num-hops", "7"])
+    sys.path.insert(0, os.path.join(REF, "search"))
+    import aceso_cost_model as cm          # noqa: the reference, imported to record its outputs
+    import aceso_prims as pr               # noqa
+    from aceso_utils import check_legality, get_config
+    from model_ops_info import get_full_op_list, get_tunable_op_list
+    args = cm.args
+    cm.read_profiled_time(model, size, dbdir)
+    full_ops = get_full_op_list(args)
+    tunable = get_tunable_op_list(args)
+    rng = random.Random(0xACE51 + sum(map(ord, case)))
+    num_gpus = nodes * gpn
+    out = {"case": case, "model_name": model, "model_size": size, "micro_batch_size": mbs_list,
+           "num_nodes": nodes, "num_gpus_per_node": gpn, "global_batch_size": gbs, "memory_limit": limit,
+           "num_layers": num_layers, "num_ops": len(full_ops), "plans": []}
+    prims = {p.name: p for p in pr.action_resource_table}
+    want = 5 if model == "gpt" else 3
+    while len(out["plans"]) < want:
+        nops, tp, dp, rc, algo, mbs = rand_plan(rng, full_ops, tunable, num_gpus, mbs_list, 4, min(gpn, 8),
+                                                uniform_stage=(len(out["plans"]) % 2 == 0))
+        if len(nops) < 2 or min(nops) < 8:
+            continue
+        config = get_config(nops, tp, dp, [0] * len(tp), mbs, gbs, full_ops, algo)
+        if not check_legality(config, args):
+            continue
+        cm.update_recompute(config)
+        cm.predict_time_breakdown(config)
+        rec = {"start": pack_plan(config), "move_once": [], "exchange": [], "tp_dp": [], "mbs": [], "mig_op": []}
+        fresh = lambda: copy.deepcopy(config)
+        S = config.num_stages
+        for b in range(S):
+            for partner in (b - 1, b + 1):
+                if 0 <= partner < S:
+                    for k in (1, 5):
+                        r = pr.action_move_once(fresh(), b, partner, k)
+                        rec["move_once"].append([b, partner, k, pack_plan(r)])
+            for action in ("inc_tp_dec_dp", "inc_dp_dec_tp"):
+                r = prims[action].apply_to(fresh(), b)
+                rec["exchange"].append([b, action, None if r is None else pack_plan(r)])
+            for action in ("inc_tp", "dec_tp", "inc_dp", "dec_dp"):
+                r = prims[action].apply_to(fresh(), b)
+                rec["tp_dp"].append([b, action, None if r is None else pack_plan(r)])
+            r = prims["dec_op"].apply_to(fresh(), b)
+            rec["mig_op"].append([b, None if r is None else pack_plan(r)])
+        for action in ("inc_mbs", "dec_mbs"):
+            r = prims[action].apply_to(fresh(), 0)
+            rec["mbs"].append([action, None if r is None else pack_plan(r)])
+        out["plans"].append(rec)
+    with open(os.path.join(HERE, f"moves_{case}.json"), "w") as f:
+        json.dump(out, f)
+    n = {k: sum(len(p[k]) for p in out["plans"]) for k in ("move_once", "exchange", "tp_dp", "mbs", "mig_op")}
+    print(f"[golden] moves {case}: {len(out['plans'])} plans, {n}")
+
+
+def run_grid(case, num_saved=4):
+    """search/gen_megatron_plan.py run as the script it is, in a scratch directory; its plan files (data the
+    reference writes) go into one fixture."""
+    import tempfile
+    model, size, db, mbs_list, nodes, gpn, gbs, limit, num_layers = CASES[case]
+    with tempfile.TemporaryDirectory() as tmp:
+        argv = reference_argv(case, ["--num-layers", str(num_layers), "--config-save-path", tmp + "/",
+                                     "--num-of-saved-configs", str(num_saved)])[1:]
+        subprocess.run([sys.executable, os.path.join(REF, "search", "gen_megatron_plan.py")] + argv, check=True, cwd=tmp,
+                       stdout=subprocess.DEVNULL)
+        files = {}
+        for n in sorted(os.listdir(tmp)):
+            if n.endswith(".json"):
+                with open(os.path.join(tmp, n)) as f:
+                    files[n] = json.load(f)
+    with open(os.path.join(HERE, f"megatron_grid_{case}.json"), "w") as f:
+        json.dump({"case": case, "num_of_saved_configs": num_saved, "num_layers": num_layers, "files": files}, f)
+    print(f"[golden] megatron grid {case}: {sorted(files)}")
+
+
 def main():
     if len(sys.argv) > 2 and sys.argv[1] == "--child":
         return child(sys.argv[2])
+    if len(sys.argv) > 3 and sys.argv[1] == "--child-variant":
+        return child_variant(sys.argv[2], sys.argv[3])
+    if len(sys.argv) > 2 and sys.argv[1] == "--child-moves":
+        return child_moves(sys.argv[2])
+    quiet = subprocess.DEVNULL if os.environ.get("GOLDEN_QUIET") else None
+    me = os.path.abspath(__file__)
     for case in CASES:
         copy_db(case)
-        subprocess.run([sys.executable, os.path.abspath(__file__), "--child", case], check=True,
-                       stdout=subprocess.DEVNULL if os.environ.get("GOLDEN_QUIET") else None)
+        subprocess.run([sys.executable, me, "--child", case], check=True, stdout=quiet)
+        for variant in VARIANTS:
+            if "collmem" in variant and CASES[case][0] == "t5":
+                continue            # (resharding is off for T5, aceso_utils.py:523-526: the switch changes nothing)
+            subprocess.run([sys.executable, me, "--child-variant", case, variant], check=True, stdout=quiet)
+    for case in MOVE_CASES:
+        subprocess.run([sys.executable, me, "--child-moves", case], check=True, stdout=quiet)
+    run_grid("gpt_1_3B")
     # the single-GPU known-answer plans and the database files they index (data files)
     kat = os.path.join(HERE, "kat")
     os.makedirs(kat, exist_ok=True)

@@ -19,12 +19,14 @@ from tests.helpers import EmuEvaluator, emu_score
 CASES = ["gpt_1_3B", "resnet_500M", "t5_770M"]
 
 
-def make_model(golden_dir, case, backend):
-    with open(os.path.join(golden_dir, f"{case}.json")) as f:
+def make_model(golden_dir, case, backend, variant=None):
+    from tests.test_oracle_golden import VARIANT_SETTINGS
+    name = f"{case}.json" if variant is None else os.path.join("variants", f"{case}__{variant}.json")
+    with open(os.path.join(golden_dir, name)) as f:
         g = json.load(f)
     st = CostModelSettings(model_name=g["model_name"], micro_batch_size=g["micro_batch_size"],
                            num_gpus_per_node=g["num_gpus_per_node"], global_batch_size=g["global_batch_size"],
-                           memory_limit=g["memory_limit"])
+                           memory_limit=g["memory_limit"], **(VARIANT_SETTINGS[variant] if variant else {}))
     m = acm.CostModel.from_directory(st, g["model_name"], g["model_size"],
                                      os.path.join(golden_dir, f"db_{case}") + "/", num_layers=g["num_layers"])
     if backend == "emu":
@@ -424,3 +426,76 @@ def test_check_recompute_without_a_recomputable_group_emu(name):
 @pytest.mark.gpu
 def test_check_recompute_without_a_recomputable_group_gpu():
     _check_no_group("gpt3_1_3b", "gpu")
+
+
+# ---- the reference's vectors for its non-default switches and for inc_gpus / dec_gpus moves ---------
+from tests.test_oracle_golden import ALL_VARIANTS
+
+
+def _run_variant(g, m):
+    cfgs = [cfg_of(g, m, p) for p in g["plans"]]
+    m.predict_time_breakdown_batch(cfgs)
+    for c, p in zip(cfgs, g["plans"]):
+        for k in ["time_list", "memory_list", "efficient_time_list"]:
+            assert getattr(c, k) == p[k], k
+        assert m.get_reserved_memory_list(c) == p["reserved_memory_list"]
+        mbs = p["micro_batch_size"]
+        for s, st in enumerate(c.stages):
+            assert list(m.predict_stage_memory(st.ops, st.recompute_ops, st.tp_size, st.dp_size, mbs, st.num_stages_behind,
+                                               st.algo, breakdown=True)) == p["stage_memory_breakdown"][s]
+        for b, partner, k, metric, v, r in p["value_after_move"]:
+            gv, gr = m.predict_value_after_move(c, b, partner, k, metric)
+            assert gv == v and list(gr) == r
+    qs = [(st.ops, p["micro_batch_size"], st.tp_size, st.dp_size, st.num_stages_behind, st.algo)
+          for c, p in zip(cfgs, g["plans"]) for st in c.stages]
+    assert m.check_recompute_batch(qs) == [r for p in g["plans"] for r in p["check_recompute"]]
+    # the batch scorer (scores, flags) and the array form of update_recompute under the same switches
+    it, pk, fe = m.score_batch(cfgs)
+    assert list(it) == [max(p["time_list"]) for p in g["plans"]] and list(pk) == [max(p["memory_list"]) for p in g["plans"]]
+    assert list(fe) == [int(max(p["memory_list"]) <= g["memory_limit"]) for p in g["plans"]]
+    out = m.update_recompute_arrays(m.encode(cfgs))
+    for k, p in enumerate(g["plans"]):
+        assert [st.recompute_ops for st in out.to_config(k, m.tables).stages] == p["check_recompute"]
+
+
+@pytest.mark.parametrize("name", ALL_VARIANTS)
+def test_non_default_switches_match_reference_emu(golden_dir, name):
+    g, m = make_model(golden_dir, *name.split("__")[:1], "emu", variant=name.split("__")[1])
+    _run_variant(g, m)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ALL_VARIANTS)
+def test_non_default_switches_match_reference_gpu(golden_dir, name):
+    g, m = make_model(golden_dir, *name.split("__")[:1], "gpu", variant=name.split("__")[1])
+    try:
+        _run_variant(g, m)
+    finally:
+        m.close()
+
+
+def _run_gpu_moves(g, m):
+    n = 0
+    for p in g["plans"]:
+        c = cfg_of(g, m, p)
+        for b, dim, inc, metric, v, r in p["value_after_gpu_move"]:
+            gv, gr = m.predict_value_after_move(c, b, None, 0, metric, inc_gpus=inc, dec_gpus=not inc, dim=dim)
+            assert gv == v and list(gr) == r
+            n += 1
+    assert n > 20
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_value_after_gpu_move_matches_reference_emu(golden_dir, case):
+    g, m = make_model(golden_dir, case, "emu")
+    _run_gpu_moves(g, m)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", CASES)
+def test_value_after_gpu_move_matches_reference_gpu(golden_dir, case):
+    g, m = make_model(golden_dir, case, "gpu")
+    try:
+        _run_gpu_moves(g, m)
+    finally:
+        m.close()

@@ -63,3 +63,21 @@ def test_c_oracle_reference_vectors(golden_dir, case):
         assert list(tl[k, :S]) == p["time_list"] and list(ml[k, :S]) == p["memory_list"]
         assert it[k] == max(p["time_list"]) and pk[k] == max(p["memory_list"])
         assert fe[k] == (max(p["memory_list"]) <= g["memory_limit"])
+
+
+from tests.test_oracle_golden import ALL_VARIANTS, load_variant
+
+
+@pytest.mark.parametrize("name", ALL_VARIANTS)
+def test_c_oracle_reference_vectors_non_default_switches(golden_dir, name):
+    """The reference's own numbers under MIN / collective memory / no shared space / no reserved space
+    (the switches that change scoring; flex_recompute and peak_mem_in_backward only steer check_recompute)."""
+    g, orc, full = load_variant(golden_dir, name)
+    co = COracle(orc, full, g["global_batch_size"])
+    cfgs = [make_config(g, p, full) for p in g["plans"]]
+    it, pk, fe, er, tl, ml = co.score_configs(cfgs, lists=True)
+    assert (er == 0).all()
+    for k, p in enumerate(g["plans"]):
+        S = len(p["time_list"])
+        assert list(tl[k, :S]) == p["time_list"] and list(ml[k, :S]) == p["memory_list"]
+        assert it[k] == max(p["time_list"]) and pk[k] == max(p["memory_list"])

@@ -93,3 +93,83 @@ def test_golden_exercises_resharding(golden_dir):
             orc.args.resharding = True
             hits += int(with_r[2] != without[2] or with_r[3] != without[3])
     assert hits >= 8
+
+
+# ---- the reference's non-default switches (tests/golden/variants, written by the reference) ------
+VARIANT_SETTINGS = {
+    "min": dict(memory_pred_type="MIN"),
+    "collmem": dict(consider_collective_memory=True),
+    "min_collmem": dict(memory_pred_type="MIN", consider_collective_memory=True),
+    "noshared": dict(consider_shared_space=False),
+    "noreserved": dict(consider_reserved_space=False),
+    "noflex": dict(flex_recompute=False),
+    "peakbwd": dict(peak_mem_in_backward=700),
+}
+
+
+def variant_files(golden_dir):
+    d = os.path.join(golden_dir, "variants")
+    return sorted(f[:-5] for f in os.listdir(d) if f.endswith(".json"))
+
+
+def load_variant(golden_dir, name):
+    case, variant = name.split("__")
+    with open(os.path.join(golden_dir, "variants", f"{name}.json")) as f:
+        g = json.load(f)
+    st = Settings(model_name=g["model_name"], micro_batch_size=g["micro_batch_size"],
+                  num_gpus_per_node=g["num_gpus_per_node"], memory_limit=g["memory_limit"], **VARIANT_SETTINGS[variant])
+    orc = Oracle(st)
+    orc.read_profiled_time(g["model_name"], g["model_size"], os.path.join(golden_dir, f"db_{case}") + "/")
+    full = get_full_op_list(g["model_name"], orc.op_list, g["num_layers"])
+    return g, orc, full
+
+
+ALL_VARIANTS = variant_files(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden"))
+
+
+def test_every_switch_has_vectors():
+    assert len(ALL_VARIANTS) == 19
+    for case in CASES:
+        for v in VARIANT_SETTINGS:
+            assert f"{case}__{v}" in ALL_VARIANTS or (case == "t5_770M" and "collmem" in v)
+
+
+@pytest.mark.parametrize("name", ALL_VARIANTS)
+def test_non_default_switches_bit_exact(golden_dir, name):
+    g, orc, full = load_variant(golden_dir, name)
+    _, plain, _ = load_case(golden_dir, name.split("__")[0])       # default switches: pinned by the base vectors
+    differs = 0
+    for p in g["plans"]:
+        c = make_config(g, p, full)
+        orc.predict_time_breakdown(c)
+        for k in ["time_list", "memory_list", "efficient_time_list"]:
+            assert getattr(c, k) == p[k], k
+        assert orc.get_reserved_memory_list(c) == p["reserved_memory_list"]
+        mbs = p["micro_batch_size"]
+        for s, st in enumerate(c.stages):
+            assert list(orc.predict_stage_memory(st.ops, st.recompute_ops, st.tp_size, st.dp_size, mbs,
+                                                 st.num_stages_behind, st.algo, breakdown=True)) == p["stage_memory_breakdown"][s]
+            assert orc.check_recompute(st.ops, mbs, st.tp_size, st.dp_size, st.num_stages_behind, st.algo) == p["check_recompute"][s]
+        for b, partner, k, metric, v, r in p["value_after_move"]:
+            gv, gr = orc.predict_value_after_move(c, b, partner, k, metric)
+            assert gv == v and list(gr) == r
+        c0 = make_config(g, p, full)
+        plain.predict_time_breakdown(c0)
+        rc0 = [plain.check_recompute(st.ops, mbs, st.tp_size, st.dp_size, st.num_stages_behind, st.algo) for st in c0.stages]
+        differs += int(c0.memory_list != p["memory_list"] or rc0 != p["check_recompute"])
+    # the switch must matter on these plans, or the vectors would pin nothing
+    assert differs > 0, name
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_value_after_gpu_move_bit_exact(golden_dir, case):
+    """predict_value_after_move with inc_gpus / dec_gpus for dim tp and dp (aceso_cost_model.py:715-728)."""
+    g, orc, full = load_case(golden_dir, case)
+    n = 0
+    for p in g["plans"]:
+        c = make_config(g, p, full)
+        for b, dim, inc, metric, v, r in p["value_after_gpu_move"]:
+            gv, gr = orc.predict_value_after_move(c, b, None, 0, metric, inc_gpus=inc, dec_gpus=not inc, dim=dim)
+            assert gv == v and list(gr) == r
+            n += 1
+    assert n > 20

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define ACE_ABI_VERSION 6
+#define ACE_ABI_VERSION 7
 #define ACE_MAX_STAGES 16      /* aceso_utils.py:502: end_num_stages = min(num_gpus, 16) */
 #define ACE_STAGE_REC 18       /* doubles per stage record, see ACE_R_* */
 
@@ -35,6 +35,7 @@ enum {
     ACE_EHIP = -3,        /* a HIP runtime call failed (ace_last_hip_error() says which) */
     ACE_ENOMEM = -4,
     ACE_EVERSION = -5,
+    ACE_EFIXED = -6,      /* the call would have to reallocate a workspace that ace_reserve() fixed */
 };
 
 /* per-plan status bytes written by ace_score_batch */
@@ -151,11 +152,20 @@ void ace_destroy(ace_handle_t *h);
  *  quantities predict_time_breakdown / predict_stage_time / predict_stage_memory are made of; for a
  *  batch of single-stage queries (batch->d_range) one record each: double[n_plans][ACE_STAGE_REC].
  * Plain scoring (no d_stage_out, no d_range) uses a workspace owned by the handle (80 bytes per plan
- * and stage, allocated on first use and grown when a larger batch arrives: that call allocates), so
- * scoring calls on one handle must be stream-ordered with respect to each other. */
+ * and stage, allocated on first use and grown when a larger batch arrives: that call allocates, unless
+ * ace_reserve() sized or fixed it beforehand), so scoring calls on one handle must be stream-ordered with
+ * respect to each other. */
 int ace_score_batch(ace_handle_t *h, const ace_batch_t *batch, double memory_limit, int strict,
                     double *d_iter_ms, double *d_peak_mb, uint8_t *d_feasible, uint8_t *d_status,
                     double *d_stage_out, void *stream);
+
+/* Size the handle's workspace for plain scoring of batches of up to max_plans plans now (max_plans = 0: leave it as
+ * it is), so that no later ace_score_batch / ace_time_score_kernel call of that size allocates.  With fixed != 0 a
+ * later call that needs a larger workspace returns ACE_EFIXED instead of freeing and reallocating it (which would
+ * synchronise the device in the middle of a stream, is invalid during stream capture and would leave a recorded
+ * graph with the address of freed memory); fixed = 0 lets the workspace grow on demand again.  This call itself
+ * may allocate: make it outside any capture.  No counterpart in the reference. */
+int ace_reserve(ace_handle_t *h, size_t max_plans, int fixed);
 
 /* The k feasible plans with the smallest iteration time, ascending, ties broken by the lower plan
  * index: the order sort_configs (aceso_utils.py:723-740) / gen_megatron_plan.py:131-135 produce.

@@ -285,6 +285,7 @@ struct ace_handle {
     uint32_t *d_win_rows;
     double *d_stage_ws;        // grow-only workspace for deferred stage tails
     size_t stage_ws_plans;     // capacity in plans
+    int stage_ws_fixed;        // ace_reserve(..., fixed): a larger batch is an error instead of a reallocation
 };
 
 // The bodies of these kernels live in ace_edit_kernels.h (shared with the host build of the tests).
@@ -331,6 +332,7 @@ const char *ace_strerror(int code) {
         case ACE_EHIP: return "HIP runtime error";
         case ACE_ENOMEM: return "out of memory";
         case ACE_EVERSION: return "ABI version mismatch";
+        case ACE_EFIXED: return "the batch needs a larger workspace than the one fixed with ace_reserve";
         default: return "unknown error";
     }
 }
@@ -532,6 +534,7 @@ static int ensure_stage_ws(ace_handle_t *h, AceKernelArgs *a) {
     const size_t need = (((size_t)a->g.P + kBlock - 1) / kBlock) * kBlock;
     if (need * ACE_MAX_STAGES * (ACE_WS_REC / 2) > 0xffffffffull) return ACE_OK;   // 32-bit record offsets: larger batches take the plain kernel
     if (need > h->stage_ws_plans) {
+        if (h->stage_ws_fixed) return ACE_EFIXED;
         if (h->d_stage_ws) ACE_HIP(hipFree(h->d_stage_ws));
         h->d_stage_ws = nullptr;
         h->stage_ws_plans = 0;
@@ -543,6 +546,22 @@ static int ensure_stage_ws(ace_handle_t *h, AceKernelArgs *a) {
 }
 
 extern "C" {
+
+int ace_reserve(ace_handle_t *h, size_t max_plans, int fixed) {
+    if (!h || max_plans > 0x7fffffffull) return ACE_EINVAL;
+    if (max_plans) {
+        AceKernelArgs a;
+        memset(&a, 0, sizeof(a));
+        a.g.P = (int32_t)max_plans;
+        const int was_fixed = h->stage_ws_fixed;
+        h->stage_ws_fixed = 0;
+        const int rc = ensure_stage_ws(h, &a);
+        h->stage_ws_fixed = was_fixed;
+        if (rc) return rc;
+    }
+    h->stage_ws_fixed = fixed ? 1 : 0;
+    return ACE_OK;
+}
 
 int ace_score_batch(ace_handle_t *h, const ace_batch_t *batch, double memory_limit, int strict, double *d_iter_ms,
                     double *d_peak_mb, uint8_t *d_feasible, uint8_t *d_status, double *d_stage_out, void *stream) {

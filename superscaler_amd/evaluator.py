@@ -16,7 +16,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libace_eva
 _lib = None
 
 EXPORTS = ["ace_abi_version", "ace_strerror", "ace_last_hip_error", "ace_create", "ace_destroy",
-           "ace_score_batch", "ace_topk_workspace_bytes", "ace_topk", "ace_time_score_kernel", "ace_apply_moves",
+           "ace_score_batch", "ace_reserve", "ace_topk_workspace_bytes", "ace_topk", "ace_time_score_kernel", "ace_apply_moves",
            "ace_recompute_groups", "ace_recompute_select", "ace_group_keys", "ace_gather_plans"]
 
 
@@ -56,6 +56,8 @@ def load_library():
     lib.ace_score_batch.argtypes = [ctypes.c_void_p, ctypes.POINTER(AceBatchStruct), ctypes.c_double, ctypes.c_int,
                                     ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                     ctypes.c_void_p, ctypes.c_void_p]
+    lib.ace_reserve.restype = ctypes.c_int
+    lib.ace_reserve.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
     lib.ace_topk_workspace_bytes.restype = ctypes.c_size_t
     lib.ace_topk_workspace_bytes.argtypes = [ctypes.c_size_t, ctypes.c_int]
     lib.ace_topk.restype = ctypes.c_int
@@ -234,7 +236,6 @@ class PlanEvaluator:
         self._deal_cache = {}
         self._topk_ws = None
         self._small = None
-        self._ws_slots = 0          # plans the handle's workspace of deferred stage tails holds (as the library sizes it)
         self._graphs_alive = 0
 
     def close(self):
@@ -280,14 +281,8 @@ class PlanEvaluator:
         else:
             it, pk, fe, st = out
         breakdown = breakdown or dbatch.ranges is not None
-        if not breakdown and self.tables.n_windows == 1:
-            # plain scoring with every row resident uses the handle's workspace, which grows (is reallocated) for a larger batch:
-            # a captured step holds its address
-            slots = -(-P // 1024) * 1024
-            if self._graphs_alive and slots > self._ws_slots:
-                raise AceError("this batch would reallocate the workspace that a captured step of this evaluator uses: "
-                               "capture after the largest batch has been scored, or use another evaluator")
-            self._ws_slots = max(self._ws_slots, slots)
+        # (plain scoring with every row resident uses the handle's workspace, which the library reallocates for a larger
+        # batch -- unless a captured step holds its address: then ace_reserve() has fixed it and the call is refused)
         # (a single-stage query has one record)
         n_rec = 1 if dbatch.ranges is not None else MAX_STAGES
         rec = torch.zeros((P, n_rec, STAGE_REC), dtype=torch.float64, device=self.device) if breakdown else None
@@ -298,12 +293,19 @@ class PlanEvaluator:
         _check(self.lib, rc, "ace_score_batch")
         return (it, pk, fe, st, rec) if breakdown else (it, pk, fe, st)
 
+    def reserve(self, max_plans: int, fixed: bool = False):
+        """Size the handle's scoring workspace for batches of up to `max_plans` plans now; `fixed`: a later, larger
+        batch is refused (AceError) instead of reallocating it (what a captured step needs)."""
+        with self._torch.cuda.device(self.device):
+            _check(self.lib, self.lib.ace_reserve(self.handle, int(max_plans), int(fixed)), "ace_reserve")
+
     def topk(self, iter_ms, feasible, k: int):
         """Device-wide top-k: (indices int64[k], times f64[k], count)."""
         torch = self._torch
         n = iter_ms.numel()
         need = self.lib.ace_topk_workspace_bytes(n, k)
         if self._topk_ws is None or self._topk_ws.numel() < need:
+            # (a captured step keeps its own reference to the workspace it recorded, so the old one stays alive for it)
             self._topk_ws = torch.empty(need, dtype=torch.uint8, device=self.device)
         idx = torch.empty(k, dtype=torch.int64, device=self.device)
         val = torch.empty(k, dtype=torch.float64, device=self.device)
@@ -558,8 +560,10 @@ class StepGraph:
         with torch.cuda.graph(self.graph):
             ev.score(dbatch, memory_limit, strict, out=self.scores)
             self.top = ev.topk(self.scores[0], self.scores[2], k)
+        self._topk_ws = ev._topk_ws               # the recorded launches write into it: it must outlive a larger topk()
         self._ev = ev
         ev._graphs_alive += 1
+        ev.reserve(0, fixed=True)                 # the handle's workspace may not move while the graph lives
 
     def replay(self):
         if self._ev is None or not self._ev.handle:
@@ -571,8 +575,11 @@ class StepGraph:
         """Forget the recorded launches (the evaluator may then score larger batches again)."""
         if self._ev is not None:
             self._ev._graphs_alive -= 1
+            if self._ev._graphs_alive == 0 and self._ev.handle:
+                self._ev.reserve(0, fixed=False)
             self._ev = None
             self.graph = None
+            self._topk_ws = None
 
     def __del__(self):
         try:

@@ -38,7 +38,7 @@ import numpy as np
 from . import opgraph as og
 from .profile_db import CostModelSettings, ProfileDB
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 MAX_STAGES = 16
 STAGE_REC = 18
 LDS_BYTES = 160 * 1024

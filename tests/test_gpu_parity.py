@@ -455,6 +455,16 @@ def test_captured_step_replays_to_the_eager_results(torch_mod):
     bigger = ev.upload(synth.make_plans(w, tables, n_plans=201000, seed_offset=13, workers=4))
     with pytest.raises(AceError):
         ev.score(bigger)
+    # ... whichever call gets there: the library itself refuses (ace_reserve fixed the workspace)
+    with pytest.raises(AceError):
+        ev.time_score_kernel(bigger, 1)
+    # a larger top-k takes a workspace of its own; the recorded one stays alive with the graph
+    ev.topk(fresh[0], fresh[2], 4096)
+    junk = [torch.full((1 << 20,), 7, dtype=torch.uint8, device="cuda") for _ in range(8)]     # what the allocator might hand out again
+    (scores, top) = g.replay()
+    torch.cuda.synchronize()
+    assert all(torch.equal(a, b) for a, b in zip(list(scores) + list(top), list(fresh) + list(ftop)))
+    del junk
     g.release()
     ev.score(bigger)
     with pytest.raises(AceError):

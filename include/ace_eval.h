@@ -159,6 +159,20 @@ int ace_score_batch(ace_handle_t *h, const ace_batch_t *batch, double memory_lim
                     double *d_iter_ms, double *d_peak_mb, uint8_t *d_feasible, uint8_t *d_status,
                     double *d_stage_out, void *stream);
 
+/* ace_score_batch for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): plain scoring (no d_stage_out, no batch->d_range) of at most
+ * ACE_STATIC_MAX_PLANS plans, with the deferred-stage-tail records in a static device array of the library
+ * (ACE_STATIC_MAX_PLANS * 1,280 bytes = 20 MiB, held by every GPU the library runs on until the process ends)
+ * instead of the handle's workspace.  It calls no hipMalloc / hipFree and no allocating library routine, and
+ * leaves the handle's workspace alone.  Same results as ace_score_batch, bit for bit.  Returns ACE_ETOOBIG for a
+ * larger batch.  The array is shared by every call on that GPU, whichever handle or stream: calls that overlap
+ * in time on one GPU race on it (order them on one stream, or with events); nothing in it has to be cleared
+ * between calls (a launch reads back only the records it wrote itself).  The handle's device must be current.
+ * No counterpart in the reference. */
+#define ACE_STATIC_MAX_PLANS 16384
+int ace_score_batch_static(ace_handle_t *h, const ace_batch_t *batch, double memory_limit, int strict,
+                           double *d_iter_ms, double *d_peak_mb, uint8_t *d_feasible, uint8_t *d_status, void *stream);
+
 /* Size the handle's workspace for plain scoring of batches of up to max_plans plans now (max_plans = 0: leave it as
  * it is), so that no later ace_score_batch / ace_time_score_kernel call of that size allocates.  With fixed != 0 a
  * later call that needs a larger workspace returns ACE_EFIXED instead of freeing and reallocating it (which would

@@ -13,10 +13,17 @@
 
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <new>
 
 #include "ace_edit_kernels.h"
 #include "ace_score_loop.h"
+
+// Scratch of ace_score_batch_static: the deferred-stage-tail records of up to ACE_STATIC_MAX_PLANS plans (the
+// layout ace_score_body's DEFER variant uses: [stage][plan slot][ACE_WS_REC]).  Every GPU the library runs on holds
+// its own copy of this array until the process ends.  In host code the array's name is only a stand-in for
+// hipGetSymbolAddress(): kernels get the per-device pointer that call returned (static_scratch_ptr), never the name.
+static __device__ __align__(256) double scratch[(size_t)ACE_STATIC_MAX_PLANS * ACE_MAX_STAGES * ACE_WS_REC];
 
 namespace {
 
@@ -27,8 +34,13 @@ constexpr int kBlock = ACE_BLOCK;        // lanes (= plans) per workgroup: 16 wa
 constexpr int kSmallBlock = 256;         // ... for small batches: 4 wavefronts, 1 per SIMD
 constexpr int kSmallBatchBlocks = 128;   // batches of fewer than this many kBlock workgroups use kSmallBlock
 constexpr uint32_t kMaxLds = 160 * 1024;  // CDNA4 LDS per workgroup
+static_assert(ACE_STATIC_MAX_PLANS % ACE_BLOCK == 0, "the static scratch holds whole workgroups");
 
 thread_local char g_hip_err[256] = "";
+
+constexpr int kMaxDevices = 64;
+double *g_static_ptr[kMaxDevices];     // device address of `scratch` by device ordinal; filled once per device
+std::mutex g_static_mutex;
 
 #define ACE_HIP(call)                                                                          \
     do {                                                                                       \
@@ -362,6 +374,22 @@ template <bool BD, bool RANGED, bool WIN, bool DEFER> static int allow_big_lds()
     return ACE_OK;
 }
 
+// The device address of `scratch` on the current device (looked up once per device).
+static int static_scratch_ptr(double **out) {
+    int dev = -1;
+    ACE_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return ACE_EINVAL;
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    if (!g_static_ptr[dev]) {
+        void *p = nullptr;
+        ACE_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return ACE_EHIP;
+        g_static_ptr[dev] = static_cast<double *>(p);
+    }
+    *out = g_static_ptr[dev];
+    return ACE_OK;
+}
+
 extern "C" {
 
 int ace_create(const ace_tables_t *t, ace_handle_t **out) {
@@ -444,7 +472,9 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     h->num_types = t->num_types; h->lds_bytes = lds_bytes;
     const size_t pos_entries = (size_t)((t->num_ops + 15) / 16) * 16 + 16;
     int rc;
+    double *scratch_here = nullptr;
     if ((rc = hipGetDevice(&h->device) == hipSuccess ? ACE_OK : ACE_EHIP) ||
+        (rc = static_scratch_ptr(&scratch_here)) ||
         (rc = upload((void **)&h->d_rows, t->rows, (size_t)t->num_types * row_bytes)) ||
         (rc = upload((void **)&h->d_pos_info, t->pos_info, (size_t)(t->num_ops + 1) * 4, pos_entries * 4)) ||
         (rc = upload((void **)&h->d_pair_kinds, t->pair_kinds, (size_t)rk_bytes)) ||
@@ -569,6 +599,24 @@ int ace_score_batch(ace_handle_t *h, const ace_batch_t *batch, double memory_lim
     int rc = fill_args(h, batch, memory_limit, strict, d_iter_ms, d_peak_mb, d_feasible, d_status, d_stage_out, &a);
     if (rc) return rc;
     if ((rc = ensure_stage_ws(h, &a))) return rc;
+    launch_score(h, a, (hipStream_t)stream);
+    ACE_HIP(hipGetLastError());
+    return ACE_OK;
+}
+
+int ace_score_batch_static(ace_handle_t *h, const ace_batch_t *batch, double memory_limit, int strict, double *d_iter_ms,
+                           double *d_peak_mb, uint8_t *d_feasible, uint8_t *d_status, void *stream) {
+    if (batch && (batch->d_range || batch->n_plans > (size_t)ACE_STATIC_MAX_PLANS)) return batch->d_range ? ACE_EINVAL : ACE_ETOOBIG;
+    AceKernelArgs a;
+    int rc = fill_args(h, batch, memory_limit, strict, d_iter_ms, d_peak_mb, d_feasible, d_status, nullptr, &a);
+    if (rc) return rc;
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev != h->device || dev < 0 || dev >= kMaxDevices) return ACE_EINVAL;
+    // (the same test as ensure_stage_ws: tables that take the kernels without deferred stage tails need no scratch)
+    const bool deferred = !(h->n_windows > 1 || h->geom.N >= 65536 || (h->geom.flags & ACE_F_COLLECTIVE_MEM));
+    // looked up by ace_create on this device; the padded plan count of either workgroup size fits: ACE_STATIC_MAX_PLANS is a multiple of kBlock
+    a.stage_ws = deferred ? g_static_ptr[dev] : nullptr;
+    if (deferred && !a.stage_ws) return ACE_EINVAL;
     launch_score(h, a, (hipStream_t)stream);
     ACE_HIP(hipGetLastError());
     return ACE_OK;

@@ -16,7 +16,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libace_eva
 _lib = None
 
 EXPORTS = ["ace_abi_version", "ace_strerror", "ace_last_hip_error", "ace_create", "ace_destroy",
-           "ace_score_batch", "ace_reserve", "ace_topk_workspace_bytes", "ace_topk", "ace_time_score_kernel", "ace_apply_moves",
+           "ace_score_batch", "ace_score_batch_static", "ace_reserve", "ace_topk_workspace_bytes", "ace_topk", "ace_time_score_kernel", "ace_apply_moves",
            "ace_recompute_groups", "ace_recompute_select", "ace_group_keys", "ace_gather_plans"]
 
 
@@ -56,6 +56,9 @@ def load_library():
     lib.ace_score_batch.argtypes = [ctypes.c_void_p, ctypes.POINTER(AceBatchStruct), ctypes.c_double, ctypes.c_int,
                                     ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                     ctypes.c_void_p, ctypes.c_void_p]
+    lib.ace_score_batch_static.restype = ctypes.c_int
+    lib.ace_score_batch_static.argtypes = [ctypes.c_void_p, ctypes.POINTER(AceBatchStruct), ctypes.c_double, ctypes.c_int,
+                                           ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
     lib.ace_reserve.restype = ctypes.c_int
     lib.ace_reserve.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
     lib.ace_topk_workspace_bytes.restype = ctypes.c_size_t

@@ -61,9 +61,40 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     const uint32_t lds_base = ace_lds_base(lds_raw);
     g.hot_off += lds_base; g.start_off += lds_base; g.out_off += lds_base; g.z_off += lds_base;
     g.rk_lds_off += lds_base; g.stg_lds_off += lds_base;
-    const long long plan = block * BLOCK + tid;
+    const long long slot = block * BLOCK + tid;                     // this lane's place in the batch (and in the workspace)
+    long long plan = slot;
+#ifndef ACE_HOST_EMU
+    if (DEFER && BLOCK >= 128) {
+        // The lanes of a wavefront walk the ops together, and every op at which one of them closes a stage takes all
+        // of them through the stage-end code: so the workgroup deals its plans to its lanes by pipeline depth
+        // (counting sort on the depth in the plan header, deepest first; plans of one depth in any order), and the
+        // sorted wavefronts to the SIMDs in turn (wavefront w runs on SIMD w % 4) so that each SIMD gets the same
+        // mix.  Only which lane scores which plan changes: results go to the plan's own index.
+        unsigned int *cnt = reinterpret_cast<unsigned int *>(lds_raw);                  // 17 bins (nothing is staged yet)
+        unsigned short *plan_of = reinterpret_cast<unsigned short *>(lds_raw + 128);     // [BLOCK]
+        uint32_t depth = 0;                                                              // lanes past the batch: last
+        if (slot < g.P) {
+            depth = a.hdr[slot].x & 0xffu;
+            depth = depth > 16u ? 16u : depth;
+        }
+        if (tid < 32) cnt[tid] = 0u;
+        ACE_SYNC();
+        const uint32_t rank = atomicAdd(&cnt[16u - depth], 1u);
+        ACE_SYNC();
+        uint32_t before = 0;
+        for (uint32_t b = 0; b < 16u - depth; ++b) before += cnt[b];
+        const uint32_t sorted = before + rank;
+        // sorted wavefront q goes to wavefront q of the workgroup in rows of four, every second row reversed
+        const uint32_t q = sorted >> 6;
+        const uint32_t wave = (q & 4u) ? (q ^ 3u) : q;
+        plan_of[(wave << 6) | (sorted & 63u)] = (unsigned short)tid;
+        ACE_SYNC();
+        plan = block * BLOCK + plan_of[tid];
+        ACE_SYNC();
+    }
+#endif
     const bool in_batch = plan < g.P;
-    const long long pl = in_batch ? plan : (long long)g.P - 1;      // slot this lane reads
+    const long long pl = in_batch ? plan : (long long)g.P - 1;      // plan this lane reads
     // where this lane's results go; a slot whose entry is not a valid index computes but writes nothing
     const long long out = a.order ? (long long)a.order[pl] : plan;
     const bool active = in_batch && out < g.P;
@@ -113,7 +144,7 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     double *rec = (BD && a.stage_out && active) ? a.stage_out + (size_t)out * rec_doubles : nullptr;
     if (DEFER) {
         // stage-major: the records of one stage of consecutive plans are adjacent (padded lanes own a slot too)
-        rec = a.stage_ws + (size_t)plan * ACE_WS_REC;
+        rec = a.stage_ws + (size_t)slot * ACE_WS_REC;
         st.ws_stride = n_blocks * (uint32_t)BLOCK * (ACE_WS_REC / 2);
     }
 

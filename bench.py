@@ -17,11 +17,16 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per plan of one scoring-kernel launch on the default workload, from two rocprofv3 --pmc
-# runs (FETCH_SIZE, then WRITE_SIZE) scaled by the readings of a plain 256 MiB copy in the same
-# runs (factors 2.000 and 1.000), keyed by (workload, ops, plans grouped at upload):
-# 1,049 B read + 681 B written with the grouped layout, 1,334 + 618 in the generator's order.
-MEASURED_TRAFFIC_BYTES_PER_PLAN = {("gpt3_13b", 523, True): 1731.0, ("gpt3_13b", 523, False): 1952.0}
+# Counter readings of the scoring kernel on the default workload, which a run of this script cannot take itself
+# (rocprofv3 --pmc passes): copied from the committed summary named in "source", which also names the library
+# build they were taken on.  HBM bytes per plan and launch = FETCH_SIZE + WRITE_SIZE, each scaled by the reading
+# of a plain 256 MiB copy in the same pass; vector instructions per op and wavefront = SQ_INSTS_VALU / SQ_WAVES /
+# ops; 14 of them are the reference's own fp64 arithmetic (nine adds / multiply-adds, five maxima).
+PROFILE_COUNTERS = {
+    ("gpt3_13b", 523): {"source": "profiles/score_kernel_gpt3_13b.md", "traffic_bytes_per_plan": 1952.0,
+                        "valu_per_op_per_wavefront": 60.1, "valu_busy": 0.88},
+}
+ESSENTIAL_VALU_PER_OP = 14
 
 
 def cpu_baseline(tables, batch, threads):
@@ -53,12 +58,14 @@ def cpu_baseline(tables, batch, threads):
             cpu_model = next((ln.split(":", 1)[1].strip() for ln in f if ln.startswith("model name")), cpu_model)
     except OSError:
         pass
-    return {"value": P / dt_all, "unit": "plans/s", "cores": threads, "kind": "port", "cpu_model": cpu_model,
-            "sample": f"all {P} plans of the same batch in {dt_all:.2f} s, C oracle (oracle/aceso_oracle.c), "
-                      f"{threads} OpenMP threads",
-            "single_core_value": n1 / dt_one, "single_core_sample": f"first {n1} plans, {dt_one:.2f} s, 1 thread",
-            "python_oracle_value": npy / dt_py,
-            "python_oracle_sample": f"first {npy} plans, {dt_py:.2f} s, pure-Python oracle, 1 process"}
+    # the stated baseline is the reference's way of running: pure Python, one process, one core
+    return {"value": npy / dt_py, "unit": "plans/s", "cores": 1, "kind": "port", "cpu_model": cpu_model,
+            "sample": f"first {npy} plans of the same batch in {dt_py:.2f} s, loop-faithful Python oracle "
+                      "(oracle/aceso_oracle.py), 1 process",
+            "c_port_value": P / dt_all, "c_port_cores": threads,
+            "c_port_sample": f"all {P} plans in {dt_all:.2f} s, C oracle (oracle/aceso_oracle.c), {threads} OpenMP threads",
+            "c_port_single_core_value": n1 / dt_one,
+            "c_port_single_core_sample": f"first {n1} plans, {dt_one:.2f} s, 1 thread"}
 
 
 def main():
@@ -72,12 +79,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--pp", type=int, nargs="+", default=None,
                     help="restrict the pipeline depths the plans are drawn from (profiling aid)")
-    ap.add_argument("--caller-order", action="store_true",
-                    help="keep the plans in the generator's order in HBM instead of grouping them by pipeline "
-                         "depth and first stage boundaries at upload (results are in the generator's order either way)")
-    ap.add_argument("--no-layout-comparison", action="store_true",
-                    help="do not also time the kernel on the plans in the generator's order (keeps a profiler's "
-                         "per-kernel average to the benchmark's own layout)")
+    ap.add_argument("--regrouped-too", action="store_true",
+                    help="also time the step on a copy of the batch regrouped on the device beforehand (by pipeline "
+                         "depth and first stage boundaries; ace_group_keys / ace_gather_plans), as a secondary figure")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="also run one plain device-to-device copy of this many MiB (a kernel of known "
                          "traffic, to scale FETCH_SIZE / WRITE_SIZE counter readings)")
@@ -104,16 +108,7 @@ def main():
     batch = synth.make_plans(w, tables, n_plans=n_plans, workers=min(16, os.cpu_count() or 1))
     gen_s = time.perf_counter() - t0
     ev = PlanEvaluator(tables, device="cuda:0")
-    d_plain = ev.upload(batch)
-    d, group_ms = d_plain, None
-    if not args.caller_order:
-        # grouped storage, made on the device from the plain upload; timed, but not part of the step
-        ev.group(d_plain)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        d = ev.group(d_plain)
-        torch.cuda.synchronize()
-        group_ms = (time.perf_counter() - t0) * 1e3
+    d = ev.upload(batch)                      # the plans as the generator emitted them
     P, N = d.n_plans, d.num_ops
     it = torch.empty(P, dtype=torch.float64, device="cuda:0")
     pk = torch.empty(P, dtype=torch.float64, device="cuda:0")
@@ -137,50 +132,61 @@ def main():
     elapsed, (idx, val, cnt) = timed(d)
     ms_per_step = elapsed / args.steps * 1e3
     plans_per_s = P * args.steps / elapsed
-    plain_plans_per_s = plans_per_s
-    if not args.caller_order and not args.no_layout_comparison:
-        elapsed_plain, (idx2, val2, cnt2) = timed(d_plain)
-        plain_plans_per_s = P * args.steps / elapsed_plain
-        assert torch.equal(idx, idx2) and torch.equal(val, val2), "grouped storage changed the ranking"
-
     # dominant kernel: the scoring kernel, timed with HIP events on its launch stream
     kern_ms = ev.time_score_kernel(d, reps=max(args.steps, 5))
-    kern_ms_caller_order = kern_ms
-    if not args.caller_order and not args.no_layout_comparison:
-        kern_ms_caller_order = ev.time_score_kernel(d_plain, reps=max(args.steps, 5))
+    secondary = {}
+    if args.regrouped_too:
+        ev.group(d)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        dg = ev.group(d)
+        torch.cuda.synchronize()
+        secondary["regrouping_ms"] = (time.perf_counter() - t0) * 1e3
+        elapsed_g, (idx2, val2, cnt2) = timed(dg)
+        assert torch.equal(idx, idx2) and torch.equal(val, val2), "grouped storage changed the ranking"
+        secondary["value_plans_regrouped_beforehand"] = P * args.steps / elapsed_g
+        secondary["kernel_ms_plans_regrouped_beforehand"] = ev.time_score_kernel(dg, reps=max(args.steps, 5))
+        elapsed, (idx, val, cnt) = timed(d)        # (leaves the generator-order results in the output tensors)
     algo_bytes = (3 * N + 19) * P            # canonical encoding: 3 bytes per op + 2 + 17 bytes of results
     moved_bytes = d.bytes_moved_per_plan * P + 17 * P
     achieved = algo_bytes / (kern_ms * 1e-3) / 1e9
     n_feasible = int(fe.sum().item())
     best = val[0].item() if n_feasible else None
+    counters = PROFILE_COUNTERS.get((w.name, N)) if P == w.n_plans and not args.pp else None
 
     out = {
         "metric": "plans scored/sec at GPT-3 13B op graph (1M plans); % HBM roofline",
         "value": plans_per_s, "unit": "plans/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f64", "data": "synthetic",
-        "config": {"workload": f"{w.name}: {N}-op graph, {P} seeded plans, D={w.num_gpus}, "
-                               f"PP in {w.pp_choices}, mbs in {w.mbs_list}, recompute p={w.recompute_p}, "
-                               f"memory cap {w.memory_limit:.0f} MB, global batch {w.global_batch}, top-{args.topk}",
-                   "step": "score kernel + device-wide top-k, inputs resident in HBM",
-                   "layout": ("plans in the generator's order" if args.caller_order else
-                              "resident plans regrouped once on the device (by pipeline depth and first two stage "
-                              "boundaries, wavefronts dealt to the workgroups) before the timed steps; results and "
-                              "top-k indices in the generator's order"),
-                   "regrouping_ms": group_ms,
-                   "value_plans_in_generator_order": plain_plans_per_s,
-                   "feasible_plans": n_feasible, "best_iter_ms": best, "plan_generation_s": round(gen_s, 1)},
+        "config": dict({"workload": f"{w.name}: {N}-op graph, {P} seeded plans, D={w.num_gpus}, "
+                                    f"PP in {w.pp_choices}, mbs in {w.mbs_list}, recompute p={w.recompute_p}, "
+                                    f"memory cap {w.memory_limit:.0f} MB, global batch {w.global_batch}, top-{args.topk}",
+                        "step": "score kernel + device-wide top-k, inputs resident in HBM",
+                        "layout": "plans in the generator's order (each workgroup of the kernel deals its 1,024 plans to "
+                                  "its lanes by pipeline depth; nothing is reordered beforehand)",
+                        "feasible_plans": n_feasible, "best_iter_ms": best, "plan_generation_s": round(gen_s, 1)},
+                       **secondary),
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS,
-                     "traffic": (MEASURED_TRAFFIC_BYTES_PER_PLAN[(w.name, N, not args.caller_order)] * P
-                                 if (w.name, N, not args.caller_order) in MEASURED_TRAFFIC_BYTES_PER_PLAN else None),
+                     "traffic": counters["traffic_bytes_per_plan"] * P if counters else None,
+                     "traffic_source": counters["source"] if counters else None,
                      "algorithmic_bytes": algo_bytes,
                      "kernel": "ace_score_kernel<BD=false,RANGED=false,WIN=false,DEFER=true>", "kernel_ms": kern_ms,
-                     "kernel_ms_plans_in_generator_order": kern_ms_caller_order,
                      "algorithmic_bytes_per_plan": 3 * N + 19,
                      "bytes_moved_per_plan": d.bytes_moved_per_plan + 17,
-                     "achieved_on_bytes_moved": moved_bytes / (kern_ms * 1e-3) / 1e9},
+                     "achieved_on_bytes_moved": moved_bytes / (kern_ms * 1e-3) / 1e9,
+                     "note": "HBM is the nominal roofline of this path (plan bytes streamed once, tables in LDS); the kernel "
+                             "itself is bound by vector-instruction issue, see roofline_valu_issue"},
     }
+    if counters:
+        # the bound that holds: one vector instruction per SIMD and quad-cycle; the time of the kernel is the number
+        # of vector instructions its wavefronts issue
+        v = counters["valu_per_op_per_wavefront"]
+        out["roofline_valu_issue"] = {"bound": "valu_issue", "unit": "vector instructions per op per wavefront",
+                                      "essential": ESSENTIAL_VALU_PER_OP, "achieved": v,
+                                      "frac": ESSENTIAL_VALU_PER_OP / v, "simd_valu_busy": counters["valu_busy"],
+                                      "source": counters["source"]}
     if args.calibration_copy_mib > 0:
         src = torch.zeros(args.calibration_copy_mib << 20, dtype=torch.uint8, device="cuda:0")
         dst = torch.empty_like(src)

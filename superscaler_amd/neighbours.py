@@ -174,6 +174,92 @@ def sample_moves(base: PlanBatch, tables: CompiledTables, n: int, rng: np.random
     return PlanBatch(np.stack(t_codes), np.stack(t_hdr)), moves
 
 
+# ---- the reference's own primitives as descriptors --------------------------------------------------------------
+# What search/aceso_prims.py's primitives do to a plan, before the update_recompute() call each of them ends with
+# (CostModel.update_recompute_arrays / update_recompute_device on the expanded batch; check_recompute does not look at
+# the recompute bits a stage had, so re-choosing them for every stage of a plan whose other stages already carry
+# check_recompute's choice gives what the primitive's own call on the touched stages gives).  Which stage, partner,
+# count or direction to try is the caller's policy (aceso_policy.py, the goal loops of prim_mig_op, the producer /
+# consumer choice of prim_tp_dp), made from predict_value_after_move / wrap_predict_delta_time as in the reference.
+
+def _plan_fields(base: PlanBatch, p: int = 0):
+    row, hdr = base.codes[p], base.hdr[p]
+    S = int(hdr[0] & 0xff)
+    gword = int(hdr[1]) | (int(hdr[2]) << 32)
+    glogs = np.array([(gword >> (4 * s)) & 15 for s in range(S)], dtype=np.int64)
+    starts, ends = _stage_bounds(row)
+    return row, hdr, S, int(hdr[0] >> 8) & 0xff, glogs, starts, ends
+
+
+def migrate_ops_move(base: PlanBatch, n_algo: int, stage: int, partner: int, num_ops: int, template: int = 0) -> np.ndarray:
+    """action_move_once (aceso_prims.py:66-134): the last `num_ops` ops of `stage` go to the stage on its right
+    (partner > stage) or its first `num_ops` to the stage on its left; they take the tp (and with it the dp) of the
+    receiving stage's nearest op (:91-92, :112-113) and keep their algorithm.  One descriptor (uint32[4])."""
+    row, _, S, _, _, starts, ends = _plan_fields(base, template)
+    if not (0 <= stage < S and 0 <= partner < S and abs(stage - partner) == 1):
+        raise ValueError("op migration goes to an adjacent stage")
+    if not 0 < num_ops < ends[stage] - starts[stage]:
+        raise ValueError("the stage must keep at least one op")       # (:84-86 returns the plan unchanged)
+    tp = (row & 7) // n_algo
+    if stage < partner:
+        cut = int(starts[partner])
+        new_cut, ref = cut - num_ops, int(tp[cut])
+    else:
+        cut = int(starts[stage])
+        new_cut, ref = cut + num_ops, int(tp[cut - 1])
+    return np.array([template | (OP_MIGRATE << 16), cut | (new_cut << 16), ref, 0], dtype=np.uint32)
+
+
+def stage_tp_step_move(base: PlanBatch, stage: int, up: bool, template: int = 0) -> np.ndarray:
+    """prim_tp_dp_exchange (aceso_prims.py:772-797): every op of `stage` one tp step up (dp halves) or down (dp
+    doubles) on the same devices.  The caller checks the legality conditions of :781 / :786-789.  One descriptor."""
+    _, _, S, _, _, starts, ends = _plan_fields(base, template)
+    if not 0 <= stage < S:
+        raise ValueError("no such stage")
+    return np.array([template | (OP_TP_STEP << 16), int(starts[stage]) | (int(ends[stage]) << 16), 1 if up else 0, 0],
+                    dtype=np.uint32)
+
+
+def device_steps_template(base: PlanBatch, tables: CompiledTables, steps, p: int = 0):
+    """prim_tp_dp (aceso_prims.py:377-485): devices move between stages; `steps` lists (stage, "tp" | "dp", +1 | -1)
+    for the producer (its tp or dp halves, :312-321) and the consumers (doubles, :302-310).  A dp step only changes the
+    stage's device count; a tp step also moves every op of the stage one tp index.  Returns (code row, header) of the
+    resulting plan, to be used as a template row (op OP_NONE)."""
+    row, hdr, S, bidx, glogs, starts, ends = _plan_fields(base, p)
+    A = tables.db.n_algo
+    row, glogs = row.copy(), glogs.copy()
+    for stage, dim, sign in steps:
+        if dim not in ("tp", "dp") or sign not in (1, -1) or not 0 <= stage < S:
+            raise ValueError(f"bad step {(stage, dim, sign)}")
+        glogs[stage] += sign
+        if dim == "tp":
+            lo, hi = int(starts[stage]), int(ends[stage])
+            t = (row[lo:hi] & 7).astype(np.int64) // A + sign
+            if t.min() < 0 or t.max() >= len(tables.db.tp_list):
+                raise ValueError("tp step leaves the profiled sizes")
+            row[lo:hi] = (row[lo:hi] & 0xF8) | (t * A + (row[lo:hi] & (A - 1))).astype(np.uint8)
+    if glogs.min() < 0:
+        raise ValueError("a stage would lose its last device")
+    h = hdr.copy()
+    _set_header(h, S, bidx, glogs, tables.settings.num_gpus_per_node)
+    return row, h
+
+
+def micro_batch_template(base: PlanBatch, tables: CompiledTables, micro_bs: int, tp_per_stage, p: int = 0):
+    """prim_mbs (aceso_prims.py:544-580): the next micro-batch size, every stage uniformly on the tp size
+    best_total_gpu_time (:509-542) chose for it (`tp_per_stage`, sizes).  Returns (code row, header)."""
+    row, hdr, S, _, glogs, starts, ends = _plan_fields(base, p)
+    A = tables.db.n_algo
+    row = row.copy()
+    for s in range(S):
+        t = tables.db.tp_list.index(int(tp_per_stage[s]))
+        lo, hi = int(starts[s]), int(ends[s])
+        row[lo:hi] = (row[lo:hi] & 0xF8) | (np.uint8(t * A) + (row[lo:hi] & (A - 1))).astype(np.uint8)
+    h = hdr.copy()
+    h[0] = S | (tables.db.mbs_list.index(int(micro_bs)) << 8)
+    return row, h
+
+
 def apply_moves_host(templates: PlanBatch, moves: np.ndarray, n_algo: int) -> PlanBatch:
     """Expand move descriptors into plans with numpy (masks over a [neighbours, ops] byte matrix)."""
     A = np.uint8(n_algo)

@@ -282,6 +282,37 @@ def test_uniform_grid_gpu(golden_dir):
     _grid_check(golden_dir, "gpu")
 
 
+def _grid_files_check(golden_dir, backend, tmp_path):
+    """The plan files the reference's own search/gen_megatron_plan.py wrote for the GPT-1.3B database
+    (tests/golden/megatron_grid_gpt_1_3B.json, made by tests/golden/make_golden.py: run_grid): same file names (the
+    truncated predicted time is part of them), same order, same JSON content."""
+    from superscaler_amd import megatron_grid
+    from superscaler_amd.plan import dump_config_to_json
+    with open(os.path.join(golden_dir, "megatron_grid_gpt_1_3B.json")) as f:
+        fx = json.load(f)
+    g, m = make_model(golden_dir, "gpt_1_3B", backend)
+    try:
+        best = megatron_grid.best_uniform_plans(m, g["num_nodes"] * g["num_gpus_per_node"], fx["num_layers"], fx["num_of_saved_configs"])
+        names = [f"{g['model_name']}_{g['model_size']}_{fx['num_layers']}layers_megatron_est_{int(t)}.json" for t, _, _ in best]
+        assert names == sorted(fx["files"], key=lambda n: int(n.rsplit("_", 1)[1][:-5])) and len(names) == fx["num_of_saved_configs"]
+        for name, (t, mem, cfg) in zip(names, best):
+            path = str(tmp_path / name)
+            dump_config_to_json(cfg, path, g["model_name"], g["model_size"], fx["num_layers"])
+            with open(path) as f:
+                assert json.load(f) == fx["files"][name], name
+    finally:
+        m.close()
+
+
+def test_uniform_grid_writes_the_reference_files_emu(golden_dir, tmp_path):
+    _grid_files_check(golden_dir, "emu", tmp_path)
+
+
+@pytest.mark.gpu
+def test_uniform_grid_writes_the_reference_files_gpu(golden_dir, tmp_path):
+    _grid_files_check(golden_dir, "gpu", tmp_path)
+
+
 @pytest.mark.gpu
 def test_recompute_arrays_gpu_equals_cpu_build():
     """2,048 GPT-3 13B plans under a 40 GB cap: the array-form greedy loop gives the same bits whether

@@ -1,0 +1,167 @@
+"""The move primitives of the reference's search (search/aceso_prims.py) against their descriptor form.
+
+tests/golden/moves_<case>.json holds what the reference itself returned (tests/golden/make_golden.py, child_moves) for
+action_move_once, prim_tp_dp_exchange, prim_tp_dp, prim_mbs and prim_mig_op on seeded legal plans whose recompute lists
+are check_recompute's own.  For every recorded result the test builds the edit from what the primitive is documented to
+do (superscaler_amd/neighbours.py: migrate_ops_move, stage_tp_step_move, device_steps_template, micro_batch_template),
+expands it with apply_moves_host -- on the GPU also with the library's ace_apply_moves -- re-chooses the recompute bits
+with update_recompute_arrays as every primitive does, and compares the whole plan (op counts, tp, dp, recompute, algo,
+micro-batch size: the reference's config_details) with the recorded one.
+
+Which stage / partner / count / direction a primitive tries is its policy and comes from the fixture here (for
+prim_tp_dp and prim_mbs: read off the recorded result, per stage); the policy calls themselves
+(predict_value_after_move, wrap_predict_delta_time) are pinned in test_cost_model_api.py."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from superscaler_amd import neighbours as nb
+from superscaler_amd.plan import PlanBatch, config_details, get_config
+from tests.test_cost_model_api import make_model
+
+MOVE_CASES = ["gpt_1_3B", "resnet_500M"]
+
+
+def unpack(g, m, d):
+    """A plan of the fixture (make_golden.pack_plan) as an AcesoConfig."""
+    digits = lambda s: [1 << int(c) for c in s]
+    bits = lambda s: [int(c) for c in s]
+    return get_config(d["num_ops_in_each_stage"], digits(d["tp_log2"]), digits(d["dp_log2"]), bits(d["recompute_ops"]),
+                      d["micro_batch_size"], g["global_batch_size"], m.graph.ops, bits(d["algo"]))
+
+
+def load(golden_dir, case, backend):
+    with open(os.path.join(golden_dir, f"moves_{case}.json")) as f:
+        moves = json.load(f)
+    g, m = make_model(golden_dir, case, backend)
+    return moves, g, m
+
+
+def expand(m, templates, moves, device):
+    """Descriptors -> plans (host numpy, or the library's kernel), then the primitives' closing update_recompute."""
+    if device:
+        d = m.evaluator.apply_moves(templates, moves)
+        return m.evaluator.download(m.update_recompute_device(d))
+    return m.update_recompute_arrays(nb.apply_moves_host(templates, moves, m.tables.db.n_algo))
+
+
+def same_plan(m, batch, k, want_cfg):
+    return config_details(batch.to_config(k, m.tables), get_string=True) == config_details(want_cfg, get_string=True)
+
+
+def steps_between(start_cfg, res_cfg):
+    """What prim_tp_dp did to each stage, read off its result: (stage, dim, +1 / -1)."""
+    steps = []
+    for s, (a, b) in enumerate(zip(start_cfg.stages, res_cfg.stages)):
+        if b.num_gpus == a.num_gpus:
+            assert b.tp_size == a.tp_size and b.dp_size == a.dp_size
+            continue
+        sign = 1 if b.num_gpus == 2 * a.num_gpus else -1
+        assert b.num_gpus * 2 == a.num_gpus or sign == 1
+        if b.tp_size == a.tp_size:
+            steps.append((s, "dp", sign))
+        else:
+            assert b.dp_size == a.dp_size
+            steps.append((s, "tp", sign))
+    return steps
+
+
+def hops_between(start_cfg, res_cfg, first):
+    """The op migrations behind a prim_mig_op result: one boundary after the other, starting next to the stage the
+    primitive was applied to (`first`) and walking away from it (aceso_prims.py:166-189)."""
+    a = np.cumsum([len(st.ops) for st in start_cfg.stages])[:-1]
+    b = np.cumsum([len(st.ops) for st in res_cfg.stages])[:-1]
+    moved = [j for j in range(len(a)) if a[j] != b[j]]          # boundary j separates stages j and j + 1
+    hops = []
+    for j in sorted(moved, key=lambda j: abs(j + 0.5 - first)):
+        if b[j] < a[j]:
+            hops.append((j, j + 1, int(a[j] - b[j])))           # stage j gives its tail to stage j + 1
+        else:
+            hops.append((j + 1, j, int(b[j] - a[j])))
+    return hops
+
+
+def run_case(golden_dir, case, backend):
+    moves, g, m = load(golden_dir, case, backend)
+    device = backend == "gpu"
+    A = m.tables.db.n_algo
+    seen = {"move_once": 0, "exchange": 0, "tp_dp": 0, "mbs": 0, "mig_op": 0}
+    failed = []
+    try:
+        for pi, rec in enumerate(moves["plans"]):
+            start_cfg = unpack(moves, m, rec["start"])
+            base = PlanBatch.from_configs([start_cfg], m.tables)
+            # the start plans carry check_recompute's own choice: re-choosing changes nothing
+            assert np.array_equal(m.update_recompute_arrays(base).codes, base.codes)
+            rows, hdrs, descs, want, tag = [base.codes[0]], [base.hdr[0]], [], [], []
+
+            def template(row, hdr):
+                rows.append(row)
+                hdrs.append(hdr)
+                return np.array([len(rows) - 1, 0, 0, 0], dtype=np.uint32)
+
+            for b, partner, k, res in rec["move_once"]:
+                descs.append(nb.migrate_ops_move(base, A, b, partner, k))
+                want.append(unpack(moves, m, res))
+                tag.append("move_once")
+            for b, action, res in rec["exchange"]:
+                if res is not None:
+                    descs.append(nb.stage_tp_step_move(base, b, up=(action == "inc_tp_dec_dp")))
+                    want.append(unpack(moves, m, res))
+                    tag.append("exchange")
+            for b, action, res in rec["tp_dp"]:
+                if res is not None:
+                    res_cfg = unpack(moves, m, res)
+                    steps = steps_between(start_cfg, res_cfg)
+                    assert (b, action.split("_")[1], 1 if action.startswith("inc") else -1) in steps
+                    descs.append(template(*nb.device_steps_template(base, m.tables, steps)))
+                    want.append(res_cfg)
+                    tag.append("tp_dp")
+            for action, res in rec["mbs"]:
+                if res is not None:
+                    res_cfg = unpack(moves, m, res)
+                    assert all(len(set(st.tp_size)) == 1 for st in res_cfg.stages)
+                    descs.append(template(*nb.micro_batch_template(base, m.tables, res_cfg.micro_bs,
+                                                                   [st.tp_size[0] for st in res_cfg.stages])))
+                    want.append(res_cfg)
+                    tag.append("mbs")
+            out = expand(m, PlanBatch(np.stack(rows), np.stack(hdrs)), np.stack(descs), device)
+            for k, (cfg, t) in enumerate(zip(want, tag)):
+                seen[t] += 1
+                if not same_plan(m, out, k, cfg):
+                    failed.append((pi, t, k))
+            # prim_mig_op: a chain of op migrations, each applied to the result of the one before
+            for b, res in rec["mig_op"]:
+                if res is None:
+                    continue
+                res_cfg = unpack(moves, m, res)
+                cur = base
+                for frm, to, k in hops_between(start_cfg, res_cfg, b):
+                    cur = nb.apply_moves_host(cur, nb.migrate_ops_move(cur, A, frm, to, k)[None, :], A)
+                got = expand(m, cur, np.zeros((1, 4), dtype=np.uint32), device)
+                seen["mig_op"] += 1
+                if not same_plan(m, got, 0, res_cfg):
+                    failed.append((pi, "mig_op", b))
+    finally:
+        if device:
+            m.close()
+    return seen, failed
+
+
+@pytest.mark.parametrize("case", MOVE_CASES)
+def test_reference_primitives_in_descriptor_form_emu(golden_dir, case):
+    seen, failed = run_case(golden_dir, case, "emu")
+    assert not failed, failed
+    assert seen["move_once"] >= 8 and seen["exchange"] >= 1 and seen["mbs"] >= 1
+    if case == "gpt_1_3B":
+        assert seen["tp_dp"] >= 4 and seen["mig_op"] >= 2
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", MOVE_CASES)
+def test_reference_primitives_in_descriptor_form_gpu(golden_dir, case):
+    seen, failed = run_case(golden_dir, case, "gpu")
+    assert not failed, failed
+    assert sum(seen.values()) > 10

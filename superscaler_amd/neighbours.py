@@ -449,7 +449,9 @@ def hill_climb(cm, start: PlanBatch, steps: int, n_neighbours: int, seed: int = 
             if visited is None:
                 # equal descriptors are equal plans: keep one of each (template < 2^16, op < 2^8, p1 < 2^8)
                 packed = (moves[:, 0] | (moves[:, 2] << 24)).astype(np.uint64) | (moves[:, 1].astype(np.uint64) << np.uint64(32))
-                moves = moves[np.unique(packed, return_index=True)[1]]
+                # (first occurrences, in the order they were drawn: among neighbours of equal time the earliest wins,
+                # as it does when the duplicates are scored too)
+                moves = moves[np.sort(np.unique(packed, return_index=True)[1])]
                 d = ev.apply_moves(templates, moves)
             else:
                 d, keys = ev.apply_moves(templates, moves, with_keys=True)

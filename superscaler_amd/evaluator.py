@@ -185,7 +185,12 @@ class DeviceBatch:
             if ranges is not None:
                 ranges = np.asarray(ranges)[perm]
             self.order = torch.from_numpy(perm.astype(np.int32)).to(device)
-        if staging is not None:
+        pinned = getattr(batch, "pinned_tensors", None) if host_codes is batch.codes else None
+        if pinned is not None:
+            # the plans were produced in page-locked memory (PlanEvaluator.pinned_plan_batch): the copy to the device reads
+            # them where they are, no staging copy on the host
+            codes = pinned[0].to(device, non_blocking=True)
+        elif staging is not None:
             stage = staging[:P * N].view(P, N)
             stage.copy_(torch.from_numpy(np.ascontiguousarray(host_codes)))
             codes = stage.to(device, non_blocking=True)
@@ -195,7 +200,10 @@ class DeviceBatch:
             codes = torch.nn.functional.pad(codes, (0, G * 16 - N))
         # [P, G, 16] -> [G, P, 16]: plan-minor, sixteen ops per 16-byte word
         self.codes = codes.view(P, G, 16).permute(1, 0, 2).contiguous()
-        self.hdr = torch.from_numpy(np.ascontiguousarray(host_hdr).view(np.int32)).to(device)
+        if pinned is not None:
+            self.hdr = pinned[1].to(device, non_blocking=True)
+        else:
+            self.hdr = torch.from_numpy(np.ascontiguousarray(host_hdr).view(np.int32)).to(device)
         self.ranges = None
         if ranges is not None:
             r = np.ascontiguousarray(ranges, dtype=np.uint32)
@@ -261,6 +269,19 @@ class PlanEvaluator:
             if msg:
                 raise ValueError(msg)
         return DeviceBatch(batch, self.device, ranges, staging, group_by_depth)
+
+    def pinned_plan_batch(self, n_plans: int) -> PlanBatch:
+        """An empty PlanBatch (codes uint8 [n_plans, N], hdr uint32 [n_plans, 4]) whose arrays live in page-locked host
+        memory: a producer that writes its plans there (synth.make_plans(out=...), neighbours on the host, a reader of
+        plan files) hands them to upload() / score_stream() without the host-side staging copy, so the transfer runs at
+        the bus's rate.  The caller must not rewrite the arrays while an upload of them is in flight."""
+        torch = self._torch
+        N = self.tables.graph.num_ops
+        tc = torch.empty((n_plans, N), dtype=torch.uint8, pin_memory=True)
+        th = torch.empty((n_plans, 4), dtype=torch.int32, pin_memory=True)
+        b = PlanBatch(tc.numpy(), th.numpy().view(np.uint32))
+        b.pinned_tensors = (tc, th)
+        return b
 
     def device_context(self):
         """Context manager that makes this evaluator's GPU the current one (for raw library calls)."""
@@ -363,8 +384,9 @@ class PlanEvaluator:
 
         def upload(b):
             # buffer `turn` was last used two batches ago, and that batch has been scored and synchronised
+            # (plans that already sit in page-locked memory need no staging buffer)
             need = b.n_plans * b.num_ops
-            if staging[turn[0]] is None or staging[turn[0]].numel() < need:
+            if getattr(b, "pinned_tensors", None) is None and (staging[turn[0]] is None or staging[turn[0]].numel() < need):
                 staging[turn[0]] = torch.empty(need, dtype=torch.uint8, pin_memory=True)
             with torch.cuda.stream(copy_stream):
                 d = self.upload(b, validate=False, staging=staging[turn[0]])

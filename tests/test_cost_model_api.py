@@ -282,6 +282,50 @@ def test_uniform_grid_gpu(golden_dir):
     _grid_check(golden_dir, "gpu")
 
 
+ATTRS = ["time_list", "memory_list", "compute_time_list", "total_gpu_time", "breakdown_ideal_time_per_gpu",
+         "breakdown_eff_loss_time_per_gpu", "breakdown_recomp_time_per_gpu", "efficient_time_list"]
+
+
+def _candidate_list_check(golden_dir, case, backend):
+    """The search's candidate loop (aceso_search.py:121-145: every new config scored, the fastest one whose memory fits
+    kept) with the candidates handed over in ONE call: predict_time_breakdown_batch fills every attribute
+    predict_time_breakdown fills, with the same values, and the selection made from them is the same."""
+    g, m = make_model(golden_dir, case, backend)
+    try:
+        one_by_one = [cfg_of(g, m, p) for p in g["plans"]]
+        for c in one_by_one:
+            m.predict_time_breakdown(c)
+        batched = [cfg_of(g, m, p) for p in g["plans"]]
+        m.predict_time_breakdown_batch(batched)
+        for a, b in zip(one_by_one, batched):
+            for k in ATTRS:
+                assert getattr(a, k) == getattr(b, k), k
+
+        def pick(configs, initial_time):
+            best, best_t = None, initial_time
+            for k, c in enumerate(configs):
+                if max(c.time_list) < best_t and max(c.memory_list) <= g["memory_limit"]:
+                    best, best_t = k, max(c.time_list)
+            return best
+        fits = [max(c.time_list) for c in one_by_one if max(c.memory_list) <= g["memory_limit"]]
+        for t0 in [float("inf")] + sorted(fits)[1:3]:
+            assert pick(one_by_one, t0) == pick(batched, t0)
+        assert (pick(batched, float("inf")) is not None) == bool(fits)
+    finally:
+        m.close()
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_candidate_list_in_one_call_emu(golden_dir, case):
+    _candidate_list_check(golden_dir, case, "emu")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", CASES)
+def test_candidate_list_in_one_call_gpu(golden_dir, case):
+    _candidate_list_check(golden_dir, case, "gpu")
+
+
 def _grid_files_check(golden_dir, backend, tmp_path):
     """The plan files the reference's own search/gen_megatron_plan.py wrote for the GPT-1.3B database
     (tests/golden/megatron_grid_gpt_1_3B.json, made by tests/golden/make_golden.py: run_grid): same file names (the

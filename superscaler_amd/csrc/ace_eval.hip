@@ -420,8 +420,8 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     const int32_t rk_bytes = t->n_pair_kinds * t->n_glog * 64;
     const int32_t stg_words = t->n_mbs * 16;
     const uint32_t rk_off = (uint32_t)t->lds_row_bytes;
-    const uint32_t stg_off = (rk_off + (uint32_t)rk_bytes + 15u) & ~15u;
-    const uint32_t lds_bytes = stg_off + (uint32_t)stg_words * 4u;
+    uint32_t stg_off, lut2_off;
+    const uint32_t lds_bytes = ace_lds_layout(rk_off, (uint32_t)rk_bytes, (uint32_t)stg_words, &stg_off, &lut2_off);
     if (lds_bytes > kMaxLds) return ACE_ETOOBIG;
     // window tables: window starts are multiples of 4 ops; every referenced row must fit the
     // resident region; every position's row offsets must point at a row start inside it
@@ -463,7 +463,7 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     g.z_shift = 3;
     while ((1 << (g.z_shift - 3)) < t->z_table_doubles) ++g.z_shift;
     g.zm_delta = (uint32_t)t->n_z << g.z_shift;
-    g.rk_lds_off = rk_off; g.stg_lds_off = stg_off;
+    g.rk_lds_off = rk_off; g.stg_lds_off = stg_off; g.lut2_lds_off = lut2_off;
     g.rk_kind_stride = (uint32_t)(t->n_glog * 64);
     g.row_bytes = (uint32_t)row_bytes;
     g.flags = t->flags; g.main_params = t->main_params; g.optimizer = t->optimizer;

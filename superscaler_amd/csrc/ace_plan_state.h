@@ -128,6 +128,7 @@ struct AceGeom {
     uint32_t z_shift;           // log2(bytes of one resharding-cost table inside a row)
     uint32_t zm_delta;          // bytes from a cost table to the memory table of the same collective (ACE_F_COLLECTIVE_MEM)
     uint32_t rk_lds_off, stg_lds_off;              // LDS byte offsets of the pair-kind and stage LUT regions
+    uint32_t lut2_lds_off;                         // ... of the per-(micro-batch, stage size) offset pairs (see ace_lds_layout)
     uint32_t rk_kind_stride;    // bytes of one pair kind (n_glog * 64)
     uint32_t row_bytes;         // bytes of one op type's row
     int32_t flags;
@@ -142,6 +143,20 @@ ACE_HD uint32_t info_row(const AceGeom &g, uint32_t i) { return (i & 0xffu) * g.
 ACE_HD uint32_t info_nextrow(const AceGeom &g, uint32_t i) { return ((i >> 8) & 0xffu) * g.row_bytes; }
 
 #define ACE_WS_REC 10          // doubles per deferred stage record (see PlanState::stash)
+
+// LDS regions behind the resident rows: pair kinds | stage LUT (one word per (micro-batch, stage size)) | per
+// (micro-batch, stage size) two words: byte offset of the stage's diag inside the cost sub-tables, and the pair-kind block
+// offset relative to it.  Returns the total LDS size.
+#ifdef ACE_HOST_EMU
+inline
+#else
+__host__ __device__ inline
+#endif
+uint32_t ace_lds_layout(uint32_t rk_off, uint32_t rk_bytes, uint32_t stg_words, uint32_t *stg_off, uint32_t *lut2_off) {
+    *stg_off = (rk_off + rk_bytes + 15u) & ~15u;
+    *lut2_off = (*stg_off + stg_words * 4u + 15u) & ~15u;
+    return *lut2_off + stg_words * 8u;
+}
 
 // COLL: consider_collective_memory (the tables carry ACE_F_COLLECTIVE_MEM).
 // BD: per-stage records for the caller.  RANGED: one stage over an op sub-range.  DEFER: stage
@@ -170,6 +185,8 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false> struct Pl
     uint64_t diag_next, rk_next;   // diags / rk_all shifted down by the stages handed out so far
     uint32_t ws_stride;         // DEFER: 16-byte units between two stages of one plan in the workspace
     uint32_t ws_off;            // DEFER: 16-byte units from the plan's first slot to the slot of the current stage (fits: see ensure_stage_ws)
+    uint64_t glogs_next;        // DEFER: glogs shifted down by the stages handed out so far
+    uint32_t lut2_lane;         // DEFER: LDS address of the offset pairs of this plan's micro-batch size
     uint64_t diags;             // the diag of every stage, 4 bits each, looked up once per plan
     uint32_t r_next;            // collective ids of the (previous op, this op) pair, fetched one op ahead
     uint32_t pair_prev;         // pair_bit of the (previous op, this op) pair
@@ -198,17 +215,22 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false> struct Pl
         ideal_hot_v = ideal_start_v = 0;
         if (bidx >= (uint32_t)g.n_mbs) { status = ACE_PLAN_MALFORMED; bidx = 0; }
         if (RANGED && (lo < 0 || hi > g.N || lo >= hi)) { status = ACE_PLAN_MALFORMED; lo = 0; hi = 1; }
-        // one LUT read per possible stage now, none where a stage begins (where few lanes are active)
         diags = 0;
-        uint64_t rks = 0;
-        for (uint32_t k = 0; k < ACE_MAX_STAGES; ++k) {
-            uint32_t glog = (uint32_t)(glogs >> (4u * k)) & 15u;
-            uint32_t w = lds.ld<uint32_t>(g.stg_lds_off + (bidx * 16u + glog) * 4u);
-            diags |= (uint64_t)(w & 15u) << (4u * k);
-            // the stage size as the pair-kind tables index it (a size outside the tables is unscorable anyway: block 0)
-            rks |= (uint64_t)(glog < (uint32_t)g.n_glog ? glog : 0u) << (4u * k);
+        glogs_next = glogs;
+        lut2_lane = g.lut2_lds_off + bidx * 128u;
+        rk_all = 0; diag_next = 0; rk_next = 0;
+        if (!DEFER) {
+            // one LUT read per possible stage now, none where a stage begins (where few lanes are active)
+            uint64_t rks = 0;
+            for (uint32_t k = 0; k < ACE_MAX_STAGES; ++k) {
+                uint32_t glog = (uint32_t)(glogs >> (4u * k)) & 15u;
+                uint32_t w = lds.ld<uint32_t>(g.stg_lds_off + (bidx * 16u + glog) * 4u);
+                diags |= (uint64_t)(w & 15u) << (4u * k);
+                // the stage size as the pair-kind tables index it (a size outside the tables is unscorable anyway: block 0)
+                rks |= (uint64_t)(glog < (uint32_t)g.n_glog ? glog : 0u) << (4u * k);
+            }
+            rewind(rks);
         }
-        rewind(rks);
         if (BD) {
             // the "ideal" pass uses tp = dp = 1 and micro-batch = micro_bs (aceso_cost_model.py:588-590):
             // the diag of (micro_bs, 1 gpu)
@@ -229,6 +251,19 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false> struct Pl
     // `tail`: also what only finish() uses (one LDS read).
     ACE_HD void start_fast(const AceGeom &g, const AceLds &lds, bool tail) {
         ++s;
+        if (DEFER) {
+            // the op loop's two offsets of the next stage are READ, as one pair of words per (micro-batch, stage size): where
+            // a stage ends a lane or two are active, but every vector instruction costs the whole wavefront an issue slot
+            const uint32_t glog = (uint32_t)glogs_next & 15u;      // (past the sixteenth stage: zero, and result() refuses such a plan)
+            glogs_next >>= 4;
+            const ace_u2 zz = lds.ld<ace_u2>(lut2_lane + glog * 8u);
+            z_v = zz.x;
+            rk_v = zz.y;
+            fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = rs_f = rs_b = mc = 0.0;
+            lastclose = false;
+            r_next = 0;
+            return;
+        }
         // the next stage's nibbles sit at the bottom of diag_next / rk_next (stages come in order; past
         // the sixteenth they read zero, and such a plan is caught by result())
         const uint32_t d = (uint32_t)diag_next & 15u;
@@ -301,9 +336,13 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false> struct Pl
     ACE_HD void replay(const AceGeom &g, const AceLds &lds, const uint32_t *pos_info, const double *ws, int s2) {
         const ace_d2 *r = reinterpret_cast<const ace_d2 *>(ws) + (size_t)((uint32_t)s2 * ws_stride);
         ace_d2 r0 = r[0], r1 = r[1], r2 = r[2], r3 = r[3], r4 = r[4];
-        if (s2 == 0) rewind(rk_all);
-        s = s2 - 1;
-        start_fast(g, lds, true);              // s = s2; per-stage offsets, mrow (called for s2 = 0, 1, ... in order)
+        s = s2;
+        {
+            const uint32_t glog = (uint32_t)(glogs >> (4u * ((uint32_t)s2 & 15u))) & 15u;
+            const uint32_t w = lds.ld<uint32_t>(g.stg_lds_off + (bidx * 16u + glog) * 4u);
+            dc_v = ace_mul24(w & 15u, (uint32_t)g.C);
+            mrow = w >> 16;
+        }
         uint64_t meta;
         __builtin_memcpy(&meta, &r4.y, 8);
         uint32_t lo32 = (uint32_t)meta, i_last = (uint32_t)(meta >> 32);

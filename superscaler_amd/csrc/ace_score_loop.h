@@ -60,7 +60,7 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     AceGeom g = a.g;
     const uint32_t lds_base = ace_lds_base(lds_raw);
     g.hot_off += lds_base; g.start_off += lds_base; g.out_off += lds_base; g.z_off += lds_base;
-    g.rk_lds_off += lds_base; g.stg_lds_off += lds_base;
+    g.rk_lds_off += lds_base; g.stg_lds_off += lds_base; g.lut2_lds_off += lds_base;
     const long long slot = block * BLOCK + tid;                     // this lane's place in the batch (and in the workspace)
     long long plan = slot;
 #ifndef ACE_HOST_EMU
@@ -129,8 +129,16 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
 
     // small tables: pair kinds and the (micro-batch, stage gpus) LUT; without windows, every row
     for (int j = tid; j < a.rk_bytes; j += BLOCK) lds_raw[a.g.rk_lds_off + j] = a.pair_kinds[j];
-    for (int j = tid; j < a.stg_words; j += BLOCK)
-        reinterpret_cast<uint32_t *>(lds_raw + a.g.stg_lds_off)[j] = a.stage_lut[j];
+    for (int j = tid; j < a.stg_words; j += BLOCK) {
+        const uint32_t w = a.stage_lut[j];
+        reinterpret_cast<uint32_t *>(lds_raw + a.g.stg_lds_off)[j] = w;
+        // entry j = micro-batch index * 16 + log2(stage size): byte offset of the stage's diag inside the cost sub-tables,
+        // and the pair-kind block of the stage size relative to it (what PlanState::start_fast hands to the op loop)
+        const uint32_t glog = (uint32_t)j & 15u;
+        const uint32_t z_v = (w & 15u) * (uint32_t)a.g.C * 8u;
+        reinterpret_cast<ace_u2 *>(lds_raw + a.g.lut2_lds_off)[j] =
+            ace_u2{z_v, ((glog < (uint32_t)a.g.n_glog ? glog : 0u) << 6) - z_v};
+    }
     stage_window<BLOCK>(a, lds_raw, w0, tid);       // every row, or the first window's
     ACE_SYNC();
 

@@ -63,10 +63,9 @@ extern "C" int ace_emu_score(const ace_tables_t *t, const uint8_t *codes /* [P][
     g.zm_delta = (uint32_t)t->n_z << g.z_shift;
     const int32_t rk_bytes = t->n_pair_kinds * t->n_glog * 64;
     g.rk_lds_off = (uint32_t)t->lds_row_bytes;
-    g.stg_lds_off = (g.rk_lds_off + (uint32_t)rk_bytes + 15u) & ~15u;
+    const uint32_t lds_bytes = ace_lds_layout(g.rk_lds_off, (uint32_t)rk_bytes, (uint32_t)t->n_mbs * 16u, &g.stg_lds_off, &g.lut2_lds_off);
     g.rk_kind_stride = (uint32_t)(t->n_glog * 64);
     g.row_bytes = (uint32_t)t->row_doubles * 8u;
-    const uint32_t lds_bytes = g.stg_lds_off + (uint32_t)t->n_mbs * 16u * 4u;
     g.flags = t->flags; g.main_params = t->main_params; g.optimizer = t->optimizer;
     g.mem_limit = memory_limit; g.strict = strict ? 1 : 0;
     if (range && !stage_out) return -1;
@@ -76,6 +75,11 @@ extern "C" int ace_emu_score(const ace_tables_t *t, const uint8_t *codes /* [P][
         memset(lds.data(), 0xff, lds.size());
         memcpy(lds.data() + g.rk_lds_off, t->pair_kinds, rk_bytes);
         memcpy(lds.data() + g.stg_lds_off, t->stage_lut, (size_t)t->n_mbs * 16 * 4);
+        for (int j = 0; j < t->n_mbs * 16; ++j) {       // (as the kernel's staging loop fills this region)
+            const uint32_t glog = (uint32_t)j & 15u, z_v = (t->stage_lut[j] & 15u) * (uint32_t)C * 8u;
+            const ace_u2 e{z_v, ((glog < (uint32_t)t->n_glog ? glog : 0u) << 6) - z_v};
+            memcpy(lds.data() + g.lut2_lds_off + 8 * j, &e, 8);
+        }
         ace_u4 h;
         memcpy(&h, hdr + 4 * p, 16);
         ace_u2 rg{0u, 0u};
@@ -156,11 +160,10 @@ extern "C" int ace_emu_kernel(const ace_tables_t *t, const uint8_t *codes, const
     g.zm_delta = (uint32_t)t->n_z << g.z_shift;
     a.rk_bytes = t->n_pair_kinds * t->n_glog * 64;
     g.rk_lds_off = (uint32_t)t->lds_row_bytes;
-    g.stg_lds_off = (g.rk_lds_off + (uint32_t)a.rk_bytes + 15u) & ~15u;
+    a.stg_words = t->n_mbs * 16;
+    const uint32_t lds_bytes = ace_lds_layout(g.rk_lds_off, (uint32_t)a.rk_bytes, (uint32_t)a.stg_words, &g.stg_lds_off, &g.lut2_lds_off);
     g.rk_kind_stride = (uint32_t)(t->n_glog * 64);
     g.row_bytes = (uint32_t)t->row_doubles * 8u;
-    a.stg_words = t->n_mbs * 16;
-    const uint32_t lds_bytes = g.stg_lds_off + (uint32_t)a.stg_words * 4u;
     g.flags = t->flags; g.main_params = t->main_params; g.optimizer = t->optimizer;
     g.mem_limit = memory_limit; g.strict = strict ? 1 : 0;
     a.n_windows = t->n_windows; a.row_doubles = t->row_doubles;

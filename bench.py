@@ -71,8 +71,8 @@ def cpu_baseline(tables, batch, threads):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="gpt3_13b")
     ap.add_argument("--plans", type=int, default=None)
     ap.add_argument("--topk", type=int, default=64)

@@ -87,6 +87,7 @@ struct TopkState {                     // lives in the caller's workspace
 __device__ __forceinline__ unsigned long long time_key(double t, uint8_t feasible) {
     // positive doubles order like their bit patterns; infeasible or NaN plans sort last
     if (!feasible || !(t == t)) return kInfKey;
+    if (t == 0.0) t = 0.0;          // (-0.0 compares equal to 0.0 in the reference's float order: one key for both)
     unsigned long long b = (unsigned long long)__double_as_longlong(t);
     return (b >> 63) ? ~b : (b | 0x8000000000000000ull);
 }
@@ -273,6 +274,315 @@ __global__ __launch_bounds__(1024) void topk_finish(TopkState *st, Cand *less, C
     }
     if (threadIdx.x == 0 && out_count) *out_count = (int)cnt;
 }
+
+// ------------------------------------------------------------------------------------------
+// top-k, short form (small k): three launches instead of seventeen.  The k-th smallest key of an evenly spaced SAMPLE
+// bounds the k-th smallest key of the whole input from above, so one pass keeps everything at or below it (about
+// n * k / kSample entries), and one workgroup then selects among those in LDS: radix select on the 96-bit order
+// (key, index), which makes ties fall to the lower index, a gather of the k winners and a small sort.
+// ------------------------------------------------------------------------------------------
+constexpr int kSample = 8192;            // sampled keys, sorted in LDS by one workgroup
+constexpr unsigned kCandCap = 12000;     // candidates the last kernel can hold in LDS (12 bytes each)
+constexpr int kShortMaxK = 256;
+constexpr size_t kShortMaxNK = 1ull << 26;   // n * k up to this: about kSample candidates expected, kCandCap is 4 sigma above
+
+struct ShortTopk { unsigned long long thr; unsigned int count; unsigned int pad; };
+
+// Which of the kRadix buckets of `hist` (LDS) holds the rem-th entry (1-based), counting buckets in order: returns the
+// bucket, the entries before it in `before` and the total in `total` to every lane of the 1024-lane workgroup (no bucket:
+// total < rem, and the return value is meaningless).  Two buckets per lane, wavefront scans, one exchange through LDS.
+__device__ __forceinline__ unsigned int short_pick(const unsigned int *hist, unsigned int rem, unsigned int *wsum /* [16 + 3] */,
+                                                   unsigned int &before, unsigned int &total) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const unsigned int h0 = hist[2 * tid], h1 = hist[2 * tid + 1];
+    unsigned int incl = h0 + h1;
+    for (int off = 1; off < 64; off <<= 1) {
+        const unsigned int v = __shfl_up(incl, off, 64);
+        if (lane >= off) incl += v;
+    }
+    if (lane == 63) wsum[wave] = incl;
+    __syncthreads();
+    unsigned int base = 0, all = 0;
+    for (int w2 = 0; w2 < 16; ++w2) {
+        const unsigned int v = wsum[w2];
+        if (w2 < wave) base += v;
+        all += v;
+    }
+    incl += base;
+    const unsigned int excl = incl - (h0 + h1);
+    if (all >= rem && excl < rem && rem <= incl) {       // exactly one lane
+        const bool second = excl + h0 < rem;
+        wsum[16] = 2 * tid + (second ? 1 : 0);
+        wsum[17] = excl + (second ? h0 : 0u);
+    }
+    __syncthreads();
+    const unsigned int bucket = wsum[16];
+    before = wsum[17];
+    total = all;
+    __syncthreads();                                       // (wsum is reused by the next call)
+    return bucket;
+}
+
+// Smallest and largest finite key of a strided view of the lanes' own keys (kmin = kInfKey: none), to every lane.  The bits
+// above the highest bit in which the two differ are common to all keys: the radix passes start below them, where the
+// histogram spreads (a pass over common bits would send every LDS atomic to one bucket, one after the other).
+// `cnt`: the lane's number of finite keys; `total` their number in all.
+__device__ __forceinline__ void short_minmax(unsigned long long mn, unsigned long long mx, unsigned long long cnt,
+                                             unsigned long long *wmm /* [48] */, unsigned long long &kmin, unsigned long long &kmax,
+                                             unsigned long long &total) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int off = 32; off > 0; off >>= 1) {
+        const unsigned long long a = __shfl_xor(mn, off, 64), b = __shfl_xor(mx, off, 64);
+        cnt += __shfl_xor(cnt, off, 64);
+        mn = a < mn ? a : mn;
+        mx = b > mx ? b : mx;
+    }
+    if (lane == 0) { wmm[3 * wave] = mn; wmm[3 * wave + 1] = mx; wmm[3 * wave + 2] = cnt; }
+    __syncthreads();
+    kmin = kInfKey; kmax = 0; total = 0;
+    for (int w2 = 0; w2 < 16; ++w2) {
+        const unsigned long long a = wmm[3 * w2], b = wmm[3 * w2 + 1];
+        kmin = a < kmin ? a : kmin;
+        kmax = b > kmax ? b : kmax;
+        total += wmm[3 * w2 + 2];
+    }
+    __syncthreads();
+}
+
+// The sample's k-th smallest key, to three radix digits below the bits all sampled keys share: the threshold is the largest key of that
+// bucket, an upper bound of the input's k-th smallest key that lets a few more entries through than the exact one would.
+__global__ __launch_bounds__(1024) void topk_sample(const double *t, const uint8_t *f, size_t n, int k, ShortTopk *st) {
+    __shared__ unsigned long long key[kSample];
+    __shared__ unsigned int hist[kRadix];
+    __shared__ unsigned int wsum[20];
+    const int tid = threadIdx.x;
+    // the sample: 64 runs of 128 consecutive entries, evenly spaced (consecutive entries share cache lines); all of a short input
+    const size_t m = n < (size_t)kSample ? n : (size_t)kSample;
+    const size_t run_step = n / 64;
+    for (int j = tid; j < kSample; j += 1024) {
+        const size_t i = n <= (size_t)kSample ? (size_t)j : (size_t)(j >> 7) * run_step + (size_t)(j & 127);
+        key[j] = (size_t)j < m ? time_key(t[i], f[i]) : kInfKey;
+    }
+    __shared__ unsigned long long wmm[48];
+    unsigned long long mn = kInfKey, mx = 0, nf = 0;
+    __syncthreads();
+    for (int j = tid; j < kSample; j += 1024) {
+        const unsigned long long x = key[j];
+        if (x != kInfKey) { mn = x < mn ? x : mn; mx = x > mx ? x : mx; ++nf; }
+    }
+    unsigned long long kmin, kmax, nfin;
+    short_minmax(mn, mx, nf, wmm, kmin, kmax, nfin);
+    int cur = (nfin == 0 || kmin == kmax) ? 0 : 64 - __clzll((long long)(kmin ^ kmax));      // the low `cur` bits vary
+    unsigned long long prefix = cur >= 64 ? 0ull : (kmin >> cur) << cur;
+    unsigned int rem = (unsigned)k;
+    bool enough = nfin >= (unsigned long long)k;           // fewer than k feasible entries in the sample: keep every feasible entry
+    for (int pass = 0; pass < 3 && enough && cur > 0; ++pass) {
+        for (int j = tid; j < kRadix; j += 1024) hist[j] = 0;
+        __syncthreads();
+        const int bits = cur < kRadixBits ? cur : kRadixBits, shift = cur - bits;
+        for (int j = tid; j < kSample; j += 1024) {
+            const unsigned long long x = key[j];
+            if (x != kInfKey && (cur >= 64 || (x >> cur) == (prefix >> cur)))
+                atomicAdd(&hist[(unsigned)((x >> shift) & ((1ull << bits) - 1ull))], 1u);
+        }
+        __syncthreads();
+        unsigned int before, total;
+        const unsigned int b = short_pick(hist, rem, wsum, before, total);
+        (void)total;
+        prefix |= (unsigned long long)b << shift;
+        rem -= before;
+        cur = shift;
+    }
+    if (tid == 0) {
+        // the largest key that starts with the digits found (all sampled keys equal: that key itself)
+        unsigned long long thr = enough ? (prefix | (cur > 0 ? ((1ull << cur) - 1ull) : 0ull)) : kInfKey;
+        if (thr == kInfKey) thr = kInfKey - 1;
+        st->thr = thr; st->count = 0; st->pad = 0;
+    }
+}
+
+constexpr int kFilterPer = 8;             // entries per lane of topk_filter
+__global__ __launch_bounds__(1024) void topk_filter(const double *t, const uint8_t *f, size_t n, ShortTopk *st, Cand *cand) {
+    // One atomic on the shared counter per WORKGROUP (atomics on one address are served one after the other, about ten
+    // nanoseconds each): the lanes count their hits in LDS first.
+    __shared__ unsigned int s_hits, s_base;
+    const unsigned long long thr = st->thr;
+    const size_t i0 = (size_t)blockIdx.x * 1024 * kFilterPer + threadIdx.x;
+    unsigned long long key[kFilterPer];
+    if (threadIdx.x == 0) s_hits = 0;
+#pragma unroll
+    for (int q = 0; q < kFilterPer; ++q) {
+        const size_t i = i0 + (size_t)q * 1024;
+        key[q] = i < n ? time_key(t[i], f[i]) : kInfKey;
+    }
+    __syncthreads();
+    unsigned int mine = 0;
+#pragma unroll
+    for (int q = 0; q < kFilterPer; ++q) mine += key[q] <= thr ? 1u : 0u;
+    unsigned int first = 0;
+    if (mine) first = atomicAdd(&s_hits, mine);
+    __syncthreads();
+    if (threadIdx.x == 0 && s_hits) s_base = atomicAdd(&st->count, s_hits);
+    __syncthreads();
+    if (mine) {
+        unsigned int p = s_base + first;
+#pragma unroll
+        for (int q = 0; q < kFilterPer; ++q) {
+            if (key[q] <= thr) {
+                if (p < kCandCap) cand[p] = Cand{key[q], (long long)(i0 + (size_t)q * 1024)};
+                ++p;
+            }
+        }
+    }
+}
+
+// Entry j of the selection's input: the candidates in LDS, or -- when more entries passed the filter than LDS holds --
+// the whole input again, read from global memory (slow, exact, and rare: see kShortMaxNK).
+struct ShortSource {
+    const unsigned long long *lkey; const unsigned int *lidx;     // LDS
+    const double *t; const uint8_t *f;                             // global
+    bool global;
+    __device__ __forceinline__ void get(size_t j, unsigned long long &key, unsigned int &idx) const {
+        if (global) { key = time_key(t[j], f[j]); idx = (unsigned int)j; }
+        else { key = lkey[j]; idx = lidx[j]; }
+    }
+};
+
+__global__ __launch_bounds__(1024) void topk_short_final(const double *t, const uint8_t *f, size_t n, ShortTopk *st, const Cand *cand,
+                                                         int k, long long *out_idx, double *out_val, int *out_count) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    unsigned long long *lkey = reinterpret_cast<unsigned long long *>(smem);                       // [kCandCap]
+    unsigned int *lidx = reinterpret_cast<unsigned int *>(smem + (size_t)kCandCap * 8);            // [kCandCap]
+    unsigned int *hist = lidx + kCandCap;                                                          // [kRadix]
+    Cand *win = reinterpret_cast<Cand *>(hist + kRadix);                                           // [kShortMaxK]
+    __shared__ unsigned int wsum[20];
+    __shared__ unsigned int s_nwin;
+    const int tid = threadIdx.x;
+    const unsigned int count = st->count;
+    ShortSource src{lkey, lidx, t, f, count > kCandCap};
+    const size_t m = src.global ? n : (size_t)count;
+    if (!src.global)
+        for (unsigned j = tid; j < count; j += 1024) { const Cand c = cand[j]; lkey[j] = c.key; lidx[j] = (unsigned int)c.idx; }
+    if (tid == 0) s_nwin = 0;
+    // radix select on the 96-bit order (key, index): 6 passes over the key bits, then 3 over the index bits of the entries
+    // whose key is the selected one -- cut short as soon as the bucket that holds the k-th entry is small enough to be sorted
+    // as it is (usually after two passes).  State is kept by every lane alike (short_pick returns the same values to all).
+    constexpr unsigned kSmall = 512;                           // bucket entries that fit the histogram's LDS as (key, index) pairs
+    Cand *bucket = reinterpret_cast<Cand *>(hist);
+    __shared__ unsigned int s_nbucket;
+    __shared__ unsigned long long wmm[48];
+    unsigned long long mn = kInfKey, mx = 0, nf = 0;
+    __syncthreads();
+    for (size_t j = tid; j < m; j += 1024) {
+        unsigned long long key; unsigned int idx;
+        src.get(j, key, idx);
+        if (key != kInfKey) { mn = key < mn ? key : mn; mx = key > mx ? key : mx; ++nf; }
+    }
+    unsigned long long kmin, kmax, nfin;
+    short_minmax(mn, mx, nf, wmm, kmin, kmax, nfin);
+    const bool all = nfin < (unsigned long long)k;             // fewer feasible entries than asked for: all of them win
+    int cur = (nfin == 0 || kmin == kmax) ? 0 : 64 - __clzll((long long)(kmin ^ kmax));      // the low `cur` key bits vary
+    unsigned long long prefix = cur >= 64 ? 0ull : (kmin >> cur) << cur;
+    unsigned int iprefix = 0, rem = (unsigned)k;
+    bool small = false;
+    int small_shift = 0, icur = 32;
+    if (tid == 0) s_nbucket = 0;
+    // key digits from the highest varying bit down, then index digits among the entries with the selected key
+    while (!all && !small && (cur > 0 || icur > 0)) {
+        for (int j = tid; j < kRadix; j += 1024) hist[j] = 0;
+        __syncthreads();
+        const bool on_key = cur > 0;
+        const int top = on_key ? cur : icur;
+        const int bits = top < kRadixBits ? top : kRadixBits, shift = top - bits;
+        for (size_t j = tid; j < m; j += 1024) {
+            unsigned long long key; unsigned int idx;
+            src.get(j, key, idx);
+            if (key == kInfKey) continue;
+            if (on_key) {
+                if (cur >= 64 || (key >> cur) == (prefix >> cur))
+                    atomicAdd(&hist[(unsigned)((key >> shift) & ((1ull << bits) - 1ull))], 1u);
+            } else if (key == prefix) {
+                if (icur >= 32 || (idx >> icur) == (iprefix >> icur)) atomicAdd(&hist[(idx >> shift) & ((1u << bits) - 1u)], 1u);
+            }
+        }
+        __syncthreads();
+        unsigned int before, total;
+        const unsigned int b = short_pick(hist, rem, wsum, before, total);
+        (void)total;
+        rem -= before;
+        if (on_key) {
+            prefix |= (unsigned long long)b << shift;
+            cur = shift;
+            if (hist[b] <= kSmall) { small = true; small_shift = shift; }
+        } else {
+            iprefix |= b << shift;
+            icur = shift;
+        }
+        __syncthreads();                                       // (hist[b] read by all before the next pass clears it)
+    }
+    // gather the winners
+    for (size_t j = tid; j < m; j += 1024) {
+        unsigned long long key; unsigned int idx;
+        src.get(j, key, idx);
+        if (key == kInfKey) continue;
+        bool wins;
+        if (all) wins = true;
+        else if (small) {
+            // the key bits from small_shift up are fixed: below the bucket -> a winner; in it -> sorted below
+            const unsigned long long hk = key >> small_shift, hp = prefix >> small_shift;
+            wins = hk < hp;
+            if (hk == hp) {
+                const unsigned int p = atomicAdd(&s_nbucket, 1u);
+                if (p < kSmall) bucket[p] = Cand{key, (long long)idx};
+            }
+        } else wins = key < prefix || (key == prefix && idx <= iprefix);
+        if (wins) {
+            const unsigned int p = atomicAdd(&s_nwin, 1u);
+            if (p < (unsigned)kShortMaxK) win[p] = Cand{key, (long long)idx};
+        }
+    }
+    __syncthreads();
+    if (small) {
+        // the `rem` smallest (key, index) of the bucket join the winners: an entry's rank is the number of entries before
+        // it in that order (the pairs are distinct), so every lane finds the place of one entry by itself
+        const unsigned int nb = s_nbucket < kSmall ? s_nbucket : kSmall;
+        const unsigned int base = s_nwin;
+        if ((unsigned)tid < nb) {
+            const Cand me = bucket[tid];
+            unsigned int rank = 0;
+            for (unsigned j = 0; j < nb; ++j) {
+                const Cand o = bucket[j];
+                rank += (o.key < me.key || (o.key == me.key && o.idx < me.idx)) ? 1u : 0u;
+            }
+            if (rank < rem && base + rank < (unsigned)kShortMaxK) win[base + rank] = me;
+        }
+        __syncthreads();
+        if (tid == 0) s_nwin = base + rem;
+    }
+    __syncthreads();
+    const unsigned int nwin = s_nwin < (unsigned)k ? s_nwin : (unsigned)k;
+    // the winners in ascending (key, index) order, by rank as above
+    for (unsigned j = tid; j < (unsigned)k; j += 1024) {
+        if (j >= nwin) {
+            out_idx[j] = -1;
+            out_val[j] = __longlong_as_double(0x7ff0000000000000ll);
+        }
+    }
+    if ((unsigned)tid < nwin) {
+        const Cand me = win[tid];
+        unsigned int rank = 0;
+        for (unsigned j = 0; j < nwin; ++j) {
+            const Cand o = win[j];
+            rank += (o.key < me.key || (o.key == me.key && o.idx < me.idx)) ? 1u : 0u;
+        }
+        unsigned long long b = me.key;
+        b = (b >> 63) ? (b & 0x7fffffffffffffffull) : ~b;
+        out_idx[rank] = me.idx;
+        out_val[rank] = __longlong_as_double((long long)b);
+    }
+    if (tid == 0 && out_count) *out_count = (int)nwin;
+}
+constexpr size_t kShortLds = (size_t)kCandCap * 12 + (size_t)kRadix * 4 + (size_t)kShortMaxK * sizeof(Cand);
 
 unsigned int next_pow2(unsigned int v) {
     unsigned int p = 1;
@@ -483,6 +793,8 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
         (rc = upload((void **)&h->d_win_pos, t->win_pos, (size_t)(t->n_windows + 1) * 4)) ||
         (rc = upload((void **)&h->d_win_row_begin, t->win_row_begin, (size_t)(t->n_windows + 1) * 4)) ||
         (rc = upload((void **)&h->d_win_rows, t->win_rows, (size_t)n_win_rows * 8)) ||
+        (rc = hipFuncSetAttribute(reinterpret_cast<const void *>(&topk_short_final), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)kShortLds) == hipSuccess ? ACE_OK : ACE_EHIP) ||
         (rc = allow_big_lds<false, false, false, false>()) || (rc = allow_big_lds<false, false, true, false>()) ||
         (rc = allow_big_lds<false, false, false, true>()) ||
         (rc = allow_big_lds<true, false, false, false>()) || (rc = allow_big_lds<true, false, true, false>()) ||
@@ -654,7 +966,8 @@ size_t ace_topk_workspace_bytes(size_t n, int k) {
     if (k <= 0) return 0;
     const unsigned cap = topk_cap(k);
     const unsigned p2 = next_pow2(2 * cap);
-    return 256 + sizeof(unsigned int) * kRadix + sizeof(Cand) * ((size_t)cap * 2 + p2);
+    // (the last part: state and candidates of the short form)
+    return 256 + sizeof(unsigned int) * kRadix + sizeof(Cand) * ((size_t)cap * 2 + p2) + 256 + sizeof(Cand) * kCandCap;
 }
 
 int ace_topk(ace_handle_t *h, const double *d_iter_ms, const uint8_t *d_feasible, size_t n, int k, int64_t *d_idx,
@@ -673,6 +986,17 @@ int ace_topk(ace_handle_t *h, const double *d_iter_ms, const uint8_t *d_feasible
     unsigned blocks = (unsigned)((n + kTopBlock * 8 - 1) / (kTopBlock * 8));
     if (blocks < 1) blocks = 1;
     if (blocks > 2048) blocks = 2048;
+    if (k <= kShortMaxK && n * (size_t)k <= kShortMaxNK && n <= 0xffffffffull) {
+        ShortTopk *sst = (ShortTopk *)(buf + p2);
+        Cand *cand = (Cand *)((unsigned char *)sst + 256);
+        hipLaunchKernelGGL(topk_sample, dim3(1), dim3(1024), 0, s, d_iter_ms, d_feasible, n, k, sst);
+        hipLaunchKernelGGL(topk_filter, dim3((unsigned)((n + 1024 * kFilterPer - 1) / (1024 * kFilterPer))), dim3(1024), 0, s, d_iter_ms,
+                           d_feasible, n, sst, cand);
+        hipLaunchKernelGGL(topk_short_final, dim3(1), dim3(1024), kShortLds, s, d_iter_ms, d_feasible, n, sst, cand, k,
+                           (long long *)d_idx, d_val, d_count);
+        ACE_HIP(hipGetLastError());
+        return ACE_OK;
+    }
     hipLaunchKernelGGL(topk_init, dim3(1), dim3(256), 0, s, st, hist, k);
     for (int pass = 0; pass < kPasses; ++pass) {
         hipLaunchKernelGGL(topk_hist, dim3(blocks), dim3(kTopBlock), 0, s, d_iter_ms, d_feasible, n, pass, st, hist);

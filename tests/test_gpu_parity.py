@@ -108,6 +108,48 @@ def test_topk_ties_pick_lowest_index(torch_mod):
     ev.close()
 
 
+def test_topk_short_form_edges(torch_mod):
+    """The three-launch form of the top-k (small k): inputs on which the sample's bound lets nearly everything through (all
+    times equal, a million of them: the last kernel then selects from global memory), heavy duplication, negative zero and
+    infinities, all infeasible, a single entry -- against a stable sort; and the same results as the multi-launch form."""
+    from superscaler_amd.evaluator import PlanEvaluator
+    torch = torch_mod
+    w = synth.WORKLOADS["gpt3_1_3b"]
+    ev = PlanEvaluator(synth.make_tables(w))
+    rng = np.random.default_rng(5)
+
+    def check(ht, hf, ks):
+        t = torch.from_numpy(ht).cuda()
+        f = torch.from_numpy(hf).cuda()
+        key = np.where((hf > 0) & ~np.isnan(ht), ht, np.inf)
+        order = np.lexsort((np.arange(len(ht)), key))
+        n_ok = int(np.isfinite(key).sum()) if not np.isinf(ht[hf > 0]).any() else None
+        for k in ks:
+            idx, val, cnt = ev.topk(t, f, k)
+            idx, val = idx.cpu().numpy(), val.cpu().numpy()
+            n = int(cnt.item())
+            if n_ok is not None:
+                assert n == min(k, n_ok)
+            assert np.array_equal(idx[:n], order[:n]) and np.array_equal(val[:n], ht[order[:n]]), (len(ht), k)
+            assert (idx[n:] == -1).all()
+
+    n = 1 << 20
+    check(np.full(n, 7.25), np.ones(n, dtype=np.uint8), [1, 64, 256])                      # one value: every entry passes the filter
+    check(rng.integers(0, 50, n).astype(np.float64), (rng.random(n) < 0.9).astype(np.uint8), [64, 200])   # 50 distinct values
+    t = rng.lognormal(3.0, 1.0, 300000)
+    t[::1000] = 0.0
+    t[1::1000] = -0.0
+    check(t, (rng.random(300000) < 0.5).astype(np.uint8), [8, 64, 256, 257, 300])           # (257, 300: the multi-launch form)
+    check(rng.random(5000), np.zeros(5000, dtype=np.uint8), [64])                           # nothing feasible
+    check(rng.random(70), np.ones(70, dtype=np.uint8), [64, 100])                           # fewer entries than the sample, than k
+    check(np.array([3.5]), np.ones(1, dtype=np.uint8), [1, 5])
+    t = rng.random(100000)
+    f = np.zeros(100000, dtype=np.uint8)
+    f[rng.choice(100000, 40, replace=False)] = 1
+    check(t, f, [64])                                                                       # fewer feasible entries than k, none in the sample
+    ev.close()
+
+
 GOLDEN = ["gpt_1_3B", "resnet_500M", "t5_770M"]
 
 

@@ -23,8 +23,8 @@ HBM_PEAK_GBPS = 8000.0
 # of a plain 256 MiB copy in the same pass; vector instructions per op and wavefront = SQ_INSTS_VALU / SQ_WAVES /
 # ops; 14 of them are the reference's own fp64 arithmetic (nine adds / multiply-adds, five maxima).
 PROFILE_COUNTERS = {
-    ("gpt3_13b", 523): {"source": "profiles/score_kernel_gpt3_13b.md", "traffic_bytes_per_plan": 1952.0,
-                        "valu_per_op_per_wavefront": 60.1, "valu_busy": 0.88},
+    ("gpt3_13b", 523): {"source": "profiles/score_kernel_gpt3_13b.md", "traffic_bytes_per_plan": 2206.0,
+                        "valu_per_op_per_wavefront": 47.4, "valu_busy": 0.85},
 }
 ESSENTIAL_VALU_PER_OP = 14
 

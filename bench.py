@@ -23,7 +23,7 @@ HBM_PEAK_GBPS = 8000.0
 # of a plain 256 MiB copy in the same pass; vector instructions per op and wavefront = SQ_INSTS_VALU / SQ_WAVES /
 # ops; 14 of them are the reference's own fp64 arithmetic (nine adds / multiply-adds, five maxima).
 PROFILE_COUNTERS = {
-    ("gpt3_13b", 523): {"source": "profiles/score_kernel_gpt3_13b.md", "traffic_bytes_per_plan": 2206.0,
+    ("gpt3_13b", 523): {"source": "profiles/score_kernel_gpt3_13b.md", "commit": "381908c", "traffic_bytes_per_plan": 2206.0,
                         "valu_per_op_per_wavefront": 47.4, "valu_busy": 0.85},
 }
 ESSENTIAL_VALU_PER_OP = 14
@@ -188,7 +188,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS,
                      "traffic": counters["traffic_bytes_per_plan"] * P if counters else None,
-                     "traffic_source": counters["source"] if counters else None,
+                     "traffic_source": f'{counters["source"]} (library sources of commit {counters["commit"]})' if counters else None,
                      "algorithmic_bytes": algo_bytes,
                      "kernel": "ace_score_kernel<BD=false,RANGED=false,WIN=false,DEFER=true>", "kernel_ms": kern_ms,
                      "algorithmic_bytes_per_plan": 3 * N + 19,

@@ -64,12 +64,13 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     const long long slot = block * BLOCK + tid;                     // this lane's place in the batch (and in the workspace)
     long long plan = slot;
 #ifndef ACE_HOST_EMU
-    if (DEFER && BLOCK >= 128) {
+    if (!RANGED && BLOCK >= 128) {
         // The lanes of a wavefront walk the ops together, and every op at which one of them closes a stage takes all
         // of them through the stage-end code: so the workgroup deals its plans to its lanes by pipeline depth
         // (counting sort on the depth in the plan header, deepest first; plans of one depth in any order), and the
         // sorted wavefronts to the SIMDs in turn (wavefront w runs on SIMD w % 4) so that each SIMD gets the same
-        // mix.  Only which lane scores which plan changes: results go to the plan's own index.
+        // mix.  Only which lane scores which plan changes: results go to the plan's own index.  (Single-stage queries
+        // are left as they come: their length, not a depth, is what would have to be sorted on.)
         unsigned int *cnt = reinterpret_cast<unsigned int *>(lds_raw);                  // 17 bins (nothing is staged yet)
         unsigned short *plan_of = reinterpret_cast<unsigned short *>(lds_raw + 128);     // [BLOCK]
         uint32_t depth = 0;                                                              // lanes past the batch: last

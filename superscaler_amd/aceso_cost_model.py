@@ -525,6 +525,12 @@ class CostModel:
         from .recompute import update_recompute_device
         return update_recompute_device(self, dbatch)
 
+    def generate_initial_config(self, num_stages, args):
+        """aceso_utils.py:710-721: the search's starting plan for `args.initial_point` (balance, imbalance_gpu,
+        imbalance_op, test, or the path of a plan file) on this model's op list; unscored."""
+        from .initial_plans import generate_initial_config
+        return generate_initial_config(num_stages, args, self.graph.ops)
+
     def predict_value_after_move(self, config, bottleneck, partner, num_ops_moved, metric, inc_gpus=False,
                                  dec_gpus=False, dim=None):
         """aceso_cost_model.py:693-739."""
@@ -659,3 +665,70 @@ def get_reserved_memory_list(config):
 
 def get_activation_size(op_name, mbs, tp, algo_index=0):
     return _m().get_activation_size(op_name, mbs, tp, algo_index)
+
+
+def reference_arg_parser():
+    """The flags of the reference's command lines that the cost model reads (aceso_utils.py:359-453), with its
+    defaults; flags of the search itself are accepted and ignored."""
+    import argparse
+    ap = argparse.ArgumentParser(allow_abbrev=False)
+    ap.add_argument("--model-name", type=str, default=None)
+    ap.add_argument("--model-size", type=str, default=None)
+    ap.add_argument("--num-layers", type=int, default=None)
+    ap.add_argument("--global-batch-size", type=int, default=None)
+    ap.add_argument("--micro-batch-size", type=int, nargs="+", default=None)
+    ap.add_argument("--num-nodes", type=int, required=True)
+    ap.add_argument("--num-gpus-per-node", type=int, required=True)
+    ap.add_argument("--memory-limit", type=int, default=28000)
+    ap.add_argument("--max-tp", type=int, default=None)
+    ap.add_argument("--profiled-time-path", type=str, required=True, help="with the trailing /")
+    ap.add_argument("--memory-pred-type", type=str, default="MAX")
+    ap.add_argument("--initial-point", type=str, default="balance")
+    ap.add_argument("--init-dim", type=str, default="tp")
+    ap.add_argument("--do-not-consider-shared-tensor-space", action="store_false", dest="consider_shared_space")
+    ap.add_argument("--do-not-consider-reserved-space", action="store_false", dest="consider_reserved_space")
+    ap.add_argument("--do-not-use-flex-recompute", action="store_false", dest="flex_recompute")
+    ap.add_argument("--peak-mem-in-backward", type=int, default=0)
+    ap.add_argument("--consider-collective-memory", action="store_true")
+    ap.add_argument("--save-to-csv", type=str, default=None)
+    return ap
+
+
+def main(argv=None, device="cuda:0") -> int:
+    """`python -m superscaler_amd.aceso_cost_model`: what the reference's module does when run as a script
+    (aceso_cost_model.py:926-932) -- read the plan file named by --initial-point, print its time and memory
+    breakdown, write the per-stage csv if --save-to-csv names one.  Takes the reference's flags."""
+    import json
+    from .plan import config_from_json, save_config_info_to_csv
+    ns, _ignored = reference_arg_parser().parse_known_args(argv)
+    ns.num_gpus = ns.num_nodes * ns.num_gpus_per_node
+    with open(ns.initial_point) as f:
+        config_dict = json.load(f)
+    # (aceso_utils.py:473-497: the plan file names the model; defaults of the micro-batch sizes by model)
+    ns.model_name, ns.model_size = config_dict["model_name"], config_dict["model_size"]
+    if ns.model_name not in ("resnet", "gpt", "t5", "scale-layer"):
+        raise RuntimeError(f"model {ns.model_name} is not supported yet.")
+    if ns.micro_batch_size is None:
+        ns.micro_batch_size = [16, 32, 48, 64] if ns.model_name == "resnet" else [1, 2, 4, 8]
+    if ns.num_layers is None:
+        from .plan import GPT_CONFIGS, T5_CONFIGS
+        if ns.model_name == "gpt":
+            ns.num_layers = GPT_CONFIGS[ns.model_size][0]
+        elif ns.model_name == "t5":
+            ns.num_layers = T5_CONFIGS[ns.model_size][0]
+        elif ns.model_name == "scale-layer":
+            raise RuntimeError("should provide --num-layers for scale-layer exp")
+    configure(ns, device)
+    read_profiled_time(config_dict["model_name"], config_dict["model_size"], ns.profiled_time_path)
+    try:
+        config = config_from_json(config_dict, _m().graph.ops)
+        predict_time_breakdown(config, print_time=True, print_memory=True)
+        if ns.save_to_csv is not None:
+            save_config_info_to_csv(config, get_reserved_memory_list(config), ns.save_to_csv)
+    finally:
+        _m().close()
+    return 0
+
+
+if __name__ == "__main__":
+    raise SystemExit(main())

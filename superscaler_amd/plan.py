@@ -322,6 +322,17 @@ def dump_config_to_json(config, file_name: str, model_name: str, model_size: str
         json.dump(config_to_json_dict(config, model_name, model_size, num_layers), f, indent=4)
 
 
+def save_config_info_to_csv(config, reserved_mem_list, file_name: str) -> None:
+    """aceso_utils.py:244-252: one line per stage of a scored plan (time, total / normal / reserved memory)."""
+    import csv
+    rows = [["stage-index", "time", "memory(total)", "memory(normal)", "memory(reserved)"]]
+    for i in range(config.num_stages):
+        rows.append([f"stage-{i}", f"{config.time_list[i]:.2f}", f"{config.memory_list[i]:.2f}",
+                     f"{(config.memory_list[i] - reserved_mem_list[i]):.2f}", f"{reserved_mem_list[i]:.2f}"])
+    with open(file_name, mode="w", newline="") as f:
+        csv.writer(f).writerows(rows)
+
+
 def check_legality(config, num_gpus: int, num_gpus_per_node: int, num_nodes: int) -> bool:
     """aceso_utils.py:760-774: stage sizes in {1,2,4,8}, all devices used, node boundaries fall on
     stage boundaries."""

@@ -146,6 +146,8 @@ class ProfileDB:
         try:
             db.inter_band = band(time_path + "p2p_inter_node.csv")
         except OSError:
+            if verbose:
+                print("inter-node bandwidth file is not found, using intra-node bandwidth instead.")
             db.inter_band = list(db.intra_band)
         return db
 

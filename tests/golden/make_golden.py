@@ -3,7 +3,9 @@
 
 Run in the build container only (it needs /root/reference):
 
-    python tests/golden/make_golden.py
+    python tests/golden/make_golden.py [base] [variants] [moves] [grid] [initial] [main] [kat]
+
+(no argument: every part).
 
 For each model family it (1) copies the few profile-database CSV files the case needs from
 the reference tree into tests/golden/db_<case>/ (data files, not source), (2) starts one
@@ -26,7 +28,11 @@ Further children of the same kind write
                                    action_move_once, prim_mig_op, prim_tp_dp, prim_mbs,
                                    prim_tp_dp_exchange) make of seeded legal plans;
   megatron_grid_<case>.json        the plan files search/gen_megatron_plan.py itself writes (run as
-                                   the script it is, in a scratch directory).
+                                   the script it is, in a scratch directory);
+  initial_<case>.json              the starting plans of the search (aceso_utils.py generate_initial_config:
+                                   balance, imbalance_gpu, imbalance_op, test) for 1 to 8 stages;
+  main_<case>.json                 what search/aceso_cost_model.py prints and saves (--save-to-csv) when run as a
+                                   script on a plan file.
 """
 import json
 import os
@@ -348,6 +354,118 @@ def run_grid(case, num_saved=4):
     print(f"[golden] megatron grid {case}: {sorted(files)}")
 
 
+def pack_plan_runs(config):
+    """A plan as run-length lists [value, count] over all its ops (any integer value, unlike pack_plan's digits)."""
+    def runs(key):
+        out = []
+        for st in config.stages:
+            for x in getattr(st, key):
+                if out and out[-1][0] == int(x):
+                    out[-1][1] += 1
+                else:
+                    out.append([int(x), 1])
+        return out
+    return {"num_ops_in_each_stage": [len(st.ops) for st in config.stages], "tp": runs("tp_size"), "dp": runs("dp_size"),
+            "recompute_ops": runs("recompute_ops"), "algo": runs("algo"), "micro_batch_size": config.micro_bs,
+            "num_gpus": [st.num_gpus for st in config.stages]}
+
+
+def child_initial(case):
+    """generate_initial_config (aceso_utils.py:537-721) for its four built-in starting points, 1 to 8 stages,
+    both values of --init-dim: the plan it returns, None, or the exception it ends with."""
+    import contextlib
+    import io
+    model, size, db, mbs_list, nodes, gpn, gbs, limit, num_layers = CASES[case]
+    extra = ["--num-layers", str(num_layers)] if num_layers else []
+    sys.argv = reference_argv(case, extra)
+    sys.path.insert(0, os.path.join(REF, "search"))
+    import aceso_utils as U                # noqa: the reference, imported to record its outputs
+    args = U.parse_args()
+    out = {"case": case, "model_name": model, "model_size": size, "micro_batch_size": mbs_list, "num_nodes": nodes,
+           "num_gpus_per_node": gpn, "global_batch_size": gbs, "num_layers": num_layers, "max_tp": args.max_tp,
+           "plans": []}
+    for flex in (True, False):
+        for init_dim in ("tp", "dp"):
+            for point in ("balance", "imbalance_gpu", "imbalance_op", "test"):
+                if init_dim == "dp" and point != "balance":
+                    continue                      # only the balanced start reads --init-dim
+                if not flex and point not in ("balance", "imbalance_op"):
+                    continue                      # only these two read --do-not-use-flex-recompute
+                for num_stages in range(1, 9):
+                    args.initial_point, args.init_dim, args.flex_recompute = point, init_dim, flex
+                    try:
+                        with contextlib.redirect_stdout(io.StringIO()):
+                            cfg = U.generate_initial_config(num_stages, args)
+                        rec = None if cfg is None else pack_plan_runs(cfg)
+                    except Exception as e:        # (the reference's own failures are part of its behaviour)
+                        rec = {"error": type(e).__name__}
+                    out["plans"].append([point, init_dim, flex, num_stages, rec])
+    with open(os.path.join(HERE, f"initial_{case}.json"), "w") as f:
+        json.dump(out, f)
+    kinds = {"plan": 0, "none": 0, "error": 0}
+    for *_, rec in out["plans"]:
+        kinds["none" if rec is None else ("error" if "error" in rec else "plan")] += 1
+    print(f"[golden] initial plans {case}: {kinds}")
+
+
+def run_main(case):
+    """search/aceso_cost_model.py run as the script it is (:926-932: read a plan file, print the time and memory
+    breakdown, --save-to-csv) in a scratch directory; its standard output and the csv file it writes go into one
+    fixture.  Plan files: the ones gen_megatron_plan.py wrote for this case (megatron_grid_<case>.json), else the
+    reference's own single-GPU plan of that model."""
+    import tempfile
+    model, size, db, mbs_list, nodes, gpn, gbs, limit, num_layers = CASES[case]
+    grid = os.path.join(HERE, f"megatron_grid_{case}.json")
+    plans = {}
+    if os.path.exists(grid):
+        with open(grid) as f:
+            plans = json.load(f)["files"]
+    else:
+        name = {"resnet_500M": "resnet_500M_mbs64_recomp.json", "t5_770M": "t5_770M_mbs2_recomp.json"}[case]
+        with open(os.path.join(REF, "search", "single_gpu_configs", name)) as f:
+            plans = {name: json.load(f)}
+    # ... and three of the seeded multi-stage plans of <case>.json (mixed tp / dp / algorithms: resharding is active),
+    # in the form read_config_from_json reads (aceso_utils.py:213-242)
+    base = os.path.join(HERE, f"{case}.json")
+    if os.path.exists(base):
+        with open(base) as f:
+            b = json.load(f)
+        for k, pl in enumerate(b["plans"][:3]):
+            per_op = {key: (json.loads(pl[key]) if isinstance(pl[key], str) else pl[key]) for key in ("tp", "dp", "recompute_ops", "algo")}
+            cuts = [0]
+            for n in pl["num_ops_in_each_stage"]:
+                cuts.append(cuts[-1] + n)
+            split = lambda xs: [xs[cuts[i]:cuts[i + 1]] for i in range(len(cuts) - 1)]
+            plans[f"seeded_plan_{k}.json"] = {
+                "model_name": model, "model_size": size, "num_layers": num_layers,
+                "micro_batch_size": pl["micro_batch_size"], "global_batch_size": gbs,
+                "num_gpus": [per_op["tp"][c] * per_op["dp"][c] for c in cuts[:-1]],
+                "num_ops_in_each_stage": pl["num_ops_in_each_stage"],
+                "model_parallel_size_of_each_op": split(per_op["tp"]), "data_parallel_size_of_each_op": split(per_op["dp"]),
+                "recompute_ops": split(per_op["recompute_ops"]), "algo_of_each_op": split(per_op["algo"])}
+    runs = []
+    with tempfile.TemporaryDirectory() as tmp:
+        for name, plan in sorted(plans.items()):
+            with open(os.path.join(tmp, name), "w") as f:
+                json.dump(plan, f)
+            single = sum(plan["num_gpus"]) == 1
+            flags = ["--initial-point", os.path.join(tmp, name), "--save-to-csv", os.path.join(tmp, "out.csv")]
+            if isinstance(plan.get("num_layers"), int):
+                flags += ["--num-layers", str(plan["num_layers"])]
+            argv = reference_argv(case, flags)[1:]
+            if single:                          # the single-GPU plans are for one node with one GPU
+                argv[argv.index("--num-nodes") + 1] = "1"
+                argv[argv.index("--num-gpus-per-node") + 1] = "1"
+            r = subprocess.run([sys.executable, os.path.join(REF, "search", "aceso_cost_model.py")] + argv, check=True,
+                               cwd=tmp, stdout=subprocess.PIPE, text=True)
+            with open(os.path.join(tmp, "out.csv")) as f:
+                csv_text = f.read()
+            runs.append({"plan_file": name, "plan": plan, "single_gpu": single, "stdout": r.stdout, "csv": csv_text})
+    with open(os.path.join(HERE, f"main_{case}.json"), "w") as f:
+        json.dump({"case": case, "runs": runs}, f)
+    print(f"[golden] command line {case}: {[r['plan_file'] for r in runs]}")
+
+
 def main():
     if len(sys.argv) > 2 and sys.argv[1] == "--child":
         return child(sys.argv[2])
@@ -355,18 +473,34 @@ def main():
         return child_variant(sys.argv[2], sys.argv[3])
     if len(sys.argv) > 2 and sys.argv[1] == "--child-moves":
         return child_moves(sys.argv[2])
+    if len(sys.argv) > 2 and sys.argv[1] == "--child-initial":
+        return child_initial(sys.argv[2])
+    # optional arguments: the parts to (re)write, of base variants moves grid initial main kat; none = all
+    parts = set(sys.argv[1:]) or {"base", "variants", "moves", "grid", "initial", "main", "kat"}
     quiet = subprocess.DEVNULL if os.environ.get("GOLDEN_QUIET") else None
     me = os.path.abspath(__file__)
     for case in CASES:
         copy_db(case)
-        subprocess.run([sys.executable, me, "--child", case], check=True, stdout=quiet)
+        if "base" in parts:
+            subprocess.run([sys.executable, me, "--child", case], check=True, stdout=quiet)
         for variant in VARIANTS:
+            if "variants" not in parts:
+                break
             if "collmem" in variant and CASES[case][0] == "t5":
                 continue            # (resharding is off for T5, aceso_utils.py:523-526: the switch changes nothing)
             subprocess.run([sys.executable, me, "--child-variant", case, variant], check=True, stdout=quiet)
     for case in MOVE_CASES:
-        subprocess.run([sys.executable, me, "--child-moves", case], check=True, stdout=quiet)
-    run_grid("gpt_1_3B")
+        if "moves" in parts:
+            subprocess.run([sys.executable, me, "--child-moves", case], check=True, stdout=quiet)
+    if "grid" in parts:
+        run_grid("gpt_1_3B")
+    for case in CASES:
+        if "initial" in parts:
+            subprocess.run([sys.executable, me, "--child-initial", case], check=True, stdout=quiet)
+        if "main" in parts:
+            run_main(case)
+    if "kat" not in parts:
+        return
     # the single-GPU known-answer plans and the database files they index (data files)
     kat = os.path.join(HERE, "kat")
     os.makedirs(kat, exist_ok=True)

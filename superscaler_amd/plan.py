@@ -322,6 +322,17 @@ def dump_config_to_json(config, file_name: str, model_name: str, model_size: str
         json.dump(config_to_json_dict(config, model_name, model_size, num_layers), f, indent=4)
 
 
+def sort_configs(config_list, sort_metric):
+    """aceso_utils.py:723-758: scored plans in ascending order of their slowest stage ("max_stage_time") or of
+    `total_gpu_time`; plans that compare equal keep their order (the reference inserts a plan in front of the first
+    one that is strictly larger).  For encoded batches the same order comes from CostModel.top_k."""
+    if sort_metric == "max_stage_time":
+        return sorted(config_list, key=lambda c: max(c.time_list))
+    if sort_metric == "total_gpu_time":
+        return sorted(config_list, key=lambda c: c.total_gpu_time)
+    raise RuntimeError(f"sort_metric {sort_metric} not supported.")
+
+
 def save_config_info_to_csv(config, reserved_mem_list, file_name: str) -> None:
     """aceso_utils.py:244-252: one line per stage of a scored plan (time, total / normal / reserved memory)."""
     import csv

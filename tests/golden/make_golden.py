@@ -400,6 +400,17 @@ def child_initial(case):
                     except Exception as e:        # (the reference's own failures are part of its behaviour)
                         rec = {"error": type(e).__name__}
                     out["plans"].append([point, init_dim, flex, num_stages, rec])
+    # sort_configs (aceso_utils.py:723-758) on lists with repeated values: the order it returns, as indices
+    import types
+    rng = random.Random(0xACE52)
+    out["sort"] = []
+    for n in (1, 2, 7, 40):
+        times = [[float(rng.randrange(5)), float(rng.randrange(5))] for _ in range(n)]
+        gpu = [float(rng.randrange(4)) for _ in range(n)]
+        objs = [types.SimpleNamespace(time_list=t, total_gpu_time=g, k=k) for k, (t, g) in enumerate(zip(times, gpu))]
+        out["sort"].append({"time_list": times, "total_gpu_time": gpu,
+                            "max_stage_time": [o.k for o in U.sort_configs(objs, "max_stage_time")],
+                            "by_total_gpu_time": [o.k for o in U.sort_configs(objs, "total_gpu_time")]})
     with open(os.path.join(HERE, f"initial_{case}.json"), "w") as f:
         json.dump(out, f)
     kinds = {"plan": 0, "none": 0, "error": 0}

@@ -67,6 +67,20 @@ def test_initial_plans_are_the_references(golden_dir, case):
         assert seen["error"] >= 4
 
 
+def test_sort_configs_orders_like_the_reference(golden_dir):
+    from superscaler_amd.plan import sort_configs
+    with open(os.path.join(golden_dir, "initial_gpt_1_3B.json")) as f:
+        fx = json.load(f)
+    assert len(fx["sort"]) == 4
+    for rec in fx["sort"]:
+        objs = [types.SimpleNamespace(time_list=t, total_gpu_time=g, k=k)
+                for k, (t, g) in enumerate(zip(rec["time_list"], rec["total_gpu_time"]))]
+        assert [o.k for o in sort_configs(objs, "max_stage_time")] == rec["max_stage_time"]
+        assert [o.k for o in sort_configs(objs, "total_gpu_time")] == rec["by_total_gpu_time"]
+    with pytest.raises(RuntimeError):
+        sort_configs([], "other")
+
+
 def run_command_line(golden_dir, case, backend, tmp_path, capsys, monkeypatch):
     from superscaler_amd import aceso_cost_model as api
     with open(os.path.join(golden_dir, f"main_{case}.json")) as f:

@@ -3,7 +3,7 @@
 
 Run in the build container only (it needs /root/reference):
 
-    python tests/golden/make_golden.py [base] [variants] [moves] [grid] [initial] [main] [kat]
+    python tests/golden/make_golden.py [base] [variants] [moves] [grid] [initial] [main] [trace] [kat]
 
 (no argument: every part).
 
@@ -32,7 +32,9 @@ Further children of the same kind write
   initial_<case>.json              the starting plans of the search (aceso_utils.py generate_initial_config:
                                    balance, imbalance_gpu, imbalance_op, test) for 1 to 8 stages;
   main_<case>.json                 what search/aceso_cost_model.py prints and saves (--save-to-csv) when run as a
-                                   script on a plan file.
+                                   script on a plan file;
+  search_trace_<case>.json         the calls the reference's own search makes into the cost model during a short run
+                                   (arguments and results).
 """
 import json
 import os
@@ -477,6 +479,109 @@ def run_main(case):
     print(f"[golden] command line {case}: {[r['plan_file'] for r in runs]}")
 
 
+TRACED = ["predict_time_breakdown", "update_recompute", "get_reserved_memory_list", "wrap_predict_delta_time",
+          "predict_stage_time_helper", "predict_stage_memory_helper", "predict_value_after_move", "check_recompute",
+          "predict_stage_time", "predict_stage_memory"]
+
+
+def child_search_trace(case, per_function=25):
+    """The reference's search (search/aceso_search.py run_search, a few trials for 2, 3 and 4 stages) with every call
+    its modules make into aceso_cost_model recorded: function, arguments, what came back.  Calls the cost model makes
+    into itself are not recorded; up to `per_function` distinct calls per function and stage count are kept."""
+    import contextlib
+    import io
+    import tempfile
+    model, size, db, mbs_list, nodes, gpn, gbs, limit, num_layers = CASES[case]
+    tmp = tempfile.mkdtemp()
+    for d in ("", "trends/", "csv/", "top_configs/"):          # (what the search's reporting writes into)
+        os.makedirs(os.path.join(tmp, d), exist_ok=True)
+    extra = ["--no-multi-process", "--time-budget-total", "1000000", "--max-num-trials", "4", "--max-num-hops", "3",
+             "--log-path", tmp + "/", "--config-save-path", tmp + "/", "--add-action-tp-dp-exchange"]
+    if num_layers:
+        extra += ["--num-layers", str(num_layers)]
+    sys.argv = reference_argv(case, extra)
+    sys.path.insert(0, os.path.join(REF, "search"))
+    import aceso_cost_model as cm              # noqa: the reference, imported to record its outputs
+    trace = {n: [] for n in TRACED}
+    seen = {n: set() for n in TRACED}
+    taken = {n: 0 for n in TRACED}                 # ... in the current run_search
+    depth = [0]
+
+    from model_ops_info import get_full_op_list
+    full_ops = get_full_op_list(cm.args)
+
+    def plain(x):
+        """JSON form: a plan as run-length lists, a list of op names (always a contiguous piece of the model) as
+        {"ops": [first position, length]}, a long list of small integers as {"runs": [[value, count], ...]}."""
+        if hasattr(x, "stages"):
+            return {"config": pack_plan_runs(x)}
+        if isinstance(x, (list, tuple)):
+            if x and all(isinstance(v, str) for v in x):
+                n = len(x)
+                start = next(k for k in range(len(full_ops) - n + 1) if full_ops[k:k + n] == list(x))
+                return {"ops": [start, n]}
+            if len(x) > 8 and all(isinstance(v, int) and not isinstance(v, bool) for v in x):
+                runs = []
+                for v in x:
+                    if runs and runs[-1][0] == v:
+                        runs[-1][1] += 1
+                    else:
+                        runs.append([v, 1])
+                return {"runs": runs}
+            return [plain(v) for v in x]
+        return x
+
+    def wrap(name, fn):
+        def traced(*a, **kw):
+            if depth[0] or taken[name] >= per_function:
+                depth[0] += 1
+                try:
+                    return fn(*a, **kw)
+                finally:
+                    depth[0] -= 1
+            args_in = plain(list(a))
+            kw_in = {k: plain(v) for k, v in kw.items()}
+            depth[0] += 1
+            try:
+                r = fn(*a, **kw)
+            finally:
+                depth[0] -= 1
+            key = json.dumps([args_in, kw_in], sort_keys=True)
+            if key in seen[name]:
+                return r
+            seen[name].add(key)
+            taken[name] += 1
+            rec = {"args": args_in, "kwargs": kw_in, "returns": plain(r)}
+            cfg = a[0] if a and hasattr(a[0], "stages") else None
+            if name == "predict_time_breakdown":
+                rec["after"] = {k: getattr(cfg, k) for k in
+                                ("time_list", "memory_list", "compute_time_list", "total_gpu_time", "efficient_time_list",
+                                 "breakdown_ideal_time_per_gpu", "breakdown_eff_loss_time_per_gpu",
+                                 "breakdown_recomp_time_per_gpu")}
+            if name == "update_recompute":
+                rec["after"] = pack_plan_runs(cfg)
+            trace[name].append(rec)
+            return r
+        return traced
+
+    for n in TRACED:
+        setattr(cm, n, wrap(n, getattr(cm, n)))
+    with contextlib.redirect_stdout(io.StringIO()):
+        import aceso_search as S                   # noqa (binds the wrapped functions; reads the database)
+        results = {}
+        for num_stages in (2, 3, 4):
+            taken.update({n: 0 for n in TRACED})
+            r = S.run_search(num_stages, queue=None)
+            results[num_stages] = None if r is None else [r[0], r[1]]
+    out = {"case": case, "model_name": model, "model_size": size, "micro_batch_size": mbs_list, "num_nodes": nodes,
+           "num_gpus_per_node": gpn, "global_batch_size": gbs, "memory_limit": limit, "num_layers": num_layers,
+           "flags": extra[:9], "best_time_and_memory": results, "calls": trace}
+    with open(os.path.join(HERE, f"search_trace_{case}.json"), "w") as f:
+        json.dump(out, f)
+    shutil.rmtree(tmp, ignore_errors=True)
+    print(f"[golden] search trace {case}: { {n: len(v) for n, v in trace.items()} }, best {results}")
+
+
 def main():
     if len(sys.argv) > 2 and sys.argv[1] == "--child":
         return child(sys.argv[2])
@@ -486,8 +591,10 @@ def main():
         return child_moves(sys.argv[2])
     if len(sys.argv) > 2 and sys.argv[1] == "--child-initial":
         return child_initial(sys.argv[2])
-    # optional arguments: the parts to (re)write, of base variants moves grid initial main kat; none = all
-    parts = set(sys.argv[1:]) or {"base", "variants", "moves", "grid", "initial", "main", "kat"}
+    if len(sys.argv) > 2 and sys.argv[1] == "--child-search-trace":
+        return child_search_trace(sys.argv[2])
+    # optional arguments: the parts to (re)write, of base variants moves grid initial main trace kat; none = all
+    parts = set(sys.argv[1:]) or {"base", "variants", "moves", "grid", "initial", "main", "trace", "kat"}
     quiet = subprocess.DEVNULL if os.environ.get("GOLDEN_QUIET") else None
     me = os.path.abspath(__file__)
     for case in CASES:
@@ -510,6 +617,9 @@ def main():
             subprocess.run([sys.executable, me, "--child-initial", case], check=True, stdout=quiet)
         if "main" in parts:
             run_main(case)
+    for case in MOVE_CASES:
+        if "trace" in parts:
+            subprocess.run([sys.executable, me, "--child-search-trace", case], check=True, stdout=quiet)
     if "kat" not in parts:
         return
     # the single-GPU known-answer plans and the database files they index (data files)

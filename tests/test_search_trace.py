@@ -1,0 +1,93 @@
+"""The calls the reference's own search makes into its cost model, replayed on this one.
+
+tests/golden/search_trace_<case>.json (tests/golden/make_golden.py, child_search_trace): search/aceso_search.py's
+run_search for 2, 3 and 4 pipeline stages, a few trials each, with every call that aceso_search.py, aceso_prims.py and
+aceso_policy.py made into aceso_cost_model recorded -- function, arguments, what came back, and for the two functions
+that write into the plan (predict_time_breakdown, update_recompute) what they left there.  The plans and stages are the
+ones real moves produce (one-op stages, stages after GPU moves, recompute lists of check_recompute's own making), the
+argument forms the ones the callers use (positional and keyword).  Every recorded call must return the same here, to
+the last bit, on the CPU build of the kernels and on the GPU."""
+import json
+import os
+
+import pytest
+
+from superscaler_amd.plan import get_config
+from tests.test_cost_model_api import make_model
+from tests.test_initial_plans import pack_runs
+
+CASES = ["gpt_1_3B", "resnet_500M"]
+BREAKDOWN = ("time_list", "memory_list", "compute_time_list", "total_gpu_time", "efficient_time_list",
+             "breakdown_ideal_time_per_gpu", "breakdown_eff_loss_time_per_gpu", "breakdown_recomp_time_per_gpu")
+
+
+def decode(x, fx, m):
+    """make_golden's `plain` undone: plans, op-name slices and run-length integer lists back to what the callers passed."""
+    if isinstance(x, dict):
+        if "config" in x:
+            d = x["config"]
+            flat = lambda runs: [v for v, n in runs for _ in range(n)]
+            return get_config(d["num_ops_in_each_stage"], flat(d["tp"]), flat(d["dp"]), flat(d["recompute_ops"]),
+                              d["micro_batch_size"], fx["global_batch_size"], m.graph.ops, flat(d["algo"]))
+        if "ops" in x:
+            return m.graph.ops[x["ops"][0]:x["ops"][0] + x["ops"][1]]
+        if "runs" in x:
+            return [v for v, n in x["runs"] for _ in range(n)]
+        raise AssertionError(x)
+    if isinstance(x, list):
+        return [decode(v, fx, m) for v in x]
+    return x
+
+
+def plain_result(r):
+    if isinstance(r, tuple):
+        return [plain_result(v) for v in r]
+    if isinstance(r, list):
+        return [plain_result(v) for v in r]
+    return r
+
+
+def replay(golden_dir, case, backend):
+    with open(os.path.join(golden_dir, f"search_trace_{case}.json")) as f:
+        fx = json.load(f)
+    g, m = make_model(golden_dir, case, backend)
+    counts = {}
+    bad = []
+    try:
+        for name, calls in fx["calls"].items():
+            counts[name] = len(calls)
+            for k, call in enumerate(calls):
+                args = decode(call["args"], fx, m)
+                kwargs = {key: decode(v, fx, m) for key, v in call["kwargs"].items()}
+                got = plain_result(getattr(m, name)(*args, **kwargs))
+                want = decode(call["returns"], fx, m) if not isinstance(call["returns"], dict) or "config" not in call["returns"] \
+                    else call["returns"]
+                ok = got == want
+                if name == "predict_time_breakdown":
+                    ok = ok and all(getattr(args[0], key) == call["after"][key] for key in BREAKDOWN)
+                if name == "update_recompute":
+                    ok = ok and pack_runs(args[0]) == call["after"]
+                if not ok:
+                    bad.append((name, k))
+    finally:
+        if backend == "gpu":
+            m.close()
+    return counts, bad
+
+
+def check(counts, bad, case):
+    assert not bad, bad[:10]
+    assert counts["predict_time_breakdown"] >= 30 and counts["update_recompute"] >= 30
+    assert counts["predict_value_after_move"] >= 60 and counts["predict_stage_time_helper"] >= 60
+    assert counts["check_recompute"] >= 30 and counts["predict_stage_time"] >= 30 and counts["predict_stage_memory"] >= 30
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_the_searchs_calls_return_what_the_reference_returned_emu(golden_dir, case):
+    check(*replay(golden_dir, case, "emu"), case)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", CASES)
+def test_the_searchs_calls_return_what_the_reference_returned_gpu(golden_dir, case):
+    check(*replay(golden_dir, case, "gpu"), case)

@@ -60,6 +60,9 @@ class CostModel:
         self.tables: CompiledTables = compile_tables(graph, db, settings)
         self.device = device
         self._evaluator = None        # created on first use: HIP must be initialised after any fork()
+        # check_recompute starts from the reference's memo table (see check_recompute_batch); False: always from the
+        # stage's own memory
+        self.reference_memo = True
         self._mbs_index = {m: k for k, m in enumerate(db.mbs_list)}
         self._type_index = {n: k for k, n in enumerate(db.op_names)}
         self._first_pos = {}
@@ -407,7 +410,20 @@ class CostModel:
         state, pending = [], []
         for k, (ops, micro_bs, tp_size, dp_size, nsb, algo_list) in enumerate(queries):
             mw, mg, mo, ma, mp, mr = self._memory_breakdown(rec[k].tolist(), nsb)
-            stage_memory = (mw + mg + mo + ma + mp + mr) + args.peak_mem_in_backward
+            stage_memory = mw + mg + mo + ma + mp + mr
+            if self.reference_memo:
+                # :828 asks predict_stage_memory_helper, whose table is keyed by the stage's first op NAME, its length and
+                # its per-op lists (:759): a stage that shares those with one asked about earlier starts from that one's
+                # memory, whatever its other ops are (possible where a model's layers differ, as T5's encoder and decoder)
+                key = (f"ops{ops[0]}{len(ops)}tp{tp_size}dp{dp_size}rc{rcs[k]}algo{algo_list}bs{micro_bs}stage{nsb}")
+                self.stage_memory_visit += 1
+                known = self.stage_memory_set.get(key)
+                if known is not None:
+                    self.stage_memory_hit += 1
+                    stage_memory = known
+                else:
+                    self.stage_memory_set[key] = stage_memory
+            stage_memory = stage_memory + args.peak_mem_in_backward
             # get_peak_activations of an all-zero recompute list is 0 (:421)
             st = {"mem": stage_memory, "saved": 0, "peak": 0, "groups": None, "stale": False}
             if stage_memory - limit > 0:

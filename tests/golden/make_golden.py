@@ -531,8 +531,52 @@ def child_search_trace(case, per_function=25):
             return [plain(v) for v in x]
         return x
 
+    # The two memo tables of the cost model (stage_memory_set :743-767, stage_time_set :769-791) are keyed by a stage's
+    # FIRST op name, its length and its per-op lists: two different stages of a model whose layers differ (T5) can share
+    # a key, so what check_recompute starts from depends on what was asked before.  Every hit inside a recorded call is
+    # recorded with it (`memo`), so that a replay can put the same entries in place.
+    events = []
+
+    def runs_of(xs):
+        out = []
+        for v in xs:
+            if out and out[-1][0] == v:
+                out[-1][1] += 1
+            else:
+                out.append([v, 1])
+        return out
+
+    def memo_event(name, a, kw):
+        if name == "predict_stage_memory_helper":
+            names = ["config", "stage_index", "ops", "recompute_ops", "tp_size", "dp_size", "base_batch_size",
+                     "num_stages_behind", "algo_list"]
+            b = dict(zip(names, a))
+            b.update(kw)
+            if b.get("ops") is None:
+                st = b["config"].stages[b["stage_index"]]
+                ops_, rc_, tp_, dp_, bs_, al_, nsb_ = st.ops, st.recompute_ops, st.tp_size, st.dp_size, st.base_bs, st.algo, st.num_stages_behind
+            else:
+                ops_, rc_, tp_, dp_, bs_, al_, nsb_ = (b["ops"], b["recompute_ops"], b["tp_size"], b["dp_size"],
+                                                       b["base_batch_size"], b["algo_list"], b["num_stages_behind"])
+            key = f"ops{ops_[0]}{len(ops_)}tp{tp_}dp{dp_}rc{rc_}algo{al_}bs{bs_}stage{nsb_}"
+            store = cm.stage_memory_set
+        else:
+            config, stage_index = a[0], a[1]
+            st = config.stages[stage_index]
+            ops_, rc_, tp_, dp_, bs_, al_, nsb_ = st.ops, st.recompute_ops, st.tp_size, st.dp_size, config.micro_bs, st.algo, None
+            key = f"ops{ops_[0]}{len(ops_)}tp{tp_}dp{dp_}rc{rc_}algo{al_}bs{bs_}"
+            store = cm.stage_time_set
+        if store.get(key) is None:
+            return None
+        return {"kind": "memory" if nsb_ is not None else "time", "first": ops_[0], "n": len(ops_), "tp": runs_of(tp_),
+                "dp": runs_of(dp_), "rc": runs_of(rc_), "algo": runs_of(al_), "bs": bs_, "nsb": nsb_, "value": store[key]}
+
     def wrap(name, fn):
         def traced(*a, **kw):
+            if name in ("predict_stage_memory_helper", "predict_stage_time_helper"):
+                e = memo_event(name, a, kw)
+                if e is not None:
+                    events.append(e)
             if depth[0] or taken[name] >= per_function:
                 depth[0] += 1
                 try:
@@ -541,6 +585,7 @@ def child_search_trace(case, per_function=25):
                     depth[0] -= 1
             args_in = plain(list(a))
             kw_in = {k: plain(v) for k, v in kw.items()}
+            first_event = len(events) - (1 if name.endswith("_helper") and events and e is not None else 0)
             depth[0] += 1
             try:
                 r = fn(*a, **kw)
@@ -552,6 +597,8 @@ def child_search_trace(case, per_function=25):
             seen[name].add(key)
             taken[name] += 1
             rec = {"args": args_in, "kwargs": kw_in, "returns": plain(r)}
+            if len(events) > first_event:
+                rec["memo"] = events[first_event:]
             cfg = a[0] if a and hasattr(a[0], "stages") else None
             if name == "predict_time_breakdown":
                 rec["after"] = {k: getattr(cfg, k) for k in
@@ -617,7 +664,7 @@ def main():
             subprocess.run([sys.executable, me, "--child-initial", case], check=True, stdout=quiet)
         if "main" in parts:
             run_main(case)
-    for case in MOVE_CASES:
+    for case in CASES:
         if "trace" in parts:
             subprocess.run([sys.executable, me, "--child-search-trace", case], check=True, stdout=quiet)
     if "kat" not in parts:

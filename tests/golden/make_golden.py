@@ -484,10 +484,16 @@ TRACED = ["predict_time_breakdown", "update_recompute", "get_reserved_memory_lis
           "predict_stage_time", "predict_stage_memory"]
 
 
-def child_search_trace(case, per_function=25):
+TRACE_EXTRAS = ["--predict-delta-time", "--add-action-finetune-dim", "--add-action-finetune-algo", "--add-action-tune-tp-dp",
+                "--finetune-after-trial", "1", "--finetune-tp-dp-after-trial"]
+
+
+def child_search_trace(case, extras=False, per_function=25):
     """The reference's search (search/aceso_search.py run_search, a few trials for 2, 3 and 4 stages) with every call
     its modules make into aceso_cost_model recorded: function, arguments, what came back.  Calls the cost model makes
-    into itself are not recorded; up to `per_function` distinct calls per function and stage count are kept."""
+    into itself are not recorded; up to `per_function` distinct calls per function and stage count are kept.
+    `extras`: with the optional actions and the delta-time prediction switched on (TRACE_EXTRAS), into
+    search_trace_<case>__extras.json."""
     import contextlib
     import io
     import tempfile
@@ -497,6 +503,8 @@ def child_search_trace(case, per_function=25):
         os.makedirs(os.path.join(tmp, d), exist_ok=True)
     extra = ["--no-multi-process", "--time-budget-total", "1000000", "--max-num-trials", "4", "--max-num-hops", "3",
              "--log-path", tmp + "/", "--config-save-path", tmp + "/", "--add-action-tp-dp-exchange"]
+    if extras:
+        extra += TRACE_EXTRAS
     if num_layers:
         extra += ["--num-layers", str(num_layers)]
     sys.argv = reference_argv(case, extra)
@@ -622,11 +630,11 @@ def child_search_trace(case, per_function=25):
             results[num_stages] = None if r is None else [r[0], r[1]]
     out = {"case": case, "model_name": model, "model_size": size, "micro_batch_size": mbs_list, "num_nodes": nodes,
            "num_gpus_per_node": gpn, "global_batch_size": gbs, "memory_limit": limit, "num_layers": num_layers,
-           "flags": extra[:9], "best_time_and_memory": results, "calls": trace}
-    with open(os.path.join(HERE, f"search_trace_{case}.json"), "w") as f:
+           "flags": extra[:9] + (TRACE_EXTRAS if extras else []), "best_time_and_memory": results, "calls": trace}
+    with open(os.path.join(HERE, f"search_trace_{case}{'__extras' if extras else ''}.json"), "w") as f:
         json.dump(out, f)
     shutil.rmtree(tmp, ignore_errors=True)
-    print(f"[golden] search trace {case}: { {n: len(v) for n, v in trace.items()} }, best {results}")
+    print(f"[golden] search trace {case}{' (extras)' if extras else ''}: { {n: len(v) for n, v in trace.items()} }, best {results}")
 
 
 def main():
@@ -639,7 +647,7 @@ def main():
     if len(sys.argv) > 2 and sys.argv[1] == "--child-initial":
         return child_initial(sys.argv[2])
     if len(sys.argv) > 2 and sys.argv[1] == "--child-search-trace":
-        return child_search_trace(sys.argv[2])
+        return child_search_trace(sys.argv[2], extras=len(sys.argv) > 3 and sys.argv[3] == "extras")
     # optional arguments: the parts to (re)write, of base variants moves grid initial main trace kat; none = all
     parts = set(sys.argv[1:]) or {"base", "variants", "moves", "grid", "initial", "main", "trace", "kat"}
     quiet = subprocess.DEVNULL if os.environ.get("GOLDEN_QUIET") else None
@@ -667,6 +675,7 @@ def main():
     for case in CASES:
         if "trace" in parts:
             subprocess.run([sys.executable, me, "--child-search-trace", case], check=True, stdout=quiet)
+            subprocess.run([sys.executable, me, "--child-search-trace", case, "extras"], check=True, stdout=quiet)
     if "kat" not in parts:
         return
     # the single-GPU known-answer plans and the database files they index (data files)

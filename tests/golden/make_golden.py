@@ -513,6 +513,8 @@ def child_search_trace(case, extras=False, per_function=25):
     trace = {n: [] for n in TRACED}
     seen = {n: set() for n in TRACED}
     taken = {n: 0 for n in TRACED}                 # ... in the current run_search
+    seconds = {n: 0.0 for n in TRACED}
+    import time
     depth = [0]
 
     from model_ops_info import get_full_op_list
@@ -595,16 +597,19 @@ def child_search_trace(case, extras=False, per_function=25):
             kw_in = {k: plain(v) for k, v in kw.items()}
             first_event = len(events) - (1 if name.endswith("_helper") and events and e is not None else 0)
             depth[0] += 1
+            t0 = time.perf_counter()
             try:
                 r = fn(*a, **kw)
             finally:
                 depth[0] -= 1
+            dt = time.perf_counter() - t0
             key = json.dumps([args_in, kw_in], sort_keys=True)
             if key in seen[name]:
                 return r
             seen[name].add(key)
             taken[name] += 1
             rec = {"args": args_in, "kwargs": kw_in, "returns": plain(r)}
+            seconds[name] += dt                    # (what the reference took for the recorded calls, on this machine)
             if len(events) > first_event:
                 rec["memo"] = events[first_event:]
             cfg = a[0] if a and hasattr(a[0], "stages") else None
@@ -630,7 +635,8 @@ def child_search_trace(case, extras=False, per_function=25):
             results[num_stages] = None if r is None else [r[0], r[1]]
     out = {"case": case, "model_name": model, "model_size": size, "micro_batch_size": mbs_list, "num_nodes": nodes,
            "num_gpus_per_node": gpn, "global_batch_size": gbs, "memory_limit": limit, "num_layers": num_layers,
-           "flags": extra[:9] + (TRACE_EXTRAS if extras else []), "best_time_and_memory": results, "calls": trace}
+           "flags": extra[:9] + (TRACE_EXTRAS if extras else []), "best_time_and_memory": results,
+           "reference_seconds": {n: round(v, 4) for n, v in seconds.items()}, "calls": trace}
     with open(os.path.join(HERE, f"search_trace_{case}{'__extras' if extras else ''}.json"), "w") as f:
         json.dump(out, f)
     shutil.rmtree(tmp, ignore_errors=True)

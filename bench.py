@@ -46,7 +46,7 @@ def cpu_baseline(tables, batch, threads):
     co.score_arrays(*[a[:n1] for a in arrays], threads=1)
     dt_one = time.perf_counter() - t0
     orc = oracle_for(tables)
-    npy = min(P, 1024)
+    npy = min(P, 8192)           # about 14 s of the Python oracle at 523 ops
     cfgs = [oracle_config(batch, p, tables) for p in range(npy)]
     t0 = time.perf_counter()
     for c in cfgs:

@@ -63,7 +63,7 @@ VARIANTS = {
     "noflex": ["--do-not-use-flex-recompute"],
     "peakbwd": ["--peak-mem-in-backward", "700"],
 }
-MOVE_CASES = ["gpt_1_3B", "resnet_500M"]
+MOVE_CASES = ["gpt_1_3B", "resnet_500M", "t5_770M"]
 
 
 def copy_db(case):
@@ -280,6 +280,7 @@ def child_moves(case):
     """What the reference's move primitives return for seeded legal plans whose recompute lists are
     check_recompute's own (as initialize_search leaves them, aceso_search.py:26-27)."""
     import copy
+    import types
     model, size, db, mbs_list, nodes, gpn, gbs, limit, num_layers = CASES[case]
     dbdir = os.path.join(HERE, f"db_{case}") + "/"
     sys.argv = reference_argv(case, ["--add-action-tp-dp-exchange", "--time-budget-total", "1000000", "--max-num-hops", "7"])
@@ -291,7 +292,7 @@ def child_moves(case):
     args = cm.args
     cm.read_profiled_time(model, size, dbdir)
     full_ops = get_full_op_list(args)
-    tunable = get_tunable_op_list(args)
+    tunable = get_tunable_op_list(args) if model != "t5" else []       # (T5's database has one algorithm per op)
     rng = random.Random(0xACE51 + sum(map(ord, case)))
     num_gpus = nodes * gpn
     out = {"case": case, "model_name": model, "model_size": size, "micro_batch_size": mbs_list,
@@ -324,8 +325,41 @@ def child_moves(case):
             for action in ("inc_tp", "dec_tp", "inc_dp", "dec_dp"):
                 r = prims[action].apply_to(fresh(), b)
                 rec["tp_dp"].append([b, action, None if r is None else pack_plan(r)])
-            r = prims["dec_op"].apply_to(fresh(), b)
-            rec["mig_op"].append([b, None if r is None else pack_plan(r)])
+            # prim_mig_op: the op migrations behind its result, in the order it made them (up to max_op_move_steps
+            # chains, each from a bottleneck stage towards a partner, :150-218) -- followed through the copies it works on
+            lineage, keep = {}, []
+            real_deepcopy, real_move = copy.deepcopy, pr.action_move_once
+
+            def deepcopy_logged(x, *a, **kw):
+                y = real_deepcopy(x, *a, **kw)
+                if hasattr(x, "stages"):
+                    lineage[id(y)] = (id(x), None)
+                    keep.extend([x, y])
+                return y
+
+            def move_logged(config, frm, to, k, *a, **kw):
+                y = real_move(config, frm, to, k, *a, **kw)
+                if y is not config:
+                    lineage[id(y)] = (id(config), [frm, to, k])
+                    keep.extend([config, y])
+                return y
+
+            pr.copy = types.SimpleNamespace(deepcopy=deepcopy_logged)
+            pr.action_move_once = move_logged
+            try:
+                start = fresh()
+                r = prims["dec_op"].apply_to(start, b)
+            finally:
+                pr.copy, pr.action_move_once = copy, real_move
+            hops = []
+            if r is not None:
+                at = id(r)
+                while at != id(start):
+                    at, move = lineage[at]
+                    if move is not None:
+                        hops.append(move)
+                hops.reverse()
+            rec["mig_op"].append([b, None if r is None else pack_plan(r), hops])
         for action in ("inc_mbs", "dec_mbs"):
             r = prims[action].apply_to(fresh(), 0)
             rec["mbs"].append([action, None if r is None else pack_plan(r)])

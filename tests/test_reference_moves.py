@@ -9,7 +9,8 @@ with update_recompute_arrays as every primitive does, and compares the whole pla
 micro-batch size: the reference's config_details) with the recorded one.
 
 Which stage / partner / count / direction a primitive tries is its policy and comes from the fixture here (for
-prim_tp_dp and prim_mbs: read off the recorded result, per stage); the policy calls themselves
+prim_tp_dp and prim_mbs: read off the recorded result, per stage; for prim_mig_op: the action_move_once calls behind
+its result, in the order it made them); the policy calls themselves
 (predict_value_after_move, wrap_predict_delta_time) are pinned in test_cost_model_api.py."""
 import json
 import os
@@ -21,7 +22,7 @@ from superscaler_amd import neighbours as nb
 from superscaler_amd.plan import PlanBatch, config_details, get_config
 from tests.test_cost_model_api import make_model
 
-MOVE_CASES = ["gpt_1_3B", "resnet_500M"]
+MOVE_CASES = ["gpt_1_3B", "resnet_500M", "t5_770M"]
 
 
 def unpack(g, m, d):
@@ -47,8 +48,13 @@ def expand(m, templates, moves, device):
     return m.update_recompute_arrays(nb.apply_moves_host(templates, moves, m.tables.db.n_algo))
 
 
-def same_plan(m, batch, k, want_cfg):
-    return config_details(batch.to_config(k, m.tables), get_string=True) == config_details(want_cfg, get_string=True)
+def same_plan(m, batch, k, want_cfg, recompute=True):
+    got = batch.to_config(k, m.tables)
+    if not recompute:
+        for cfg in (got, want_cfg):
+            for st in cfg.stages:
+                st.recompute_ops = [0] * len(st.ops)
+    return config_details(got, get_string=True) == config_details(want_cfg, get_string=True)
 
 
 def steps_between(start_cfg, res_cfg):
@@ -68,23 +74,9 @@ def steps_between(start_cfg, res_cfg):
     return steps
 
 
-def hops_between(start_cfg, res_cfg, first):
-    """The op migrations behind a prim_mig_op result: one boundary after the other, starting next to the stage the
-    primitive was applied to (`first`) and walking away from it (aceso_prims.py:166-189)."""
-    a = np.cumsum([len(st.ops) for st in start_cfg.stages])[:-1]
-    b = np.cumsum([len(st.ops) for st in res_cfg.stages])[:-1]
-    moved = [j for j in range(len(a)) if a[j] != b[j]]          # boundary j separates stages j and j + 1
-    hops = []
-    for j in sorted(moved, key=lambda j: abs(j + 0.5 - first)):
-        if b[j] < a[j]:
-            hops.append((j, j + 1, int(a[j] - b[j])))           # stage j gives its tail to stage j + 1
-        else:
-            hops.append((j + 1, j, int(b[j] - a[j])))
-    return hops
-
-
 def run_case(golden_dir, case, backend):
     moves, g, m = load(golden_dir, case, backend)
+    m.reference_memo = False        # (each primitive result is compared on its own: no history)
     device = backend == "gpu"
     A = m.tables.db.n_algo
     seen = {"move_once": 0, "exchange": 0, "tp_dp": 0, "mbs": 0, "mig_op": 0}
@@ -133,16 +125,24 @@ def run_case(golden_dir, case, backend):
                 if not same_plan(m, out, k, cfg):
                     failed.append((pi, t, k))
             # prim_mig_op: a chain of op migrations, each applied to the result of the one before
-            for b, res in rec["mig_op"]:
+            for b, res, hops in rec["mig_op"]:
                 if res is None:
                     continue
                 res_cfg = unpack(moves, m, res)
                 cur = base
-                for frm, to, k in hops_between(start_cfg, res_cfg, b):
-                    cur = nb.apply_moves_host(cur, nb.migrate_ops_move(cur, A, frm, to, k)[None, :], A)
+                # the recorded action_move_once calls (stage, the partner it works towards, op count): each moves the ops
+                # to the adjacent stage on the partner's side (aceso_prims.py:88-133)
+                for frm, towards, k in hops:
+                    cur = nb.apply_moves_host(cur, nb.migrate_ops_move(cur, A, frm, frm + (1 if towards > frm else -1), k)[None, :], A)
                 got = expand(m, cur, np.zeros((1, 4), dtype=np.uint32), device)
                 seen["mig_op"] += 1
-                if not same_plan(m, got, 0, res_cfg):
+                # Every move settles the recompute bits of the two stages it touches (:104-108) through check_recompute,
+                # whose starting memory comes from a memo table that two different T5 stages can share an entry of
+                # (aceso_cost_model.py:759): after several moves a T5 plan's bits depend on what the reference was asked
+                # before.  For T5 chains of more than one move the rest of the plan is compared; the bits are pinned
+                # call by call in test_search_trace.py.
+                history_free = case != "t5_770M" or len(hops) <= 1
+                if not same_plan(m, got, 0, res_cfg, recompute=history_free):
                     failed.append((pi, "mig_op", b))
     finally:
         if device:
@@ -154,7 +154,9 @@ def run_case(golden_dir, case, backend):
 def test_reference_primitives_in_descriptor_form_emu(golden_dir, case):
     seen, failed = run_case(golden_dir, case, "emu")
     assert not failed, failed
-    assert seen["move_once"] >= 8 and seen["exchange"] >= 1 and seen["mbs"] >= 1
+    assert seen["move_once"] >= 8 and seen["mbs"] >= 1
+    assert seen["exchange"] >= 1 or case == "t5_770M"       # (the reference's exchange returned None for every T5 start)
+    assert seen["mig_op"] >= 2
     if case == "gpt_1_3B":
         assert seen["tp_dp"] >= 4 and seen["mig_op"] >= 2
 

@@ -123,6 +123,22 @@ def cross_node_bits(stage_gpus: Sequence[int], gpus_per_node: int) -> int:
     return bits
 
 
+def _flat_ints(stages, key: str, count: int) -> np.ndarray:
+    """The per-op list `key` of all stages as one int64 array of `count` entries (ValueError if the lengths do not add
+    up).  Small non-negative values, the usual case, go through bytes(): three times faster than numpy's own conversion
+    of a Python list."""
+    flat = []
+    for st in stages:
+        flat += getattr(st, key)
+    try:
+        a = np.frombuffer(bytes(flat), dtype=np.uint8).astype(np.int64)
+    except (ValueError, TypeError):          # a value outside 0..255, or not a plain int
+        a = np.fromiter(flat, dtype=np.int64, count=len(flat))
+    if len(a) != count:
+        raise ValueError(f"{key}: {len(a)} entries for {count} ops")
+    return a
+
+
 @dataclass
 class PlanBatch:
     codes: np.ndarray        # uint8 [P, N]
@@ -186,10 +202,7 @@ class PlanBatch:
             if total != N:
                 raise ValueError(f"plan {p} has {total} ops, the op graph {N}")
             # the per-op lists of all stages, flattened once each
-            tp = np.fromiter(chain(st.tp_size for st in stages), dtype=np.int64, count=N)
-            dp = np.fromiter(chain(st.dp_size for st in stages), dtype=np.int64, count=N)
-            al = np.fromiter(chain(st.algo for st in stages), dtype=np.int64, count=N)
-            rc = np.fromiter(chain(st.recompute_ops for st in stages), dtype=np.int64, count=N)
+            tp, dp, al, rc = (_flat_ints(stages, key, N) for key in ("tp_size", "dp_size", "algo", "recompute_ops"))
             g_of_op = np.repeat(np.asarray(gl, dtype=np.int64), lens)
             bad = np.flatnonzero(tp * dp != g_of_op)
             if len(bad):

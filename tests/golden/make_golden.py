@@ -34,7 +34,9 @@ Further children of the same kind write
   main_<case>.json                 what search/aceso_cost_model.py prints and saves (--save-to-csv) when run as a
                                    script on a plan file;
   search_trace_<case>.json         the calls the reference's own search makes into the cost model during a short run
-                                   (arguments and results).
+                                   (arguments and results);
+  search_binding_<case>.json       what the same search finds when its cost model is replaced by this repository's
+                                   binding, beside what it found with its own.
 """
 import json
 import os
@@ -677,6 +679,59 @@ def child_search_trace(case, extras=False, per_function=25):
     print(f"[golden] search trace {case}{' (extras)' if extras else ''}: { {n: len(v) for n, v in trace.items()} }, best {results}")
 
 
+def child_binding_search(case):
+    """The reference's search run a second time with its cost model REPLACED by this repository's binding
+    (superscaler_amd/binding/aceso_cost_model.py, scoring through the CPU build of the kernel source, tests/emu): same
+    flags and stage counts as child_search_trace.  Writes what both runs found into search_binding_<case>.json; the
+    two must be equal (tests/test_search_trace.py checks the file)."""
+    import contextlib
+    import importlib.util
+    import io
+    import tempfile
+    model, size, db, mbs_list, nodes, gpn, gbs, limit, num_layers = CASES[case]
+    tmp = tempfile.mkdtemp()
+    for d in ("", "trends/", "csv/", "top_configs/"):
+        os.makedirs(os.path.join(tmp, d), exist_ok=True)
+    extra = ["--no-multi-process", "--time-budget-total", "1000000", "--max-num-trials", "4", "--max-num-hops", "3",
+             "--log-path", tmp + "/", "--config-save-path", tmp + "/", "--add-action-tp-dp-exchange"]
+    if num_layers:
+        extra += ["--num-layers", str(num_layers)]
+    sys.argv = reference_argv(case, extra)
+    root = os.path.dirname(os.path.dirname(HERE))
+    sys.path.insert(0, os.path.join(REF, "search"))
+    sys.path.insert(0, root)
+    # the CPU build of the kernels behind the evaluator (there is no GPU in the build container)
+    import superscaler_amd.aceso_cost_model as gpu
+    from tests.helpers import EmuEvaluator
+
+    def emu_of(self):
+        if "_emu" not in self.__dict__:
+            self.__dict__["_emu"] = EmuEvaluator(self.tables)
+        return self.__dict__["_emu"]
+    gpu.CostModel.evaluator = property(emu_of)
+    spec = importlib.util.spec_from_file_location("aceso_cost_model", os.path.join(root, "superscaler_amd", "binding",
+                                                                                   "aceso_cost_model.py"))
+    mod = importlib.util.module_from_spec(spec)
+    sys.modules["aceso_cost_model"] = mod          # what aceso_search / aceso_prims import
+    spec.loader.exec_module(mod)
+    with contextlib.redirect_stdout(io.StringIO()):
+        import aceso_search as S                   # noqa: the reference's search, unchanged
+        found = {}
+        for num_stages in (2, 3, 4):
+            r = S.run_search(num_stages, queue=None)
+            found[str(num_stages)] = None if r is None else [r[0], r[1], r[2]]
+    with open(os.path.join(HERE, f"search_trace_{case}.json")) as f:
+        ref = json.load(f)["best_time_and_memory"]
+    out = {"case": case, "flags": extra[:7] + ["--add-action-tp-dp-exchange"], "with_the_binding": {k: (v[:2] if v else None) for k, v in found.items()},
+           "explored_with_the_binding": {k: (v[2] if v else None) for k, v in found.items()},
+           "with_the_reference_cost_model": ref}
+    with open(os.path.join(HERE, f"search_binding_{case}.json"), "w") as f:
+        json.dump(out, f, indent=1)
+    shutil.rmtree(tmp, ignore_errors=True)
+    same = out["with_the_binding"] == {k: v for k, v in ref.items()}
+    print(f"[golden] search over the binding {case}: {out['with_the_binding']} -- {'same as' if same else 'DIFFERENT FROM'} the reference's own")
+
+
 def main():
     if len(sys.argv) > 2 and sys.argv[1] == "--child":
         return child(sys.argv[2])
@@ -686,6 +741,8 @@ def main():
         return child_moves(sys.argv[2])
     if len(sys.argv) > 2 and sys.argv[1] == "--child-initial":
         return child_initial(sys.argv[2])
+    if len(sys.argv) > 2 and sys.argv[1] == "--child-binding-search":
+        return child_binding_search(sys.argv[2])
     if len(sys.argv) > 2 and sys.argv[1] == "--child-search-trace":
         return child_search_trace(sys.argv[2], extras=len(sys.argv) > 3 and sys.argv[3] == "extras")
     # optional arguments: the parts to (re)write, of base variants moves grid initial main trace kat; none = all
@@ -716,6 +773,7 @@ def main():
         if "trace" in parts:
             subprocess.run([sys.executable, me, "--child-search-trace", case], check=True, stdout=quiet)
             subprocess.run([sys.executable, me, "--child-search-trace", case, "extras"], check=True, stdout=quiet)
+            subprocess.run([sys.executable, me, "--child-binding-search", case], check=True, stdout=quiet)
     if "kat" not in parts:
         return
     # the single-GPU known-answer plans and the database files they index (data files)

@@ -732,6 +732,61 @@ def child_binding_search(case):
     print(f"[golden] search over the binding {case}: {out['with_the_binding']} -- {'same as' if same else 'DIFFERENT FROM'} the reference's own")
 
 
+def child_binding_grid(case, num_saved=4):
+    """search/gen_megatron_plan.py run as a script over this repository's binding (see child_binding_search): the
+    plan files it writes must be the ones it wrote with the reference's own cost model (megatron_grid_<case>.json).
+    Adds the comparison to search_binding_<case>.json."""
+    import contextlib
+    import importlib.util
+    import io
+    import runpy
+    import tempfile
+    model, size, db, mbs_list, nodes, gpn, gbs, limit, num_layers = CASES[case]
+    tmp = tempfile.mkdtemp()
+    sys.argv = reference_argv(case, ["--num-layers", str(num_layers), "--config-save-path", tmp + "/",
+                                     "--num-of-saved-configs", str(num_saved)])
+    root = os.path.dirname(os.path.dirname(HERE))
+    sys.path.insert(0, os.path.join(REF, "search"))
+    sys.path.insert(0, root)
+    import superscaler_amd.aceso_cost_model as gpu
+    from tests.helpers import EmuEvaluator
+
+    def emu_of(self):
+        if "_emu" not in self.__dict__:
+            self.__dict__["_emu"] = EmuEvaluator(self.tables)
+        return self.__dict__["_emu"]
+    gpu.CostModel.evaluator = property(emu_of)
+    spec = importlib.util.spec_from_file_location("aceso_cost_model", os.path.join(root, "superscaler_amd", "binding",
+                                                                                   "aceso_cost_model.py"))
+    mod = importlib.util.module_from_spec(spec)
+    sys.modules["aceso_cost_model"] = mod
+    spec.loader.exec_module(mod)
+    cwd = os.getcwd()
+    os.chdir(tmp)
+    try:
+        with contextlib.redirect_stdout(io.StringIO()):
+            runpy.run_path(os.path.join(REF, "search", "gen_megatron_plan.py"), run_name="__main__")
+    finally:
+        os.chdir(cwd)
+    files = {}
+    for n in sorted(os.listdir(tmp)):
+        if n.endswith(".json"):
+            with open(os.path.join(tmp, n)) as f:
+                files[n] = json.load(f)
+    with open(os.path.join(HERE, f"megatron_grid_{case}.json")) as f:
+        ref_files = json.load(f)["files"]
+    path = os.path.join(HERE, f"search_binding_{case}.json")
+    with open(path) as f:
+        out = json.load(f)
+    out["grid_files_with_the_binding"] = sorted(files)
+    out["grid_files_with_the_reference_cost_model"] = sorted(ref_files)
+    out["grid_files_identical"] = files == ref_files
+    with open(path, "w") as f:
+        json.dump(out, f, indent=1)
+    shutil.rmtree(tmp, ignore_errors=True)
+    print(f"[golden] gen_megatron_plan over the binding {case}: {sorted(files)} -- {'identical' if files == ref_files else 'DIFFERENT'}")
+
+
 def main():
     if len(sys.argv) > 2 and sys.argv[1] == "--child":
         return child(sys.argv[2])
@@ -741,6 +796,8 @@ def main():
         return child_moves(sys.argv[2])
     if len(sys.argv) > 2 and sys.argv[1] == "--child-initial":
         return child_initial(sys.argv[2])
+    if len(sys.argv) > 2 and sys.argv[1] == "--child-binding-grid":
+        return child_binding_grid(sys.argv[2])
     if len(sys.argv) > 2 and sys.argv[1] == "--child-binding-search":
         return child_binding_search(sys.argv[2])
     if len(sys.argv) > 2 and sys.argv[1] == "--child-search-trace":
@@ -774,6 +831,8 @@ def main():
             subprocess.run([sys.executable, me, "--child-search-trace", case], check=True, stdout=quiet)
             subprocess.run([sys.executable, me, "--child-search-trace", case, "extras"], check=True, stdout=quiet)
             subprocess.run([sys.executable, me, "--child-binding-search", case], check=True, stdout=quiet)
+            if os.path.exists(os.path.join(HERE, f"megatron_grid_{case}.json")):
+                subprocess.run([sys.executable, me, "--child-binding-grid", case], check=True, stdout=quiet)
     if "kat" not in parts:
         return
     # the single-GPU known-answer plans and the database files they index (data files)

@@ -127,6 +127,11 @@ def test_the_references_search_over_the_binding_found_the_same_plans(golden_dir,
     assert fx["with_the_binding"] == fx["with_the_reference_cost_model"]
     assert all(v is not None and v[0] > 0 for v in fx["with_the_binding"].values())
     assert all(n >= 4 for n in fx["explored_with_the_binding"].values())
+    if case == "gpt_1_3B":
+        # search/gen_megatron_plan.py, run as the script it is over the binding, wrote the plan files it writes with
+        # the reference's own cost model (child_binding_grid)
+        assert fx["grid_files_identical"] is True and len(fx["grid_files_with_the_binding"]) == 4
+        assert fx["grid_files_with_the_binding"] == fx["grid_files_with_the_reference_cost_model"]
     # aceso_search.py:4, aceso_prims.py:7, gen_megatron_plan.py:8 import these names from aceso_cost_model
     wanted = {"read_profiled_time", "predict_time_breakdown", "update_recompute", "get_reserved_memory_list",
               "wrap_predict_delta_time", "predict_stage_time_helper", "predict_value_after_move", "check_recompute",

@@ -64,6 +64,7 @@ class CostModel:
         # stage's own memory
         self.reference_memo = True
         self._record_cache = {}       # single-stage records by (first op, micro-batch index, stage size, code bytes)
+        self._record_cache_max = 8192 # emptied when it has grown beyond this many records
         self._tp_lut = np.zeros(max(db.tp_list) + 1, dtype=np.uint8)      # tp size -> its index in the database
         self._tp_lut[np.asarray(db.tp_list)] = np.arange(len(db.tp_list), dtype=np.uint8)
         self._mbs_index = {m: k for k, m in enumerate(db.mbs_list)}
@@ -291,6 +292,8 @@ class CostModel:
         keys = [(int(ranges[p, 0]), int(hdr[p, 0]) >> 8, int(hdr[p, 1]), codes[p, ranges[p, 0]:ranges[p, 1]].tobytes())
                 for p in range(P)]
         cache = self._record_cache
+        if len(cache) > self._record_cache_max:
+            cache.clear()            # (before the look-ups below: what this call hits must still be there when it is read)
         out = np.empty((P, STAGE_REC), dtype=np.float64)
         miss = [p for p in range(P) if keys[p] not in cache]
         if miss:
@@ -302,8 +305,6 @@ class CostModel:
             it, pk, fe, st, rec = self.evaluator.score_host(PlanBatch(codes[todo], hdr[todo]), breakdown=True,
                                                             ranges=ranges[todo])
             self._raise_for_status(st)
-            if len(cache) + len(todo) > 8192:
-                cache.clear()
             for j, p in enumerate(todo):
                 cache[keys[p]] = (rec[j, 0, :].copy(), int(hdr[p, 0]) & 0xff)
         for p in range(P):

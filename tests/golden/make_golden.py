@@ -537,7 +537,7 @@ def child_search_trace(case, extras=False, per_function=25):
     tmp = tempfile.mkdtemp()
     for d in ("", "trends/", "csv/", "top_configs/"):          # (what the search's reporting writes into)
         os.makedirs(os.path.join(tmp, d), exist_ok=True)
-    extra = ["--no-multi-process", "--time-budget-total", "1000000", "--max-num-trials", "4", "--max-num-hops", "3",
+    extra = ["--no-multi-process", "--time-budget-total", "1000000", "--max-num-trials", os.environ.get("GOLDEN_TRIALS", "4"), "--max-num-hops", os.environ.get("GOLDEN_HOPS", "3"),
              "--log-path", tmp + "/", "--config-save-path", tmp + "/", "--add-action-tp-dp-exchange"]
     if extras:
         extra += TRACE_EXTRAS
@@ -692,7 +692,7 @@ def child_binding_search(case):
     tmp = tempfile.mkdtemp()
     for d in ("", "trends/", "csv/", "top_configs/"):
         os.makedirs(os.path.join(tmp, d), exist_ok=True)
-    extra = ["--no-multi-process", "--time-budget-total", "1000000", "--max-num-trials", "4", "--max-num-hops", "3",
+    extra = ["--no-multi-process", "--time-budget-total", "1000000", "--max-num-trials", os.environ.get("GOLDEN_TRIALS", "4"), "--max-num-hops", os.environ.get("GOLDEN_HOPS", "3"),
              "--log-path", tmp + "/", "--config-save-path", tmp + "/", "--add-action-tp-dp-exchange"]
     if num_layers:
         extra += ["--num-layers", str(num_layers)]

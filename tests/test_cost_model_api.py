@@ -574,3 +574,20 @@ def test_value_after_gpu_move_matches_reference_gpu(golden_dir, case):
         _run_gpu_moves(g, m)
     finally:
         m.close()
+
+
+def test_record_cache_survives_its_own_eviction(golden_dir):
+    """Single-stage records are kept by their kernel inputs and the table is emptied when it has grown too large: a call
+    some of whose queries are in the table and some not must get all its records also when the table is emptied on that
+    call (the emptying once happened between the look-up and the read: KeyError in a long search)."""
+    g, m = make_model(golden_dir, "resnet_500M", "emu")
+    ops = m.graph.ops
+    q = lambda lo, n, bit: (ops[lo:lo + n], [bit] * n, [1] * n, [1] * n, 32, 0, [0] * n)
+    first = m._stage_records([q(3, 5, 0)])
+    m._record_cache_max = 1
+    both = m._stage_records([q(3, 5, 0), q(20, 7, 1)])             # one known, one new, table at its limit
+    assert np.array_equal(both[0], first[0], equal_nan=True)
+    more = m._stage_records([q(20, 7, 1), q(3, 5, 0), q(40, 4, 0), q(41, 4, 1)])
+    assert np.array_equal(more[0], both[1], equal_nan=True) and np.array_equal(more[1], first[0], equal_nan=True)
+    fresh = make_model(golden_dir, "resnet_500M", "emu")[1]
+    assert np.array_equal(fresh._stage_records([q(40, 4, 0), q(41, 4, 1)]), more[2:], equal_nan=True)

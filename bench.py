@@ -190,7 +190,8 @@ def main():
                      "traffic": counters["traffic_bytes_per_plan"] * P if counters else None,
                      "traffic_source": f'{counters["source"]} (library sources of commit {counters["commit"]})' if counters else None,
                      "algorithmic_bytes": algo_bytes,
-                     "kernel": "ace_score_kernel<BD=false,RANGED=false,WIN=false,DEFER=true>", "kernel_ms": kern_ms,
+                     "kernel": ("ace_score_kernel<BD=false,RANGED=false,WIN=true,DEFER=false>" if tables.n_windows > 1 else
+                                "ace_score_kernel<BD=false,RANGED=false,WIN=false,DEFER=true>"), "kernel_ms": kern_ms,
                      "algorithmic_bytes_per_plan": 3 * N + 19,
                      "bytes_moved_per_plan": d.bytes_moved_per_plan + 17,
                      "achieved_on_bytes_moved": moved_bytes / (kern_ms * 1e-3) / 1e9,

@@ -679,11 +679,39 @@ def child_search_trace(case, extras=False, per_function=25):
     print(f"[golden] search trace {case}{' (extras)' if extras else ''}: { {n: len(v) for n, v in trace.items()} }, best {results}")
 
 
+def child_search_results(case):
+    """The reference's search with its own cost model and nothing recorded but what it found (the flags of
+    child_search_trace; GOLDEN_TRIALS / GOLDEN_HOPS set the length): one JSON line on standard output."""
+    import contextlib
+    import io
+    import tempfile
+    model, size, db, mbs_list, nodes, gpn, gbs, limit, num_layers = CASES[case]
+    tmp = tempfile.mkdtemp()
+    for d in ("", "trends/", "csv/", "top_configs/"):
+        os.makedirs(os.path.join(tmp, d), exist_ok=True)
+    extra = ["--no-multi-process", "--time-budget-total", "1000000", "--max-num-trials", os.environ.get("GOLDEN_TRIALS", "4"), "--max-num-hops", os.environ.get("GOLDEN_HOPS", "3"),
+             "--log-path", tmp + "/", "--config-save-path", tmp + "/", "--add-action-tp-dp-exchange"]
+    if num_layers:
+        extra += ["--num-layers", str(num_layers)]
+    sys.argv = reference_argv(case, extra)
+    sys.path.insert(0, os.path.join(REF, "search"))
+    found = {}
+    with contextlib.redirect_stdout(io.StringIO()):
+        import aceso_search as S                   # noqa: the reference, run to record what it finds
+        for num_stages in (2, 3, 4):
+            r = S.run_search(num_stages, queue=None)
+            found[str(num_stages)] = None if r is None else [r[0], r[1], r[2]]
+    shutil.rmtree(tmp, ignore_errors=True)
+    print(json.dumps(found))
+
+
 def child_binding_search(case):
     """The reference's search run a second time with its cost model REPLACED by this repository's binding
     (superscaler_amd/binding/aceso_cost_model.py, scoring through the CPU build of the kernel source, tests/emu): same
     flags and stage counts as child_search_trace.  Writes what both runs found into search_binding_<case>.json; the
-    two must be equal (tests/test_search_trace.py checks the file)."""
+    two must be equal (tests/test_search_trace.py checks the file).  With GOLDEN_TRIALS / GOLDEN_HOPS in the environment
+    (the committed long runs: 40 trials of 7 hops, the hop count of the reference's scripts; about twenty minutes a
+    model) both searches are run at that length and the record goes to search_binding_<case>__long.json."""
     import contextlib
     import importlib.util
     import io
@@ -720,12 +748,24 @@ def child_binding_search(case):
         for num_stages in (2, 3, 4):
             r = S.run_search(num_stages, queue=None)
             found[str(num_stages)] = None if r is None else [r[0], r[1], r[2]]
-    with open(os.path.join(HERE, f"search_trace_{case}.json")) as f:
-        ref = json.load(f)["best_time_and_memory"]
+    long_run = "GOLDEN_TRIALS" in os.environ or "GOLDEN_HOPS" in os.environ
+    explored_ref = None
+    if long_run:
+        # another length than the recorded trace's: the reference's own run of that length, in a process of its own
+        r = subprocess.run([sys.executable, os.path.abspath(__file__), "--child-search-results", case], check=True,
+                           stdout=subprocess.PIPE, text=True)
+        own = json.loads(r.stdout.strip().splitlines()[-1])
+        ref = {k: (v[:2] if v else None) for k, v in own.items()}
+        explored_ref = {k: (v[2] if v else None) for k, v in own.items()}
+    else:
+        with open(os.path.join(HERE, f"search_trace_{case}.json")) as f:
+            ref = json.load(f)["best_time_and_memory"]
     out = {"case": case, "flags": extra[:7] + ["--add-action-tp-dp-exchange"], "with_the_binding": {k: (v[:2] if v else None) for k, v in found.items()},
            "explored_with_the_binding": {k: (v[2] if v else None) for k, v in found.items()},
            "with_the_reference_cost_model": ref}
-    with open(os.path.join(HERE, f"search_binding_{case}.json"), "w") as f:
+    if explored_ref is not None:
+        out["explored_with_the_reference_cost_model"] = explored_ref
+    with open(os.path.join(HERE, f"search_binding_{case}{'__long' if long_run else ''}.json"), "w") as f:
         json.dump(out, f, indent=1)
     shutil.rmtree(tmp, ignore_errors=True)
     same = out["with_the_binding"] == {k: v for k, v in ref.items()}
@@ -796,6 +836,8 @@ def main():
         return child_moves(sys.argv[2])
     if len(sys.argv) > 2 and sys.argv[1] == "--child-initial":
         return child_initial(sys.argv[2])
+    if len(sys.argv) > 2 and sys.argv[1] == "--child-search-results":
+        return child_search_results(sys.argv[2])
     if len(sys.argv) > 2 and sys.argv[1] == "--child-binding-grid":
         return child_binding_grid(sys.argv[2])
     if len(sys.argv) > 2 and sys.argv[1] == "--child-binding-search":

@@ -145,3 +145,16 @@ def test_the_references_search_over_the_binding_found_the_same_plans(golden_dir,
     assert wanted <= exported
     import superscaler_amd.aceso_cost_model as api
     assert all(callable(getattr(api, name)) for name in exported - {"parse_args"})
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_the_long_search_over_the_binding_found_the_same_plans(golden_dir, case):
+    """The same comparison at ten times the length: 40 trials of up to 7 hops (the hop count of the reference's own
+    search scripts), both runs made by the fixture generator at that length (GOLDEN_TRIALS=40 GOLDEN_HOPS=7)."""
+    with open(os.path.join(golden_dir, f"search_binding_{case}__long.json")) as f:
+        fx = json.load(f)
+    assert fx["flags"][fx["flags"].index("--max-num-trials") + 1] == "40" and fx["flags"][fx["flags"].index("--max-num-hops") + 1] == "7"
+    assert set(fx["with_the_binding"]) == {"2", "3", "4"}
+    assert fx["with_the_binding"] == fx["with_the_reference_cost_model"]
+    assert fx["explored_with_the_binding"] == fx["explored_with_the_reference_cost_model"]
+    assert all(n >= 20 for n in fx["explored_with_the_binding"].values())

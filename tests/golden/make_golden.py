@@ -665,7 +665,7 @@ def child_search_trace(case, extras=False, per_function=25):
     with contextlib.redirect_stdout(io.StringIO()):
         import aceso_search as S                   # noqa (binds the wrapped functions; reads the database)
         results = {}
-        for num_stages in (2, 3, 4):
+        for num_stages in [int(x) for x in os.environ.get("GOLDEN_STAGES", "2,3,4").split(",")]:
             taken.update({n: 0 for n in TRACED})
             r = S.run_search(num_stages, queue=None)
             results[num_stages] = None if r is None else [r[0], r[1]]
@@ -691,6 +691,7 @@ def child_search_results(case):
         os.makedirs(os.path.join(tmp, d), exist_ok=True)
     extra = ["--no-multi-process", "--time-budget-total", "1000000", "--max-num-trials", os.environ.get("GOLDEN_TRIALS", "4"), "--max-num-hops", os.environ.get("GOLDEN_HOPS", "3"),
              "--log-path", tmp + "/", "--config-save-path", tmp + "/", "--add-action-tp-dp-exchange"]
+    extra += os.environ.get("GOLDEN_FLAGS", "").split()        # (further flags of the reference, for both runs alike)
     if num_layers:
         extra += ["--num-layers", str(num_layers)]
     sys.argv = reference_argv(case, extra)
@@ -698,7 +699,7 @@ def child_search_results(case):
     found = {}
     with contextlib.redirect_stdout(io.StringIO()):
         import aceso_search as S                   # noqa: the reference, run to record what it finds
-        for num_stages in (2, 3, 4):
+        for num_stages in [int(x) for x in os.environ.get("GOLDEN_STAGES", "2,3,4").split(",")]:
             r = S.run_search(num_stages, queue=None)
             found[str(num_stages)] = None if r is None else [r[0], r[1], r[2]]
     shutil.rmtree(tmp, ignore_errors=True)
@@ -722,6 +723,7 @@ def child_binding_search(case):
         os.makedirs(os.path.join(tmp, d), exist_ok=True)
     extra = ["--no-multi-process", "--time-budget-total", "1000000", "--max-num-trials", os.environ.get("GOLDEN_TRIALS", "4"), "--max-num-hops", os.environ.get("GOLDEN_HOPS", "3"),
              "--log-path", tmp + "/", "--config-save-path", tmp + "/", "--add-action-tp-dp-exchange"]
+    extra += os.environ.get("GOLDEN_FLAGS", "").split()        # (further flags of the reference, for both runs alike)
     if num_layers:
         extra += ["--num-layers", str(num_layers)]
     sys.argv = reference_argv(case, extra)
@@ -745,10 +747,10 @@ def child_binding_search(case):
     with contextlib.redirect_stdout(io.StringIO()):
         import aceso_search as S                   # noqa: the reference's search, unchanged
         found = {}
-        for num_stages in (2, 3, 4):
+        for num_stages in [int(x) for x in os.environ.get("GOLDEN_STAGES", "2,3,4").split(",")]:
             r = S.run_search(num_stages, queue=None)
             found[str(num_stages)] = None if r is None else [r[0], r[1], r[2]]
-    long_run = "GOLDEN_TRIALS" in os.environ or "GOLDEN_HOPS" in os.environ
+    long_run = any(k in os.environ for k in ("GOLDEN_TRIALS", "GOLDEN_HOPS", "GOLDEN_FLAGS", "GOLDEN_STAGES"))
     explored_ref = None
     if long_run:
         # another length than the recorded trace's: the reference's own run of that length, in a process of its own
@@ -760,12 +762,14 @@ def child_binding_search(case):
     else:
         with open(os.path.join(HERE, f"search_trace_{case}.json")) as f:
             ref = json.load(f)["best_time_and_memory"]
-    out = {"case": case, "flags": extra[:7] + ["--add-action-tp-dp-exchange"], "with_the_binding": {k: (v[:2] if v else None) for k, v in found.items()},
+    out = {"case": case, "flags": extra[:7] + ["--add-action-tp-dp-exchange"] + os.environ.get("GOLDEN_FLAGS", "").split(),
+           "stage_counts": os.environ.get("GOLDEN_STAGES", "2,3,4"), "with_the_binding": {k: (v[:2] if v else None) for k, v in found.items()},
            "explored_with_the_binding": {k: (v[2] if v else None) for k, v in found.items()},
            "with_the_reference_cost_model": ref}
     if explored_ref is not None:
         out["explored_with_the_reference_cost_model"] = explored_ref
-    with open(os.path.join(HERE, f"search_binding_{case}{'__long' if long_run else ''}.json"), "w") as f:
+    suffix = os.environ.get("GOLDEN_SUFFIX", "__long") if long_run else ""
+    with open(os.path.join(HERE, f"search_binding_{case}{suffix}.json"), "w") as f:
         json.dump(out, f, indent=1)
     shutil.rmtree(tmp, ignore_errors=True)
     same = out["with_the_binding"] == {k: v for k, v in ref.items()}

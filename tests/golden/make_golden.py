@@ -3,7 +3,7 @@
 
 Run in the build container only (it needs /root/reference):
 
-    python tests/golden/make_golden.py [base] [variants] [moves] [grid] [initial] [main] [trace] [kat]
+    python tests/golden/make_golden.py [base] [variants] [moves] [grid] [initial] [main] [trace] [sweep] [kat]
 
 (no argument: every part).
 
@@ -36,7 +36,9 @@ Further children of the same kind write
   search_trace_<case>.json         the calls the reference's own search makes into the cost model during a short run
                                    (arguments and results);
   search_binding_<case>.json       what the same search finds when its cost model is replaced by this repository's
-                                   binding, beside what it found with its own.
+                                   binding, beside what it found with its own; ...__sweep_<name>.json: the same under
+                                   further settings of the reference (BINDING_SWEEPS); ...__long.json: at ten times
+                                   the length.
 """
 import json
 import os
@@ -520,6 +522,22 @@ TRACED = ["predict_time_breakdown", "update_recompute", "get_reserved_memory_lis
           "predict_stage_time", "predict_stage_memory"]
 
 
+# The search comparison of child_binding_search under further settings of the reference: name -> (flags, stage counts)
+BINDING_SWEEPS = {
+    "extras": ("--predict-delta-time --add-action-finetune-dim --add-action-finetune-algo --add-action-tune-tp-dp "
+               "--finetune-after-trial 1 --finetune-tp-dp-after-trial", "2,3,4"),
+    "min": ("--memory-pred-type MIN", "2,3,4"),
+    "noflex": ("--do-not-use-flex-recompute", "2,3,4"),
+    "peakbwd": ("--peak-mem-in-backward 700", "2,3,4"),
+    "noreserved": ("--do-not-consider-reserved-space", "2,3,4"),
+    "noshared": ("--do-not-consider-shared-tensor-space", "2,3,4"),
+    "stages1568": ("", "1,5,6,8"),
+    "imbgpu": ("--initial-point imbalance_gpu", "2,3,4"),
+    "collmem": ("--consider-collective-memory", "2,3,4"),          # (not for T5: resharding is off there)
+    "imbop": ("--initial-point imbalance_op", "2,3,4"),            # (GPT only: the reference's own start for ResNet
+                                                                   #  assumes ResNet-50's 33 layers and fails on this model)
+}
+
 TRACE_EXTRAS = ["--predict-delta-time", "--add-action-finetune-dim", "--add-action-finetune-algo", "--add-action-tune-tp-dp",
                 "--finetune-after-trial", "1", "--finetune-tp-dp-after-trial"]
 
@@ -848,8 +866,9 @@ def main():
         return child_binding_search(sys.argv[2])
     if len(sys.argv) > 2 and sys.argv[1] == "--child-search-trace":
         return child_search_trace(sys.argv[2], extras=len(sys.argv) > 3 and sys.argv[3] == "extras")
-    # optional arguments: the parts to (re)write, of base variants moves grid initial main trace kat; none = all
-    parts = set(sys.argv[1:]) or {"base", "variants", "moves", "grid", "initial", "main", "trace", "kat"}
+    # optional arguments: the parts to (re)write, of base variants moves grid initial main trace sweep kat; none = all
+    # (the long search comparison, search_binding_<case>__long.json, is made by hand: see child_binding_search)
+    parts = set(sys.argv[1:]) or {"base", "variants", "moves", "grid", "initial", "main", "trace", "sweep", "kat"}
     quiet = subprocess.DEVNULL if os.environ.get("GOLDEN_QUIET") else None
     me = os.path.abspath(__file__)
     for case in CASES:
@@ -879,6 +898,12 @@ def main():
             subprocess.run([sys.executable, me, "--child-binding-search", case], check=True, stdout=quiet)
             if os.path.exists(os.path.join(HERE, f"megatron_grid_{case}.json")):
                 subprocess.run([sys.executable, me, "--child-binding-grid", case], check=True, stdout=quiet)
+        if "sweep" in parts:
+            for name, (flags, stages) in BINDING_SWEEPS.items():
+                if (name == "collmem" and CASES[case][0] == "t5") or (name == "imbop" and CASES[case][0] != "gpt"):
+                    continue
+                env = dict(os.environ, GOLDEN_FLAGS=flags, GOLDEN_STAGES=stages, GOLDEN_SUFFIX=f"__sweep_{name}")
+                subprocess.run([sys.executable, me, "--child-binding-search", case], check=True, stdout=quiet, env=env)
     if "kat" not in parts:
         return
     # the single-GPU known-answer plans and the database files they index (data files)

@@ -158,3 +158,22 @@ def test_the_long_search_over_the_binding_found_the_same_plans(golden_dir, case)
     assert fx["with_the_binding"] == fx["with_the_reference_cost_model"]
     assert fx["explored_with_the_binding"] == fx["explored_with_the_reference_cost_model"]
     assert all(n >= 20 for n in fx["explored_with_the_binding"].values())
+
+
+def test_the_search_over_the_binding_under_further_settings(golden_dir):
+    """The same comparison (short searches) under the reference's other settings: the optional actions with the
+    delta-time prediction, MIN memory prediction, no flex recompute, a backward peak, no reserved / no shared space,
+    collective memory, 1 / 5 / 6 / 8 stages, the other starting points (make_golden.BINDING_SWEEPS): 27 records, each
+    with the same best plans and the same number of explored plans on both sides."""
+    import glob
+    files = sorted(glob.glob(os.path.join(golden_dir, "search_binding_*__sweep_*.json")))
+    assert len(files) == 27
+    names = set()
+    for path in files:
+        with open(path) as f:
+            fx = json.load(f)
+        names.add(os.path.basename(path).split("__sweep_")[1][:-5])
+        assert fx["with_the_binding"] == fx["with_the_reference_cost_model"], path
+        assert fx["explored_with_the_binding"] == fx["explored_with_the_reference_cost_model"], path
+        assert any(v is not None for v in fx["with_the_binding"].values()), path
+    assert names == {"extras", "min", "noflex", "peakbwd", "noreserved", "noshared", "stages1568", "imbgpu", "collmem", "imbop"}

@@ -3,9 +3,9 @@
 
 Run in the build container only (it needs /root/reference):
 
-    python tests/golden/make_golden.py [base] [variants] [moves] [grid] [initial] [main] [trace] [sweep] [kat]
+    python tests/golden/make_golden.py [base] [variants] [moves] [grid] [initial] [main] [trace] [sweep] [kat] [big]
 
-(no argument: every part).
+(no argument: every part but `big`, the search comparison on GPT-13B with 32 GPUs, which takes a quarter of an hour).
 
 For each model family it (1) copies the few profile-database CSV files the case needs from
 the reference tree into tests/golden/db_<case>/ (data files, not source), (2) starts one
@@ -38,7 +38,7 @@ Further children of the same kind write
   search_binding_<case>.json       what the same search finds when its cost model is replaced by this repository's
                                    binding, beside what it found with its own; ...__sweep_<name>.json: the same under
                                    further settings of the reference (BINDING_SWEEPS); ...__long.json: at ten times
-                                   the length.
+                                   the length; search_binding_gpt_13B__big.json: GPT-13B on 4 nodes of 8 GPUs.
 """
 import json
 import os
@@ -55,6 +55,12 @@ CASES = {
     "gpt_1_3B": ("gpt", "1_3B", "profiler/profiled-time-eurosys", [1, 2, 4, 8], 2, 4, 512, 12000, 24),
     "resnet_500M": ("resnet", "500M", "profiler/profiled-time-miniset", [32, 64], 1, 4, 768, 12000, None),
     "t5_770M": ("t5", "770M", "profiler/profiled-time-miniset", [1, 2, 4, 8], 1, 4, 512, 9000, 24),
+}
+
+# a larger setting for the search comparison only (child_binding_search): 32 GPUs, tp up to 8; its database files are
+# the ones the known-answer tests already hold (tests/golden/kat)
+BIG_CASES = {
+    "gpt_13B": ("gpt", "13B", "profiler/profiled-time-eurosys", [1, 2, 4, 8], 4, 8, 1024, 28000, 40),
 }
 
 # non-default switches of the cost model (aceso_utils.py:405, 423-430, 448)
@@ -133,8 +139,8 @@ def rand_plan(rng, full_ops, tunable, num_gpus, mbs_list, max_stages, max_tp, un
 
 
 def reference_argv(case, extra=()):
-    model, size, db, mbs_list, nodes, gpn, gbs, limit, num_layers = CASES[case]
-    dbdir = os.path.join(HERE, f"db_{case}") + "/"
+    model, size, db, mbs_list, nodes, gpn, gbs, limit, num_layers = {**CASES, **BIG_CASES}[case]
+    dbdir = os.path.join(HERE, "kat" if case in BIG_CASES else f"db_{case}") + "/"
     return ["golden", "--model-name", model, "--model-size", size,
             "--num-nodes", str(nodes), "--num-gpus-per-node", str(gpn),
             "--global-batch-size", str(gbs), "--memory-limit", str(limit),
@@ -703,7 +709,7 @@ def child_search_results(case):
     import contextlib
     import io
     import tempfile
-    model, size, db, mbs_list, nodes, gpn, gbs, limit, num_layers = CASES[case]
+    model, size, db, mbs_list, nodes, gpn, gbs, limit, num_layers = {**CASES, **BIG_CASES}[case]
     tmp = tempfile.mkdtemp()
     for d in ("", "trends/", "csv/", "top_configs/"):
         os.makedirs(os.path.join(tmp, d), exist_ok=True)
@@ -735,7 +741,7 @@ def child_binding_search(case):
     import importlib.util
     import io
     import tempfile
-    model, size, db, mbs_list, nodes, gpn, gbs, limit, num_layers = CASES[case]
+    model, size, db, mbs_list, nodes, gpn, gbs, limit, num_layers = {**CASES, **BIG_CASES}[case]
     tmp = tempfile.mkdtemp()
     for d in ("", "trends/", "csv/", "top_configs/"):
         os.makedirs(os.path.join(tmp, d), exist_ok=True)
@@ -898,6 +904,11 @@ def main():
             subprocess.run([sys.executable, me, "--child-binding-search", case], check=True, stdout=quiet)
             if os.path.exists(os.path.join(HERE, f"megatron_grid_{case}.json")):
                 subprocess.run([sys.executable, me, "--child-binding-grid", case], check=True, stdout=quiet)
+    if "big" in parts:
+        # (about a quarter of an hour)
+        env = dict(os.environ, GOLDEN_SUFFIX="__big", GOLDEN_STAGES="4,5,6,8,16", GOLDEN_TRIALS="8", GOLDEN_HOPS="5")
+        subprocess.run([sys.executable, me, "--child-binding-search", "gpt_13B"], check=True, stdout=quiet, env=env)
+    for case in CASES:
         if "sweep" in parts:
             for name, (flags, stages) in BINDING_SWEEPS.items():
                 if (name == "collmem" and CASES[case][0] == "t5") or (name == "imbop" and CASES[case][0] != "gpt"):

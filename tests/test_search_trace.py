@@ -177,3 +177,16 @@ def test_the_search_over_the_binding_under_further_settings(golden_dir):
         assert fx["explored_with_the_binding"] == fx["explored_with_the_reference_cost_model"], path
         assert any(v is not None for v in fx["with_the_binding"].values()), path
     assert names == {"extras", "min", "noflex", "peakbwd", "noreserved", "noshared", "stages1568", "imbgpu", "collmem", "imbop"}
+
+
+def test_the_search_over_the_binding_on_32_gpus(golden_dir):
+    """GPT-13B (523 ops) on 4 nodes of 8 GPUs -- tensor parallelism up to 8, stages across node boundaries -- with 4, 5, 6, 8
+    and 16 pipeline stages, 8 trials of up to 5 hops: same best plans and same number of explored plans (437 to 17,270)
+    over the binding as with the reference's own cost model."""
+    with open(os.path.join(golden_dir, "search_binding_gpt_13B__big.json")) as f:
+        fx = json.load(f)
+    assert set(fx["with_the_binding"]) == {"4", "5", "6", "8", "16"}
+    assert fx["with_the_binding"] == fx["with_the_reference_cost_model"]
+    assert fx["explored_with_the_binding"] == fx["explored_with_the_reference_cost_model"]
+    assert all(v is not None and v[1] <= 28000 for v in fx["with_the_binding"].values())
+    assert max(fx["explored_with_the_binding"].values()) > 10000

@@ -65,6 +65,11 @@ class CostModel:
         self.reference_memo = True
         self._record_cache = {}       # single-stage records by (first op, micro-batch index, stage size, code bytes)
         self._record_cache_max = 8192 # emptied when it has grown beyond this many records
+        # predict_value_after_move: how many op counts a scan over them may be evaluated ahead (0: never); the scans seen
+        # lately with their evaluated-ahead results
+        self.look_ahead = 32
+        self._scans = {}
+        self.scan_ahead_used, self.scan_ahead_evaluated, self.scan_ahead_dropped = 0, 0, 0
         self._tp_lut = np.zeros(max(db.tp_list) + 1, dtype=np.uint8)      # tp size -> its index in the database
         self._tp_lut[np.asarray(db.tp_list)] = np.arange(len(db.tp_list), dtype=np.uint8)
         self._mbs_index = {m: k for k, m in enumerate(db.mbs_list)}
@@ -320,6 +325,11 @@ class CostModel:
         if len(ops) == 0:
             return 0 / 1000
         r = self._stage_records([(ops, recompute_ops, tp_size, dp_size, base_batch_size, 0, algo_list)])[0].tolist()
+        return self._stage_time_of(r, delta, on_the_right, decrease)
+
+    @staticmethod
+    def _stage_time_of(r, delta=False, on_the_right=False, decrease=True):
+        """The sum of aceso_cost_model.py:505-512 over one stage record."""
         fwd_comp, bwd_comp, in_comm, out_comm, recomp_time = r[R_FWD], r[R_BWD], r[R_IN_COMM], r[R_OUT_COMM], r[R_RECOMP]
         if not delta:
             sum_time = fwd_comp + bwd_comp + in_comm + out_comm + recomp_time
@@ -420,9 +430,12 @@ class CostModel:
             if si < len(rc) - 1:
                 rc[si + 1] = 1
 
-    def check_recompute_batch(self, queries):
+    def check_recompute_batch(self, queries, memo=None, starts=None):
         """check_recompute for many stages at once, identical to calling it one by one.
         queries: [(ops, micro_bs, tp_size, dp_size, num_stages_behind, algo_list)]; returns the recompute lists.
+        `memo` (default: `self.reference_memo`): whether the starting memory goes through the reference's memo table;
+        `starts`, a list, receives per query (memo key, starting memory as evaluated) -- both are for the evaluate-ahead
+        of predict_value_after_move, which works off the table and applies it when a result is used.
 
         Which op group a greedy round takes (:794-806) depends only on the group sums and on which
         groups earlier rounds took, not on the memory figures; those only decide whether the round
@@ -434,7 +447,10 @@ class CostModel:
         stage evaluations."""
         args = self.settings
         n = len(queries)
+        use_memo = self.reference_memo if memo is None else memo
         if not args.flex_recompute:
+            if starts is not None:
+                starts.extend((None, None) for _ in queries)
             return [[1] * len(q[0]) for q in queries]
         rcs = [[0] * len(q[0]) for q in queries]
         if n == 0:
@@ -483,11 +499,14 @@ class CostModel:
         for k, (ops, micro_bs, tp_size, dp_size, nsb, algo_list) in enumerate(queries):
             mw, mg, mo, ma, mp, mr = self._memory_breakdown(rec[k].tolist(), nsb)
             stage_memory = mw + mg + mo + ma + mp + mr
-            if self.reference_memo:
+            if use_memo or starts is not None:
                 # :828 asks predict_stage_memory_helper, whose table is keyed by the stage's first op NAME, its length and
                 # its per-op lists (:759): a stage that shares those with one asked about earlier starts from that one's
                 # memory, whatever its other ops are (possible where a model's layers differ, as T5's encoder and decoder)
                 key = (f"ops{ops[0]}{len(ops)}tp{tp_size}dp{dp_size}rc{rcs[k]}algo{algo_list}bs{micro_bs}stage{nsb}")
+                if starts is not None:
+                    starts.append((key, stage_memory))
+            if use_memo:
                 self.stage_memory_visit += 1
                 known = self.stage_memory_set.get(key)
                 if known is not None:
@@ -599,6 +618,10 @@ class CostModel:
                                  dec_gpus=False, dim=None):
         """aceso_cost_model.py:693-739."""
         st = config.stages[bottleneck]
+        if self.look_ahead > 0 and not inc_gpus and not dec_gpus and partner is not None and bottleneck != partner:
+            ahead = self._scan_step(st, config.micro_bs, bottleneck < partner, num_ops_moved, metric)
+            if ahead is not None:
+                return ahead
         ops, tp_size, dp_size = list(st.ops), list(st.tp_size), list(st.dp_size)
         algo_list, recompute_ops = list(st.algo), list(st.recompute_ops)
         if num_ops_moved > 0:
@@ -624,6 +647,97 @@ class CostModel:
         else:
             raise RuntimeError(f"metric {metric} not implemented.")
         return value, recompute_ops
+
+    # ---- predict_value_after_move over a scan of op counts ------------------------------------------------------------
+    # The reference's op migration (aceso_prims.py:168-185, :252-271) asks predict_value_after_move for the same stage
+    # with 0, 1, 2, ... ops taken off one end until a value falls below its goal, and again from 0 for the next goal.
+    # One such call is a check_recompute (two or three launches) and a stage evaluation, each for ONE stage: launch
+    # latency, not scoring.  Once a scan is recognised (the same stage contents, the next op count) the coming op counts
+    # are evaluated together, a window that doubles while the scan goes on, and the later calls are answered from that.
+    # What a call returns and what it leaves in the memo table are the same as without: a result evaluated ahead is
+    # computed off the table (from the stage's own memory) and the table is consulted and written when the result is
+    # used; where the table then holds another starting memory for the key, the result is dropped and the call takes
+    # the ordinary path.
+
+    _SCANS_KEPT = 16
+
+    def _scan_step(self, st, micro_bs, to_the_right, num_ops_moved, metric):
+        """predict_value_after_move(..., num_ops_moved, metric) from a result evaluated ahead: (value, recompute list),
+        or None when the call is to take the ordinary path."""
+        if metric in ("time", "time_with_efficiency"):
+            on_time = True
+        elif metric == "memory":
+            on_time = False
+        else:
+            return None
+        a = self.settings
+        try:
+            key = (tuple(st.ops), bytes(st.tp_size), bytes(st.dp_size), bytes(st.algo), micro_bs, st.num_stages_behind,
+                   to_the_right, on_time, a.memory_limit, a.flex_recompute, a.peak_mem_in_backward)
+        except (ValueError, TypeError):           # a size beyond a byte: not worth a second encoding
+            return None
+        scan = self._scans.get(key)
+        if scan is None:
+            if len(self._scans) >= self._SCANS_KEPT:
+                del self._scans[next(iter(self._scans))]
+            self._scans[key] = {"last": num_ops_moved, "window": 0, "ahead": {}}
+            return None
+        if num_ops_moved <= 0:
+            scan["last"] = num_ops_moved
+            return None
+        entry = scan["ahead"].get(num_ops_moved)
+        if entry is None:
+            step = num_ops_moved - scan["last"]
+            scan["last"] = num_ops_moved
+            if not 0 < step <= 8:
+                scan["window"] = 0
+                return None
+            scan["window"] = min(max(4, 2 * scan["window"]), self.look_ahead)
+            self._scan_ahead(scan, st, micro_bs, to_the_right, num_ops_moved, step, on_time)
+            entry = scan["ahead"].get(num_ops_moved)
+            if entry is None:
+                return None
+        else:
+            scan["last"] = num_ops_moved
+        rc, value, memo_key, start = entry
+        if memo_key is not None and self.reference_memo:
+            known = self.stage_memory_set.get(memo_key)
+            if known is not None and known != start:
+                self.scan_ahead_dropped += 1      # check_recompute would start elsewhere (see check_recompute_batch)
+                return None
+            self.stage_memory_visit += 1
+            if known is not None:
+                self.stage_memory_hit += 1
+            else:
+                self.stage_memory_set[memo_key] = start
+        self.scan_ahead_used += 1
+        return value, list(rc)
+
+    def _scan_ahead(self, scan, st, micro_bs, to_the_right, first, step, on_time):
+        """Evaluate `scan["window"]` op counts from `first` on, `step` apart, for stage `st`."""
+        n, nsb = len(st.ops), st.num_stages_behind
+        counts = [k for k in range(first, first + step * scan["window"], step) if k < n]
+        if not counts:
+            return
+        ops, tp_size, dp_size, algo = list(st.ops), list(st.tp_size), list(st.dp_size), list(st.algo)
+        parts = []
+        for k in counts:
+            sl = slice(None, -k) if to_the_right else slice(k, None)
+            parts.append((ops[sl], tp_size[sl], dp_size[sl], algo[sl]))
+        starts = []
+        rcs = self.check_recompute_batch([(o, micro_bs, t, d, nsb, g) for o, t, d, g in parts], memo=False, starts=starts)
+        # (predict_stage_time evaluates with no stage behind, predict_stage_memory with the stage's own count)
+        rec = self._stage_records([(o, rc, t, d, micro_bs, 0 if on_time else nsb, g)
+                                   for (o, t, d, g), rc in zip(parts, rcs)])
+        for j, k in enumerate(counts):
+            r = rec[j].tolist()
+            if on_time:
+                value = self._stage_time_of(r)
+            else:
+                mw, mg, mo, ma, mp, mr = self._memory_breakdown(r, nsb)
+                value = mw + mg + mo + ma + mp + mr
+            scan["ahead"][k] = (bytes(rcs[j]), value, starts[j][0], starts[j][1])
+        self.scan_ahead_evaluated += len(counts)
 
     def wrap_predict_delta_time(self, config, longest_stage, shortest_stage, num_ops_moved, decrease=True):
         """aceso_cost_model.py:885-922."""

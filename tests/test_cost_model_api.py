@@ -591,3 +591,64 @@ def test_record_cache_survives_its_own_eviction(golden_dir):
     assert np.array_equal(more[0], both[1], equal_nan=True) and np.array_equal(more[1], first[0], equal_nan=True)
     fresh = make_model(golden_dir, "resnet_500M", "emu")[1]
     assert np.array_equal(fresh._stage_records([q(40, 4, 0), q(41, 4, 1)]), more[2:], equal_nan=True)
+
+
+def _scan_twice(m, cfg, stage, partner, metric, step=1):
+    """The op migration's call pattern (aceso_prims.py:168-185): every op count from 0 up, then again from 0."""
+    out = []
+    for _ in range(2):
+        for k in range(0, len(cfg.stages[stage].ops), step):
+            value, rc = m.predict_value_after_move(cfg, stage, partner, k, metric)
+            out.append((k, value, list(rc)))
+    return out
+
+
+def _scans_check(golden_dir, case, backend):
+    """predict_value_after_move answers a scan over op counts from results evaluated ahead: values, recompute lists, the
+    memo table and its counters must be those of the one-by-one path (look_ahead = 0), also where the table holds
+    another stage's memory under a scanned stage's key (the reference's key collisions, forced here)."""
+    g, plain = make_model(golden_dir, case, backend)
+    _, ahead = make_model(golden_dir, case, backend)
+    try:
+        plain.look_ahead = 0
+        assert ahead.look_ahead > 0
+        for m in (plain, ahead):
+            m.settings.memory_limit = g["memory_limit"] * 0.6                # most stages must recompute
+        plans = [p for p in g["plans"] if len(p["num_ops_in_each_stage"]) > 1][:3]
+        recomputing = 0
+        for pi, p in enumerate(plans):
+            cfg_a, cfg_b = cfg_of(g, plain, p), cfg_of(g, ahead, p)
+            for stage, partner in ((0, 1), (1, 0)):
+                for metric, step in (("time_with_efficiency", 1), ("memory", 1), ("time", 3)):
+                    if pi == 1 and metric == "memory":
+                        # a collision on the way: some scanned key already holds another start
+                        st = cfg_a.stages[stage]
+                        k = max(1, len(st.ops) // 2)
+                        sl = slice(None, -k) if stage < partner else slice(k, None)
+                        key = (f"ops{st.ops[sl][0]}{len(st.ops[sl])}tp{st.tp_size[sl]}dp{st.dp_size[sl]}rc{[0] * len(st.ops[sl])}"
+                               f"algo{st.algo[sl]}bs{cfg_a.micro_bs}stage{st.num_stages_behind}")
+                        for m in (plain, ahead):
+                            m.stage_memory_set[key] = g["memory_limit"] * 0.9
+                    want = _scan_twice(plain, cfg_a, stage, partner, metric, step)
+                    got = _scan_twice(ahead, cfg_b, stage, partner, metric, step)
+                    assert got == want, (case, pi, stage, partner, metric)
+                    recomputing += sum(sum(rc) for _, _, rc in want)
+                    assert ahead.stage_memory_set == plain.stage_memory_set
+                    assert (ahead.stage_memory_visit, ahead.stage_memory_hit) == (plain.stage_memory_visit, plain.stage_memory_hit)
+        assert ahead.scan_ahead_used > 0 and plain.scan_ahead_used == 0
+        assert ahead.scan_ahead_dropped > 0                    # the forced collision was met
+        assert recomputing > 0                                 # and the limit did make stages recompute
+    finally:
+        plain.close()
+        ahead.close()
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_scans_over_op_counts_emu(golden_dir, case):
+    _scans_check(golden_dir, case, "emu")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", CASES)
+def test_scans_over_op_counts_gpu(golden_dir, case):
+    _scans_check(golden_dir, case, "gpu")

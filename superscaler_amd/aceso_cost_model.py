@@ -78,6 +78,7 @@ class CostModel:
         for i, name in enumerate(graph.ops):
             self._first_pos.setdefault(name, []).append(i)
         self._slice_cache = {}
+        self._op_types = np.asarray([self._type_index[name] for name in graph.ops], dtype=np.int64)
         # memo caches with the reference's keys and hit counters (aceso_cost_model.py:743-791)
         self.stage_memory_set, self.stage_memory_visit, self.stage_memory_hit = {}, 0, 0
         self.stage_time_set, self.stage_time_visit, self.stage_time_hit = {}, 0, 0
@@ -284,7 +285,10 @@ class CostModel:
             bidx = self._mbs_index[micro_bs]
             if not 0 <= nsb < MAX_STAGES:
                 raise ValueError("num_stages_behind outside 0..15")
-            r = (np.asarray(rc) == 1).astype(np.uint8)
+            if isinstance(rc, bytearray):                    # (check_recompute_batch's own trial states)
+                r = (np.frombuffer(rc, dtype=np.uint8) == 1).astype(np.uint8)
+            else:
+                r = (np.asarray(rc) == 1).astype(np.uint8)
             codes[p, lo:lo + n] = base | (r << 3)
             codes[p, lo] |= 1 << 4
             hdr[p, 0] = (nsb + 1) | (bidx << 8)
@@ -361,6 +365,26 @@ class CostModel:
         """aceso_cost_model.py:487-491: one raw table entry."""
         return float(self.db.tables["activations"][self._type_index[op_name], self._mbs_index[mbs],
                                                     int(math.log(tp, 2)), algo_index])
+
+    def _activation_sizes(self, ops, micro_bs, tp_size, dp_size, algo_list, factor):
+        """[get_activation_size(ops[i], micro_bs // dp_size[i], tp_size[i], algo_list[i]) * factor for every i], as Python
+        floats (the same table entries and the same product, taken with one indexing operation)."""
+        n = len(ops)
+        try:
+            lo = self._locate(ops)
+            types = self._op_types[lo:lo + n]
+        except ValueError:                      # not a slice of the model's op sequence: by name
+            types = np.fromiter((self._type_index[name] for name in ops), dtype=np.int64, count=n)
+        def mapped(values, fn):
+            # fn over a list with few distinct values
+            a = np.asarray(values, dtype=np.int64)
+            distinct = np.unique(a)
+            return np.asarray([fn(int(v)) for v in distinct], dtype=np.int64)[np.searchsorted(distinct, a)]
+
+        mbs = mapped(dp_size, lambda d: self._mbs_index[micro_bs // d])
+        tps = mapped(tp_size, lambda t: int(math.log(t, 2)))
+        algos = np.asarray(algo_list, dtype=np.int64)
+        return (self.db.tables["activations"][types, mbs, tps, algos] * float(factor)).tolist()
 
     def predict_stage_memory_helper(self, config, stage_index, ops=None, recompute_ops=None, tp_size=None,
                                     dp_size=None, base_batch_size=None, num_stages_behind=None, algo_list=None):
@@ -462,13 +486,17 @@ class CostModel:
             return (q[0], rc, q[2], q[3], q[1], q[4], q[5])
 
         def build_groups(k):
+            # (:835-848; the activation sizes are get_activation_size's table entries, looked up for the whole stage at
+            # once: this loop is the host's largest share of a check_recompute call)
             ops, micro_bs, tp_size, dp_size, nsb, algo_list = queries[k]
+            sizes = self._activation_sizes(ops, micro_bs, tp_size, dp_size, algo_list, nsb + 1)
             groups = {}
-            for index in range(len(ops)):
-                g = groups.setdefault(ops[index], {"index": [], "activation_size": [], "recomputed": False, "sum_size": 0})
+            for index, name in enumerate(ops):
+                g = groups.get(name)
+                if g is None:
+                    g = groups[name] = {"index": [], "activation_size": [], "recomputed": False, "sum_size": 0}
+                sz = sizes[index]
                 g["index"].append(index)
-                sz = self.get_activation_size(ops[index], micro_bs // dp_size[index], tp_size[index],
-                                              algo_list[index]) * (nsb + 1)
                 g["activation_size"].append(sz)
                 g["sum_size"] += sz
             return groups
@@ -478,12 +506,12 @@ class CostModel:
             (recompute lists, group lengths)."""
             ops = queries[k][0]
             trial = {name: dict(g) for name, g in groups.items()}
-            cur, states, chain, gain = list(rcs[k]), [], [], 0.0
+            cur, states, chain, gain = bytearray(rcs[k]), [], [], 0.0
             while True:
                 idx, sizes = self._next_recompute_op_group(ops, trial, math.inf)
                 if idx is None:
                     break
-                cur = list(cur)
+                cur = bytearray(cur)
                 self._mark_recompute(cur, idx)
                 chain.append(len(idx))
                 states.append(cur)
@@ -533,7 +561,7 @@ class CostModel:
             launch, plan = [], {}
             for k in pending:
                 st = state[k]
-                states = [list(rcs[k])] if st["stale"] else []       # a prefix round: its own state is not evaluated yet
+                states = [bytearray(rcs[k])] if st["stale"] else []  # a prefix round: its own state is not evaluated yet
                 more, chain = chain_of(k, st["groups"], st["mem"] - limit, st["stale"])
                 plan[k] = (len(launch), chain, int(st["stale"]))
                 launch.extend(query(k, rc) for rc in states + more)
@@ -680,7 +708,7 @@ class CostModel:
         if scan is None:
             if len(self._scans) >= self._SCANS_KEPT:
                 del self._scans[next(iter(self._scans))]
-            self._scans[key] = {"last": num_ops_moved, "window": 0, "ahead": {}}
+            self._scans[key] = {"last": num_ops_moved, "window": 0, "ahead": {}, "dropped": False}
             return None
         if num_ops_moved <= 0:
             scan["last"] = num_ops_moved
@@ -689,7 +717,7 @@ class CostModel:
         if entry is None:
             step = num_ops_moved - scan["last"]
             scan["last"] = num_ops_moved
-            if not 0 < step <= 8:
+            if not 0 < step <= 8 or scan["dropped"]:
                 scan["window"] = 0
                 return None
             scan["window"] = min(max(4, 2 * scan["window"]), self.look_ahead)
@@ -703,7 +731,10 @@ class CostModel:
         if memo_key is not None and self.reference_memo:
             known = self.stage_memory_set.get(memo_key)
             if known is not None and known != start:
-                self.scan_ahead_dropped += 1      # check_recompute would start elsewhere (see check_recompute_batch)
+                # check_recompute would start elsewhere (see check_recompute_batch); the keys of a scan's other op counts
+                # tend to be taken likewise: nothing more is evaluated ahead for this stage
+                self.scan_ahead_dropped += 1
+                scan["dropped"] = True
                 return None
             self.stage_memory_visit += 1
             if known is not None:

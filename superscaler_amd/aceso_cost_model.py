@@ -721,7 +721,13 @@ class CostModel:
                 scan["window"] = 0
                 return None
             scan["window"] = min(max(4, 2 * scan["window"]), self.look_ahead)
-            self._scan_ahead(scan, st, micro_bs, to_the_right, num_ops_moved, step, on_time)
+            try:
+                self._scan_ahead(scan, st, micro_bs, to_the_right, num_ops_moved, step, on_time)
+            except Exception:
+                # whatever a later op count's stage raises belongs to the call that asks for it (if one ever does): this
+                # call takes the ordinary path, and so do the rest of the scan's
+                scan["dropped"] = True
+                return None
             entry = scan["ahead"].get(num_ops_moved)
             if entry is None:
                 return None

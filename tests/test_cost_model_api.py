@@ -652,3 +652,19 @@ def test_scans_over_op_counts_emu(golden_dir, case):
 @pytest.mark.parametrize("case", CASES)
 def test_scans_over_op_counts_gpu(golden_dir, case):
     _scans_check(golden_dir, case, "gpu")
+
+
+def test_a_failing_evaluation_ahead_leaves_the_call_to_the_ordinary_path(golden_dir, monkeypatch):
+    """Whatever evaluating later op counts raises must not surface in the call that only asked for an earlier one."""
+    g, plain = make_model(golden_dir, "gpt_1_3B", "emu")
+    _, ahead = make_model(golden_dir, "gpt_1_3B", "emu")
+    plain.look_ahead = 0
+
+    def boom(*a, **k):
+        raise KeyError("a later op count's stage")
+    monkeypatch.setattr(ahead, "_scan_ahead", boom)
+    p = [p for p in g["plans"] if len(p["num_ops_in_each_stage"]) > 1][0]
+    want = _scan_twice(plain, cfg_of(g, plain, p), 0, 1, "time")
+    got = _scan_twice(ahead, cfg_of(g, ahead, p), 0, 1, "time")
+    assert got == want and ahead.scan_ahead_used == 0
+    assert ahead.stage_memory_set == plain.stage_memory_set

@@ -3,7 +3,7 @@
 
 Run in the build container only (it needs /root/reference):
 
-    python tests/golden/make_golden.py [base] [variants] [moves] [grid] [initial] [main] [trace] [sweep] [kat] [big]
+    python tests/golden/make_golden.py [base] [variants] [moves] [grid] [initial] [main] [reports] [trace] [sweep] [kat] [big]
 
 (no argument: every part but `big`, the search comparison on GPT-13B with 32 GPUs, which takes a quarter of an hour).
 
@@ -855,6 +855,106 @@ def child_binding_grid(case, num_saved=4):
     print(f"[golden] gen_megatron_plan over the binding {case}: {sorted(files)} -- {'identical' if files == ref_files else 'DIFFERENT'}")
 
 
+def child_reports(case):
+    """The search's reporting helpers (aceso_utils.py:776-829, :254-260, :852-927) on the recorded plans of
+    <case>.json (their time and memory lists as the reference's cost model left them): the plan summary line and the
+    recompute / algo listings, the result block of print_search_details with the three CSV files it writes, and
+    save_and_print_top_configs on result tables with ties, empty and non-positive entries: printed text, file texts and
+    the plan files copied, into reports_<case>.json."""
+    import contextlib
+    import io
+    import tempfile
+    model, size, db, mbs_list, nodes, gpn, gbs, limit, num_layers = CASES[case]
+    extra = ["--num-layers", str(num_layers)] if num_layers else []
+    sys.argv = reference_argv(case, extra)
+    sys.path.insert(0, os.path.join(REF, "search"))
+    import aceso_utils as U                # noqa: the reference, imported to record its outputs
+    from model_ops_info import get_full_op_list
+    args = U.parse_args()
+    ops = get_full_op_list(args)
+    with open(os.path.join(HERE, f"{case}.json")) as f:
+        recorded = json.load(f)
+    rng = random.Random(0xACE53)
+    out = {"case": case, "summaries": [], "details": [], "top": []}
+
+    def files_under(root):
+        got = {}
+        for d, _, names in os.walk(root):
+            for n in names:
+                with open(os.path.join(d, n), newline="") as f:
+                    got[os.path.relpath(os.path.join(d, n), root)] = f.read()
+        return got
+
+    def config_of(p):
+        c = U.get_config(p["num_ops_in_each_stage"], p["tp"], p["dp"], p["recompute_ops"], p["micro_batch_size"], gbs, ops,
+                         p["algo"])
+        c.time_list, c.memory_list = list(p["time_list"]), list(p["memory_list"])
+        return c
+
+    for k, p in enumerate(recorded["plans"][:6]):
+        c = config_of(p)
+        c.history = "earlier line\n" if k % 2 else ""
+        buf = io.StringIO()
+        with contextlib.redirect_stdout(buf):
+            U.print_simple_config_info(c, info=f"trial {k}", add_history=bool(k % 3), print_recompute_ops=k < 3,
+                                       print_debug_info=k != 4)
+        out["summaries"].append({"plan": k, "info": f"trial {k}", "add_history": bool(k % 3), "print_recompute_ops": k < 3,
+                                 "print_debug_info": k != 4, "history_before": "earlier line\n" if k % 2 else "",
+                                 "stdout": buf.getvalue(), "history_after": c.history})
+    for k, p in enumerate(recorded["plans"][:3] + [None]):
+        tmp = tempfile.mkdtemp()
+        for d in ("csv", "trends"):
+            os.makedirs(os.path.join(tmp, d))
+        args.config_save_path = args.log_path = tmp + "/"
+        args.config_suffix, args.print_recompute_ops, args.initial_point, args.max_num_hops = f"sfx{k}", k == 1, "balance", 7
+        c = None if p is None else config_of(p)
+        if c is not None:
+            c.history = f"history of plan {k}\n"
+        trials = k + 2
+        search_times = [rng.random() * 9 for _ in range(trials)]
+        config_times = [rng.random() * 5000 for _ in range(trials)]
+        targets, hops = [rng.randrange(9) for _ in range(4)], [rng.randrange(9) for _ in range(7)]
+        reserved = [] if p is None else list(p["reserved_memory_list"])
+        num_stages = 3 if p is None else len(p["num_ops_in_each_stage"])
+        buf = io.StringIO()
+        with contextlib.redirect_stdout(buf):
+            U.print_search_details(c, args, num_stages, targets, hops, search_times, config_times, reserved, 1234 + k)
+        out["details"].append({"plan": None if p is None else k, "suffix": f"sfx{k}", "print_recompute_ops": k == 1,
+                               "num_stages": num_stages, "targets": targets, "hops": hops, "search_times": search_times,
+                               "config_times": config_times, "reserved": reserved, "explored": 1234 + k,
+                               "stdout": buf.getvalue(), "files": files_under(tmp)})
+        shutil.rmtree(tmp, ignore_errors=True)
+    tables = [
+        ({1: (5000.0, 9000.4, 10, 1.0, []), 2: (4000.0, 8000.5, 20, 2.0, []), 3: (4000.0, 7000.0, 30, 3.0, []),
+          4: (6000.0, 1.0, 40, 4.0, [])}, 1, 4, 3, [1, 2, 3, 4]),
+        ({1: None, 2: (0.0, 1.0, 2, 1.0, []), 3: (-5.0, 1.0, 3, 1.0, []), 5: (7000.25, 11000.5, 4, 1.0, [])}, 1, 6, 4, [5]),
+        ({2: (3000.0, 100.0, 1, 1.0, []), 3: (2999.999, 100.6, 2, 1.0, []), 4: (float(2 ** 30), 1.0, 3, 1.0, []),
+          5: (3000.0, 99.5, 4, 1.0, [])}, 2, 5, 1, [2, 3]),
+        ({}, 1, 3, 2, []),
+        ({1: (100.0, 1.0, 1, 1.0, []), 2: (90.0, 2.0, 2, 1.0, []), 3: (80.0, 3.0, 3, 1.0, [])}, 2, 3, 5, [2]),
+    ]
+    for k, (results, start, end, saved, with_files) in enumerate(tables):
+        tmp = tempfile.mkdtemp()
+        os.makedirs(os.path.join(tmp, "top_configs"))
+        args.config_save_path, args.config_suffix = tmp + "/", f"run{k}"
+        args.start_num_stages, args.end_num_stages, args.num_of_saved_configs = start, end, saved
+        for n in with_files:
+            with open(os.path.join(tmp, f"{model}_{size}_{n}stages_run{k}.json"), "w") as f:
+                f.write(f"plan file of {n} stages")
+        buf = io.StringIO()
+        with contextlib.redirect_stdout(buf):
+            U.save_and_print_top_configs(results, args)
+        out["top"].append({"results": {str(n): (None if r is None else list(r)) for n, r in results.items()},
+                           "start": start, "end": end, "saved": saved, "with_files": with_files, "suffix": f"run{k}",
+                           "stdout": buf.getvalue(), "copied": sorted(os.listdir(os.path.join(tmp, "top_configs")))})
+        shutil.rmtree(tmp, ignore_errors=True)
+    out["format_size_list"] = [[x, U.format_size_list(x)] for x in ([[1, 1], [2, 4, 2]], [[8]], [], [[0, 1], [1, 1], [4, 2]])]
+    with open(os.path.join(HERE, f"reports_{case}.json"), "w") as f:
+        json.dump(out, f)
+    print(f"[golden] search reports {case}: {len(out['summaries'])} summaries, {len(out['details'])} result blocks, "
+          f"{len(out['top'])} rankings")
+
+
 def main():
     if len(sys.argv) > 2 and sys.argv[1] == "--child":
         return child(sys.argv[2])
@@ -866,15 +966,17 @@ def main():
         return child_initial(sys.argv[2])
     if len(sys.argv) > 2 and sys.argv[1] == "--child-search-results":
         return child_search_results(sys.argv[2])
+    if len(sys.argv) > 2 and sys.argv[1] == "--child-reports":
+        return child_reports(sys.argv[2])
     if len(sys.argv) > 2 and sys.argv[1] == "--child-binding-grid":
         return child_binding_grid(sys.argv[2])
     if len(sys.argv) > 2 and sys.argv[1] == "--child-binding-search":
         return child_binding_search(sys.argv[2])
     if len(sys.argv) > 2 and sys.argv[1] == "--child-search-trace":
         return child_search_trace(sys.argv[2], extras=len(sys.argv) > 3 and sys.argv[3] == "extras")
-    # optional arguments: the parts to (re)write, of base variants moves grid initial main trace sweep kat; none = all
+    # optional arguments: the parts to (re)write, of base variants moves grid initial main reports trace sweep kat; none = all
     # (the long search comparison, search_binding_<case>__long.json, is made by hand: see child_binding_search)
-    parts = set(sys.argv[1:]) or {"base", "variants", "moves", "grid", "initial", "main", "trace", "sweep", "kat"}
+    parts = set(sys.argv[1:]) or {"base", "variants", "moves", "grid", "initial", "main", "reports", "trace", "sweep", "kat"}
     quiet = subprocess.DEVNULL if os.environ.get("GOLDEN_QUIET") else None
     me = os.path.abspath(__file__)
     for case in CASES:
@@ -897,6 +999,8 @@ def main():
             subprocess.run([sys.executable, me, "--child-initial", case], check=True, stdout=quiet)
         if "main" in parts:
             run_main(case)
+        if "reports" in parts:
+            subprocess.run([sys.executable, me, "--child-reports", case], check=True, stdout=quiet)
     for case in CASES:
         if "trace" in parts:
             subprocess.run([sys.executable, me, "--child-search-trace", case], check=True, stdout=quiet)

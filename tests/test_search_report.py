@@ -1,0 +1,118 @@
+"""The search's reporting helpers (superscaler_amd/search_report.py) against what the reference's own printed and wrote
+(tests/golden/reports_<case>.json, written by tests/golden/make_golden.py, child_reports, from
+search/aceso_utils.py:776-829, :254-260, :852-927): plan summary lines and histories, the result block of a stage count with
+its three CSV files, and the final ranking of the stage counts (stable on equal times; empty, non-positive and
+out-of-range entries) with the plan files it copies."""
+import contextlib
+import io
+import json
+import os
+import types
+
+import pytest
+
+from superscaler_amd import opgraph as og
+from superscaler_amd import search_report as sr
+from superscaler_amd.plan import get_config
+
+CASES = ["gpt_1_3B", "resnet_500M", "t5_770M"]
+
+
+def load(golden_dir, case):
+    with open(os.path.join(golden_dir, f"reports_{case}.json")) as f:
+        fx = json.load(f)
+    with open(os.path.join(golden_dir, f"{case}.json")) as f:
+        g = json.load(f)
+    return fx, g
+
+
+def op_list(golden_dir, case, g):
+    from superscaler_amd.profile_db import CostModelSettings, ProfileDB
+    st = CostModelSettings(model_name=g["model_name"], micro_batch_size=g["micro_batch_size"],
+                           num_gpus_per_node=g["num_gpus_per_node"], global_batch_size=g["global_batch_size"],
+                           memory_limit=g["memory_limit"])
+    db = ProfileDB.from_directory(g["model_name"], g["model_size"], os.path.join(golden_dir, f"db_{case}") + "/", st)
+    return og.OpGraph.build(g["model_name"], db.op_names, g["num_layers"]).ops
+
+
+def config_of(g, ops, p):
+    c = get_config(p["num_ops_in_each_stage"], p["tp"], p["dp"], p["recompute_ops"], p["micro_batch_size"],
+                   g["global_batch_size"], ops, p["algo"])
+    c.time_list, c.memory_list = list(p["time_list"]), list(p["memory_list"])
+    return c
+
+
+def files_under(root):
+    got = {}
+    for d, _, names in os.walk(root):
+        for n in names:
+            with open(os.path.join(d, n), newline="") as f:
+                got[os.path.relpath(os.path.join(d, n), root)] = f.read()
+    return got
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_plan_summaries(golden_dir, case):
+    fx, g = load(golden_dir, case)
+    ops = op_list(golden_dir, case, g)
+    assert len(fx["summaries"]) == 6
+    for rec in fx["summaries"]:
+        c = config_of(g, ops, g["plans"][rec["plan"]])
+        c.history = rec["history_before"]
+        buf = io.StringIO()
+        with contextlib.redirect_stdout(buf):
+            sr.print_simple_config_info(c, info=rec["info"], add_history=rec["add_history"],
+                                        print_recompute_ops=rec["print_recompute_ops"], print_debug_info=rec["print_debug_info"])
+        assert buf.getvalue() == rec["stdout"], rec["plan"]
+        assert c.history == rec["history_after"]
+    for sizes, text in fx["format_size_list"]:
+        assert sr.format_size_list(sizes) == text
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_result_blocks_and_their_files(golden_dir, case, tmp_path):
+    fx, g = load(golden_dir, case)
+    ops = op_list(golden_dir, case, g)
+    assert [d["plan"] for d in fx["details"]] == [0, 1, 2, None]
+    for k, rec in enumerate(fx["details"]):
+        root = tmp_path / f"run{k}"
+        for d in ("csv", "trends"):
+            os.makedirs(root / d)
+        args = types.SimpleNamespace(model_name=g["model_name"], model_size=g["model_size"], config_save_path=f"{root}/",
+                                     log_path=f"{root}/", config_suffix=rec["suffix"], initial_point="balance",
+                                     max_num_hops=7, print_recompute_ops=rec["print_recompute_ops"])
+        c = None
+        if rec["plan"] is not None:
+            c = config_of(g, ops, g["plans"][rec["plan"]])
+            c.history = f"history of plan {rec['plan']}\n"
+        buf = io.StringIO()
+        with contextlib.redirect_stdout(buf):
+            sr.print_search_details(c, args, rec["num_stages"], rec["targets"], rec["hops"], rec["search_times"],
+                                    rec["config_times"], rec["reserved"], rec["explored"])
+        assert buf.getvalue() == rec["stdout"], k
+        assert files_under(root) == rec["files"], k
+        assert len(rec["files"]) == (3 if c is not None else 1)
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_ranking_of_the_stage_counts(golden_dir, case, tmp_path):
+    fx, g = load(golden_dir, case)
+    assert len(fx["top"]) == 5
+    for k, rec in enumerate(fx["top"]):
+        root = tmp_path / f"top{k}"
+        os.makedirs(root / "top_configs")
+        for n in rec["with_files"]:
+            (root / f"{g['model_name']}_{g['model_size']}_{n}stages_{rec['suffix']}.json").write_text(f"plan file of {n} stages")
+        args = types.SimpleNamespace(model_name=g["model_name"], model_size=g["model_size"], config_save_path=f"{root}/",
+                                     config_suffix=rec["suffix"], start_num_stages=rec["start"], end_num_stages=rec["end"],
+                                     num_of_saved_configs=rec["saved"], global_batch_size=g["global_batch_size"])
+        results = {int(n): (None if r is None else tuple(r)) for n, r in rec["results"].items()}
+        buf = io.StringIO()
+        with contextlib.redirect_stdout(buf):
+            sr.save_and_print_top_configs(results, args)
+        assert buf.getvalue() == rec["stdout"], k
+        assert sorted(os.listdir(root / "top_configs")) == rec["copied"], k
+    # equal times keep the order in which the stage counts were met; a time at the sentinel value is never ranked
+    ties = {2: (3000.0, 1.0, 1, 1.0, []), 3: (2999.999, 1.0, 1, 1.0, []), 4: (float(2 ** 30), 1.0, 1, 1.0, []), 5: (3000.0, 1.0, 1, 1.0, [])}
+    assert sr.rank_stage_counts(ties, 2, 5) == [3, 2, 5]
+    assert sr.rank_stage_counts(ties, 3, 4) == [3]

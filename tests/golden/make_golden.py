@@ -763,11 +763,8 @@ def child_binding_search(case):
             self.__dict__["_emu"] = EmuEvaluator(self.tables)
         return self.__dict__["_emu"]
     gpu.CostModel.evaluator = property(emu_of)
-    spec = importlib.util.spec_from_file_location("aceso_cost_model", os.path.join(root, "superscaler_amd", "binding",
-                                                                                   "aceso_cost_model.py"))
-    mod = importlib.util.module_from_spec(spec)
-    sys.modules["aceso_cost_model"] = mod          # what aceso_search / aceso_prims import
-    spec.loader.exec_module(mod)
+    from superscaler_amd.run_reference import install_binding
+    install_binding(os.path.join(REF, "search"))   # registers what aceso_search / aceso_prims import
     with contextlib.redirect_stdout(io.StringIO()):
         import aceso_search as S                   # noqa: the reference's search, unchanged
         found = {}
@@ -824,11 +821,8 @@ def child_binding_grid(case, num_saved=4):
             self.__dict__["_emu"] = EmuEvaluator(self.tables)
         return self.__dict__["_emu"]
     gpu.CostModel.evaluator = property(emu_of)
-    spec = importlib.util.spec_from_file_location("aceso_cost_model", os.path.join(root, "superscaler_amd", "binding",
-                                                                                   "aceso_cost_model.py"))
-    mod = importlib.util.module_from_spec(spec)
-    sys.modules["aceso_cost_model"] = mod
-    spec.loader.exec_module(mod)
+    from superscaler_amd.run_reference import install_binding
+    install_binding(os.path.join(REF, "search"))
     cwd = os.getcwd()
     os.chdir(tmp)
     try:

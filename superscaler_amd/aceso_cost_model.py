@@ -689,6 +689,38 @@ class CostModel:
 
     _SCANS_KEPT = 16
 
+    def _scan_entry(self, key, count, evaluate):
+        """The scan with this key and what was evaluated ahead for op count `count`: (scan, entry), entry None when the
+        call is to take the ordinary path.  `evaluate(scan, step)` fills scan["ahead"] for `scan["window"]` op counts
+        from `count` on, `step` apart; it is called when `count` continues the scan and is not there yet."""
+        scan = self._scans.get(key)
+        if scan is None:
+            if len(self._scans) >= self._SCANS_KEPT:
+                del self._scans[next(iter(self._scans))]
+            self._scans[key] = {"last": count, "window": 0, "ahead": {}, "dropped": False}
+            return None, None
+        if count <= 0:
+            scan["last"] = count
+            return scan, None
+        entry = scan["ahead"].get(count)
+        if entry is not None:
+            scan["last"] = count
+            return scan, entry
+        step = count - scan["last"]
+        scan["last"] = count
+        if not 0 < step <= 8 or scan["dropped"]:
+            scan["window"] = 0
+            return scan, None
+        scan["window"] = min(max(4, 2 * scan["window"]), self.look_ahead)
+        try:
+            evaluate(scan, step)
+        except Exception:
+            # whatever a later op count's stage raises belongs to the call that asks for it (if one ever does): this
+            # call takes the ordinary path, and so do the rest of the scan's
+            scan["dropped"] = True
+            return scan, None
+        return scan, scan["ahead"].get(count)
+
     def _scan_step(self, st, micro_bs, to_the_right, num_ops_moved, metric):
         """predict_value_after_move(..., num_ops_moved, metric) from a result evaluated ahead: (value, recompute list),
         or None when the call is to take the ordinary path."""
@@ -704,35 +736,10 @@ class CostModel:
                    to_the_right, on_time, a.memory_limit, a.flex_recompute, a.peak_mem_in_backward)
         except (ValueError, TypeError):           # a size beyond a byte: not worth a second encoding
             return None
-        scan = self._scans.get(key)
-        if scan is None:
-            if len(self._scans) >= self._SCANS_KEPT:
-                del self._scans[next(iter(self._scans))]
-            self._scans[key] = {"last": num_ops_moved, "window": 0, "ahead": {}, "dropped": False}
-            return None
-        if num_ops_moved <= 0:
-            scan["last"] = num_ops_moved
-            return None
-        entry = scan["ahead"].get(num_ops_moved)
+        scan, entry = self._scan_entry(key, num_ops_moved,
+                                       lambda sc, step: self._scan_ahead(sc, st, micro_bs, to_the_right, num_ops_moved, step, on_time))
         if entry is None:
-            step = num_ops_moved - scan["last"]
-            scan["last"] = num_ops_moved
-            if not 0 < step <= 8 or scan["dropped"]:
-                scan["window"] = 0
-                return None
-            scan["window"] = min(max(4, 2 * scan["window"]), self.look_ahead)
-            try:
-                self._scan_ahead(scan, st, micro_bs, to_the_right, num_ops_moved, step, on_time)
-            except Exception:
-                # whatever a later op count's stage raises belongs to the call that asks for it (if one ever does): this
-                # call takes the ordinary path, and so do the rest of the scan's
-                scan["dropped"] = True
-                return None
-            entry = scan["ahead"].get(num_ops_moved)
-            if entry is None:
-                return None
-        else:
-            scan["last"] = num_ops_moved
+            return None
         rc, value, memo_key, start = entry
         if memo_key is not None and self.reference_memo:
             known = self.stage_memory_set.get(memo_key)
@@ -776,6 +783,40 @@ class CostModel:
             scan["ahead"][k] = (bytes(rcs[j]), value, starts[j][0], starts[j][1])
         self.scan_ahead_evaluated += len(counts)
 
+    def _delta_scan_step(self, config, st, longest_stage, right, num_ops_moved, decrease):
+        """wrap_predict_delta_time from a result evaluated ahead (the op migration asks for 1, 2, 3, ... moved ops of one
+        stage in turn when --predict-delta-time is on, aceso_prims.py:174-177), or None for the ordinary path."""
+        try:
+            nb = None
+            if not decrease:
+                other = config.stages[longest_stage + 1] if right else config.stages[longest_stage - 1]
+                nb = (other.tp_size[0], other.dp_size[0]) if right else (other.tp_size[-1], other.dp_size[-1])
+            key = ("delta", tuple(st.ops), bytes(st.recompute_ops), bytes(st.tp_size), bytes(st.dp_size), bytes(st.algo),
+                   config.micro_bs, right, decrease, nb)
+        except (ValueError, TypeError, IndexError):
+            return None
+
+        def evaluate(scan, step):
+            n = len(st.ops)
+            counts = [k for k in range(num_ops_moved, num_ops_moved + step * scan["window"], step) if k < n]
+            queries = []
+            for k in counts:
+                sl = slice(n - k, None) if right else slice(0, k)
+                if decrease:
+                    rc, tp, dp = list(st.recompute_ops[sl]), st.tp_size[sl], st.dp_size[sl]
+                else:
+                    rc, tp, dp = [0] * k, [nb[0]] * k, [nb[1]] * k
+                queries.append((st.ops[sl], rc, tp, dp, config.micro_bs, 0, st.algo[sl]))
+            rec = self._stage_records(queries)
+            for j, k in enumerate(counts):
+                scan["ahead"][k] = self._stage_time_of(rec[j].tolist(), delta=True, on_the_right=right, decrease=decrease)
+            self.scan_ahead_evaluated += len(counts)
+
+        scan, value = self._scan_entry(key, num_ops_moved, evaluate)
+        if value is not None:
+            self.scan_ahead_used += 1
+        return value
+
     def wrap_predict_delta_time(self, config, longest_stage, shortest_stage, num_ops_moved, decrease=True):
         """aceso_cost_model.py:885-922."""
         st = config.stages[longest_stage]
@@ -783,6 +824,10 @@ class CostModel:
         if longest_stage == shortest_stage:
             raise RuntimeError("")
         right = longest_stage < shortest_stage
+        if self.look_ahead > 0 and 0 < num_ops_moved < num_ops:
+            ahead = self._delta_scan_step(config, st, longest_stage, right, num_ops_moved, decrease)
+            if ahead is not None:
+                return ahead
         sl = slice(num_ops - num_ops_moved, None) if right else slice(0, num_ops_moved)
         ops, algo_list = st.ops[sl], st.algo[sl]
         if decrease:

@@ -633,6 +633,13 @@ def _scans_check(golden_dir, case, backend):
                     got = _scan_twice(ahead, cfg_b, stage, partner, metric, step)
                     assert got == want, (case, pi, stage, partner, metric)
                     recomputing += sum(sum(rc) for _, _, rc in want)
+                # the same scan with --predict-delta-time (aceso_prims.py:174-177): wrap_predict_delta_time per op count
+                for decrease in (True, False):
+                    for step in (1, 2):
+                        counts = list(range(0, len(cfg_a.stages[stage].ops), step)) * 2
+                        want_d = [plain.wrap_predict_delta_time(cfg_a, stage, partner, k, decrease) for k in counts]
+                        got_d = [ahead.wrap_predict_delta_time(cfg_b, stage, partner, k, decrease) for k in counts]
+                        assert got_d == want_d, (case, pi, stage, partner, decrease, step)
                     assert ahead.stage_memory_set == plain.stage_memory_set
                     assert (ahead.stage_memory_visit, ahead.stage_memory_hit) == (plain.stage_memory_visit, plain.stage_memory_hit)
         assert ahead.scan_ahead_used > 0 and plain.scan_ahead_used == 0

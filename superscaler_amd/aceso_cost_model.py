@@ -252,8 +252,54 @@ class CostModel:
     def _stage_records(self, queries) -> np.ndarray:
         """One GPU launch for single-stage queries [(ops, recompute_ops, tp, dp, micro_bs, num_stages_behind, algo)];
         returns the stage records [len(queries), STAGE_REC].  Cross-node flags are off, as in
-        predict_stage_time (aceso_cost_model.py:494-495)."""
-        tb = self.tables
+        predict_stage_time (aceso_cost_model.py:494-495).
+
+        Records already computed for the same stage (same op range, per-op lists and micro-batch size) are reused: the
+        search asks about the stage it has just run check_recompute on, and about the same stages again and again.  The
+        table is keyed by the query's lists as bytes, so a query that is in it costs no encoding either.  The number of
+        stages behind is not part of the key: it enters only the record's total-memory field, which nothing on the host
+        reads (cleared below where it would be another stage count's)."""
+        P = len(queries)
+        cache = self._record_cache
+        if len(cache) > self._record_cache_max:
+            cache.clear()            # (before the look-ups below: what this call hits must still be there when it is read)
+        keys, los, todo, first = [], [], [], {}
+        for p, (ops, rc, tp, dp, micro_bs, nsb, algo) in enumerate(queries):
+            n = len(ops)
+            if n == 0:
+                raise ValueError("empty stage")
+            if not 0 <= nsb < MAX_STAGES:
+                raise ValueError("num_stages_behind outside 0..15")
+            lo = self._locate(ops)
+            try:
+                key = (lo, n, micro_bs, bytes(tp), bytes(dp), bytes(algo), bytes(rc))
+            except (ValueError, TypeError):          # an entry that is no small integer: evaluated, not kept
+                key = ("unkeyed", p)
+            keys.append(key)
+            los.append(lo)
+            if key not in cache and key not in first:        # (equal queries inside one call are evaluated once)
+                first[key] = p
+                todo.append(p)
+        if todo:
+            codes, hdr, ranges = self._encode_stage_queries([queries[p] for p in todo], [los[p] for p in todo])
+            it, pk, fe, st, rec = self.evaluator.score_host(PlanBatch(codes, hdr), breakdown=True, ranges=ranges)
+            self._raise_for_status(st)
+            for j, p in enumerate(todo):
+                cache[keys[p]] = (rec[j, 0, :].copy(), queries[p][5] + 1)
+        out = np.empty((P, STAGE_REC), dtype=np.float64)
+        for p in range(P):
+            r, stages = cache[keys[p]]
+            out[p] = r
+            if stages != queries[p][5] + 1:
+                out[p, R_STAGE_MB] = math.nan
+        for key in first:
+            if key[0] == "unkeyed":
+                del cache[key]
+        return out
+
+    def _encode_stage_queries(self, queries, los):
+        """Codes, headers and op ranges of single-stage queries as the ranged kernel reads them; `los`: where each
+        query's op list starts in the model's op sequence."""
         N, A = self.graph.num_ops, self.db.n_algo
         tp_index = {t: k for k, t in enumerate(self.db.tp_list)}
         P = len(queries)
@@ -264,12 +310,9 @@ class CostModel:
         # checked and encoded once)
         shared = {}
         for p, (ops, rc, tp, dp, micro_bs, nsb, algo) in enumerate(queries):
-            n = len(ops)
-            if n == 0:
-                raise ValueError("empty stage")
+            n, lo = len(ops), los[p]
             who = (id(ops), id(tp), id(dp), id(algo), micro_bs)
             if who not in shared:
-                lo = self._locate(ops)
                 dp_a = np.asarray(dp, dtype=np.int64)
                 tp_a = np.asarray(tp, dtype=np.int64)
                 for d in set(dp_a.tolist()):
@@ -280,12 +323,10 @@ class CostModel:
                 for x in set(tp_a.tolist()):
                     tp_index[x]                              # KeyError for a tp size that was not profiled
                 t = self._tp_lut[tp_a]
-                shared[who] = (lo, g, t * A + np.asarray(algo, dtype=np.uint8))
-            lo, g, base = shared[who]
+                shared[who] = (g, t * A + np.asarray(algo, dtype=np.uint8))
+            g, base = shared[who]
             bidx = self._mbs_index[micro_bs]
-            if not 0 <= nsb < MAX_STAGES:
-                raise ValueError("num_stages_behind outside 0..15")
-            if isinstance(rc, bytearray):                    # (check_recompute_batch's own trial states)
+            if isinstance(rc, (bytes, bytearray)):           # (check_recompute_batch's own trial states)
                 r = (np.frombuffer(rc, dtype=np.uint8) == 1).astype(np.uint8)
             else:
                 r = (np.asarray(rc) == 1).astype(np.uint8)
@@ -294,34 +335,7 @@ class CostModel:
             hdr[p, 0] = (nsb + 1) | (bidx << 8)
             hdr[p, 1] = g.bit_length() - 1
             ranges[p] = (lo, lo + n)
-        # Records already computed for the same stage (same op range, per-op codes, micro-batch size and stage size) are
-        # reused: the search asks about the stage it has just run check_recompute on, and about the same stages again
-        # and again.  The number of stages behind is not part of the key: it enters only the record's total-memory
-        # field, which nothing on the host reads (cleared below where it would be another stage count's).
-        keys = [(int(ranges[p, 0]), int(hdr[p, 0]) >> 8, int(hdr[p, 1]), codes[p, ranges[p, 0]:ranges[p, 1]].tobytes())
-                for p in range(P)]
-        cache = self._record_cache
-        if len(cache) > self._record_cache_max:
-            cache.clear()            # (before the look-ups below: what this call hits must still be there when it is read)
-        out = np.empty((P, STAGE_REC), dtype=np.float64)
-        miss = [p for p in range(P) if keys[p] not in cache]
-        if miss:
-            # (equal queries inside one call are evaluated once)
-            first = {}
-            for p in miss:
-                first.setdefault(keys[p], p)
-            todo = sorted(first.values())
-            it, pk, fe, st, rec = self.evaluator.score_host(PlanBatch(codes[todo], hdr[todo]), breakdown=True,
-                                                            ranges=ranges[todo])
-            self._raise_for_status(st)
-            for j, p in enumerate(todo):
-                cache[keys[p]] = (rec[j, 0, :].copy(), int(hdr[p, 0]) & 0xff)
-        for p in range(P):
-            r, stages = cache[keys[p]]
-            out[p] = r
-            if stages != (int(hdr[p, 0]) & 0xff):
-                out[p, R_STAGE_MB] = math.nan
-        return out
+        return codes, hdr, ranges
 
     def predict_stage_time(self, ops, recompute_ops, tp_size, dp_size, base_batch_size, algo_list,
                            delta=False, on_the_right=False, decrease=True):

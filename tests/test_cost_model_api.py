@@ -577,7 +577,7 @@ def test_value_after_gpu_move_matches_reference_gpu(golden_dir, case):
 
 
 def test_record_cache_survives_its_own_eviction(golden_dir):
-    """Single-stage records are kept by their kernel inputs and the table is emptied when it has grown too large: a call
+    """Single-stage records are kept by their queries' lists and the table is emptied when it has grown too large: a call
     some of whose queries are in the table and some not must get all its records also when the table is emptied on that
     call (the emptying once happened between the look-up and the read: KeyError in a long search)."""
     g, m = make_model(golden_dir, "resnet_500M", "emu")

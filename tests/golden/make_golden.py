@@ -943,6 +943,18 @@ def child_reports(case):
                            "stdout": buf.getvalue(), "copied": sorted(os.listdir(os.path.join(tmp, "top_configs")))})
         shutil.rmtree(tmp, ignore_errors=True)
     out["format_size_list"] = [[x, U.format_size_list(x)] for x in ([[1, 1], [2, 4, 2]], [[8]], [], [[0, 1], [1, 1], [4, 2]])]
+    # config_details as the visited sets key on it (aceso_utils.py:117-135), and check_legality (:760-774) on stage
+    # sizes around the node boundaries
+    import types
+    out["config_details"] = [U.config_details(config_of(p), get_string=True) for p in recorded["plans"][:3]]
+    out["legality"] = []
+    for _ in range(200):
+        n_stages = rng.randrange(1, 7)
+        gpus = [rng.choice([1, 1, 2, 2, 4, 4, 8, 8, 3, 16]) for _ in range(n_stages)]
+        cfg = types.SimpleNamespace(num_stages=n_stages, stages=[types.SimpleNamespace(num_gpus=g) for g in gpus])
+        args.num_nodes, args.num_gpus_per_node = rng.choice([1, 2, 4]), rng.choice([2, 4, 8])
+        args.num_gpus = rng.choice([sum(gpus), sum(gpus), args.num_nodes * args.num_gpus_per_node])
+        out["legality"].append([gpus, args.num_gpus, args.num_gpus_per_node, args.num_nodes, U.check_legality(cfg, args)])
     with open(os.path.join(HERE, f"reports_{case}.json"), "w") as f:
         json.dump(out, f)
     print(f"[golden] search reports {case}: {len(out['summaries'])} summaries, {len(out['details'])} result blocks, "

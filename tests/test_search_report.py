@@ -67,6 +67,15 @@ def test_plan_summaries(golden_dir, case):
         assert c.history == rec["history_after"]
     for sizes, text in fx["format_size_list"]:
         assert sr.format_size_list(sizes) == text
+    from superscaler_amd.plan import check_legality, config_details
+    for p, text in zip(g["plans"], fx["config_details"]):
+        assert config_details(config_of(g, ops, p), get_string=True) == text
+    verdicts = set()
+    for gpus, num_gpus, per_node, nodes, legal in fx["legality"]:
+        cfg = types.SimpleNamespace(num_stages=len(gpus), stages=[types.SimpleNamespace(num_gpus=n) for n in gpus])
+        assert check_legality(cfg, num_gpus, per_node, nodes) == legal, (gpus, num_gpus, per_node, nodes)
+        verdicts.add(legal)
+    assert verdicts == {True, False} and len(fx["legality"]) == 200
 
 
 @pytest.mark.parametrize("case", CASES)

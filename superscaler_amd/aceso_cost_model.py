@@ -728,7 +728,7 @@ class CostModel:
         scan["window"] = min(max(4, 2 * scan["window"]), self.look_ahead)
         try:
             evaluate(scan, step)
-        except (KeyError, ValueError, TypeError, IndexError, RuntimeError):
+        except (KeyError, ValueError, TypeError, IndexError, RuntimeError, ArithmeticError):
             # whatever a later op count's stage raises belongs to the call that asks for it (if one ever does): this
             # call takes the ordinary path, and so do the rest of the scan's
             scan["dropped"] = True

@@ -600,6 +600,7 @@ struct ace_handle {
     // device copies
     double *d_rows;
     uint32_t *d_pos_info;
+    ace_u4 *d_pos4;            // per position, for the assembly op loop (null when the rows are windowed)
     uint8_t *d_pair_kinds;
     uint32_t *d_stage_lut;
     double *d_nbm1;
@@ -682,6 +683,29 @@ template <bool BD, bool RANGED, bool WIN, bool DEFER> static int allow_big_lds()
         ACE_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&ace_score_kernel<BD, RANGED, WIN, false, kBlock, true>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
     return ACE_OK;
+}
+
+// Per op position, what the assembly form of the op loop (ace_score_loop_asm.inc) reads with scalar loads: the LDS
+// address of the position's row at its hot sub-table and at its collective-cost tables, the LDS address of the
+// pair-kind block of the (this op, next op) pair, and two flags (bit 0: the rule "ordinary op followed by a layer
+// start" does NOT apply here, bit 1: ordinary op).  Positions past the last op point at row 0 and pair kind 0.
+static int upload_pos4(ace_handle *h, const ace_tables_t *t, size_t pos_entries, uint32_t rk_off) {
+    h->d_pos4 = nullptr;
+    if (t->n_windows != 1) return ACE_OK;
+    ace_u4 *p4 = new (std::nothrow) ace_u4[pos_entries];
+    if (!p4) return ACE_ENOMEM;
+    const uint32_t row_bytes = (uint32_t)t->row_doubles * 8u, kind_stride = (uint32_t)t->n_glog * 64u;
+    for (size_t i = 0; i < pos_entries; ++i) {
+        const uint32_t info = i < (size_t)t->num_ops ? t->pos_info[i] : 0u;
+        const uint32_t row = (info & 0xffu) * row_bytes;
+        p4[i].x = row + (uint32_t)t->hot_off * 8u;
+        p4[i].y = row + (uint32_t)t->z_off * 8u;
+        p4[i].z = rk_off + ((info >> 16) & 0xffu) * kind_stride;
+        p4[i].w = (((info >> 24) & 1u) ^ 1u) | (((info >> 25) & 1u) << 1);
+    }
+    const int rc = upload((void **)&h->d_pos4, p4, pos_entries * sizeof(ace_u4));
+    delete[] p4;
+    return rc;
 }
 
 // The device address of `scratch` on the current device (looked up once per device).
@@ -787,6 +811,7 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
         (rc = static_scratch_ptr(&scratch_here)) ||
         (rc = upload((void **)&h->d_rows, t->rows, (size_t)t->num_types * row_bytes)) ||
         (rc = upload((void **)&h->d_pos_info, t->pos_info, (size_t)(t->num_ops + 1) * 4, pos_entries * 4)) ||
+        (rc = upload_pos4(h, t, pos_entries, rk_off)) ||
         (rc = upload((void **)&h->d_pair_kinds, t->pair_kinds, (size_t)rk_bytes)) ||
         (rc = upload((void **)&h->d_stage_lut, t->stage_lut, (size_t)stg_words * 4)) ||
         (rc = upload((void **)&h->d_nbm1, t->nb_minus_1, (size_t)t->n_mbs * 8)) ||
@@ -809,6 +834,7 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
 void ace_destroy(ace_handle_t *h) {
     if (!h) return;
     (void)hipFree(h->d_rows); (void)hipFree(h->d_pos_info); (void)hipFree(h->d_pair_kinds);
+    if (h->d_pos4) (void)hipFree(h->d_pos4);
     (void)hipFree(h->d_stage_lut); (void)hipFree(h->d_nbm1); (void)hipFree(h->d_win_pos);
     (void)hipFree(h->d_win_row_begin); (void)hipFree(h->d_win_rows);
     if (h->d_stage_ws) (void)hipFree(h->d_stage_ws);
@@ -830,7 +856,7 @@ static int fill_args(ace_handle_t *h, const ace_batch_t *b, double memory_limit,
     a->hdr = reinterpret_cast<const ace_u4 *>(b->d_hdr);
     a->range = reinterpret_cast<const ace_u2 *>(b->d_range);
     a->order = b->d_order;
-    a->rows = h->d_rows; a->pos_info = h->d_pos_info; a->pair_kinds = h->d_pair_kinds; a->stage_lut = h->d_stage_lut;
+    a->rows = h->d_rows; a->pos_info = h->d_pos_info; a->pos4 = h->d_pos4; a->pair_kinds = h->d_pair_kinds; a->stage_lut = h->d_stage_lut;
     a->nbm1 = h->d_nbm1; a->win_pos = h->d_win_pos; a->win_row_begin = h->d_win_row_begin; a->win_rows = h->d_win_rows;
     a->n_windows = h->n_windows; a->row_doubles = h->row_doubles; a->rk_bytes = h->rk_bytes; a->stg_words = h->stg_words;
     a->iter_ms = d_iter_ms; a->peak_mb = d_peak_mb; a->feasible = d_feasible; a->status = d_status; a->stage_out = d_stage_out;

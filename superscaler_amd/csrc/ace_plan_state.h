@@ -222,13 +222,7 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false> struct Pl
         if (!DEFER) {
             // one LUT read per possible stage now, none where a stage begins (where few lanes are active)
             uint64_t rks = 0;
-            for (uint32_t k = 0; k < ACE_MAX_STAGES; ++k) {
-                uint32_t glog = (uint32_t)(glogs >> (4u * k)) & 15u;
-                uint32_t w = lds.ld<uint32_t>(g.stg_lds_off + (bidx * 16u + glog) * 4u);
-                diags |= (uint64_t)(w & 15u) << (4u * k);
-                // the stage size as the pair-kind tables index it (a size outside the tables is unscorable anyway: block 0)
-                rks |= (uint64_t)(glog < (uint32_t)g.n_glog ? glog : 0u) << (4u * k);
-            }
+            stage_nibbles(g, lds, diags, rks);
             rewind(rks);
         }
         if (BD) {
@@ -237,6 +231,18 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false> struct Pl
             uint32_t d = lds.ld<uint32_t>(g.stg_lds_off + (bidx * 16u + 0u) * 4u) & 15u;
             ideal_hot_v = ace_mul24(d, (uint32_t)g.C * ACE_HOT_STRIDE);
             ideal_start_v = ace_mul24(d, (uint32_t)g.C * ACE_START_STRIDE);
+        }
+    }
+
+    // Per stage, four bits each (stage 0 lowest): the diag of the stage's (micro-batch, stage size) pair, and the stage
+    // size as the pair-kind tables index it (a size outside the tables is unscorable anyway: block 0).
+    ACE_HD void stage_nibbles(const AceGeom &g, const AceLds &lds, uint64_t &dg, uint64_t &rks) const {
+        dg = 0; rks = 0;
+        for (uint32_t k = 0; k < ACE_MAX_STAGES; ++k) {
+            uint32_t glog = (uint32_t)(glogs >> (4u * k)) & 15u;
+            uint32_t w = lds.ld<uint32_t>(g.stg_lds_off + (bidx * 16u + glog) * 4u);
+            dg |= (uint64_t)(w & 15u) << (4u * k);
+            rks |= (uint64_t)(glog < (uint32_t)g.n_glog ? glog : 0u) << (4u * k);
         }
     }
 
@@ -308,7 +314,8 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false> struct Pl
         const double coll = COLL ? mc : 0.0;
         if (g.flags & ACE_F_NO_RESERVED) return 0.0;
         if (g.flags & ACE_F_RESERVED_MIN) return ace_max(ace_max(rfm, rbm), ace_max(W, coll));
-        return ace_max(rfm + rbm, W) + coll;
+        // (the sum below is never -0.0, so adding the reference's integer 0 would change nothing)
+        return COLL ? ace_max(rfm + rbm, W) + coll : ace_max(rfm + rbm, W);
     }
 
     // DEFER: park the finished stage in the plan's workspace slot `s`: ten values in five 16-byte
@@ -493,7 +500,7 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false> struct Pl
     }
 
     ACE_HD void result(const AceGeom &g, double nbm1, double &iter_ms, double &peak_mb, uint8_t &feasible, uint8_t &st) {
-        if (!RANGED && s != S) status = ACE_PLAN_MALFORMED;   // every stage end also opened the next stage
+        if (!RANGED && (s != S || S > ACE_MAX_STAGES)) status = ACE_PLAN_MALFORMED;   // every stage end also opened the next stage
         // max over stages of t_s*(nb-1) + sum(t): rounding is monotonic, so the maximum is attained
         // at the largest t_s and equals this expression bit for bit
         iter_ms = max_t * nbm1 + sum_t;

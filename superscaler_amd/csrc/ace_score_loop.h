@@ -13,6 +13,10 @@
 #define ACE_ANY(x) __any(x)
 #endif
 
+#ifndef ACE_HOST_EMU
+#include "ace_score_loop_asm.inc"
+#endif
+
 struct AceKernelArgs {
     AceGeom g;
     const ace_u4 *codes;        // [G][P] 16 op bytes each
@@ -21,6 +25,8 @@ struct AceKernelArgs {
     const uint32_t *order;      // [P] result index of the plan in each slot, or null (slot i -> result i)
     const double *rows;         // [n_types][row_doubles]
     const uint32_t *pos_info;   // [N + 1], padded to 16 * G + 16 entries
+    const ace_u4 *pos4;         // [16 * G + 16] per position: LDS address of its row's hot sub-table, of its cost tables, of the
+                                //   pair-kind block of the (this, next) pair; bit 0: no layer start follows an ordinary op here, bit 1: ordinary op
     const uint8_t *pair_kinds;  // -> LDS
     const uint32_t *stage_lut;  // -> LDS
     const double *nbm1;         // [n_mbs]
@@ -45,6 +51,37 @@ template <int BLOCK> ACE_HD void stage_window(const AceKernelArgs &a, unsigned c
         for (int j = tid; j < n16; j += BLOCK) dst[j] = src[j];
     }
 }
+
+#ifndef ACE_HOST_EMU
+// The op loop of the plain scoring kernel in gfx950 assembly (ace_score_loop_asm.inc; written by
+// gen_score_loop_asm.py, which describes it): walks all ops of this lane's plan, parks every finished stage in the
+// lane's workspace records like PlanState::stash(), and returns the number of stages closed.  LDS addresses in `pos4`
+// are absolute: the caller checks that the workgroup's LDS array starts at address 0.
+__device__ __forceinline__ uint32_t ace_score_loop_asm(const AceKernelArgs &a, const AceGeom &g, uint64_t dg, uint64_t rks,
+                                                       uint32_t code_off, double *rec, uint32_t ws_stride) {
+    uint32_t cnt;
+    const uint64_t gstride = (uint64_t)(uint32_t)g.P * 16u;
+    const uint32_t gs_lo = (uint32_t)gstride, gs_hi = (uint32_t)(gstride >> 32);
+    const uint32_t c8 = (uint32_t)g.C * 8u;
+#define ACE_LOOP_ASM_RUN(TEXT)                                                                                          \
+    asm volatile(TEXT : [cnt] "=&v"(cnt)                                                                               \
+                 : [dg] "v"(dg), [rk] "v"(rks), [codeoff] "v"(code_off), [rec] "v"(rec), [codes] "s"(a.codes),         \
+                   [pos] "s"(a.pos4), [c8] "s"(c8), [zshift] "s"(g.z_shift), [n_ops] "s"(g.N), [n_groups] "s"(g.G),     \
+                   [gstride_lo] "s"(gs_lo), [gstride_hi] "s"(gs_hi), [wsstride] "s"(ws_stride)                          \
+                 : ACE_LOOP_ASM_CLOBBERS)
+    if (g.flags & ACE_F_RESHARDING) {
+        if (g.flags & ACE_F_NO_RESERVED) ACE_LOOP_ASM_RUN(ACE_LOOP_ASM_RSH1_NONE);
+        else if (g.flags & ACE_F_RESERVED_MIN) ACE_LOOP_ASM_RUN(ACE_LOOP_ASM_RSH1_MIN);
+        else ACE_LOOP_ASM_RUN(ACE_LOOP_ASM_RSH1_MAX);
+    } else {
+        if (g.flags & ACE_F_NO_RESERVED) ACE_LOOP_ASM_RUN(ACE_LOOP_ASM_RSH0_NONE);
+        else if (g.flags & ACE_F_RESERVED_MIN) ACE_LOOP_ASM_RUN(ACE_LOOP_ASM_RSH0_MIN);
+        else ACE_LOOP_ASM_RUN(ACE_LOOP_ASM_RSH0_MAX);
+    }
+#undef ACE_LOOP_ASM_RUN
+    return cnt;
+}
+#endif
 
 // BD: also write per-stage records.  RANGED: each plan is one stage over an op sub-range.
 // WIN: the rows of all op types do not fit in LDS together; restage at window boundaries.
@@ -160,6 +197,16 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     int w = w0 + 1;
     int next_win = WIN ? a.win_pos[w] : 0x7fffffff;
     ace_u4 cw = a.codes[(size_t)grp_begin * g.P + pl];     // sixteen op bytes of this plan
+#ifndef ACE_HOST_EMU
+    if (DEFER && lds_base == 0u && a.pos4) {
+        // the assembly form of the loop below (same operations per plan, same results)
+        if (!(cw.x & 0x10u)) st.status = ACE_PLAN_MALFORMED;    // the first op must open a stage
+        uint64_t dg, rks;
+        st.stage_nibbles(g, lds, dg, rks);
+        st.s = (int)ace_score_loop_asm(a, g, dg, rks, (uint32_t)pl * 16u, rec, st.ws_stride);
+        grp_end = grp_begin;
+    } else
+#endif
     if (!RANGED) st.begin(g, lds, 0, cw.x & 0xffu, a.pos_info[0]);
     uint32_t pinfo = grp_begin ? a.pos_info[(grp_begin << 4) - 1] : 0u;    // descriptor of the previous group's last position
     for (int grp = grp_begin; grp < grp_end; ++grp) {

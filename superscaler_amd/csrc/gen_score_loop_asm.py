@@ -1,0 +1,374 @@
+"""Writes ace_score_loop_asm.inc: the op loop of the plain scoring kernel (deferred stage tails) as gfx950 assembly.
+
+    python3 superscaler_amd/csrc/gen_score_loop_asm.py
+
+The loop is the one ace_score_body() runs in C++ (ace_score_loop.h, PlanState::step / stash / start_fast of
+ace_plan_state.h, DEFER variant), written out by hand so that
+  * the 0/1 factors of the recompute rules become execution masks: the recompute bit, the recompute-pair bit and
+    the stage-start bit of an op are tested with one byte-select compare each, and the conditional additions run
+    under the resulting lane mask (an addition that does not happen and an addition of +0.0 give the same bits);
+  * the table reads of op k+1 are issued before op k's values are used (two alternating register sets);
+  * every position-dependent address comes ready-made from a per-position table (four words per op position,
+    read with scalar loads one 4-op word ahead) instead of being derived per op.
+Floating-point operations and their order per plan are exactly those of the C++ loop, so results are bit-identical.
+
+One text per (resharding on / off, reserved-memory rule); each is a C string literal macro that ace_score_loop.h
+pastes into an asm statement.  Register use: v28-v127 and s24-s99 belong to the loop; operands live below.
+"""
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+# ---- vector registers ---------------------------------------------------------------------------------------
+FB, RCS = "v[32:33]", "v[34:35]"            # quad v[32:35]: stash record 0 = {fwd + bwd, recompute sum}
+RSF, RSB = "v[36:37]", "v[38:39]"           # quad v[36:39]: record 1 = {resharding fwd, bwd}
+W_, A_ = "v[40:41]", "v[42:43]"             # quad v[40:43]: record 2 = {weights, activations}
+SAVED, PKT = "v[44:45]", "v[46:47]"         # quad v[44:47]: record 3 = {saved, closed peak}
+RES, META = "v[48:49]", "v[50:51]"          # quad v[48:51]: record 4 = {reserved term, meta}
+FWD, BWD, RUN, PEAK = "v[52:53]", "v[54:55]", "v[56:57]", "v[58:59]"
+RFM = ["v[60:61]", "v[64:65]"]              # reserved maxima, alternating between consecutive ops
+RBM = ["v[62:63]", "v[66:67]"]
+
+
+def E(x):                                   # hot entry of an op: {fwd, bwd} {weights, act} {reserved fwd, bwd}
+    b = 68 + 12 * x
+    return dict(q0=f"v[{b}:{b+3}]", q1=f"v[{b+4}:{b+7}]", q2=f"v[{b+8}:{b+11}]", fwd=f"v[{b}:{b+1}]",
+                bwd=f"v[{b+2}:{b+3}]", w=f"v[{b+4}:{b+5}]", act=f"v[{b+6}:{b+7}]", rf=f"v[{b+8}:{b+9}]",
+                rb=f"v[{b+10}:{b+11}]")
+
+
+def ZV(x):                                  # collective costs of an op's input: forward, backward
+    b = 92 + 4 * x
+    return f"v[{b}:{b+1}]", f"v[{b+2}:{b+3}]"
+
+
+def R(x):                                   # collective ids of an op pair (byte from the pair table)
+    return f"v{100 + x}"
+
+
+WORD = [f"v{102 + j}" for j in range(4)]    # code words of the current 16-op group
+NEXT = [f"v{106 + j}" for j in range(4)]    # ... of the next group
+
+
+def D(y):                                   # per 4-op word: next-op bytes, code*8, code*8+next code, rc bit, pair bit
+    b = 110 + 5 * y
+    return dict(nw=f"v{b}", w8=f"v{b+1}", cn=f"v{b+2}", r8=f"v{b+3}", p8=f"v{b+4}")
+
+
+ZV_, RK, WSOFF, WSOFF64, FMETA, CNT = "v120", "v121", "v122", "v[122:123]", "v124", "v125"   # (v123 stays zero)
+DG, DG_LO, RKS, RKS_LO = "v[28:29]", "v28", "v[30:31]", "v30"   # per stage, 4 bits each, next stage lowest: diag; pair-table block
+T0, T1, T01, T2 = "v126", "v127", "v[126:127]", "v33"
+
+# ---- scalar registers ---------------------------------------------------------------------------------------
+ALL = "s[24:25]"
+CPTR, CPTR_LO, CPTR_HI = "s[26:27]", "s26", "s27"
+GRP, K07, K08, POSBASE, LEFT, K1F = "s30", "s39", "s40", "s41", "s31", "s38"
+PPTR, PPTR_LO, PPTR_HI = "s[36:37]", "s36", "s37"
+M_RC, M_P, M_ST, M_KP = "s[42:43]", "s[44:45]", "s[46:47]", "s[48:49]"
+ORD, ORD_LO, ORD_HI = "s[50:51]", "s50", "s51"
+MASK = [f"s{52 + j}" for j in range(4)]
+PLANT = [f"s{56 + j}" for j in range(4)]
+PREVFL = "s62"
+S0, S1, S2, S23 = "s96", "s97", "s98", "s[98:99]"
+
+
+def P(y, q):                                # position entry q of the word in buffer y: hot, z, pair-table address, flags
+    b = 64 + 16 * y + 4 * q
+    return dict(hot=f"s{b}", z=f"s{b+1}", pk=f"s{b+2}", fl=f"s{b+3}")
+
+
+def PBUF(y):
+    return f"s[{64 + 16 * y}:{79 + 16 * y}]"
+
+
+class Gen:
+    def __init__(self, rsh, mode):
+        self.rsh, self.mode, self.lines = rsh, mode, []
+
+    def o(self, s):
+        self.lines.append(s)
+
+    def c(self, s):
+        self.lines.append("; " + s)
+
+    # -- pieces ------------------------------------------------------------------------------------------------
+    def prep(self, y, wa, wb):
+        d = D(y)
+        self.c(f"word-level: next-op bytes, code*8, code*8+next code, recompute bit, recompute-pair bit (buffer {y})")
+        self.o(f"v_alignbit_b32 {d['nw']}, {wb}, {wa}, 8")
+        self.o(f"v_and_b32 {d['w8']}, {K07}, {wa}")
+        self.o(f"v_lshlrev_b32 {d['w8']}, 3, {d['w8']}")
+        self.o(f"v_and_or_b32 {d['cn']}, {d['nw']}, {K07}, {d['w8']}")
+        self.o(f"v_and_b32 {d['r8']}, {K08}, {wa}")
+        self.o(f"v_lshrrev_b32 {d['p8']}, 1, {d['nw']}")
+        self.o(f"v_bitop3_b32 {d['p8']}, {d['r8']}, {d['nw']}, {d['p8']} bitop3:0x40")
+
+    def stage_start(self):
+        """z_v and the pair-table block of the stage that begins: the next nibbles of the packed per-stage lists."""
+        self.o(f"v_and_b32 {T0}, 15, {DG_LO}")
+        self.o(f"v_mul_u32_u24 {ZV_}, {T0}, %[c8]")
+        self.o(f"v_lshrrev_b64 {DG}, 4, {DG}")
+        self.o(f"v_and_b32 {T0}, 15, {RKS_LO}")
+        self.o(f"v_lshlrev_b32 {RK}, 6, {T0}")
+        self.o(f"v_lshrrev_b64 {RKS}, 4, {RKS}")
+
+    def issue(self, k1):
+        """Address arithmetic and LDS reads of op k1 (0..16; 16 = first op of the next group)."""
+        j1, b1 = k1 >> 2, k1 & 3
+        y1, x1 = j1 & 1, k1 & 1
+        d, p, e = D(y1), P(y1, b1), E(x1)
+        sel = f"dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_{b1}"
+        self.c(f"op {k1}: table reads")
+        self.o(f"v_add_u32_sdwa {T0}, {ZV_}, {d['w8']} {sel}")
+        self.o(f"v_mad_u32_u24 {T1}, {T0}, 6, {p['hot']}")
+        self.o(f"ds_read_b128 {e['q0']}, {T1}")
+        self.o(f"ds_read_b128 {e['q1']}, {T1} offset:16")
+        self.o(f"ds_read_b128 {e['q2']}, {T1} offset:32")
+        if not self.rsh:
+            return
+        self.o(f"v_add_u32_sdwa {T1}, {RK}, {d['cn']} {sel}")
+        self.o(f"v_add_u32_e32 {T1}, {p['pk']}, {T1}")
+        self.o(f"ds_read_u8 {R(1 - x1)}, {T1}")            # ids of the (k1, k1 + 1) pair
+        self.o(f"v_add_u32_e32 {T0}, {p['z']}, {T0}")
+        self.o("s_waitcnt lgkmcnt(4)")                       # the ids of the (k1 - 1, k1) pair are in
+        zf, zb = ZV(x1)
+        self.o(f"v_and_b32 {T1}, 15, {R(x1)}")
+        self.o(f"v_lshrrev_b32 {T2}, 4, {R(x1)}")
+        self.o(f"v_lshl_add_u32 {T1}, {T1}, %[zshift], {T0}")
+        self.o(f"v_lshl_add_u32 {T2}, {T2}, %[zshift], {T0}")
+        self.o(f"ds_read_b64 {zf}, {T1}")
+        self.o(f"ds_read_b64 {zb}, {T2}")
+
+    def reserved(self, cur):
+        if self.mode == "max":          # max(rf + rb, W)
+            self.o(f"v_add_f64 {RES}, {RFM[cur]}, {RBM[cur]}")
+            self.o(f"v_max_f64 {RES}, {RES}, {W_}")
+        elif self.mode == "min":        # max(max(rf, rb), max(W, 0))
+            self.o(f"v_max_f64 {RES}, {RFM[cur]}, {RBM[cur]}")
+            self.o(f"v_max_f64 {T01}, {W_}, 0")
+            self.o(f"v_max_f64 {RES}, {RES}, {T01}")
+        else:
+            self.o(f"v_mov_b64 {RES}, 0")
+
+    def slot(self, k):
+        j, b = k >> 2, k & 3
+        y, x, x1 = j & 1, k & 1, (k + 1) & 1
+        d, p, e = D(y), P(y, b), E(x)
+        cur, nxt = k & 1, (k + 1) & 1          # reserved maxima: read `cur`, write `nxt`
+        L = f"{k}_%="
+        self.c(f"================ op {k} of the group")
+        if b == 0:
+            self.c("position entries of the next word")
+            self.o(f"s_load_dwordx16 {PBUF((j + 1) & 1)}, {PPTR}, {64 * (j + 1)}")
+        if b == 2:
+            self.o("s_waitcnt lgkmcnt(0)")
+        if k == 11:
+            self.next_group_words()
+        if b == 3:
+            if j < 3:
+                self.prep((j + 1) & 1, WORD[j + 1], WORD[j + 2] if j + 2 < 4 else NEXT[0])
+            else:
+                self.prep(0, NEXT[0], NEXT[1])
+        sel = f"src0_sel:BYTE_{b} src1_sel:DWORD"
+        self.o(f"v_cmp_ne_u32_sdwa {M_RC}, {d['r8']}, 0 {sel}")
+        self.o(f"v_cmp_ne_u32_sdwa {M_P}, {d['p8']}, 0 {sel}")
+        self.o(f"v_cmp_gt_u32_sdwa {M_ST}, {d['nw']}, 15 {sel}")
+        self.o(f"s_cmp_lg_u64 {M_ST}, 0")
+        self.o(f"s_cbranch_scc0 L_ns_{L}")
+        self.c("lanes whose next op opens a stage: that stage's table offsets; its first op pays no resharding")
+        self.o(f"s_mov_b64 exec, {M_ST}")
+        self.stage_start()
+        if self.rsh:
+            self.o("s_waitcnt lgkmcnt(2)")
+            self.o(f"v_mov_b32 {R(x1)}, 0")
+        self.o(f"s_mov_b64 exec, {ALL}")
+        self.o(f"L_ns_{L}:")
+        self.issue(k + 1)
+        if not self.rsh:
+            self.o("s_waitcnt lgkmcnt(3)")
+        self.c(f"op {k}: sums")
+        zf, zb = ZV(x)
+        self.o(f"v_add_f64 {FWD}, {FWD}, {e['fwd']}")
+        self.o(f"v_add_f64 {BWD}, {BWD}, {e['bwd']}")
+        self.o(f"v_add_f64 {W_}, {W_}, {e['w']}")
+        self.o(f"v_add_f64 {A_}, {A_}, {e['act']}")
+        if self.rsh:
+            self.o(f"v_add_f64 {RSF}, {RSF}, {zf}")
+            self.o(f"v_add_f64 {RSB}, {RSB}, {zb}")
+        self.o(f"v_max_f64 {RFM[nxt]}, {RFM[cur]}, {e['rf']}")
+        self.o(f"v_max_f64 {RBM[nxt]}, {RBM[cur]}, {e['rb']}")
+        self.o(f"s_mov_b64 exec, {M_RC}")
+        self.o(f"v_add_f64 {RCS}, {RCS}, {e['fwd']}")
+        self.o(f"s_cbranch_scc0 L_ne_{L}")
+        self.c("lanes whose stage ends with this op: park the stage's values, start the next stage from zero")
+        self.o(f"s_mov_b64 exec, {M_ST}")
+        self.o(f"v_add_f64 {FB}, {FWD}, {BWD}")
+        prevfl = P(y, b - 1)["fl"] if b else PREVFL
+        self.o(f"s_bitcmp1_b32 {prevfl}, 1")
+        self.o(f"s_cselect_b32 {ORD_HI}, 0x3ff00000, 0")
+        self.o(f"v_mul_f64 {PKT}, {RUN}, {ORD}")
+        self.o(f"v_max_f64 {PKT}, {PEAK}, {PKT}")
+        self.reserved(cur)
+        wsrc = WORD[j]
+        self.o(f"v_bfe_u32 v50, {wsrc}, {8 * b}, 3")
+        self.o(f"v_lshl_or_b32 v50, v50, 19, {FMETA}")
+        self.o(f"s_add_u32 {S0}, {POSBASE}, {k}")
+        self.o(f"v_mov_b32 v51, {S0}")
+        self.o(f"v_bfe_u32 {T0}, {d['nw']}, {8 * b}, 3")
+        self.o(f"s_add_u32 {S0}, {S0}, 1")
+        self.o(f"v_lshl_or_b32 {FMETA}, {T0}, 16, {S0}")
+        self.o(f"v_cmp_gt_u32_e32 vcc, 16, {CNT}")
+        self.o("s_and_b64 exec, exec, vcc")
+        self.o(f"v_lshl_add_u64 {T01}, {WSOFF64}, 4, %[rec]")
+        self.o(f"global_store_dwordx4 {T01}, v[32:35], off")
+        self.o(f"global_store_dwordx4 {T01}, v[36:39], off offset:16")
+        self.o(f"global_store_dwordx4 {T01}, v[40:43], off offset:32")
+        self.o(f"global_store_dwordx4 {T01}, v[44:47], off offset:48")
+        self.o(f"global_store_dwordx4 {T01}, v[48:51], off offset:64")
+        self.o(f"v_add_u32_e32 {WSOFF}, %[wsstride], {WSOFF}")
+        self.o(f"s_mov_b64 exec, {M_ST}")
+        self.o(f"v_add_u32_e32 {CNT}, 1, {CNT}")
+        for r in (FWD, BWD, RUN, PEAK, RFM[nxt], RBM[nxt]):
+            self.o(f"v_mov_b64 {r}, 0")
+        self.o("s_nop 1")
+        for r in (RCS, RSF, RSB, W_, A_, SAVED):
+            self.o(f"v_mov_b64 {r}, 0")
+        self.o(f"L_ne_{L}:")
+        self.c("recompute pair (this op, next op): saved activations, running segment, peak")
+        self.o(f"s_bitcmp1_b32 {p['fl']}, 0")
+        self.o(f"s_cselect_b64 {M_KP}, {M_P}, 0")
+        self.o(f"s_mov_b64 exec, {M_P}")
+        self.o(f"v_add_f64 {RUN}, {RUN}, {e['act']}")
+        self.o(f"s_mov_b64 exec, {M_KP}")
+        self.o(f"v_add_f64 {SAVED}, {SAVED}, {e['act']}")
+        self.o(f"s_andn2_b64 exec, {ALL}, {M_KP}")
+        self.o(f"v_max_f64 {PEAK}, {PEAK}, {RUN}")
+        self.o(f"v_mov_b64 {RUN}, 0")
+        self.o(f"s_mov_b64 exec, {ALL}")
+        if b == 3:
+            self.o(f"s_mov_b32 {PREVFL}, {p['fl']}")
+
+    def word_masks(self, tag):
+        """MASK[j] / PLANT[j] of the four words of a group from LEFT = N - (first position of that group):
+        code bytes of positions past the last op read as zero, and the byte right after the last op gets a
+        stage-start bit, which is what ends the plan's last stage."""
+        for j in range(4):
+            self.o(f"s_sub_i32 {S0}, {LEFT}, {4 * j}")
+            self.o(f"s_min_i32 {S1}, {S0}, 4")
+            self.o(f"s_max_i32 {S1}, {S1}, 0")
+            self.o(f"s_lshl_b32 {S1}, {S1}, 3")
+            self.o(f"s_bfm_b64 {S23}, {S1}, 0")
+            self.o(f"s_and_b32 {MASK[j]}, {S2}, {K1F}")
+            self.o(f"s_lshl_b64 {S23}, 16, {S1}")
+            self.o(f"s_cmp_ge_i32 {S0}, 0")
+            self.o(f"s_cselect_b32 {PLANT[j]}, {S2}, 0")
+
+    def apply_masks(self, regs, tag):
+        self.o(f"s_cmp_ge_i32 {LEFT}, 16")
+        self.o(f"s_cbranch_scc1 L_full_{tag}_%=")
+        self.word_masks(tag)
+        for j in range(4):
+            self.o(f"v_and_b32 {regs[j]}, {MASK[j]}, {regs[j]}")
+            self.o(f"v_or_b32 {regs[j]}, {PLANT[j]}, {regs[j]}")
+        self.o(f"s_branch L_masked_{tag}_%=")
+        self.o(f"L_full_{tag}_%=:")
+        for j in range(4):
+            self.o(f"v_and_b32 {regs[j]}, {K1F}, {regs[j]}")
+        self.o(f"L_masked_{tag}_%=:")
+
+    def next_group_words(self):
+        self.c("the next group's code words have arrived (zeros after the last group): padding and end-of-plan mark")
+        self.o("s_waitcnt vmcnt(0)")
+        self.o(f"s_sub_i32 {LEFT}, %[n_ops], {POSBASE}")
+        self.o(f"s_sub_i32 {LEFT}, {LEFT}, 16")
+        self.apply_masks(NEXT, "nx")
+
+    def build(self):
+        o, c = self.o, self.c
+        c("---- set-up")
+        o(f"s_mov_b64 {ALL}, exec")
+        o(f"v_mov_b64 {DG}, %[dg]")
+        o(f"v_mov_b64 {RKS}, %[rk]")
+        o(f"s_mov_b64 {CPTR}, %[codes]")
+        o(f"s_mov_b64 {PPTR}, %[pos]")
+        o(f"s_mov_b32 {K07}, 0x07070707")
+        o(f"s_mov_b32 {K08}, 0x08080808")
+        o(f"s_mov_b32 {K1F}, 0x1f1f1f1f")
+        o(f"s_mov_b32 {ORD_LO}, 0")
+        o(f"s_mov_b32 {GRP}, 0")
+        o(f"s_mov_b32 {POSBASE}, 0")
+        o(f"s_mov_b32 {PREVFL}, 0")
+        o(f"global_load_dwordx4 v[102:105], %[codeoff], {CPTR}")
+        o(f"s_load_dwordx16 {PBUF(0)}, {PPTR}, 0")
+        for r in (FWD, BWD, RUN, PEAK, RFM[0], RBM[0], RCS, RSF, RSB, W_, A_, SAVED):
+            o(f"v_mov_b64 {r}, 0")
+        o(f"v_mov_b32 {WSOFF}, 0")
+        o("v_mov_b32 v123, 0")
+        o(f"v_mov_b32 {CNT}, 0")
+        o(f"v_mov_b32 {R(0)}, 0")
+        self.stage_start()
+        o("s_waitcnt vmcnt(0) lgkmcnt(0)")
+        o(f"s_mov_b32 {LEFT}, %[n_ops]")
+        self.apply_masks(WORD, "w0")
+        o(f"v_and_b32 {T0}, 7, {WORD[0]}")
+        o(f"v_lshlrev_b32 {FMETA}, 16, {T0}")
+        self.prep(0, WORD[0], WORD[1])
+        self.issue(0)
+        c("---- one 16-op group per iteration")
+        o("L_group_%=:")
+        o(f"s_add_u32 {S0}, {GRP}, 1")
+        o(f"s_cmp_lt_u32 {S0}, %[n_groups]")
+        o("s_cbranch_scc0 L_last_%=")
+        o(f"s_add_u32 {CPTR_LO}, {CPTR_LO}, %[gstride_lo]")
+        o(f"s_addc_u32 {CPTR_HI}, {CPTR_HI}, %[gstride_hi]")
+        o(f"global_load_dwordx4 v[106:109], %[codeoff], {CPTR}")
+        o("s_branch L_loaded_%=")
+        o("L_last_%=:")
+        for r in NEXT:
+            o(f"v_mov_b32 {r}, 0")
+        o("L_loaded_%=:")
+        for k in range(16):
+            self.slot(k)
+        c("---- next group")
+        for j in range(4):
+            o(f"v_mov_b32 {WORD[j]}, {NEXT[j]}")
+        o(f"s_add_u32 {PPTR_LO}, {PPTR_LO}, 256")
+        o(f"s_addc_u32 {PPTR_HI}, {PPTR_HI}, 0")
+        o(f"s_add_u32 {POSBASE}, {POSBASE}, 16")
+        o(f"s_add_u32 {GRP}, {GRP}, 1")
+        o(f"s_cmp_lt_u32 {GRP}, %[n_groups]")
+        o("s_cbranch_scc1 L_group_%=")
+        o("s_waitcnt vmcnt(0) lgkmcnt(0)")
+        o(f"v_mov_b32 %[cnt], {CNT}")
+        return self.lines
+
+
+def c_string(lines):
+    out = []
+    for ln in lines:
+        assert '"' not in ln and "\\" not in ln
+        out.append('    "' + ln + '\\n"')
+    return " \\\n".join(out)
+
+
+def main():
+    parts = ["// Generated by gen_score_loop_asm.py -- do not edit.  gfx950 assembly of the plain scoring kernel's op loop",
+             "// (deferred stage tails), one text per (resharding, reserved-memory rule); see the generator for the design.",
+             "#pragma once", ""]
+    for rsh in (1, 0):
+        for mode in ("max", "min", "none"):
+            g = Gen(bool(rsh), mode)
+            parts.append(f"#define ACE_LOOP_ASM_RSH{rsh}_{mode.upper()} \\")
+            parts.append(c_string(g.build()))
+            parts.append("")
+    clob = ", ".join(f'"v{i}"' for i in range(28, 128)) + ", " + ", ".join(f'"s{i}"' for i in range(24, 100) if i not in (32, 33))   # (s32 / s33 are the ABI's stack registers)
+    parts.append(f"#define ACE_LOOP_ASM_CLOBBERS {clob}, \"vcc\", \"scc\", \"memory\"")
+    parts.append("")
+    path = os.path.join(HERE, "ace_score_loop_asm.inc")
+    with open(path, "w") as f:
+        f.write("\n".join(parts))
+    print("wrote", path)
+
+
+if __name__ == "__main__":
+    main()

@@ -757,6 +757,10 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     uint32_t stg_off, lut2_off;
     const uint32_t lds_bytes = ace_lds_layout(rk_off, (uint32_t)rk_bytes, (uint32_t)stg_words, &stg_off, &lut2_off);
     if (lds_bytes > kMaxLds) return ACE_ETOOBIG;
+    // (the in-kernel sort keeps its bins and its permutation in the first 128 + 2 * kBlock bytes of LDS before the
+    // tables are staged there: tiny tables still get that much)
+    const uint32_t lds_floor = 128u + 2u * (uint32_t)kBlock;
+    const uint32_t lds_alloc = lds_bytes < lds_floor ? lds_floor : lds_bytes;
     // window tables: window starts are multiples of 4 ops; every referenced row must fit the
     // resident region; every position's row offsets must point at a row start inside it
     const int32_t n_win_rows = t->win_row_begin[t->n_windows];
@@ -803,7 +807,7 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     g.flags = t->flags; g.main_params = t->main_params; g.optimizer = t->optimizer;
     g.mem_limit = 0.0; g.strict = 0;
     h->n_windows = t->n_windows; h->row_doubles = t->row_doubles; h->rk_bytes = rk_bytes; h->stg_words = stg_words;
-    h->num_types = t->num_types; h->lds_bytes = lds_bytes;
+    h->num_types = t->num_types; h->lds_bytes = lds_alloc;
     const size_t pos_entries = (size_t)((t->num_ops + 15) / 16) * 16 + 16;
     int rc;
     double *scratch_here = nullptr;

@@ -180,7 +180,8 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false> struct Pl
     double fwd, bwd, rcs, W, A, saved, run, peak, rfm, rbm, rs_f, rs_b, mc;
     double id_fwd, id_bwd;
     bool lastclose;
-    uint32_t first_meta;        // DEFER: first op of the current stage: position | code << 16
+    uint32_t replay_first;      // DEFER: first op of the stage replay() is called for next (stages follow each other) ...
+    uint32_t replay_code;       // ... and its code (before the first call: the code of the plan's first op)
     uint64_t rk_all;            // per stage (4 bits each): the stage size as the pair-kind tables index it
     uint64_t diag_next, rk_next;   // diags / rk_all shifted down by the stages handed out so far
     uint32_t ws_stride;         // DEFER: 16-byte units between two stages of one plan in the workspace
@@ -204,7 +205,7 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false> struct Pl
         s = -1;
         sum_t = 0.0; max_t = 0.0; max_mem = 0.0;
         status = 0;
-        lastclose = false; first_meta = 0; r_next = 0; pair_prev = 0;
+        lastclose = false; replay_first = 0; replay_code = 0; r_next = 0; pair_prev = 0;
         ws_stride = ACE_WS_REC / 2;
         ws_off = 0;
         fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = rs_f = rs_b = mc = 0.0;
@@ -321,13 +322,16 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false> struct Pl
     // DEFER: park the finished stage in the plan's workspace slot `s`: ten values in five 16-byte
     // stores (a store from a lane or two costs as much as one from sixty-four, so what can be
     // folded here without a table lookup is: fwd + bwd, the closed peak segment, the reserved term).
-    ACE_HD void stash(const AceGeom &g, double *ws, uint32_t i_last, uint32_t c_last, bool prev_ordinary) {
+    ACE_HD void stash(const AceGeom &g, double *ws, uint32_t i_last, uint32_t c_last, uint32_t c_next, bool prev_ordinary) {
         if (ws == nullptr || s < 0 || s >= ACE_MAX_STAGES) return;
         // stages are stashed in order, once each: slot s of this plan is ws_off further on (a running
         // offset instead of s * ws_stride, which would be a slow 32-bit multiply per stage end)
         ace_d2 *r = reinterpret_cast<ace_d2 *>(ws) + ws_off;
         ws_off += ws_stride;
-        uint64_t meta = (uint64_t)(first_meta | (c_last << 19)) | ((uint64_t)i_last << 32);
+        // what replay() needs besides the sums: the position of the stage's last op, its code and the code of the op
+        // after it (the next stage's first): code * 8 + next code in byte (position % 4) of the low word (the other
+        // bytes are not read: the assembly form of the loop stores its whole word of such bytes)
+        uint64_t meta = ((uint64_t)i_last << 32) | (uint64_t)(((c_last << 3) | c_next) << (8u * (i_last & 3u)));
         double meta_d;
         __builtin_memcpy(&meta_d, &meta, 8);
         const double fb = fwd + bwd;                                    // the first sum of :579
@@ -339,7 +343,8 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false> struct Pl
         r[4] = ace_d2{reserved_term(g), meta_d};
     }
 
-    // DEFER: evaluate stage `s2` from its stashed record (called for s2 = 0, 1, ... in order).
+    // DEFER: evaluate stage `s2` from its stashed record (called for s2 = 0, 1, ... in order, after replay_code has
+    // been set to the code of the plan's first op).
     ACE_HD void replay(const AceGeom &g, const AceLds &lds, const uint32_t *pos_info, const double *ws, int s2) {
         const ace_d2 *r = reinterpret_cast<const ace_d2 *>(ws) + (size_t)((uint32_t)s2 * ws_stride);
         ace_d2 r0 = r[0], r1 = r[1], r2 = r[2], r3 = r[3], r4 = r[4];
@@ -352,10 +357,14 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false> struct Pl
         }
         uint64_t meta;
         __builtin_memcpy(&meta, &r4.y, 8);
-        uint32_t lo32 = (uint32_t)meta, i_last = (uint32_t)(meta >> 32);
-        uint32_t i_first = lo32 & 0xffffu, c_first = (lo32 >> 16) & 7u, c_last = (lo32 >> 19) & 7u;
+        uint32_t i_last = (uint32_t)(meta >> 32);
+        const uint32_t cc = ((uint32_t)meta >> (8u * (i_last & 3u))) & 63u;
+        uint32_t i_first = s2 == 0 ? 0u : replay_first;
+        const uint32_t c_first = replay_code & 7u, c_last = cc >> 3;
         if (i_first >= (uint32_t)g.N) i_first = 0;     // garbage only if the plan was malformed
         if (i_last >= (uint32_t)g.N) i_last = 0;
+        replay_first = i_last + 1u;
+        replay_code = cc & 7u;
         start_lookups(g, lds, info_row(g, pos_info[i_first]), c_first);
         // finish() recombines: (fb + 0) = fb; the peak is closed already; max(reserved + 0, W) = reserved
         fwd = r0.x; bwd = 0.0; rcs = r0.y; rs_f = r1.x; rs_b = r1.y; W = r2.x; A = r2.y; saved = r3.x;
@@ -408,8 +417,7 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false> struct Pl
     ACE_HD void begin(const AceGeom &g, const AceLds &lds, int i, uint32_t byte, uint32_t info) {
         if (!(byte & 0x10u)) status = ACE_PLAN_MALFORMED;    // the first op must open a stage
         start_fast(g, lds, !DEFER);
-        if (DEFER) first_meta = (uint32_t)i | ((byte & 7u) << 16);
-        else start_lookups(g, lds, info_row(g, info), byte & 7u);
+        if (!DEFER) start_lookups(g, lds, info_row(g, info), byte & 7u);
     }
 
     // One op at position i.  `byte` is its code byte, `nbyte` the next op's (0 after the last op, where `plan_end` is set instead),
@@ -466,7 +474,7 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false> struct Pl
         const bool last = RANGED ? (i + 1 == hi) : (((nbyte >> 4) & 1u) || plan_end);
         if (last) {
             // :439 "i + 1 == len(ops) - 1": the (previous, this) pair closes the last segment
-            if (DEFER) stash(g, rec, (uint32_t)i, c, (pinfo >> 25) & 1u);
+            if (DEFER) stash(g, rec, (uint32_t)i, c, nc, (pinfo >> 25) & 1u);
             else {
                 lastclose = pair_prev & (pinfo >> 25) & 1u;
                 finish(g, lds, row, c, rec);
@@ -474,8 +482,7 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false> struct Pl
             if (!RANGED) {
                 // (after the plan's last op this opens a stage that stays empty: s == S in the end)
                 start_fast(g, lds, !DEFER);
-                if (DEFER) first_meta = (uint32_t)(i + 1) | (nc << 16);
-                else if (i + 1 < g.N) start_lookups(g, lds, info_nextrow(g, info), nc);
+                if (!DEFER && i + 1 < g.N) start_lookups(g, lds, info_nextrow(g, info), nc);
             }
             // the reserved maxima run over every op but the stage's last (get_reserved_memory :453-460):
             // the stage that ended took them as they were before this op, the new one starts from zero

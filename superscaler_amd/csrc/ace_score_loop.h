@@ -58,7 +58,7 @@ template <int BLOCK> ACE_HD void stage_window(const AceKernelArgs &a, unsigned c
 // lane's workspace records like PlanState::stash(), and returns the number of stages closed.  LDS addresses in `pos4`
 // are absolute: the caller checks that the workgroup's LDS array starts at address 0.
 __device__ __forceinline__ uint32_t ace_score_loop_asm(const AceKernelArgs &a, const AceGeom &g, uint64_t dg, uint64_t rks,
-                                                       uint32_t code_off, double *rec, uint32_t ws_stride) {
+                                                       uint32_t code_off, double *rec, uint32_t ws_stride, uint32_t prio = 0) {
     uint32_t cnt;
     const uint64_t gstride = (uint64_t)(uint32_t)g.P * 16u;
     const uint32_t gs_lo = (uint32_t)gstride, gs_hi = (uint32_t)(gstride >> 32);
@@ -67,7 +67,7 @@ __device__ __forceinline__ uint32_t ace_score_loop_asm(const AceKernelArgs &a, c
     asm volatile(TEXT : [cnt] "=&v"(cnt)                                                                               \
                  : [dg] "v"(dg), [rk] "v"(rks), [codeoff] "v"(code_off), [rec] "v"(rec), [codes] "s"(a.codes),         \
                    [pos] "s"(a.pos4), [c8] "s"(c8), [zshift] "s"(g.z_shift), [n_ops] "s"(g.N), [n_groups] "s"(g.G),     \
-                   [gstride_lo] "s"(gs_lo), [gstride_hi] "s"(gs_hi), [wsstride] "s"(ws_stride)                          \
+                   [gstride_lo] "s"(gs_lo), [gstride_hi] "s"(gs_hi), [wsstride] "s"(ws_stride), [prio] "s"(prio)        \
                  : ACE_LOOP_ASM_CLOBBERS)
     if (g.flags & ACE_F_RESHARDING) {
         if (g.flags & ACE_F_NO_RESERVED) ACE_LOOP_ASM_RUN(ACE_LOOP_ASM_RSH1_NONE);
@@ -100,14 +100,17 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     g.rk_lds_off += lds_base; g.stg_lds_off += lds_base; g.lut2_lds_off += lds_base;
     const long long slot = block * BLOCK + tid;                     // this lane's place in the batch (and in the workspace)
     long long plan = slot;
+    uint32_t prio = 0;                                              // issue priority of this wavefront in the op loop
 #ifndef ACE_HOST_EMU
     if (!RANGED && BLOCK >= 128) {
         // The lanes of a wavefront walk the ops together, and every op at which one of them closes a stage takes all
         // of them through the stage-end code: so the workgroup deals its plans to its lanes by pipeline depth
         // (counting sort on the depth in the plan header, deepest first; plans of one depth in any order), and the
         // sorted wavefronts to the SIMDs in turn (wavefront w runs on SIMD w % 4) so that each SIMD gets the same
-        // mix.  Only which lane scores which plan changes: results go to the plan's own index.  (Single-stage queries
-        // are left as they come: their length, not a depth, is what would have to be sorted on.)
+        // mix.  The wavefronts with the deeper plans get the higher issue priority: they have the most instructions
+        // to issue and would otherwise be the last to finish, alone on their SIMDs.  Only which lane scores which
+        // plan changes: results go to the plan's own index.  (Single-stage queries are left as they come: their
+        // length, not a depth, is what would have to be sorted on.)
         unsigned int *cnt = reinterpret_cast<unsigned int *>(lds_raw);                  // 17 bins (nothing is staged yet)
         unsigned short *plan_of = reinterpret_cast<unsigned short *>(lds_raw + 128);     // [BLOCK]
         uint32_t depth = 0;                                                              // lanes past the batch: last
@@ -128,6 +131,10 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
         plan_of[(wave << 6) | (sorted & 63u)] = (unsigned short)tid;
         ACE_SYNC();
         plan = block * BLOCK + plan_of[tid];
+        if (BLOCK >= 1024) {
+            const uint32_t pw = (uint32_t)tid >> 6, qs = (pw & 4u) ? (pw ^ 3u) : pw;       // the sorted slice this wavefront walks
+            prio = __builtin_amdgcn_readfirstlane(3u - (qs >> 2));
+        }
         ACE_SYNC();
     }
 #endif
@@ -197,19 +204,25 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     int w = w0 + 1;
     int next_win = WIN ? a.win_pos[w] : 0x7fffffff;
     ace_u4 cw = a.codes[(size_t)grp_begin * g.P + pl];     // sixteen op bytes of this plan
+    const uint32_t first_code = cw.x & 7u;
+    int grp_stop = grp_end;
 #ifndef ACE_HOST_EMU
     if (DEFER && lds_base == 0u && a.pos4) {
         // the assembly form of the loop below (same operations per plan, same results)
         if (!(cw.x & 0x10u)) st.status = ACE_PLAN_MALFORMED;    // the first op must open a stage
         uint64_t dg, rks;
         st.stage_nibbles(g, lds, dg, rks);
-        st.s = (int)ace_score_loop_asm(a, g, dg, rks, (uint32_t)pl * 16u, rec, st.ws_stride);
-        grp_end = grp_begin;
+#ifdef PROBE_NOLOOP
+        st.s = 0;
+#else
+        st.s = (int)ace_score_loop_asm(a, g, dg, rks, (uint32_t)pl * 16u, rec, st.ws_stride, prio);
+#endif
+        grp_stop = grp_begin;
     } else
 #endif
     if (!RANGED) st.begin(g, lds, 0, cw.x & 0xffu, a.pos_info[0]);
     uint32_t pinfo = grp_begin ? a.pos_info[(grp_begin << 4) - 1] : 0u;    // descriptor of the previous group's last position
-    for (int grp = grp_begin; grp < grp_end; ++grp) {
+    for (int grp = grp_begin; grp < grp_stop; ++grp) {
         const int base = grp << 4;
         // the sixteen position descriptors of this group: scalar loads (the array is padded)
         const ace_u4 *ip = reinterpret_cast<const ace_u4 *>(a.pos_info + base);
@@ -261,6 +274,7 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     }
     if (DEFER) {
         const int n_st = st.s;
+        st.replay_code = first_code;
         for (int s2 = 0; s2 < ACE_MAX_STAGES; ++s2) {
             const bool live = s2 < n_st;
             if (!ACE_ANY(live)) break;

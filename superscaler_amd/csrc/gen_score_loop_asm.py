@@ -55,7 +55,7 @@ def D(y):                                   # per 4-op word: next-op bytes, code
     return dict(nw=f"v{b}", w8=f"v{b+1}", cn=f"v{b+2}", r8=f"v{b+3}", p8=f"v{b+4}")
 
 
-ZV_, RK, WSOFF, WSOFF64, FMETA, CNT = "v120", "v121", "v122", "v[122:123]", "v124", "v125"   # (v123 stays zero)
+ZV_, RK, WSOFF, WSOFF64, CNT = "v120", "v121", "v122", "v[122:123]", "v125"   # (v123 stays zero)
 DG, DG_LO, RKS, RKS_LO = "v[28:29]", "v28", "v[30:31]", "v30"   # per stage, 4 bits each, next stage lowest: diag; pair-table block
 T0, T1, T01, T2 = "v126", "v127", "v[126:127]", "v33"
 
@@ -209,14 +209,9 @@ class Gen:
         self.o(f"v_mul_f64 {PKT}, {RUN}, {ORD}")
         self.o(f"v_max_f64 {PKT}, {PEAK}, {PKT}")
         self.reserved(cur)
-        wsrc = WORD[j]
-        self.o(f"v_bfe_u32 v50, {wsrc}, {8 * b}, 3")
-        self.o(f"v_lshl_or_b32 v50, v50, 19, {FMETA}")
         self.o(f"s_add_u32 {S0}, {POSBASE}, {k}")
-        self.o(f"v_mov_b32 v51, {S0}")
-        self.o(f"v_bfe_u32 {T0}, {d['nw']}, {8 * b}, 3")
-        self.o(f"s_add_u32 {S0}, {S0}, 1")
-        self.o(f"v_lshl_or_b32 {FMETA}, {T0}, 16, {S0}")
+        self.o(f"v_mov_b32 v50, {d['cn']}")                  # the record's last words: code*8 + next code of this word's ops,
+        self.o(f"v_mov_b32 v51, {S0}")                       # position of the stage's last op
         self.o(f"v_cmp_gt_u32_e32 vcc, 16, {CNT}")
         self.o("s_and_b64 exec, exec, vcc")
         self.o(f"v_lshl_add_u64 {T01}, {WSOFF64}, 4, %[rec]")
@@ -228,11 +223,25 @@ class Gen:
         self.o(f"v_add_u32_e32 {WSOFF}, %[wsstride], {WSOFF}")
         self.o(f"s_mov_b64 exec, {M_ST}")
         self.o(f"v_add_u32_e32 {CNT}, 1, {CNT}")
-        for r in (FWD, BWD, RUN, PEAK, RFM[nxt], RBM[nxt]):
-            self.o(f"v_mov_b64 {r}, 0")
-        self.o("s_nop 1")
-        for r in (RCS, RSF, RSB, W_, A_, SAVED):
-            self.o(f"v_mov_b64 {r}, 0")
+        self.o(f"v_mov_b64 {RUN}, 0")
+        self.o(f"v_mov_b64 {PEAK}, 0")
+        if self.rsh and os.environ.get('ACE_ZERO_LDS') == '1':
+            # the other sums restart from the zeros of collective table 0 (LDS reads instead of vector moves); they
+            # are next used after the wait that follows the next op's table reads
+            self.o(f"v_mov_b32 {T0}, {p['z']}")
+            self.o(f"v_mov_b64 {SAVED}, 0")
+            quad = "v[60:63]" if nxt == 0 else "v[64:67]"
+            self.o(f"ds_read_b128 v[52:55], {T0}")
+            self.o(f"ds_read_b128 v[36:39], {T0}")
+            self.o(f"ds_read_b128 v[40:43], {T0}")
+            self.o(f"ds_read_b128 {quad}, {T0}")
+            self.o(f"ds_read_b64 {RCS}, {T0}")
+        else:
+            for r in (FWD, BWD, RFM[nxt], RBM[nxt]):
+                self.o(f"v_mov_b64 {r}, 0")
+            self.o("s_nop 1")
+            for r in (RCS, W_, A_, SAVED) + ((RSF, RSB) if self.rsh else ()):
+                self.o(f"v_mov_b64 {r}, 0")
         self.o(f"L_ne_{L}:")
         self.c("recompute pair (this op, next op): saved activations, running segment, peak")
         self.o(f"s_bitcmp1_b32 {p['fl']}, 0")
@@ -286,6 +295,13 @@ class Gen:
     def build(self):
         o, c = self.o, self.c
         c("---- set-up")
+        if True:
+            c("issue priority of this wavefront (the deeper its plans, the higher)")
+            for lvl in (3, 2, 1):
+                o(f"s_cmp_eq_u32 %[prio], {lvl}")
+                o(f"s_cbranch_scc0 L_np{lvl}_%=")
+                o(f"s_setprio {lvl}")
+                o(f"L_np{lvl}_%=:")
         o(f"s_mov_b64 {ALL}, exec")
         o(f"v_mov_b64 {DG}, %[dg]")
         o(f"v_mov_b64 {RKS}, %[rk]")
@@ -310,8 +326,6 @@ class Gen:
         o("s_waitcnt vmcnt(0) lgkmcnt(0)")
         o(f"s_mov_b32 {LEFT}, %[n_ops]")
         self.apply_masks(WORD, "w0")
-        o(f"v_and_b32 {T0}, 7, {WORD[0]}")
-        o(f"v_lshlrev_b32 {FMETA}, 16, {T0}")
         self.prep(0, WORD[0], WORD[1])
         self.issue(0)
         c("---- one 16-op group per iteration")
@@ -339,6 +353,7 @@ class Gen:
         o(f"s_cmp_lt_u32 {GRP}, %[n_groups]")
         o("s_cbranch_scc1 L_group_%=")
         o("s_waitcnt vmcnt(0) lgkmcnt(0)")
+        o("s_setprio 0")
         o(f"v_mov_b32 %[cnt], {CNT}")
         return self.lines
 

@@ -39,6 +39,7 @@ void score_one(const ace_tables_t *t, const AceGeom &g, std::vector<unsigned cha
     }
     if (DEFER) {
         const int n_st = s.s;
+        s.replay_code = codes[0] & 7u;
         for (int s2 = 0; s2 < n_st && s2 < ACE_MAX_STAGES; ++s2) s.replay(g, view, pos, rec, s2);
         s.s = n_st;              // replay() walks s again; result() checks the count of the op loop
     }

@@ -212,11 +212,7 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
         if (!(cw.x & 0x10u)) st.status = ACE_PLAN_MALFORMED;    // the first op must open a stage
         uint64_t dg, rks;
         st.stage_nibbles(g, lds, dg, rks);
-#ifdef PROBE_NOLOOP
-        st.s = 0;
-#else
         st.s = (int)ace_score_loop_asm(a, g, dg, rks, (uint32_t)pl * 16u, rec, st.ws_stride, prio);
-#endif
         grp_stop = grp_begin;
     } else
 #endif

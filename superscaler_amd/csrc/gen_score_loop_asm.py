@@ -225,18 +225,7 @@ class Gen:
         self.o(f"v_add_u32_e32 {CNT}, 1, {CNT}")
         self.o(f"v_mov_b64 {RUN}, 0")
         self.o(f"v_mov_b64 {PEAK}, 0")
-        if self.rsh and os.environ.get('ACE_ZERO_LDS') == '1':
-            # the other sums restart from the zeros of collective table 0 (LDS reads instead of vector moves); they
-            # are next used after the wait that follows the next op's table reads
-            self.o(f"v_mov_b32 {T0}, {p['z']}")
-            self.o(f"v_mov_b64 {SAVED}, 0")
-            quad = "v[60:63]" if nxt == 0 else "v[64:67]"
-            self.o(f"ds_read_b128 v[52:55], {T0}")
-            self.o(f"ds_read_b128 v[36:39], {T0}")
-            self.o(f"ds_read_b128 v[40:43], {T0}")
-            self.o(f"ds_read_b128 {quad}, {T0}")
-            self.o(f"ds_read_b64 {RCS}, {T0}")
-        else:
+        if True:
             for r in (FWD, BWD, RFM[nxt], RBM[nxt]):
                 self.o(f"v_mov_b64 {r}, 0")
             self.o("s_nop 1")
@@ -295,13 +284,12 @@ class Gen:
     def build(self):
         o, c = self.o, self.c
         c("---- set-up")
-        if True:
-            c("issue priority of this wavefront (the deeper its plans, the higher)")
-            for lvl in (3, 2, 1):
-                o(f"s_cmp_eq_u32 %[prio], {lvl}")
-                o(f"s_cbranch_scc0 L_np{lvl}_%=")
-                o(f"s_setprio {lvl}")
-                o(f"L_np{lvl}_%=:")
+        c("issue priority of this wavefront (the deeper its plans, the higher)")
+        for lvl in (3, 2, 1):
+            o(f"s_cmp_eq_u32 %[prio], {lvl}")
+            o(f"s_cbranch_scc0 L_np{lvl}_%=")
+            o(f"s_setprio {lvl}")
+            o(f"L_np{lvl}_%=:")
         o(f"s_mov_b64 {ALL}, exec")
         o(f"v_mov_b64 {DG}, %[dg]")
         o(f"v_mov_b64 {RKS}, %[rk]")

@@ -687,11 +687,11 @@ template <bool BD, bool RANGED, bool WIN, bool DEFER> static int allow_big_lds()
 
 // Per op position, what the assembly form of the op loop (ace_score_loop_asm.inc) reads with scalar loads: the LDS
 // address of the position's row at its hot sub-table and at its collective-cost tables, the LDS address of the
-// pair-kind block of the (this op, next op) pair, and two flags (bit 0: the rule "ordinary op followed by a layer
+// 32-bit pair-kind block of the (this op, next op) pair, and two flags (bit 0: the rule "ordinary op followed by a layer
 // start" does NOT apply here, bit 1: ordinary op).  Positions past the last op point at row 0 and pair kind 0.
-static int upload_pos4(ace_handle *h, const ace_tables_t *t, size_t pos_entries, uint32_t rk_off) {
+static int upload_pos4(ace_handle *h, const ace_tables_t *t, size_t pos_entries, uint32_t pk32_off) {
     h->d_pos4 = nullptr;
-    if (t->n_windows != 1) return ACE_OK;
+    if (t->n_windows != 1 || !pk32_off) return ACE_OK;
     ace_u4 *p4 = new (std::nothrow) ace_u4[pos_entries];
     if (!p4) return ACE_ENOMEM;
     const uint32_t row_bytes = (uint32_t)t->row_doubles * 8u, kind_stride = (uint32_t)t->n_glog * 64u;
@@ -700,7 +700,7 @@ static int upload_pos4(ace_handle *h, const ace_tables_t *t, size_t pos_entries,
         const uint32_t row = (info & 0xffu) * row_bytes;
         p4[i].x = row + (uint32_t)t->hot_off * 8u;
         p4[i].y = row + (uint32_t)t->z_off * 8u;
-        p4[i].z = rk_off + ((info >> 16) & 0xffu) * kind_stride;
+        p4[i].z = pk32_off + ((info >> 16) & 0xffu) * kind_stride * 4u;
         p4[i].w = (((info >> 24) & 1u) ^ 1u) | (((info >> 25) & 1u) << 1);
     }
     const int rc = upload((void **)&h->d_pos4, p4, pos_entries * sizeof(ace_u4));
@@ -740,7 +740,7 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     const int C = t->n_tp * t->n_algo;
     // sub-tables must lie inside a row and be 16-byte aligned
     const int64_t hot_end = (int64_t)t->hot_off + (int64_t)(t->n_diag + 1) * C * 6;
-    const int64_t start_end = (int64_t)t->start_off + (int64_t)t->n_diag * C * 4;
+    const int64_t start_end = (int64_t)t->start_off + (int64_t)t->n_diag * C * 3;
     const int64_t out_end = (int64_t)t->out_off + (int64_t)t->n_mbs * t->n_tp * t->n_algo * 2;
     if ((t->flags & ACE_F_COLLECTIVE_MEM) && !(t->flags & ACE_F_RESHARDING)) return ACE_EINVAL;
     const int64_t z_end = (int64_t)t->z_off + (int64_t)t->n_z * t->z_table_doubles * ((t->flags & ACE_F_COLLECTIVE_MEM) ? 2 : 1);
@@ -755,8 +755,19 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     const int32_t stg_words = t->n_mbs * 16;
     const uint32_t rk_off = (uint32_t)t->lds_row_bytes;
     uint32_t stg_off, lut2_off;
-    const uint32_t lds_bytes = ace_lds_layout(rk_off, (uint32_t)rk_bytes, (uint32_t)stg_words, &stg_off, &lut2_off);
+    uint32_t lds_bytes = ace_lds_layout(rk_off, (uint32_t)rk_bytes, (uint32_t)stg_words, &stg_off, &lut2_off);
     if (lds_bytes > kMaxLds) return ACE_ETOOBIG;
+    // the assembly loop's pair-kind table, where every row is resident, the table has room and its entries can hold
+    // the offsets (otherwise plain scoring takes the C++ form of the loop)
+    uint32_t pk32_off = 0;
+    if (t->n_windows == 1) {
+        uint32_t off;
+        const uint32_t end = ace_lds_pk32(lds_bytes, (uint32_t)rk_bytes, &off);
+        if (end <= kMaxLds && ((int64_t)(t->n_z > 0 ? t->n_z : 1) * t->z_table_doubles * 8) <= 65536) {
+            pk32_off = off;
+            lds_bytes = end;
+        }
+    }
     // (the in-kernel sort keeps its bins and its permutation in the first 128 + 2 * kBlock bytes of LDS before the
     // tables are staged there: tiny tables still get that much)
     const uint32_t lds_floor = 128u + 2u * (uint32_t)kBlock;
@@ -801,7 +812,7 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     g.z_shift = 3;
     while ((1 << (g.z_shift - 3)) < t->z_table_doubles) ++g.z_shift;
     g.zm_delta = (uint32_t)t->n_z << g.z_shift;
-    g.rk_lds_off = rk_off; g.stg_lds_off = stg_off; g.lut2_lds_off = lut2_off;
+    g.rk_lds_off = rk_off; g.stg_lds_off = stg_off; g.lut2_lds_off = lut2_off; g.pk32_lds_off = pk32_off;
     g.rk_kind_stride = (uint32_t)(t->n_glog * 64);
     g.row_bytes = (uint32_t)row_bytes;
     g.flags = t->flags; g.main_params = t->main_params; g.optimizer = t->optimizer;
@@ -815,7 +826,7 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
         (rc = static_scratch_ptr(&scratch_here)) ||
         (rc = upload((void **)&h->d_rows, t->rows, (size_t)t->num_types * row_bytes)) ||
         (rc = upload((void **)&h->d_pos_info, t->pos_info, (size_t)(t->num_ops + 1) * 4, pos_entries * 4)) ||
-        (rc = upload_pos4(h, t, pos_entries, rk_off)) ||
+        (rc = upload_pos4(h, t, pos_entries, pk32_off)) ||
         (rc = upload((void **)&h->d_pair_kinds, t->pair_kinds, (size_t)rk_bytes)) ||
         (rc = upload((void **)&h->d_stage_lut, t->stage_lut, (size_t)stg_words * 4)) ||
         (rc = upload((void **)&h->d_nbm1, t->nb_minus_1, (size_t)t->n_mbs * 8)) ||

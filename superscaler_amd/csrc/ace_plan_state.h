@@ -117,7 +117,7 @@ struct alignas(16) ace_u4 { uint32_t x, y, z, w; };
 struct alignas(8) ace_u2 { uint32_t x, y; };
 
 #define ACE_HOT_STRIDE 48u     // bytes per (diag, code) entry of the hot sub-table
-#define ACE_START_STRIDE 32u
+#define ACE_START_STRIDE 24u    // ... of the start sub-table: input MB, input / intra-node bandwidth, input / inter-node bandwidth
 
 // Geometry and constants every lane reads (kernel arguments -> scalar registers).
 struct AceGeom {
@@ -129,6 +129,7 @@ struct AceGeom {
     uint32_t zm_delta;          // bytes from a cost table to the memory table of the same collective (ACE_F_COLLECTIVE_MEM)
     uint32_t rk_lds_off, stg_lds_off;              // LDS byte offsets of the pair-kind and stage LUT regions
     uint32_t lut2_lds_off;                         // ... of the per-(micro-batch, stage size) offset pairs (see ace_lds_layout)
+    uint32_t pk32_lds_off;                         // ... of the pair-kind table in the assembly loop's form (0: LDS has no room for it)
     uint32_t rk_kind_stride;    // bytes of one pair kind (n_glog * 64)
     uint32_t row_bytes;         // bytes of one op type's row
     int32_t flags;
@@ -156,6 +157,17 @@ uint32_t ace_lds_layout(uint32_t rk_off, uint32_t rk_bytes, uint32_t stg_words, 
     *stg_off = (rk_off + rk_bytes + 15u) & ~15u;
     *lut2_off = (*stg_off + stg_words * 4u + 15u) & ~15u;
     return *lut2_off + stg_words * 8u;
+}
+// The assembly form of the op loop reads the pair kinds as 32-bit entries (one per byte of the table above: byte offset
+// of the forward collective's cost table | that of the backward collective's << 16), placed behind everything else.
+#ifdef ACE_HOST_EMU
+inline
+#else
+__host__ __device__ inline
+#endif
+uint32_t ace_lds_pk32(uint32_t lds_end, uint32_t rk_bytes, uint32_t *pk32_off) {
+    *pk32_off = (lds_end + 15u) & ~15u;
+    return *pk32_off + rk_bytes * 4u;
 }
 
 // COLL: consider_collective_memory (the tables carry ACE_F_COLLECTIVE_MEM).
@@ -296,15 +308,11 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false> struct Pl
         out_cross = (cross >> (16u + sidx)) & 1u;
         t_first = c >> g.A_shift;
         uint32_t a = row + g.start_off + (dc_v + c) * ACE_START_STRIDE;
-        ace_d2 e0 = lds.ld<ace_d2>(a);          // input size, size / intra-node bandwidth
-        ace_d2 e1 = lds.ld<ace_d2>(a + 16);     // size / inter-node bandwidth, pad
-        inputs = e0.x;
-        in_comm = in_cross ? e1.x : e0.y;
+        inputs = lds.ld<double>(a);                                 // input size
+        in_comm = lds.ld<double>(a + (in_cross ? 16u : 8u));        // size / inter- or intra-node bandwidth
         if (BD) {
             uint32_t ai = row + g.start_off + ideal_start_v + (c & (uint32_t)(g.n_algo - 1)) * ACE_START_STRIDE;
-            ace_d2 i0 = lds.ld<ace_d2>(ai);
-            ace_d2 i1 = lds.ld<ace_d2>(ai + 16);
-            id_in = in_cross ? i1.x : i0.y;
+            id_in = lds.ld<double>(ai + (in_cross ? 16u : 8u));
             id_fwd = 0.0; id_bwd = 0.0;
         }
     }

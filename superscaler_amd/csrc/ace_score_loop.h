@@ -26,7 +26,7 @@ struct AceKernelArgs {
     const double *rows;         // [n_types][row_doubles]
     const uint32_t *pos_info;   // [N + 1], padded to 16 * G + 16 entries
     const ace_u4 *pos4;         // [16 * G + 16] per position: LDS address of its row's hot sub-table, of its cost tables, of the
-                                //   pair-kind block of the (this, next) pair; bit 0: no layer start follows an ordinary op here, bit 1: ordinary op
+                                //   32-bit pair-kind block of the (this, next) pair; bit 0: no layer start follows an ordinary op here, bit 1: ordinary op
     const uint8_t *pair_kinds;  // -> LDS
     const uint32_t *stage_lut;  // -> LDS
     const double *nbm1;         // [n_mbs]
@@ -66,7 +66,7 @@ __device__ __forceinline__ uint32_t ace_score_loop_asm(const AceKernelArgs &a, c
 #define ACE_LOOP_ASM_RUN(TEXT)                                                                                          \
     asm volatile(TEXT : [cnt] "=&v"(cnt)                                                                               \
                  : [dg] "v"(dg), [rk] "v"(rks), [codeoff] "v"(code_off), [rec] "v"(rec), [codes] "s"(a.codes),         \
-                   [pos] "s"(a.pos4), [c8] "s"(c8), [zshift] "s"(g.z_shift), [n_ops] "s"(g.N), [n_groups] "s"(g.G),     \
+                   [pos] "s"(a.pos4), [c8] "s"(c8), [n_ops] "s"(g.N), [n_groups] "s"(g.G),                                \
                    [gstride_lo] "s"(gs_lo), [gstride_hi] "s"(gs_hi), [wsstride] "s"(ws_stride), [prio] "s"(prio)        \
                  : ACE_LOOP_ASM_CLOBBERS)
     if (g.flags & ACE_F_RESHARDING) {
@@ -173,7 +173,12 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
         while (w0 + 1 < a.n_windows && a.win_pos[w0 + 1] <= (grp_begin << 4)) ++w0;
 
     // small tables: pair kinds and the (micro-batch, stage gpus) LUT; without windows, every row
-    for (int j = tid; j < a.rk_bytes; j += BLOCK) lds_raw[a.g.rk_lds_off + j] = a.pair_kinds[j];
+    for (int j = tid; j < a.rk_bytes; j += BLOCK) {
+        const uint32_t r = a.pair_kinds[j];
+        lds_raw[a.g.rk_lds_off + j] = (unsigned char)r;
+        if (DEFER && a.g.pk32_lds_off)
+            reinterpret_cast<uint32_t *>(lds_raw + a.g.pk32_lds_off)[j] = ((r & 15u) << a.g.z_shift) | (((r >> 4) << a.g.z_shift) << 16);
+    }
     for (int j = tid; j < a.stg_words; j += BLOCK) {
         const uint32_t w = a.stage_lut[j];
         reinterpret_cast<uint32_t *>(lds_raw + a.g.stg_lds_off)[j] = w;

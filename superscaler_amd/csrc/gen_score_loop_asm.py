@@ -42,7 +42,7 @@ def ZV(x):                                  # collective costs of an op's input:
     return f"v[{b}:{b+1}]", f"v[{b+2}:{b+3}]"
 
 
-def R(x):                                   # collective ids of an op pair (byte from the pair table)
+def R(x):                                   # cost-table byte offsets (forward | backward << 16) of an op pair
     return f"v{100 + x}"
 
 
@@ -127,15 +127,14 @@ class Gen:
         if not self.rsh:
             return
         self.o(f"v_add_u32_sdwa {T1}, {RK}, {d['cn']} {sel}")
-        self.o(f"v_add_u32_e32 {T1}, {p['pk']}, {T1}")
-        self.o(f"ds_read_u8 {R(1 - x1)}, {T1}")            # ids of the (k1, k1 + 1) pair
+        self.o(f"v_lshl_add_u32 {T1}, {T1}, 2, {p['pk']}")
+        self.o(f"ds_read_b32 {R(1 - x1)}, {T1}")           # cost-table offsets of the (k1, k1 + 1) pair
         self.o(f"v_add_u32_e32 {T0}, {p['z']}, {T0}")
-        self.o("s_waitcnt lgkmcnt(4)")                       # the ids of the (k1 - 1, k1) pair are in
+        self.o("s_waitcnt lgkmcnt(4)")                       # those of the (k1 - 1, k1) pair are in
         zf, zb = ZV(x1)
-        self.o(f"v_and_b32 {T1}, 15, {R(x1)}")
-        self.o(f"v_lshrrev_b32 {T2}, 4, {R(x1)}")
-        self.o(f"v_lshl_add_u32 {T1}, {T1}, %[zshift], {T0}")
-        self.o(f"v_lshl_add_u32 {T2}, {T2}, %[zshift], {T0}")
+        wsel = "dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_"
+        self.o(f"v_add_u32_sdwa {T1}, {T0}, {R(x1)} {wsel}0")
+        self.o(f"v_add_u32_sdwa {T2}, {T0}, {R(x1)} {wsel}1")
         self.o(f"ds_read_b64 {zf}, {T1}")
         self.o(f"ds_read_b64 {zb}, {T2}")
 

@@ -9,7 +9,7 @@ maxima of table entries:
   row[type]  per op type, contiguous (staged in LDS as a unit):
      hot   [diag][code][6]   fwd us, bwd us, weights MB, activations MB (x1.5 / 0 rule of
                              :386-391 applied), fwd_reserved MB, bwd_reserved MB
-     start [diag][code][4]   input MB, input/intra-node-bandwidth, input/inter-node-bandwidth, 0
+     start [diag][code][3]   input MB, input/intra-node-bandwidth, input/inter-node-bandwidth
                              (:319-336 for the stage's first op, with the index quirks of :275-299)
      out   [mbs][tp][algo][2] output/intra-bandwidth, output/inter-bandwidth (indexed the way
                              :321-326 mixes the first op's tp with the last op's mbs and algo)
@@ -38,7 +38,7 @@ import numpy as np
 from . import opgraph as og
 from .profile_db import CostModelSettings, ProfileDB
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 MAX_STAGES = 16
 STAGE_REC = 18
 LDS_BYTES = 160 * 1024
@@ -274,7 +274,8 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
     # ---- rows ------------------------------------------------------------------------------
     hot_off = 0
     start_off = hot_off + (ND + 1) * C * 6      # diag ND: all NaN, where unscorable (micro-batch, stage size) pairs point
-    out_off = start_off + ND * C * 4
+    out_off = start_off + ND * C * 3
+    out_off += out_off & 1                     # (16-byte aligned: its entries are read as pairs)
     z_off = out_off + M * T * A * 2
     z_table_doubles = 1
     while z_table_doubles < ND * C:
@@ -299,7 +300,7 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
     for ty, name in enumerate(db.op_names):
         fl = int(graph.flags[ty])
         hot = np.full((ND + 1, C, 6), nan)
-        start = np.full((ND, C, 4), nan)
+        start = np.full((ND, C, 3), nan)
         z = np.full((max(NZ, 1), ND, C), nan)
         z[0] = 0.0
         zm = np.full((max(NZ, 1), ND, C), nan)
@@ -321,7 +322,7 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
                     hot[d, c] = (float(tb["fwd"][ty, m, t, a]), float(tb["bwd"][ty, m, t, a]),
                                  float(tb["weights"][ty, m, t, a]), act, rf, rb)
                     insz = float(tb["input_size"][ty, m, t, a])
-                    start[d, c] = (insz, db.p2p_time(insz, db.intra_band), db.p2p_time(insz, db.inter_band), 0.0)
+                    start[d, c] = (insz, db.p2p_time(insz, db.intra_band), db.p2p_time(insz, db.inter_band))
                     for k, (prim, n) in enumerate(z_keys):
                         z[k + 1, d, c] = db.reshard_time(og.PRIM_NAMES[prim], n, insz)
                         # get_reshard_memory: the data itself, times the group size for the gathering collectives

@@ -25,7 +25,7 @@ def test_every_declared_symbol_is_exported():
     for n in names:
         assert hasattr(lib, n), f"{n} is declared in include/ace_eval.h but not exported"
     assert sorted(evaluator.EXPORTS) == names
-    assert lib.ace_abi_version() == 7
+    assert lib.ace_abi_version() == 8
 
 
 def test_error_strings_and_argument_checks():

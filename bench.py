@@ -18,14 +18,19 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 # Counter readings of the scoring kernel on the default workload, which a run of this script cannot take itself
-# (rocprofv3 --pmc passes): copied from the committed summary named in "source", which also names the library
-# build they were taken on.  HBM bytes per plan and launch = FETCH_SIZE + WRITE_SIZE, each scaled by the reading
-# of a plain 256 MiB copy in the same pass; vector instructions per op and wavefront = SQ_INSTS_VALU / SQ_WAVES /
-# ops; 14 of them are the reference's own fp64 arithmetic (nine adds / multiply-adds, five maxima).
+# (rocprofv3 --pmc passes): copied from the committed summary named in "source".  "library" is
+# superscaler_amd.build.source_hash() of the library sources they were taken on: when the sources no longer hash to
+# it the readings are left out of the line (with a note) instead of being reported for another kernel.
+# HBM bytes per plan and launch = FETCH_SIZE + WRITE_SIZE, each scaled by the reading of a plain 256 MiB copy in
+# the same pass; vector instructions per op and wavefront = SQ_INSTS_VALU / SQ_WAVES / ops; 14 of them are the
+# reference's own fp64 arithmetic (nine adds / multiply-adds, five maxima).
 PROFILE_COUNTERS = {
-    ("gpt3_13b", 523): {"source": "profiles/score_kernel_gpt3_13b.md", "commit": "381908c", "traffic_bytes_per_plan": 2206.0,
-                        "valu_per_op_per_wavefront": 47.4, "valu_busy": 0.85},
+    ("gpt3_13b", 523): {"source": "profiles/score_kernel_gpt3_13b.md", "library": "unset", "traffic_bytes_per_plan": 0.0,
+                        "valu_per_op_per_wavefront": 0.0, "valu_busy": 0.0},
 }
+# the other configured workloads, timed after the headline measurement (kernel only, HIP events on the launch stream)
+OTHER_WORKLOADS = ("gpt3_1_3b", "t5_770m", "wresnet_1b", "gpt3_175b")
+OTHER_PLANS = 262144
 ESSENTIAL_VALU_PER_OP = 14
 
 
@@ -68,6 +73,33 @@ def cpu_baseline(tables, batch, threads):
             "c_port_single_core_sample": f"first {n1} plans, {dt_one:.2f} s, 1 thread"}
 
 
+def kernel_name(tables):
+    return ("ace_score_kernel<BD=false,RANGED=false,WIN=true,DEFER=false>" if tables.n_windows > 1 else
+            "ace_score_kernel<BD=false,RANGED=false,WIN=false,DEFER=true>")
+
+
+def other_workloads(steps):
+    """Scoring kernel alone on the other configured workloads: {name: kernel, ms, bytes per plan, roofline fraction}."""
+    from superscaler_amd import synth
+    from superscaler_amd.evaluator import PlanEvaluator
+    out = {}
+    for name in OTHER_WORKLOADS:
+        w = synth.WORKLOADS[name]
+        tables = synth.make_tables(w)
+        batch = synth.make_plans(w, tables, n_plans=OTHER_PLANS, workers=min(16, os.cpu_count() or 1))
+        ev = PlanEvaluator(tables, device="cuda:0")
+        d = ev.upload(batch)
+        ev.time_score_kernel(d, reps=20)
+        ms = ev.time_score_kernel(d, reps=max(steps, 20))
+        bpp = 3 * d.num_ops + 19
+        gbps = bpp * d.n_plans / (ms * 1e-3) / 1e9
+        out[name] = {"kernel": kernel_name(tables), "ops": d.num_ops, "plans": d.n_plans, "kernel_ms": ms,
+                     "plans_per_s_kernel": d.n_plans / (ms * 1e-3), "algorithmic_bytes_per_plan": bpp,
+                     "achieved_GBps": gbps, "frac": gbps / HBM_PEAK_GBPS}
+        ev.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -80,6 +112,8 @@ def main():
     ap.add_argument("--pp", type=int, nargs="+", default=None,
                     help="restrict the pipeline depths the plans are drawn from (profiling aid)")
     ap.add_argument("--no-pcie-rate", action="store_true", help="skip the host-memory-in measurement")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="skip the kernel timings of the other configured workloads (config.other_workloads)")
     ap.add_argument("--regrouped-too", action="store_true",
                     help="also time the step on a copy of the batch regrouped on the device beforehand (by pipeline "
                          "depth and first stage boundaries; ace_group_keys / ace_gather_plans), as a secondary figure")
@@ -171,6 +205,12 @@ def main():
     n_feasible = int(fe.sum().item())
     best = val[0].item() if n_feasible else None
     counters = PROFILE_COUNTERS.get((w.name, N)) if P == w.n_plans and not args.pp else None
+    counters_note = None
+    from superscaler_amd import build as lib_build
+    if counters and counters["library"] != lib_build.source_hash():
+        counters_note = (f'the counter readings of {counters["source"]} were taken on library sources {counters["library"]}; '
+                         f"these sources hash to {lib_build.source_hash()}: readings left out")
+        counters = None
 
     out = {
         "metric": "plans scored/sec at GPT-3 13B op graph (1M plans); % HBM roofline",
@@ -188,15 +228,14 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS,
                      "traffic": counters["traffic_bytes_per_plan"] * P if counters else None,
-                     "traffic_source": f'{counters["source"]} (library sources of commit {counters["commit"]})' if counters else None,
+                     "traffic_source": f'{counters["source"]} (library sources {counters["library"]})' if counters else counters_note,
                      "algorithmic_bytes": algo_bytes,
-                     "kernel": ("ace_score_kernel<BD=false,RANGED=false,WIN=true,DEFER=false>" if tables.n_windows > 1 else
-                                "ace_score_kernel<BD=false,RANGED=false,WIN=false,DEFER=true>"), "kernel_ms": kern_ms,
+                     "kernel": kernel_name(tables), "kernel_ms": kern_ms,
                      "algorithmic_bytes_per_plan": 3 * N + 19,
                      "bytes_moved_per_plan": d.bytes_moved_per_plan + 17,
                      "achieved_on_bytes_moved": moved_bytes / (kern_ms * 1e-3) / 1e9,
-                     "note": "HBM is the nominal roofline of this path (plan bytes streamed once, tables in LDS); the kernel "
-                             "itself is bound by vector-instruction issue, see roofline_valu_issue"},
+                     "note": "HBM is the nominal roofline of this path (plan bytes streamed once, tables in LDS); inside the CU "
+                             "the kernel is held by vector-instruction issue and LDS reads, see roofline_valu_issue"},
     }
     if counters:
         # the bound that holds: one vector instruction per SIMD and quad-cycle; the time of the kernel is the number
@@ -215,6 +254,8 @@ def main():
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(tables, batch, threads=min(16, os.cpu_count() or 1))
     ev.close()
+    if not args.no_other_workloads and args.workload == "gpt3_13b" and not args.pp:
+        out["config"]["other_workloads"] = other_workloads(args.steps)
     print(json.dumps(out))
 
 

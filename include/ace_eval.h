@@ -204,8 +204,10 @@ int ace_topk(ace_handle_t *h, const double *d_iter_ms, const uint8_t *d_feasible
  *                    the moved ops take); 2 one tp step for the ops p0 = first | last + 1 << 16 (p1 = 1 up, 0 down);
  *                    3 toggle the recompute bit of the ops p0 = first | last + 1 << 16; 4 toggle the algorithm of op p0;
  *  d_codes_out:      uint8[ceil(num_ops / 16)][n_moves][16];  d_hdr_out: uint32[n_moves][4];
- *  d_keys_out:       NULL, or uint64[n_moves] that the CALLER HAS ZEROED: receives a 64-bit key of every
- *                    plan's bytes (equal plans -> equal keys; for visited sets, aceso_search.py:47,105).
+ *  d_keys_out:       NULL, or uint64[n_moves][2] that the CALLER HAS ZEROED: receives a 128-bit key of every
+ *                    plan's bytes (equal plans -> equal keys; for visited sets, aceso_search.py:47,105; the reference's
+ *                    sets hold the plans' full strings, aceso_utils.py:831-850: two distinct plans share a key with a
+ *                    probability of about n^2 / 2^129 for n plans).
  * The caller decides which moves are legal; the kernel only edits bytes. */
 int ace_apply_moves(const uint8_t *d_template_codes, const uint32_t *d_template_hdr, int n_templates,
                     const uint32_t *d_moves, size_t n_moves, int num_ops, int n_algo, uint8_t *d_codes_out,

@@ -417,6 +417,12 @@ class CostModel:
         self.stage_memory_set[key] = v
         return v
 
+    def clear_memo(self):
+        """Empties the two memo tables and their counters (the reference keeps them for the life of its process,
+        aceso_cost_model.py:743-791; a host that runs many searches in one process clears them in between)."""
+        self.stage_memory_set, self.stage_memory_visit, self.stage_memory_hit = {}, 0, 0
+        self.stage_time_set, self.stage_time_visit, self.stage_time_hit = {}, 0, 0
+
     def predict_stage_time_helper(self, config, stage_index):
         """aceso_cost_model.py:773-791."""
         st = config.stages[stage_index]

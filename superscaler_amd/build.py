@@ -8,7 +8,7 @@ ROOT = os.path.dirname(HERE)
 LIB = os.path.join(HERE, "libace_eval.so")
 SOURCES = [os.path.join(HERE, "csrc", "ace_eval.hip")]
 HEADERS = [os.path.join(HERE, "csrc", "ace_plan_state.h"), os.path.join(HERE, "csrc", "ace_score_loop.h"),
-           os.path.join(HERE, "csrc", "ace_edit_kernels.h"),
+           os.path.join(HERE, "csrc", "ace_score_loop_asm.inc"), os.path.join(HERE, "csrc", "ace_edit_kernels.h"),
            os.path.join(ROOT, "include", "ace_eval.h")]
 
 # -ffp-contract=off: the scoring arithmetic must round exactly like the reference's Python floats,
@@ -16,6 +16,18 @@ HEADERS = [os.path.join(HERE, "csrc", "ace_plan_state.h"), os.path.join(HERE, "c
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-shared", "-fPIC", "-ffp-contract=off",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(HERE, "csrc")]
+
+
+def source_hash() -> str:
+    """sha256 over the library's sources (the files `build` compiles, in a fixed order): names what a set of
+    profile readings was taken on."""
+    import hashlib
+    h = hashlib.sha256()
+    for path in sorted(SOURCES + HEADERS):
+        h.update(os.path.basename(path).encode() + b"\0")
+        with open(path, "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
 
 
 def build(verbose: bool = True) -> str:

@@ -1,4 +1,4 @@
-// Kernels that edit or inspect plan bytes (move descriptors -> plans with 64-bit keys; the two
+// Kernels that edit or inspect plan bytes (move descriptors -> plans with 128-bit keys; the two
 // selection steps of check_recompute's greedy loop), each as a function of its work-item index:
 // the __global__ kernels in ace_eval.hip are one-line wrappers, and the host build of the tests
 // (ACE_HOST_EMU) runs the same functions on the CPU with guard pages behind every array.
@@ -21,6 +21,18 @@ ACE_HD unsigned long long plan_key_word(uint32_t a, uint32_t b, uint32_t c, uint
     y = (y + x) * 0xBF58476D1CE4E5B9ull;
     y = (y ^ (y >> 27)) * 0x94D049BB133111EBull;
     return x ^ y ^ (y >> 31);
+}
+
+// The second half of a plan's 128-bit key: the same construction with other odd multipliers.
+ACE_HD unsigned long long plan_key_word2(uint32_t a, uint32_t b, uint32_t c, uint32_t d, uint32_t idx) {
+    unsigned long long x = ((unsigned long long)d << 32 | b) + 0xD6E8FEB86659FD93ull * (2ull * idx + 1ull);
+    unsigned long long y = ((unsigned long long)c << 32 | a) ^ (x >> 31);
+    x = (x ^ (x >> 32)) * 0xFF51AFD7ED558CCDull;
+    x = (x ^ (x >> 29)) * 0xC4CEB9FE1A85EC53ull;
+    x ^= x >> 32;
+    y = (y + x) * 0xFF51AFD7ED558CCDull;
+    y = (y ^ (y >> 29)) * 0xC4CEB9FE1A85EC53ull;
+    return x ^ y ^ (y >> 32);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -72,13 +84,17 @@ ACE_HD void apply_moves_body(unsigned long long id, const ace_u4 *tmpl_codes, co
     }
     codes_out[(size_t)g * n + k] = ace_u4{w[0], w[1], w[2], w[3]};
     if (key_out) {
-        // 64-bit key of the whole plan: XOR of one mixed value per 16-byte word (and one for the header)
+        // 128-bit key of the whole plan, two words per plan: each the XOR of one mixed value per 16-byte word (and one
+        // for the header), from two different mixing functions
         unsigned long long hsh = plan_key_word(w[0], w[1], w[2], w[3], (uint32_t)g + 1u);
+        unsigned long long hsh2 = plan_key_word2(w[0], w[1], w[2], w[3], (uint32_t)g + 1u);
         if (g == 0) {
             const ace_u4 hh = tmpl_hdr[t];
             hsh ^= plan_key_word(hh.x, hh.y, hh.z, 0u, 0u);      // (the fourth header word follows from the others)
+            hsh2 ^= plan_key_word2(hh.x, hh.y, hh.z, 0u, 0u);
         }
-        ACE_ATOMIC_XOR(&key_out[k], hsh);
+        ACE_ATOMIC_XOR(&key_out[2 * k], hsh);
+        ACE_ATOMIC_XOR(&key_out[2 * k + 1], hsh2);
     }
 }
 

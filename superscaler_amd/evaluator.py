@@ -429,7 +429,7 @@ class PlanEvaluator:
         d_mv = torch.from_numpy(np.ascontiguousarray(moves, dtype=np.uint32).view(np.int32)).to(self.device)
         codes = torch.empty((G, n, 16), dtype=torch.uint8, device=self.device)
         hdr = torch.empty((n, 4), dtype=torch.int32, device=self.device)
-        keys = torch.zeros(n, dtype=torch.int64, device=self.device) if with_keys else None
+        keys = torch.zeros((n, 2), dtype=torch.int64, device=self.device) if with_keys else None
         with torch.cuda.device(self.device):
             rc = self.lib.ace_apply_moves(d_tc.data_ptr(), d_th.data_ptr(), T, d_mv.data_ptr(), n, N,
                                           self.tables.db.n_algo, codes.data_ptr(), hdr.data_ptr(),

@@ -363,31 +363,66 @@ def _key_word(a, b, c, d, idx):
     return x ^ y ^ (y >> u(31))
 
 
+_J0, _J1, _J2 = np.uint64(0xD6E8FEB86659FD93), np.uint64(0xFF51AFD7ED558CCD), np.uint64(0xC4CEB9FE1A85EC53)
+
+
+def _key_word2(a, b, c, d, idx):
+    """The second mixing function of the library's 128-bit plan keys."""
+    u = np.uint64
+    x = ((d << u(32)) | b) + _J0 * (u(2) * idx + u(1))
+    y = ((c << u(32)) | a) ^ (x >> u(31))
+    x = (x ^ (x >> u(32))) * _J1
+    x = (x ^ (x >> u(29))) * _J2
+    x = x ^ (x >> u(32))
+    y = (y + x) * _J1
+    y = (y ^ (y >> u(29))) * _J2
+    return x ^ y ^ (y >> u(32))
+
+
 def plan_keys_host(batch: PlanBatch) -> np.ndarray:
-    """The 64-bit plan keys ace_apply_moves writes, computed on the host (uint64[n_plans])."""
+    """The 128-bit plan keys ace_apply_moves writes, computed on the host (uint64[n_plans, 2])."""
     P, N = batch.codes.shape
     G = (N + 15) // 16
     padded = np.zeros((P, G * 16), dtype=np.uint8)
     padded[:, :N] = batch.codes
     w = padded.view(np.uint32).reshape(P, G, 4).astype(np.uint64)
     idx = (np.arange(G, dtype=np.uint64) + np.uint64(1))[None, :]
+    h = batch.hdr.astype(np.uint64)
+    zero = np.zeros(P, dtype=np.uint64)
+    keys = np.empty((P, 2), dtype=np.uint64)
     with np.errstate(over="ignore"):
-        keys = np.bitwise_xor.reduce(_key_word(w[:, :, 0], w[:, :, 1], w[:, :, 2], w[:, :, 3], idx), axis=1)
-        h = batch.hdr.astype(np.uint64)
-        keys ^= _key_word(h[:, 0], h[:, 1], h[:, 2], np.zeros(P, dtype=np.uint64), np.uint64(0))
+        for col, mix in enumerate((_key_word, _key_word2)):
+            keys[:, col] = np.bitwise_xor.reduce(mix(w[:, :, 0], w[:, :, 1], w[:, :, 2], w[:, :, 3], idx), axis=1)
+            keys[:, col] ^= mix(h[:, 0], h[:, 1], h[:, 2], zero, np.uint64(0))
     return keys
 
 
+KEY128 = np.dtype([("a", "<u8"), ("b", "<u8")])
+
+
+def as_key128(keys) -> np.ndarray:
+    """uint64[n, 2] (what ace_apply_moves / plan_keys_host give) as one 128-bit record per plan."""
+    k = np.asarray(keys)
+    if k.dtype == KEY128:
+        return k
+    k = np.ascontiguousarray(k, dtype=np.uint64)
+    if k.ndim != 2 or k.shape[1] != 2:
+        raise ValueError("plan keys are pairs of 64-bit words")
+    return k.view(KEY128).ravel()
+
+
 class VisitedKeys:
-    """A visited set over 64-bit plan keys (for neighbours that only exist on the device): two sorted
+    """A visited set over 128-bit plan keys (for neighbours that only exist on the device): two sorted
     arrays, a large one and a small one that takes the new keys and is folded into the large one
-    when it has grown (so marking costs a merge of the small array only)."""
+    when it has grown (so marking costs a merge of the small array only).  Two plans are taken for the
+    same plan when both 64-bit halves of their keys agree; the reference's sets compare the plans' full
+    strings (aceso_utils.py:831-850)."""
 
     SMALL_LIMIT = 65536
 
     def __init__(self):
-        self._sorted = np.empty(0, dtype=np.uint64)
-        self._small = np.empty(0, dtype=np.uint64)
+        self._sorted = np.empty(0, dtype=KEY128)
+        self._small = np.empty(0, dtype=KEY128)
 
     def __len__(self):
         return len(self._sorted) + len(self._small)
@@ -401,6 +436,7 @@ class VisitedKeys:
 
     def unseen(self, keys: np.ndarray) -> np.ndarray:
         """Mask of the keys not marked before that do not repeat an earlier entry of `keys`."""
+        keys = as_key128(keys)
         _, first = np.unique(keys, return_index=True)
         mask = np.zeros(len(keys), dtype=bool)
         mask[first] = True
@@ -410,12 +446,12 @@ class VisitedKeys:
         return mask
 
     def mark(self, keys: np.ndarray) -> None:
-        k = np.unique(np.asarray(keys, dtype=np.uint64))
+        k = np.unique(as_key128(keys))
         k = k[self._absent(self._sorted, k)]              # (the two arrays stay disjoint: __len__ is their sum)
         self._small = np.union1d(self._small, k)
         if len(self._small) > self.SMALL_LIMIT:
             self._sorted = np.union1d(self._sorted, self._small)
-            self._small = np.empty(0, dtype=np.uint64)
+            self._small = np.empty(0, dtype=KEY128)
 
 
 def hill_climb(cm, start: PlanBatch, steps: int, n_neighbours: int, seed: int = 0, max_move: int = 8,
@@ -428,7 +464,7 @@ def hill_climb(cm, start: PlanBatch, steps: int, n_neighbours: int, seed: int = 
     replaced by check_recompute's choice before it is scored, as the reference's primitives do
     (aceso_prims.py:107-108).  With `device_moves` the neighbours never exist on the host: the move
     descriptors (16 bytes each) are expanded by the library on the device and only the winner is
-    rebuilt here; `visited` is then a VisitedKeys (64-bit keys of the plan bytes, computed by the
+    rebuilt here; `visited` is then a VisitedKeys (128-bit keys of the plan bytes, computed by the
     same kernel, before any recompute bits are re-chosen) and `greedy_recompute` runs check_recompute's
     loop on the device as well (CostModel.update_recompute_device).
     Returns (plan, iteration ms, peak MB)."""
@@ -455,7 +491,7 @@ def hill_climb(cm, start: PlanBatch, steps: int, n_neighbours: int, seed: int = 
                 d = ev.apply_moves(templates, moves)
             else:
                 d, keys = ev.apply_moves(templates, moves, with_keys=True)
-                keys = keys.cpu().numpy().view(np.uint64)
+                keys = as_key128(keys.cpu().numpy().view(np.uint64))
                 keep = np.flatnonzero(visited.unseen(keys))
                 if len(keep) == 0:
                     if on_step is not None:

@@ -27,7 +27,7 @@ def main(argv=None):
     ap.add_argument("--topk", type=int, default=64)
     ap.add_argument("--greedy-recompute", action="store_true")
     ap.add_argument("--device-moves", action="store_true",
-                    help="expand the move descriptors on the device (visited set over 64-bit plan keys)")
+                    help="expand the move descriptors on the device (visited set over 128-bit plan keys)")
     ap.add_argument("--workers", type=int, default=16)
     ap.add_argument("--distinct-batches", type=int, default=0,
                     help="generate only this many different batches and cycle through them (0 = all different); "

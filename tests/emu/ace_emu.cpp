@@ -235,14 +235,14 @@ extern "C" int ace_emu_apply_moves(const uint8_t *tmpl_codes, const uint32_t *tm
     const ace_u4 *mv = (const ace_u4 *)pool.place(moves, (size_t)n * 16);
     ace_u4 *co = (ace_u4 *)pool.place(nullptr, (size_t)n * cb);
     ace_u4 *ho = (ace_u4 *)pool.place(nullptr, (size_t)n * 16);
-    unsigned long long *ko = keys_out ? (unsigned long long *)pool.place(keys_out, (size_t)n * 8, 8) : nullptr;
+    unsigned long long *ko = keys_out ? (unsigned long long *)pool.place(keys_out, (size_t)n * 16, 8) : nullptr;
     // (the library launches whole workgroups of 256: ids past n * G must fall out at the first test)
     const unsigned long long total = ((unsigned long long)n * G + 255) / 256 * 256;
     for (unsigned long long id = 0; id < total; ++id)
         apply_moves_body(id, tc, th, n_templates, mv, (unsigned long long)n, G, n_algo == 2 ? 1 : 0, co, ho, ko);
     memcpy(codes_out, co, (size_t)n * cb);
     memcpy(hdr_out, ho, (size_t)n * 16);
-    if (keys_out) memcpy(keys_out, ko, (size_t)n * 8);
+    if (keys_out) memcpy(keys_out, ko, (size_t)n * 16);
     return 0;
 }
 

@@ -162,7 +162,7 @@ def main(workload, mode, n):
             mv = np.ascontiguousarray(moves, dtype=np.uint32)
             co = np.zeros((G, m, 16), dtype=np.uint8)
             ho = np.zeros((m, 4), dtype=np.uint32)
-            ko = np.zeros(m, dtype=np.uint64) if keys else None
+            ko = np.zeros((m, 2), dtype=np.uint64) if keys else None
             assert lib.ace_emu_apply_moves(tc.ctypes.data, th.ctypes.data, T, mv.ctypes.data, m, N, tables.db.n_algo,
                                            co.ctypes.data, ho.ctypes.data, ko.ctypes.data if keys else None) == 0
             return co, ho, ko

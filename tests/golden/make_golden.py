@@ -703,6 +703,33 @@ def child_search_trace(case, extras=False, per_function=25):
     print(f"[golden] search trace {case}{' (extras)' if extras else ''}: { {n: len(v) for n, v in trace.items()} }, best {results}")
 
 
+PER_OP_LISTS = ("model_parallel_size_of_each_op", "data_parallel_size_of_each_op", "recompute_ops", "algo_of_each_op")
+
+
+def dumped_plan(tmp, num_stages):
+    """The plan file run_search wrote for this stage count (aceso_search.py:293-294, dump_config_to_json), as a dict;
+    its per-op lists (one list per stage) as runs [[value, count], ...] to keep the fixture small."""
+    import glob
+    files = sorted(glob.glob(os.path.join(tmp, f"*_{num_stages}stages_*.json")))
+    if not files:
+        return None
+    with open(files[-1]) as f:
+        plan = json.load(f)
+    for key in PER_OP_LISTS:
+        stages = []
+        for xs in plan[key]:
+            runs = []
+            for v in xs:
+                if runs and runs[-1][0] == v:
+                    runs[-1][1] += 1
+                else:
+                    runs.append([v, 1])
+            stages.append(runs)
+        plan[key] = stages
+    plan["per_op_lists_as_runs"] = True
+    return plan
+
+
 def child_search_results(case):
     """The reference's search with its own cost model and nothing recorded but what it found (the flags of
     child_search_trace; GOLDEN_TRIALS / GOLDEN_HOPS set the length): one JSON line on standard output."""
@@ -725,9 +752,70 @@ def child_search_results(case):
         import aceso_search as S                   # noqa: the reference, run to record what it finds
         for num_stages in [int(x) for x in os.environ.get("GOLDEN_STAGES", "2,3,4").split(",")]:
             r = S.run_search(num_stages, queue=None)
-            found[str(num_stages)] = None if r is None else [r[0], r[1], r[2]]
+            found[str(num_stages)] = None if r is None else [r[0], r[1], r[2], dumped_plan(tmp, num_stages)]
     shutil.rmtree(tmp, ignore_errors=True)
     print(json.dumps(found))
+
+
+def child_score_plans(name):
+    """search_binding_<name>.json: the plan files the two searches wrote, scored by the REFERENCE's cost model
+    (read_config_from_json, predict_time_breakdown) under the record's flags; [max(time_list), max(memory_list)] per side
+    and stage count into the record ("plan_scores_by_the_reference").  The number a search returns is the best time it
+    saw; with the fine-tuning actions switched on the plan it writes can differ from the plan that time belongs to, so
+    the tests compare re-scored plans with these scores."""
+    import contextlib
+    import io
+    import tempfile
+    path = os.path.join(HERE, f"search_binding_{name}.json")
+    with open(path) as f:
+        fx = json.load(f)
+    case = fx["case"]
+    model, size, db, mbs_list, nodes, gpn, gbs, limit, num_layers = {**CASES, **BIG_CASES}[case]
+    flags = [x for x in fx["flags"] if x not in ("--no-multi-process", "--add-action-tp-dp-exchange")]
+    drop = {"--time-budget-total", "--max-num-trials", "--max-num-hops"}
+    extra, skip = [], False
+    for x in flags:
+        if skip:
+            skip = False
+            continue
+        if x in drop:
+            skip = True
+            continue
+        extra.append(x)
+    if num_layers:
+        extra += ["--num-layers", str(num_layers)]
+    tmp = tempfile.mkdtemp()
+    sys.argv = reference_argv(case, extra + ["--log-path", tmp + "/", "--config-save-path", tmp + "/"])
+    sys.path.insert(0, os.path.join(REF, "search"))
+    scores = {}
+    with contextlib.redirect_stdout(io.StringIO()):
+        import aceso_cost_model as CM                 # noqa: the reference, imported to record its outputs
+        import aceso_utils as U                       # noqa
+        args = CM.args
+        CM.read_profiled_time(args.model_name, args.model_size, args.profiled_time_path)
+        for side in ("best_plan_with_the_binding", "best_plan_with_the_reference_cost_model"):
+            scores[side] = {}
+            for stages, plan in fx[side].items():
+                if plan is None:
+                    scores[side][stages] = None
+                    continue
+                d = dict(plan)
+                if d.pop("per_op_lists_as_runs", False):
+                    for key in PER_OP_LISTS:
+                        d[key] = [[v for v, k in runs for _ in range(k)] for runs in plan[key]]
+                fn = os.path.join(tmp, "plan.json")
+                with open(fn, "w") as f:
+                    json.dump(d, f)
+                args.initial_point = fn
+                cfg = U.read_config_from_json(args)
+                CM.predict_time_breakdown(cfg)
+                scores[side][stages] = [max(cfg.time_list), max(cfg.memory_list)]
+    fx["plan_scores_by_the_reference"] = scores
+    with open(path, "w") as f:
+        json.dump(fx, f, separators=(",", ":"))
+    shutil.rmtree(tmp, ignore_errors=True)
+    same = sum(scores["best_plan_with_the_binding"][k] == (fx["with_the_binding"][k]) for k in fx["with_the_binding"])
+    print(f"[golden] plans of search_binding_{name} scored by the reference: {same} of {len(fx['with_the_binding'])} equal to what the search returned")
 
 
 def child_binding_search(case):
@@ -770,31 +858,32 @@ def child_binding_search(case):
         found = {}
         for num_stages in [int(x) for x in os.environ.get("GOLDEN_STAGES", "2,3,4").split(",")]:
             r = S.run_search(num_stages, queue=None)
-            found[str(num_stages)] = None if r is None else [r[0], r[1], r[2]]
+            found[str(num_stages)] = None if r is None else [r[0], r[1], r[2], dumped_plan(tmp, num_stages)]
     long_run = any(k in os.environ for k in ("GOLDEN_TRIALS", "GOLDEN_HOPS", "GOLDEN_FLAGS", "GOLDEN_STAGES"))
-    explored_ref = None
-    if long_run:
-        # another length than the recorded trace's: the reference's own run of that length, in a process of its own
-        r = subprocess.run([sys.executable, os.path.abspath(__file__), "--child-search-results", case], check=True,
-                           stdout=subprocess.PIPE, text=True)
-        own = json.loads(r.stdout.strip().splitlines()[-1])
-        ref = {k: (v[:2] if v else None) for k, v in own.items()}
-        explored_ref = {k: (v[2] if v else None) for k, v in own.items()}
-    else:
+    # the reference's own run with the same flags, in a process of its own
+    r = subprocess.run([sys.executable, os.path.abspath(__file__), "--child-search-results", case], check=True,
+                       stdout=subprocess.PIPE, text=True)
+    own = json.loads(r.stdout.strip().splitlines()[-1])
+    ref = {k: (v[:2] if v else None) for k, v in own.items()}
+    explored_ref = {k: (v[2] if v else None) for k, v in own.items()}
+    if not long_run:
         with open(os.path.join(HERE, f"search_trace_{case}.json")) as f:
-            ref = json.load(f)["best_time_and_memory"]
+            assert ref == json.load(f)["best_time_and_memory"], "the reference's search is not deterministic?" 
     out = {"case": case, "flags": extra[:7] + ["--add-action-tp-dp-exchange"] + os.environ.get("GOLDEN_FLAGS", "").split(),
            "stage_counts": os.environ.get("GOLDEN_STAGES", "2,3,4"), "with_the_binding": {k: (v[:2] if v else None) for k, v in found.items()},
            "explored_with_the_binding": {k: (v[2] if v else None) for k, v in found.items()},
            "with_the_reference_cost_model": ref}
-    if explored_ref is not None:
-        out["explored_with_the_reference_cost_model"] = explored_ref
+    out["explored_with_the_reference_cost_model"] = explored_ref
+    # the plan files the two searches wrote (dump_config_to_json), so that the recorded numbers can be re-scored
+    out["best_plan_with_the_binding"] = {k: (v[3] if v else None) for k, v in found.items()}
+    out["best_plan_with_the_reference_cost_model"] = {k: (v[3] if v else None) for k, v in own.items()}
     suffix = os.environ.get("GOLDEN_SUFFIX", "__long") if long_run else ""
     with open(os.path.join(HERE, f"search_binding_{case}{suffix}.json"), "w") as f:
-        json.dump(out, f, indent=1)
+        json.dump(out, f, separators=(",", ":"))
     shutil.rmtree(tmp, ignore_errors=True)
     same = out["with_the_binding"] == {k: v for k, v in ref.items()}
     print(f"[golden] search over the binding {case}: {out['with_the_binding']} -- {'same as' if same else 'DIFFERENT FROM'} the reference's own")
+    subprocess.run([sys.executable, os.path.abspath(__file__), "--child-score-plans", f"{case}{suffix}"], check=True)
 
 
 def child_binding_grid(case, num_saved=4):
@@ -976,6 +1065,8 @@ def main():
         return child_reports(sys.argv[2])
     if len(sys.argv) > 2 and sys.argv[1] == "--child-binding-grid":
         return child_binding_grid(sys.argv[2])
+    if len(sys.argv) > 2 and sys.argv[1] == "--child-score-plans":
+        return child_score_plans(sys.argv[2])
     if len(sys.argv) > 2 and sys.argv[1] == "--child-binding-search":
         return child_binding_search(sys.argv[2])
     if len(sys.argv) > 2 and sys.argv[1] == "--child-search-trace":

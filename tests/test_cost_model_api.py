@@ -675,3 +675,39 @@ def test_a_failing_evaluation_ahead_leaves_the_call_to_the_ordinary_path(golden_
     got = _scan_twice(ahead, cfg_of(g, ahead, p), 0, 1, "time")
     assert got == want and ahead.scan_ahead_used == 0
     assert ahead.stage_memory_set == plain.stage_memory_set
+
+
+def test_t5_memo_collision_host_api_and_batched_forms(golden_dir):
+    """The reference's memo table of stage memory is keyed by a stage's first op NAME, its length and its per-op lists
+    (aceso_cost_model.py:743-767): in T5 an all-encoder stage and a stage of the same length that runs on into the
+    decoder share a key.  check_recompute on the second one then starts from the first one's memory if that was asked
+    about before -- in the reference and, with `reference_memo` (the default), here.  Without the table (and in the
+    batched forms, which have none) every stage starts from its own memory.  This pins which answer each path gives."""
+    g, m = make_model(golden_dir, "t5_770M", "emu")
+    ops = m.graph.ops
+    n, mbs = 120, 4
+    A, B = ops[1:1 + n], ops[274:274 + n]
+    assert A[0] == B[0] == "enc-1st-layernorm" and A != B and any(o.startswith("dec") for o in B)
+    lists = ([1] * n, [1] * n, 1, [0] * n)              # tp, dp, stages behind, algo
+    m.clear_memo()
+    alone = m.check_recompute(B, mbs, *lists)
+    m.clear_memo()
+    first = m.check_recompute(A, mbs, *lists)
+    after_a = m.check_recompute(B, mbs, *lists)          # same key as A: starts from A's memory
+    assert sum(alone) == 46 and sum(after_a) == 118 and sum(first) == 116
+    # the table switched off: history does not matter
+    m.clear_memo()
+    m.reference_memo = False
+    assert m.check_recompute(A, mbs, *lists) == first and m.check_recompute(B, mbs, *lists) == alone
+    m.reference_memo = True
+    # the batched form without the table gives every stage its own answer whatever was asked before ...
+    m.clear_memo()
+    m.check_recompute(A, mbs, *lists)
+    q = lambda o: (o, mbs) + lists
+    assert m.check_recompute_batch([q(A), q(B)], memo=False) == [first, alone]
+    # ... and with the table it is the one-by-one sequence
+    m.clear_memo()
+    assert m.check_recompute_batch([q(A), q(B)], memo=True) == [first, after_a]
+    assert len(m.stage_memory_set) > 0
+    m.clear_memo()
+    assert len(m.stage_memory_set) == 0 and m.stage_memory_visit == 0

@@ -70,13 +70,17 @@ def test_plan_keys_separate_distinct_plans_and_key_set_behaves():
     base = synth.make_plans(w, tables, n_plans=3, seed_offset=8)
     nb = PlanBatch.concat([make_neighbours(base.slice(p, p + 1), tables, 4000, np.random.default_rng(p)) for p in range(3)])
     keys = plan_keys_host(nb)
+    assert keys.shape == (nb.n_plans, 2) and keys.dtype == np.uint64
     first = VisitedPlans().unseen(nb)
-    assert len(np.unique(keys)) == int(first.sum())            # no collision, no split
+    as_tuples = [tuple(k) for k in keys.tolist()]
+    assert len(set(as_tuples)) == int(first.sum())             # no collision, no split
+    # (either half alone separates these plans too: the two mixing functions are independent)
+    assert len(np.unique(keys[:, 0])) == int(first.sum()) and len(np.unique(keys[:, 1])) == int(first.sum())
     vk = VisitedKeys()
     assert np.array_equal(vk.unseen(keys), first)
     vk.mark(keys[:5000])
-    seen = set(keys[:5000].tolist())
-    want = first & ~np.array([k in seen for k in keys.tolist()])
+    seen = set(as_tuples[:5000])
+    want = first & ~np.array([k in seen for k in as_tuples])
     assert np.array_equal(vk.unseen(keys), want)
     assert len(vk) == len(seen)
     # the same after the small array has been folded into the large one, and with keys marked twice
@@ -84,13 +88,38 @@ def test_plan_keys_separate_distinct_plans_and_key_set_behaves():
     vk.mark(keys[4000:5000])
     assert len(vk._small) == 0 and len(vk) == len(seen) and np.array_equal(vk.unseen(keys), want)
     vk.mark(keys[4500:5500])
-    seen |= set(keys[5000:5500].tolist())
-    want = first & ~np.array([k in seen for k in keys.tolist()])
+    seen |= set(as_tuples[5000:5500])
+    want = first & ~np.array([k in seen for k in as_tuples])
     assert len(vk) == len(seen) and np.array_equal(vk.unseen(keys), want)
-    # a header-only change (another micro-batch size) changes the key
+    # a header-only change (another micro-batch size) changes both halves of the key
     h = nb.hdr.copy()
     h[:, 0] ^= 1 << 8
     assert not np.any(plan_keys_host(PlanBatch(nb.codes, h)) == keys)
+
+
+def test_plans_that_collide_in_one_half_of_the_key_stay_distinct():
+    """Two plans whose first 64-bit key words are equal (a collision of one mixing function: crafted here by
+    overwriting that word, which is what a 64-bit visited set would have seen) are still two plans to VisitedKeys, in
+    the batch, in the small array and in the large one; the reference's string sets never confuse plans
+    (aceso_utils.py:831-850)."""
+    w = synth.WORKLOADS["gpt3_1_3b"]
+    tables = synth.make_tables(w)
+    nb = make_neighbours(synth.make_plans(w, tables, n_plans=1, seed_offset=3), tables, 64, np.random.default_rng(0))
+    keys = plan_keys_host(nb)
+    distinct = np.flatnonzero(VisitedPlans().unseen(nb))[:6]
+    k = keys[distinct].copy()
+    k[:, 0] = k[0, 0]                                 # all six collide in the first half
+    assert len({tuple(x) for x in k.tolist()}) == 6
+    vk = VisitedKeys()
+    assert vk.unseen(k).all()                         # within one batch
+    vk.mark(k[:2])
+    assert vk.unseen(k).tolist() == [False, False, True, True, True, True]     # against the small array
+    vk.SMALL_LIMIT = 1
+    vk.mark(k[2:4])
+    assert len(vk._small) == 0 and len(vk) == 4
+    assert vk.unseen(k).tolist() == [False, False, False, False, True, True]   # against the large array
+    # and the same plan twice is one plan
+    assert vk.unseen(np.concatenate([k[4:5], k[4:5]])).tolist() == [True, False]
 
 
 @pytest.mark.gpu
@@ -168,7 +197,7 @@ def test_moves_expand_on_the_device_like_on_the_host(name):
         d2, keys = ev.apply_moves(templates, moves, with_keys=True)
         keys = keys.cpu().numpy().view(np.uint64)
         assert np.array_equal(keys, plan_keys_host(host))
-        assert len(np.unique(keys)) == int(VisitedPlans().unseen(host).sum())
+        assert len({tuple(k) for k in keys.tolist()}) == int(VisitedPlans().unseen(host).sum())
         vk = VisitedKeys()
         first = vk.unseen(keys)
         assert np.array_equal(first, VisitedPlans().unseen(host))

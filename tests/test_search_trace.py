@@ -114,24 +114,99 @@ def test_the_searchs_calls_return_what_the_reference_returned_gpu(golden_dir, ca
     check(counts, bad, case)
 
 
-@pytest.mark.parametrize("case", CASES)
-def test_the_references_search_over_the_binding_found_the_same_plans(golden_dir, case):
-    """tests/golden/make_golden.py (child_binding_search) ran the reference's unchanged aceso_search.py a second time
-    with its cost model module replaced by superscaler_amd/binding/aceso_cost_model.py (scoring through the CPU build
-    of the kernel source) and recorded what both runs found: the best time and memory per stage count must be the
-    same numbers.  (That run needs the reference's files and happens where the fixtures are written; this test checks
-    its record, and that the binding still exports what the reference's callers import.)"""
-    with open(os.path.join(golden_dir, f"search_binding_{case}.json")) as f:
+# ---- the searches over the binding: what they found, re-scored by today's code -------------------------------------
+# tests/golden/make_golden.py (child_binding_search) ran the reference's unchanged aceso_search.py twice, once with its
+# cost model module replaced by superscaler_amd/binding/aceso_cost_model.py (scoring through the CPU build of the kernel
+# source) and once on its own cost model, and kept per stage count what each run returned (best time, its peak
+# memory, explored plans) and the plan file each wrote (aceso_utils.py:137-211; per-op lists as runs).  Those runs need
+# the reference's files and happen where the fixtures are written.  The tests below run today's code on the records:
+# every kept plan is scored again -- CPU build of the kernels here, the library on the GPU -- and must give, to the
+# last bit, the time and memory the REFERENCE's cost model gave for that plan file (child_score_plans:
+# "plan_scores_by_the_reference"), for the plan the binding's search wrote and for the one the reference's own wrote.
+# (The number a search returns is the best time it saw; with the fine-tuning actions on, the plan it writes can be
+# another one, so the returned numbers are compared between the two runs and the plans are compared by their scores.)
+
+SWEEP_SETTINGS = {
+    "extras": {}, "stages1568": {}, "imbgpu": {}, "imbop": {},
+    "min": dict(memory_pred_type="MIN"), "noflex": dict(flex_recompute=False), "peakbwd": dict(peak_mem_in_backward=700),
+    "noreserved": dict(consider_reserved_space=False), "noshared": dict(consider_shared_space=False),
+    "collmem": dict(consider_collective_memory=True),
+}
+# (model, size, database directory under tests/golden, micro-batch sizes, gpus per node, global batch, memory limit, layers)
+BINDING_CASES = {
+    "gpt_1_3B": ("gpt", "1_3B", "db_gpt_1_3B", [1, 2, 4, 8], 4, 512, 12000, 24),
+    "resnet_500M": ("resnet", "500M", "db_resnet_500M", [32, 64], 4, 768, 12000, None),
+    "t5_770M": ("t5", "770M", "db_t5_770M", [1, 2, 4, 8], 4, 512, 9000, 24),
+    "gpt_13B": ("gpt", "13B", "kat", [1, 2, 4, 8], 8, 1024, 28000, 40),
+}
+
+
+def binding_model(golden_dir, case, backend, **settings):
+    from superscaler_amd import aceso_cost_model as acm
+    from superscaler_amd.profile_db import CostModelSettings
+    from tests.helpers import EmuEvaluator
+    model, size, db, mbs, gpn, gbs, limit, layers = BINDING_CASES[case]
+    st = CostModelSettings(model_name=model, micro_batch_size=mbs, num_gpus_per_node=gpn, global_batch_size=gbs,
+                           memory_limit=limit, **settings)
+    m = acm.CostModel.from_directory(st, model, size, os.path.join(golden_dir, db) + "/", num_layers=layers)
+    if backend == "emu":
+        m._evaluator = EmuEvaluator(m.tables)
+    return m
+
+
+def rescore(m, fx):
+    """Scores every plan the record keeps; returns how many, after checking each against the recorded numbers."""
+    from superscaler_amd.plan import config_from_json
+    n = 0
+    for side, numbers in (("best_plan_with_the_binding", "with_the_binding"),
+                          ("best_plan_with_the_reference_cost_model", "with_the_reference_cost_model")):
+        for stages, plan in fx[side].items():
+            want = fx["plan_scores_by_the_reference"][side][stages]
+            assert (plan is None) == (want is None) == (fx[numbers][stages] is None), (side, stages)
+            if plan is None:
+                continue
+            assert plan["per_op_lists_as_runs"] and plan["num_stages"] == int(stages)
+            d = dict(plan)
+            for key in ("model_parallel_size_of_each_op", "data_parallel_size_of_each_op", "recompute_ops", "algo_of_each_op"):
+                d[key] = [[v for v, k in runs for _ in range(k)] for runs in plan[key]]
+            c = config_from_json(d, m.graph.ops)
+            m.predict_time_breakdown(c)
+            assert [max(c.time_list), max(c.memory_list)] == want, (side, stages)
+            n += 1
+    return n
+
+
+def check_record(golden_dir, name, backend, case=None, **settings):
+    with open(os.path.join(golden_dir, f"search_binding_{name}.json")) as f:
         fx = json.load(f)
-    assert set(fx["with_the_binding"]) == {"2", "3", "4"}
-    assert fx["with_the_binding"] == fx["with_the_reference_cost_model"]
+    m = binding_model(golden_dir, case or fx["case"], backend, **settings)
+    try:
+        n = rescore(m, fx)
+    finally:
+        if backend == "gpu":
+            m.close()
+    # the two searches returned the same numbers after the same number of explored plans, and wrote the same plan files
+    assert fx["with_the_binding"] == fx["with_the_reference_cost_model"], name
+    assert fx["best_plan_with_the_binding"] == fx["best_plan_with_the_reference_cost_model"], name
+    assert fx["explored_with_the_binding"] == fx["explored_with_the_reference_cost_model"], name
+    return fx, n
+
+
+def _found_the_same_plans(golden_dir, case, backend):
+    fx, n = check_record(golden_dir, case, backend)
+    assert set(fx["with_the_binding"]) == {"2", "3", "4"} and n == 6
     assert all(v is not None and v[0] > 0 for v in fx["with_the_binding"].values())
-    assert all(n >= 4 for n in fx["explored_with_the_binding"].values())
+    assert all(k >= 4 for k in fx["explored_with_the_binding"].values())
     if case == "gpt_1_3B":
         # search/gen_megatron_plan.py, run as the script it is over the binding, wrote the plan files it writes with
         # the reference's own cost model (child_binding_grid)
         assert fx["grid_files_identical"] is True and len(fx["grid_files_with_the_binding"]) == 4
         assert fx["grid_files_with_the_binding"] == fx["grid_files_with_the_reference_cost_model"]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_the_references_search_over_the_binding_found_the_same_plans(golden_dir, case):
+    _found_the_same_plans(golden_dir, case, "emu")
     # aceso_search.py:4, aceso_prims.py:7, gen_megatron_plan.py:8 import these names from aceso_cost_model
     wanted = {"read_profiled_time", "predict_time_breakdown", "update_recompute", "get_reserved_memory_list",
               "wrap_predict_delta_time", "predict_stage_time_helper", "predict_value_after_move", "check_recompute",
@@ -147,46 +222,75 @@ def test_the_references_search_over_the_binding_found_the_same_plans(golden_dir,
     assert all(callable(getattr(api, name)) for name in exported - {"parse_args"})
 
 
+@pytest.mark.gpu
 @pytest.mark.parametrize("case", CASES)
-def test_the_long_search_over_the_binding_found_the_same_plans(golden_dir, case):
+def test_the_references_search_over_the_binding_found_the_same_plans_gpu(golden_dir, case):
+    _found_the_same_plans(golden_dir, case, "gpu")
+
+
+def _long_search(golden_dir, case, backend):
     """The same comparison at ten times the length: 40 trials of up to 7 hops (the hop count of the reference's own
     search scripts), both runs made by the fixture generator at that length (GOLDEN_TRIALS=40 GOLDEN_HOPS=7)."""
-    with open(os.path.join(golden_dir, f"search_binding_{case}__long.json")) as f:
-        fx = json.load(f)
+    fx, n = check_record(golden_dir, f"{case}__long", backend)
     assert fx["flags"][fx["flags"].index("--max-num-trials") + 1] == "40" and fx["flags"][fx["flags"].index("--max-num-hops") + 1] == "7"
-    assert set(fx["with_the_binding"]) == {"2", "3", "4"}
-    assert fx["with_the_binding"] == fx["with_the_reference_cost_model"]
-    assert fx["explored_with_the_binding"] == fx["explored_with_the_reference_cost_model"]
-    assert all(n >= 20 for n in fx["explored_with_the_binding"].values())
+    assert set(fx["with_the_binding"]) == {"2", "3", "4"} and n == 6
+    assert all(k >= 20 for k in fx["explored_with_the_binding"].values())
 
 
-def test_the_search_over_the_binding_under_further_settings(golden_dir):
+@pytest.mark.parametrize("case", CASES)
+def test_the_long_search_over_the_binding_found_the_same_plans(golden_dir, case):
+    _long_search(golden_dir, case, "emu")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", CASES)
+def test_the_long_search_over_the_binding_found_the_same_plans_gpu(golden_dir, case):
+    _long_search(golden_dir, case, "gpu")
+
+
+def _further_settings(golden_dir, backend):
     """The same comparison (short searches) under the reference's other settings: the optional actions with the
     delta-time prediction, MIN memory prediction, no flex recompute, a backward peak, no reserved / no shared space,
     collective memory, 1 / 5 / 6 / 8 stages, the other starting points (make_golden.BINDING_SWEEPS): 27 records, each
-    with the same best plans and the same number of explored plans on both sides."""
+    with the same best plans and the same number of explored plans on both sides; every plan re-scored under the
+    record's settings."""
     import glob
     files = sorted(glob.glob(os.path.join(golden_dir, "search_binding_*__sweep_*.json")))
     assert len(files) == 27
-    names = set()
+    names, plans = set(), 0
     for path in files:
-        with open(path) as f:
-            fx = json.load(f)
-        names.add(os.path.basename(path).split("__sweep_")[1][:-5])
-        assert fx["with_the_binding"] == fx["with_the_reference_cost_model"], path
-        assert fx["explored_with_the_binding"] == fx["explored_with_the_reference_cost_model"], path
-        assert any(v is not None for v in fx["with_the_binding"].values()), path
-    assert names == {"extras", "min", "noflex", "peakbwd", "noreserved", "noshared", "stages1568", "imbgpu", "collmem", "imbop"}
+        name = os.path.basename(path)[len("search_binding_"):-5]
+        sweep = name.split("__sweep_")[1]
+        names.add(sweep)
+        fx, n = check_record(golden_dir, name, backend, **SWEEP_SETTINGS[sweep])
+        assert n >= 2, path
+        plans += n
+    assert names == set(SWEEP_SETTINGS) and plans >= 140
+
+
+def test_the_search_over_the_binding_under_further_settings(golden_dir):
+    _further_settings(golden_dir, "emu")
+
+
+@pytest.mark.gpu
+def test_the_search_over_the_binding_under_further_settings_gpu(golden_dir):
+    _further_settings(golden_dir, "gpu")
+
+
+def _on_32_gpus(golden_dir, backend):
+    """GPT-13B (523 ops) on 4 nodes of 8 GPUs -- tensor parallelism up to 8, stages across node boundaries -- with 4, 5, 6, 8
+    and 16 pipeline stages, 8 trials of up to 5 hops: same best plans and same number of explored plans (437 to 17,270)
+    over the binding as with the reference's own cost model; the ten plans re-scored."""
+    fx, n = check_record(golden_dir, "gpt_13B__big", backend)
+    assert set(fx["with_the_binding"]) == {"4", "5", "6", "8", "16"} and n == 10
+    assert all(v is not None and v[1] <= 28000 for v in fx["with_the_binding"].values())
+    assert max(fx["explored_with_the_binding"].values()) > 10000
 
 
 def test_the_search_over_the_binding_on_32_gpus(golden_dir):
-    """GPT-13B (523 ops) on 4 nodes of 8 GPUs -- tensor parallelism up to 8, stages across node boundaries -- with 4, 5, 6, 8
-    and 16 pipeline stages, 8 trials of up to 5 hops: same best plans and same number of explored plans (437 to 17,270)
-    over the binding as with the reference's own cost model."""
-    with open(os.path.join(golden_dir, "search_binding_gpt_13B__big.json")) as f:
-        fx = json.load(f)
-    assert set(fx["with_the_binding"]) == {"4", "5", "6", "8", "16"}
-    assert fx["with_the_binding"] == fx["with_the_reference_cost_model"]
-    assert fx["explored_with_the_binding"] == fx["explored_with_the_reference_cost_model"]
-    assert all(v is not None and v[1] <= 28000 for v in fx["with_the_binding"].values())
-    assert max(fx["explored_with_the_binding"].values()) > 10000
+    _on_32_gpus(golden_dir, "emu")
+
+
+@pytest.mark.gpu
+def test_the_search_over_the_binding_on_32_gpus_gpu(golden_dir):
+    _on_32_gpus(golden_dir, "gpu")

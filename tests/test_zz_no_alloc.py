@@ -11,12 +11,13 @@ from superscaler_amd import synth
 pytestmark = pytest.mark.gpu
 
 
-def _raw_scores(ev, torch, entry, d, limit):
-    P = d.n_plans
-    it = torch.full((P,), -1.0, dtype=torch.float64, device=ev.device)
-    pk = torch.full((P,), -1.0, dtype=torch.float64, device=ev.device)
-    fe = torch.full((P,), 9, dtype=torch.uint8, device=ev.device)
-    st = torch.full((P,), 9, dtype=torch.uint8, device=ev.device)
+def _outputs(ev, torch, P):
+    return (torch.full((P,), -1.0, dtype=torch.float64, device=ev.device), torch.full((P,), -1.0, dtype=torch.float64, device=ev.device),
+            torch.full((P,), 9, dtype=torch.uint8, device=ev.device), torch.full((P,), 9, dtype=torch.uint8, device=ev.device))
+
+
+def _raw_call(ev, torch, entry, d, limit, outs):
+    it, pk, fe, st = outs
     stream = ctypes.c_void_p(torch.cuda.current_stream(ev.device).cuda_stream)
     with ev.device_context():
         if entry == "static":
@@ -27,7 +28,12 @@ def _raw_scores(ev, torch, entry, d, limit):
                                         fe.data_ptr(), st.data_ptr(), None, stream)
     assert rc == 0, ev.lib.ace_strerror(rc)
     torch.cuda.synchronize()
-    return [t.cpu().numpy() for t in (it, pk, fe, st)]
+
+
+def _raw_scores(ev, torch, entry, d, limit):
+    outs = _outputs(ev, torch, d.n_plans)
+    _raw_call(ev, torch, entry, d, limit, outs)
+    return [t.cpu().numpy() for t in outs]
 
 
 @pytest.mark.parametrize("name,sizes", [("gpt3_13b", (16384, 5000)), ("gpt3_1_3b", (3000, 64)), ("wresnet_1b", (2048, 700))])
@@ -37,13 +43,23 @@ def test_static_entry_point_equals_score_batch(name, sizes):
     w = synth.WORKLOADS[name]
     tables = synth.make_tables(w)
     limit = float(tables.settings.memory_limit)
-    ev = PlanEvaluator(tables)
+    ev = PlanEvaluator(tables)          # the handle the static entry point is called on: ace_score_batch never runs on it
+    ref = PlanEvaluator(tables)         # a second handle, for what ace_score_batch returns
     try:
         batches = [synth.make_plans(w, tables, n_plans=n, seed_offset=40 + k) for k, n in enumerate(sizes)]
         dev = [ev.upload(b) for b in batches]
-        want = [_raw_scores(ev, torch, "plain", d, limit) for d in dev]
+        want = [_raw_scores(ref, torch, "plain", ref.upload(b), limit) for b in batches]
+        # the handle has no workspace of its own and may not get one: a call that allocated would fail with ACE_EFIXED
+        with ev.device_context():
+            assert ev.lib.ace_reserve(ev.handle, 0, 1) == 0
+        outs = [_outputs(ev, torch, d.n_plans) for d in dev]
+        torch.cuda.synchronize()
         free0 = torch.cuda.mem_get_info()[0]
-        got = [_raw_scores(ev, torch, "static", d, limit) for d in dev]          # two calls in a row, the second smaller
+        for d, o in zip(dev, outs):                                              # two calls in a row, the second smaller
+            _raw_call(ev, torch, "static", d, limit, o)
+        # outputs were allocated beforehand: the device's free memory is what it was
+        assert torch.cuda.mem_get_info()[0] == free0
+        got = [[t.cpu().numpy() for t in o] for o in outs]
         for g, x in zip(got, want):
             for a, b in zip(g, x):
                 assert np.array_equal(a, b, equal_nan=True)
@@ -51,8 +67,13 @@ def test_static_entry_point_equals_score_batch(name, sizes):
         # the second call again after the first (records of the larger batch are still in the scratch)
         again = _raw_scores(ev, torch, "static", dev[1], limit)
         assert all(np.array_equal(a, b, equal_nan=True) for a, b in zip(again, want[1]))
-        # (outputs of _raw_scores are the only tensors made in between: at most a few MiB of cached blocks)
-        assert free0 - torch.cuda.mem_get_info()[0] < (8 << 20)
+        # the plain entry point on this handle would have to allocate its workspace now: refused, as fixed above
+        # (tables whose rows are windowed need no workspace)
+        o = _outputs(ev, torch, dev[0].n_plans)
+        with ev.device_context():
+            rc = ev.lib.ace_score_batch(ev.handle, ctypes.byref(dev[0].struct), limit, 0, o[0].data_ptr(), o[1].data_ptr(),
+                                        o[2].data_ptr(), o[3].data_ptr(), None, None)
+        assert rc == (0 if tables.n_windows > 1 else -6), rc
         # beyond the stated maximum: refused, nothing launched
         big = ev.upload(synth.make_plans(w, tables, n_plans=16385, seed_offset=44))
         it = torch.zeros(16385, dtype=torch.float64, device=ev.device)
@@ -63,3 +84,4 @@ def test_static_entry_point_equals_score_batch(name, sizes):
         assert rc == -2 and ev.lib.ace_strerror(rc)
     finally:
         ev.close()
+        ref.close()

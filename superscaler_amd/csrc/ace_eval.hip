@@ -600,7 +600,9 @@ struct ace_handle {
     // device copies
     double *d_rows;
     uint32_t *d_pos_info;
-    ace_u4 *d_pos4;            // per position, for the assembly op loop (null when the rows are windowed)
+    uint32_t *d_pos_types;     // d_pos_info with row indices in place of LDS slots (windowed rows, at most 256 of them; else null)
+    ace_u4 *d_pos4;            // per position, for the assembly op loop (null when its pair-kind table has no room in LDS)
+    ace_u4 *d_win_dma;         // windowed rows: the LDS-direct loads that stage each window, per wavefront (assembly op loop), or null
     uint8_t *d_pair_kinds;
     uint32_t *d_stage_lut;
     double *d_nbm1;
@@ -691,7 +693,7 @@ template <bool BD, bool RANGED, bool WIN, bool DEFER> static int allow_big_lds()
 // start" does NOT apply here, bit 1: ordinary op).  Positions past the last op point at row 0 and pair kind 0.
 static int upload_pos4(ace_handle *h, const ace_tables_t *t, size_t pos_entries, uint32_t pk32_off) {
     h->d_pos4 = nullptr;
-    if (t->n_windows != 1 || !pk32_off) return ACE_OK;
+    if (!pk32_off) return ACE_OK;
     ace_u4 *p4 = new (std::nothrow) ace_u4[pos_entries];
     if (!p4) return ACE_ENOMEM;
     const uint32_t row_bytes = (uint32_t)t->row_doubles * 8u, kind_stride = (uint32_t)t->n_glog * 64u;
@@ -705,6 +707,65 @@ static int upload_pos4(ace_handle *h, const ace_tables_t *t, size_t pos_entries,
     }
     const int rc = upload((void **)&h->d_pos4, p4, pos_entries * sizeof(ace_u4));
     delete[] p4;
+    return rc;
+}
+
+// Windowed rows: the position descriptors with each row's index in `rows` where its LDS slot is.
+static int upload_pos_types(ace_handle *h, const ace_tables_t *t, size_t pos_entries) {
+    h->d_pos_types = nullptr;
+    if (t->n_windows <= 1 || t->num_types > 256) return ACE_OK;
+    uint32_t *pt = new (std::nothrow) uint32_t[pos_entries];
+    if (!pt) return ACE_ENOMEM;
+    ace_pos_types(t, pt, pos_entries);
+    const int rc = upload((void **)&h->d_pos_types, pt, pos_entries * 4);
+    delete[] pt;
+    return rc;
+}
+
+// Windowed rows, for the assembly op loop: the rows of window w as LDS-direct loads of at most 1 KB (64 lanes x 16 bytes),
+// dealt to the sixteen wavefronts of a workgroup in turn: [window][wavefront][j] = {byte offset in rows, LDS address, bytes, 0}.
+static int upload_win_dma(ace_handle *h, const ace_tables_t *t) {
+    h->d_win_dma = nullptr;
+    if (t->n_windows <= 1 || !h->d_pos4 || !h->d_pos_types) return ACE_OK;
+    const uint64_t row_bytes = (uint64_t)t->row_doubles * 8u;
+    if ((uint64_t)t->num_types * row_bytes > 0xffffffffull) return ACE_OK;
+    const uint32_t per_row = (uint32_t)((row_bytes + 1023u) / 1024u);
+    uint32_t most = 0;
+    for (int w = 0; w < t->n_windows; ++w) {
+        const uint32_t n = (uint32_t)(t->win_row_begin[w + 1] - t->win_row_begin[w]) * per_row;
+        most = n > most ? n : most;
+    }
+    const int32_t J = (int32_t)((most + 15u) / 16u);
+    if (J <= 0) return ACE_OK;
+    // If no window's rows overlap those of the window before it in LDS, a window can be fetched while the one before it
+    // is walked (the loop then asks for window w + 1 when it enters window w: one more, empty, window ends the table).
+    uint32_t ahead = 1;
+    for (int w = 0; w + 1 < t->n_windows && ahead; ++w)
+        for (int r = t->win_row_begin[w]; r < t->win_row_begin[w + 1] && ahead; ++r)
+            for (int q = t->win_row_begin[w + 1]; q < t->win_row_begin[w + 2]; ++q) {
+                const uint64_t a0 = t->win_rows[2 * r + 1], b0 = t->win_rows[2 * q + 1];
+                if (a0 < b0 + row_bytes && b0 < a0 + row_bytes) { ahead = 0; break; }
+            }
+    const size_t entries = 2u + (size_t)(t->n_windows + 1) * 16u * (size_t)J;      // (two entries of header)
+    ace_u4 *d0 = new (std::nothrow) ace_u4[entries];
+    if (!d0) return ACE_ENOMEM;
+    for (size_t i = 0; i < entries; ++i) d0[i] = ace_u4{0u, 0u, 0u, 0u};
+    const uint64_t rows_at = (uint64_t)(uintptr_t)h->d_rows, win_at = (uint64_t)(uintptr_t)h->d_win_pos;
+    d0[0] = ace_u4{(uint32_t)rows_at, (uint32_t)(rows_at >> 32), (uint32_t)win_at, (uint32_t)(win_at >> 32)};
+    d0[1] = ace_u4{(uint32_t)J, (uint32_t)J * 256u, ahead, 0u};
+    ace_u4 *d = d0 + 2;
+    for (int w = 0; w < t->n_windows; ++w) {
+        uint32_t c = 0;
+        for (int r = t->win_row_begin[w]; r < t->win_row_begin[w + 1]; ++r)
+            for (uint32_t k = 0; k < per_row; ++k, ++c) {
+                const uint64_t left = row_bytes - (uint64_t)k * 1024u;
+                d[((size_t)w * 16u + (c & 15u)) * (size_t)J + (c >> 4)] =
+                    ace_u4{(uint32_t)(t->win_rows[2 * r] * row_bytes + k * 1024u), t->win_rows[2 * r + 1] + k * 1024u,
+                           (uint32_t)(left < 1024u ? left : 1024u), 0u};
+            }
+    }
+    const int rc = upload((void **)&h->d_win_dma, d0, entries * sizeof(ace_u4));
+    delete[] d0;
     return rc;
 }
 
@@ -757,10 +818,10 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     uint32_t stg_off, lut2_off;
     uint32_t lds_bytes = ace_lds_layout(rk_off, (uint32_t)rk_bytes, (uint32_t)stg_words, &stg_off, &lut2_off);
     if (lds_bytes > kMaxLds) return ACE_ETOOBIG;
-    // the assembly loop's pair-kind table, where every row is resident, the table has room and its entries can hold
-    // the offsets (otherwise plain scoring takes the C++ form of the loop)
+    // the assembly loop's pair-kind table, where the table has room and its entries can hold the offsets (otherwise plain
+    // scoring takes the C++ form of the loop)
     uint32_t pk32_off = 0;
-    if (t->n_windows == 1) {
+    if (t->n_windows == 1 || t->num_types <= 256) {        // (windowed rows: the loop's caller needs d_pos_types as well)
         uint32_t off;
         const uint32_t end = ace_lds_pk32(lds_bytes, (uint32_t)rk_bytes, &off);
         if (end <= kMaxLds && ((int64_t)(t->n_z > 0 ? t->n_z : 1) * t->z_table_doubles * 8) <= 65536) {
@@ -827,16 +888,18 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
         (rc = upload((void **)&h->d_rows, t->rows, (size_t)t->num_types * row_bytes)) ||
         (rc = upload((void **)&h->d_pos_info, t->pos_info, (size_t)(t->num_ops + 1) * 4, pos_entries * 4)) ||
         (rc = upload_pos4(h, t, pos_entries, pk32_off)) ||
+        (rc = upload_pos_types(h, t, pos_entries)) ||
         (rc = upload((void **)&h->d_pair_kinds, t->pair_kinds, (size_t)rk_bytes)) ||
         (rc = upload((void **)&h->d_stage_lut, t->stage_lut, (size_t)stg_words * 4)) ||
         (rc = upload((void **)&h->d_nbm1, t->nb_minus_1, (size_t)t->n_mbs * 8)) ||
         (rc = upload((void **)&h->d_win_pos, t->win_pos, (size_t)(t->n_windows + 1) * 4)) ||
         (rc = upload((void **)&h->d_win_row_begin, t->win_row_begin, (size_t)(t->n_windows + 1) * 4)) ||
         (rc = upload((void **)&h->d_win_rows, t->win_rows, (size_t)n_win_rows * 8)) ||
+        (rc = upload_win_dma(h, t)) ||
         (rc = hipFuncSetAttribute(reinterpret_cast<const void *>(&topk_short_final), hipFuncAttributeMaxDynamicSharedMemorySize,
                                   (int)kShortLds) == hipSuccess ? ACE_OK : ACE_EHIP) ||
         (rc = allow_big_lds<false, false, false, false>()) || (rc = allow_big_lds<false, false, true, false>()) ||
-        (rc = allow_big_lds<false, false, false, true>()) ||
+        (rc = allow_big_lds<false, false, false, true>()) || (rc = allow_big_lds<false, false, true, true>()) ||
         (rc = allow_big_lds<true, false, false, false>()) || (rc = allow_big_lds<true, false, true, false>()) ||
         (rc = allow_big_lds<true, true, false, false>()) || (rc = allow_big_lds<true, true, true, false>())) {
         ace_destroy(h);
@@ -848,8 +911,9 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
 
 void ace_destroy(ace_handle_t *h) {
     if (!h) return;
-    (void)hipFree(h->d_rows); (void)hipFree(h->d_pos_info); (void)hipFree(h->d_pair_kinds);
+    (void)hipFree(h->d_rows); (void)hipFree(h->d_pos_info); (void)hipFree(h->d_pos_types); (void)hipFree(h->d_pair_kinds);
     if (h->d_pos4) (void)hipFree(h->d_pos4);
+    if (h->d_win_dma) (void)hipFree(h->d_win_dma);
     (void)hipFree(h->d_stage_lut); (void)hipFree(h->d_nbm1); (void)hipFree(h->d_win_pos);
     (void)hipFree(h->d_win_row_begin); (void)hipFree(h->d_win_rows);
     if (h->d_stage_ws) (void)hipFree(h->d_stage_ws);
@@ -871,7 +935,7 @@ static int fill_args(ace_handle_t *h, const ace_batch_t *b, double memory_limit,
     a->hdr = reinterpret_cast<const ace_u4 *>(b->d_hdr);
     a->range = reinterpret_cast<const ace_u2 *>(b->d_range);
     a->order = b->d_order;
-    a->rows = h->d_rows; a->pos_info = h->d_pos_info; a->pos4 = h->d_pos4; a->pair_kinds = h->d_pair_kinds; a->stage_lut = h->d_stage_lut;
+    a->rows = h->d_rows; a->pos_info = h->d_pos_info; a->pos_types = h->d_pos_types; a->pos4 = h->d_pos4; a->win_dma = h->d_win_dma; a->pair_kinds = h->d_pair_kinds; a->stage_lut = h->d_stage_lut;
     a->nbm1 = h->d_nbm1; a->win_pos = h->d_win_pos; a->win_row_begin = h->d_win_row_begin; a->win_rows = h->d_win_rows;
     a->n_windows = h->n_windows; a->row_doubles = h->row_doubles; a->rk_bytes = h->rk_bytes; a->stg_words = h->stg_words;
     a->iter_ms = d_iter_ms; a->peak_mb = d_peak_mb; a->feasible = d_feasible; a->status = d_status; a->stage_out = d_stage_out;
@@ -905,6 +969,7 @@ static void launch_score_w(const ace_handle_t *h, const AceKernelArgs &a, hipStr
 static void launch_score(const ace_handle_t *h, const AceKernelArgs &a, hipStream_t s) {
     if (a.range) launch_score_w<true, true>(h, a, s);
     else if (a.stage_out) launch_score_w<true, false>(h, a, s);
+    else if (a.stage_ws && h->n_windows > 1) launch_score_b<false, false, true, true>(h, a, s);
     else if (a.stage_ws) launch_score_b<false, false, false, true>(h, a, s);
     else launch_score_w<false, false>(h, a, s);
 }
@@ -913,7 +978,7 @@ static void launch_score(const ace_handle_t *h, const AceKernelArgs &a, hipStrea
 // per-plan workspace; the handle keeps one and grows it on demand.
 static int ensure_stage_ws(ace_handle_t *h, AceKernelArgs *a) {
     a->stage_ws = nullptr;
-    if (a->range || a->stage_out || h->n_windows > 1 || h->geom.N >= 65536 || (h->geom.flags & ACE_F_COLLECTIVE_MEM)) return ACE_OK;
+    if (a->range || a->stage_out || (h->n_windows > 1 && !h->d_pos_types) || h->geom.N >= 65536 || (h->geom.flags & ACE_F_COLLECTIVE_MEM)) return ACE_OK;
     const size_t need = (((size_t)a->g.P + kBlock - 1) / kBlock) * kBlock;
     if (need * ACE_MAX_STAGES * (ACE_WS_REC / 2) > 0xffffffffull) return ACE_OK;   // 32-bit record offsets: larger batches take the plain kernel
     if (need > h->stage_ws_plans) {
@@ -966,7 +1031,7 @@ int ace_score_batch_static(ace_handle_t *h, const ace_batch_t *batch, double mem
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev != h->device || dev < 0 || dev >= kMaxDevices) return ACE_EINVAL;
     // (the same test as ensure_stage_ws: tables that take the kernels without deferred stage tails need no scratch)
-    const bool deferred = !(h->n_windows > 1 || h->geom.N >= 65536 || (h->geom.flags & ACE_F_COLLECTIVE_MEM));
+    const bool deferred = !((h->n_windows > 1 && !h->d_pos_types) || h->geom.N >= 65536 || (h->geom.flags & ACE_F_COLLECTIVE_MEM));
     // looked up by ace_create on this device; the padded plan count of either workgroup size fits: ACE_STATIC_MAX_PLANS is a multiple of kBlock
     a.stage_ws = deferred ? g_static_ptr[dev] : nullptr;
     if (deferred && !a.stage_ws) return ACE_EINVAL;

@@ -33,6 +33,12 @@
 struct AceLds {
     const unsigned char *base;
     uint32_t size;
+    const unsigned char *grows = nullptr;     // the table rows as the caller holds them (behind the caller's guard pages)
+    template <class T> T gld(uint32_t off) const {
+        T v;
+        memcpy(&v, grows + off, sizeof(T));
+        return v;
+    }
     template <class T> T ld(uint32_t off) const {
         if ((uint64_t)off + sizeof(T) > size || (off % (sizeof(T) > 16 ? 16 : sizeof(T))) != 0) {
             fprintf(stderr, "ace emu: LDS access out of bounds/misaligned: off=%u size=%zu lds=%u\n", off, sizeof(T), size);
@@ -54,6 +60,12 @@ static inline double ace_max(double a, double b) { return a > b ? a : b; }
 // instructions per op.  ace_lds_base() exposes it as a number, and the caller adds it to the
 // wave-uniform region offsets once (scalar arithmetic), so per-lane address math never sees it.
 struct AceLds {
+    const unsigned char *grows;     // the table rows in global memory (replay of deferred stage tails over windowed rows)
+    template <class T> ACE_HD T gld(uint32_t off) const {
+        T v;
+        __builtin_memcpy(&v, grows + off, sizeof(T));
+        return v;
+    }
     template <class T> ACE_HD T ld(uint32_t addr) const {
 #if defined(__HIP_DEVICE_COMPILE__)
         typedef const unsigned char __attribute__((address_space(3))) *lptr;
@@ -66,7 +78,7 @@ struct AceLds {
 #endif
     }
 };
-ACE_HD AceLds ace_make_lds(const unsigned char *, uint32_t) { return AceLds{}; }
+ACE_HD AceLds ace_make_lds(const unsigned char *, uint32_t) { return AceLds{nullptr}; }
 ACE_HD uint32_t ace_lds_base(const unsigned char *lds) {
 #if defined(__HIP_DEVICE_COMPILE__)
     typedef const unsigned char __attribute__((address_space(3))) *lptr;
@@ -174,7 +186,14 @@ uint32_t ace_lds_pk32(uint32_t lds_end, uint32_t rk_bytes, uint32_t *pk32_off) {
 // BD: per-stage records for the caller.  RANGED: one stage over an op sub-range.  DEFER: stage
 // tails are not evaluated where the stage ends (where only the few lanes that cut at this op are
 // active) but stashed to a per-plan workspace and replayed after the op loop with every lane busy.
-template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false> struct PlanState {
+// GROWS (with DEFER): the rows are windowed, so replay() looks the stage boundaries up in the rows' global copy (`gr`: the
+// geometry with row offsets as they are there).
+template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false, bool GROWS = false> struct PlanState {
+    template <class T> ACE_HD static T row_ld(const AceLds &lds, uint32_t a) {
+        if (GROWS) return lds.template gld<T>(a);
+        return lds.template ld<T>(a);
+    }
+
     // plan constants
     int S;
     uint32_t bidx;
@@ -308,8 +327,8 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false> struct Pl
         out_cross = (cross >> (16u + sidx)) & 1u;
         t_first = c >> g.A_shift;
         uint32_t a = row + g.start_off + (dc_v + c) * ACE_START_STRIDE;
-        inputs = lds.ld<double>(a);                                 // input size
-        in_comm = lds.ld<double>(a + (in_cross ? 16u : 8u));        // size / inter- or intra-node bandwidth
+        inputs = row_ld<double>(lds, a);                                 // input size
+        in_comm = row_ld<double>(lds, a + (in_cross ? 16u : 8u));        // size / inter- or intra-node bandwidth
         if (BD) {
             uint32_t ai = row + g.start_off + ideal_start_v + (c & (uint32_t)(g.n_algo - 1)) * ACE_START_STRIDE;
             id_in = lds.ld<double>(ai + (in_cross ? 16u : 8u));
@@ -388,7 +407,7 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false> struct Pl
         if (m_last >= (uint32_t)g.n_mbs) m_last = 0;   // only for plans whose sums are NaN already
         // output_size[ops[-1]][mbs[-1]][tp[0]][algo[-1]]  (sic, aceso_cost_model.py:321-326)
         uint32_t oidx = ((m_last * (uint32_t)g.n_tp + t_first) << g.A_shift) + a_last;
-        ace_d2 oe = lds.ld<ace_d2>(lastrow + g.out_off + oidx * 16u);
+        ace_d2 oe = row_ld<ace_d2>(lds, lastrow + g.out_off + oidx * 16u);
         double out_comm = out_cross ? oe.y : oe.x;
         double in_c = in_comm + rs_f * 1000.0;      // :352
         double out_c = out_comm + rs_b * 1000.0;    // :353

@@ -25,6 +25,7 @@ struct AceKernelArgs {
     const uint32_t *order;      // [P] result index of the plan in each slot, or null (slot i -> result i)
     const double *rows;         // [n_types][row_doubles]
     const uint32_t *pos_info;   // [N + 1], padded to 16 * G + 16 entries
+    const uint32_t *pos_types;  // windowed rows: the same with each row's index in `rows` in place of its LDS slot (null: more than 256 rows)
     const ace_u4 *pos4;         // [16 * G + 16] per position: LDS address of its row's hot sub-table, of its cost tables, of the
                                 //   32-bit pair-kind block of the (this, next) pair; bit 0: no layer start follows an ordinary op here, bit 1: ordinary op
     const uint8_t *pair_kinds;  // -> LDS
@@ -33,12 +34,30 @@ struct AceKernelArgs {
     const int32_t *win_pos;     // [n_windows + 1], multiples of 4
     const int32_t *win_row_begin;
     const uint32_t *win_rows;   // pairs (type, lds byte offset)
+    const ace_u4 *win_dma;      // what the assembly op loop stages the windows from (see ace_score_loop_asm), or null
     int32_t n_windows, row_doubles, rk_bytes, stg_words;
     double *iter_ms, *peak_mb;
     uint8_t *feasible, *status;
     double *stage_out;          // [P][ACE_MAX_STAGES][ACE_STAGE_REC], single-stage queries [P][ACE_STAGE_REC]
     double *stage_ws;           // [ACE_MAX_STAGES][plans rounded up to whole workgroups][ACE_WS_REC] for deferred stage tails
 };
+
+// Windowed rows: the position descriptors (pos_info) with each row's index in `rows` where its LDS slot is; positions
+// past the last op read zero.  (Host side: what the library uploads as AceKernelArgs::pos_types.)
+inline void ace_pos_types(const ace_tables_t *t, uint32_t *out, size_t entries) {
+    const uint32_t row_bytes = (uint32_t)t->row_doubles * 8u;
+    int w = 0;
+    for (size_t i = 0; i < entries; ++i) {
+        out[i] = 0u;
+        if (i >= (size_t)t->num_ops) continue;
+        while (w + 1 < t->n_windows && (size_t)t->win_pos[w + 1] <= i) ++w;
+        const uint32_t info = t->pos_info[i], slot_off = (info & 0xffu) * row_bytes;
+        uint32_t type = 0;
+        for (int r = t->win_row_begin[w]; r < t->win_row_begin[w + 1]; ++r)
+            if (t->win_rows[2 * r + 1] == slot_off) type = t->win_rows[2 * r];
+        out[i] = (info & 0xffff0000u) | type;
+    }
+}
 
 // Copy the rows window `w` needs from global memory into LDS (whole workgroup).
 template <int BLOCK> ACE_HD void stage_window(const AceKernelArgs &a, unsigned char *lds_raw, int w, int tid) {
@@ -57,12 +76,36 @@ template <int BLOCK> ACE_HD void stage_window(const AceKernelArgs &a, unsigned c
 // gen_score_loop_asm.py, which describes it): walks all ops of this lane's plan, parks every finished stage in the
 // lane's workspace records like PlanState::stash(), and returns the number of stages closed.  LDS addresses in `pos4`
 // are absolute: the caller checks that the workgroup's LDS array starts at address 0.
+// WIN: the rows are windowed; the loop restages them itself.  a.win_dma: {address of the rows, address of the window
+// starts, J, bytes of descriptors per window}, then per window and wavefront (sixteen) J descriptors {byte offset in the
+// rows, LDS address, bytes (at most 1,024), 0} of LDS-direct loads.
+template <bool WIN>
 __device__ __forceinline__ uint32_t ace_score_loop_asm(const AceKernelArgs &a, const AceGeom &g, uint64_t dg, uint64_t rks,
-                                                       uint32_t code_off, double *rec, uint32_t ws_stride, uint32_t prio = 0) {
+                                                       uint32_t code_off, double *rec, uint32_t ws_stride, uint32_t prio, uint32_t wave) {
     uint32_t cnt;
     const uint64_t gstride = (uint64_t)(uint32_t)g.P * 16u;
     const uint32_t gs_lo = (uint32_t)gstride, gs_hi = (uint32_t)(gstride >> 32);
     const uint32_t c8 = (uint32_t)g.C * 8u;
+    if (WIN) {
+#define ACE_LOOP_ASM_RUN(TEXT)                                                                                          \
+    asm volatile(TEXT : [cnt] "=&v"(cnt)                                                                               \
+                 : [dg] "v"(dg), [rk] "v"(rks), [codeoff] "v"(code_off), [rec] "v"(rec), [codes] "s"(a.codes),         \
+                   [pos] "s"(a.pos4), [c8] "s"(c8), [n_ops] "s"(g.N), [n_groups] "s"(g.G),                                \
+                   [gstride_lo] "s"(gs_lo), [gstride_hi] "s"(gs_hi), [wsstride] "s"(ws_stride), [prio] "s"(prio),       \
+                   [dma] "s"(a.win_dma), [wave] "s"(wave)                                                               \
+                 : ACE_LOOP_ASM_CLOBBERS)
+        if (g.flags & ACE_F_RESHARDING) {
+            if (g.flags & ACE_F_NO_RESERVED) ACE_LOOP_ASM_RUN(ACE_LOOP_ASM_WIN_RSH1_NONE);
+            else if (g.flags & ACE_F_RESERVED_MIN) ACE_LOOP_ASM_RUN(ACE_LOOP_ASM_WIN_RSH1_MIN);
+            else ACE_LOOP_ASM_RUN(ACE_LOOP_ASM_WIN_RSH1_MAX);
+        } else {
+            if (g.flags & ACE_F_NO_RESERVED) ACE_LOOP_ASM_RUN(ACE_LOOP_ASM_WIN_RSH0_NONE);
+            else if (g.flags & ACE_F_RESERVED_MIN) ACE_LOOP_ASM_RUN(ACE_LOOP_ASM_WIN_RSH0_MIN);
+            else ACE_LOOP_ASM_RUN(ACE_LOOP_ASM_WIN_RSH0_MAX);
+        }
+#undef ACE_LOOP_ASM_RUN
+        return cnt;
+    }
 #define ACE_LOOP_ASM_RUN(TEXT)                                                                                          \
     asm volatile(TEXT : [cnt] "=&v"(cnt)                                                                               \
                  : [dg] "v"(dg), [rk] "v"(rks), [codeoff] "v"(code_off), [rec] "v"(rec), [codes] "s"(a.codes),         \
@@ -86,12 +129,13 @@ __device__ __forceinline__ uint32_t ace_score_loop_asm(const AceKernelArgs &a, c
 // BD: also write per-stage records.  RANGED: each plan is one stage over an op sub-range.
 // WIN: the rows of all op types do not fit in LDS together; restage at window boundaries.
 // DEFER: stage tails are stashed in the workspace and evaluated after the op loop, when all lanes
-// are active again (needs every row resident, so never together with WIN).
+// are active again (together with WIN the boundary lookups of that evaluation read the rows in global memory,
+// a.pos_types naming each position's row there).
 // `tid` lane of workgroup `block` of `n_blocks`, BLOCK lanes each; `lds_raw`: the workgroup's LDS (`lds_bytes` long).
 template <bool BD, bool RANGED, bool WIN, bool DEFER, int BLOCK, bool COLL = false>
 ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint32_t lds_bytes, int tid, long long block,
                            uint32_t n_blocks) {
-    static_assert(!DEFER || (!BD && !RANGED && !WIN && !COLL), "deferred stage tails: plain scoring only");
+    static_assert(!DEFER || (!BD && !RANGED && !COLL), "deferred stage tails: plain scoring only");
     // region offsets as absolute LDS addresses for the reads (see AceLds); the staging loops below
     // write through `lds_raw` with the plain offsets of a.g
     AceGeom g = a.g;
@@ -192,8 +236,9 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     stage_window<BLOCK>(a, lds_raw, w0, tid);       // every row, or the first window's
     ACE_SYNC();
 
-    const AceLds lds = ace_make_lds(lds_raw, lds_bytes);
-    PlanState<BD, RANGED, DEFER, COLL> st;
+    AceLds lds = ace_make_lds(lds_raw, lds_bytes);
+    lds.grows = reinterpret_cast<const unsigned char *>(a.rows);
+    PlanState<BD, RANGED, DEFER, COLL, DEFER && WIN> st;
     const ace_u4 h = a.hdr[pl];
     st.init(g, lds, h, range);
     const double nbm1 = a.nbm1[st.bidx];
@@ -212,12 +257,13 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     const uint32_t first_code = cw.x & 7u;
     int grp_stop = grp_end;
 #ifndef ACE_HOST_EMU
-    if (DEFER && lds_base == 0u && a.pos4) {
+    if (DEFER && lds_base == 0u && a.pos4 && (!WIN || (BLOCK == 1024 && a.win_dma))) {
         // the assembly form of the loop below (same operations per plan, same results)
         if (!(cw.x & 0x10u)) st.status = ACE_PLAN_MALFORMED;    // the first op must open a stage
         uint64_t dg, rks;
         st.stage_nibbles(g, lds, dg, rks);
-        st.s = (int)ace_score_loop_asm(a, g, dg, rks, (uint32_t)pl * 16u, rec, st.ws_stride, prio);
+        st.s = (int)ace_score_loop_asm<WIN>(a, g, dg, rks, (uint32_t)pl * 16u, rec, st.ws_stride, prio,
+                                            (uint32_t)__builtin_amdgcn_readfirstlane(tid >> 6));
         grp_stop = grp_begin;
     } else
 #endif
@@ -279,7 +325,15 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
         for (int s2 = 0; s2 < ACE_MAX_STAGES; ++s2) {
             const bool live = s2 < n_st;
             if (!ACE_ANY(live)) break;
-            if (live) st.replay(g, lds, a.pos_info, rec, s2);
+            if (!live) continue;
+            if (WIN) {
+                // (row offsets as the rows lie in global memory)
+                AceGeom gr = g;
+                gr.start_off -= lds_base; gr.out_off -= lds_base;
+                gr.row_bytes = (uint32_t)a.row_doubles * 8u;
+                st.replay(gr, lds, a.pos_types, rec, s2);
+            } else
+                st.replay(g, lds, a.pos_info, rec, s2);
         }
         st.s = n_st;             // replay() walks s again; result() checks the count of the op loop
     }

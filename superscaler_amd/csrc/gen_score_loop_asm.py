@@ -69,6 +69,8 @@ ORD, ORD_LO, ORD_HI = "s[50:51]", "s50", "s51"
 MASK = [f"s{52 + j}" for j in range(4)]
 PLANT = [f"s{56 + j}" for j in range(4)]
 PREVFL = "s62"
+NEXTWIN, WIN, DMAOFF, DMACNT, ARRIVED = "s29", "s34", "s63", "s28", "s35"   # windowed rows: next window's first position, window index, ...
+DMAPTR = "s[60:61]"
 S0, S1, S2, S23 = "s96", "s97", "s98", "s[98:99]"
 
 
@@ -82,8 +84,8 @@ def PBUF(y):
 
 
 class Gen:
-    def __init__(self, rsh, mode):
-        self.rsh, self.mode, self.lines = rsh, mode, []
+    def __init__(self, rsh, mode, win=False):
+        self.rsh, self.mode, self.win, self.lines = rsh, mode, win, []
 
     def o(self, s):
         self.lines.append(s)
@@ -138,6 +140,62 @@ class Gen:
         self.o(f"ds_read_b64 {zf}, {T1}")
         self.o(f"ds_read_b64 {zb}, {T2}")
 
+    def dma(self, L):
+        """This wavefront's LDS-direct loads of the window whose descriptors start at byte DMAOFF of the table; header
+        in s[52:59] (rows, window starts, descriptors per wavefront, bytes per window, fetch-ahead flag)."""
+        self.o(f"v_mbcnt_lo_u32_b32 {T0}, -1, 0")
+        self.o(f"v_mbcnt_hi_u32_b32 {T0}, -1, {T0}")
+        self.o(f"v_lshlrev_b32 {T0}, 4, {T0}")
+        self.o(f"s_lshl_b32 {S0}, s56, 4")
+        self.o(f"s_mul_i32 {S0}, {S0}, %[wave]")
+        self.o(f"s_add_u32 {DMAOFF}, {DMAOFF}, {S0}")
+        self.o(f"s_add_u32 {DMAOFF}, {DMAOFF}, 32")
+        self.o(f"s_mov_b32 {DMACNT}, s56")
+        self.o(f"L_dma_{L}:")
+        self.o(f"s_load_dwordx4 s[96:99], {DMAPTR}, {DMAOFF}")
+        self.o("s_waitcnt lgkmcnt(0)")
+        self.o(f"v_cmp_gt_u32_e32 vcc, s98, {T0}")
+        self.o("s_mov_b64 exec, vcc")
+        self.o("s_mov_b32 m0, s97")
+        self.o(f"v_add_u32_e32 {T1}, s96, {T0}")
+        self.o("s_nop 0")
+        self.o(f"global_load_lds_dwordx4 {T1}, s[52:53]")
+        self.o(f"s_mov_b64 exec, {ALL}")
+        self.o(f"s_add_u32 {DMAOFF}, {DMAOFF}, 16")
+        self.o(f"s_sub_u32 {DMACNT}, {DMACNT}, 1")
+        self.o(f"s_cmp_lg_u32 {DMACNT}, 0")
+        self.o(f"s_cbranch_scc1 L_dma_{L}")
+
+    def window_switch(self, k1, L):
+        """Windowed rows: if op k1 of the group (0..16) is the first of the next window, every wavefront of the workgroup
+        stops here until that window's rows are in LDS.  Each wavefront copies its share of a window with LDS-direct
+        loads (descriptors {byte offset in the rows, LDS address, bytes} per window and wavefront).  Where consecutive
+        windows lie apart in LDS the loads of a window were issued when the window before it was entered, and here
+        those of the window after it are; otherwise the window is fetched here, between two barriers."""
+        self.c("rows of the next window, if it starts with the next op")
+        self.o(f"s_add_u32 {S0}, {POSBASE}, {k1}")
+        self.o(f"s_cmp_eq_u32 {S0}, {NEXTWIN}")
+        self.o(f"s_cbranch_scc0 L_nw_{L}")
+        self.o(f"s_load_dwordx8 s[52:59], {DMAPTR}, 0")
+        self.o("s_waitcnt vmcnt(0) lgkmcnt(0)")             # this wavefront's reads of the old rows and its loads so far have landed
+        self.o("s_barrier")
+        self.o(f"s_mov_b32 {ARRIVED}, 1")                   # (so have the next group's code words, if they were asked for)
+        self.o(f"s_add_u32 {WIN}, {WIN}, 1")
+        self.o(f"s_add_u32 {S0}, {WIN}, s58")
+        self.o(f"s_mul_i32 {DMAOFF}, {S0}, s57")
+        self.dma(L)
+        self.o(f"s_lshl_b32 {S0}, {WIN}, 2")
+        self.o(f"s_add_u32 {S0}, {S0}, 4")
+        self.o(f"s_load_dword {NEXTWIN}, s[54:55], {S0}")
+        self.o("s_cmp_eq_u32 s58, 1")
+        self.o(f"s_cbranch_scc1 L_wa_{L}")
+        self.o("s_waitcnt vmcnt(0)")
+        self.o("s_barrier")
+        self.o(f"L_wa_{L}:")
+        self.o("s_waitcnt lgkmcnt(0)")
+        self.o(f"L_nw_{L}:")
+        self.o(f"s_cmp_lg_u64 {M_ST}, 0")                   # (what the branch to the stage-end code tests)
+
     def reserved(self, cur):
         if self.mode == "max":          # max(rf + rb, W)
             self.o(f"v_add_f64 {RES}, {RFM[cur]}, {RBM[cur]}")
@@ -182,6 +240,8 @@ class Gen:
             self.o(f"v_mov_b32 {R(x1)}, 0")
         self.o(f"s_mov_b64 exec, {ALL}")
         self.o(f"L_ns_{L}:")
+        if self.win and b == 3:
+            self.window_switch(k + 1, L)
         self.issue(k + 1)
         if not self.rsh:
             self.o("s_waitcnt lgkmcnt(3)")
@@ -275,7 +335,14 @@ class Gen:
 
     def next_group_words(self):
         self.c("the next group's code words have arrived (zeros after the last group): padding and end-of-plan mark")
+        if self.win:
+            # (not if a window was entered since the words were asked for: they were waited for there, and the window
+            # loads now in flight need not be)
+            self.o(f"s_cmp_eq_u32 {ARRIVED}, 1")
+            self.o("s_cbranch_scc1 L_arr_%=")
         self.o("s_waitcnt vmcnt(0)")
+        if self.win:
+            self.o("L_arr_%=:")
         self.o(f"s_sub_i32 {LEFT}, %[n_ops], {POSBASE}")
         self.o(f"s_sub_i32 {LEFT}, {LEFT}, 16")
         self.apply_masks(NEXT, "nx")
@@ -301,6 +368,19 @@ class Gen:
         o(f"s_mov_b32 {GRP}, 0")
         o(f"s_mov_b32 {POSBASE}, 0")
         o(f"s_mov_b32 {PREVFL}, 0")
+        if self.win:
+            o(f"s_mov_b64 {DMAPTR}, %[dma]")
+            o(f"s_mov_b32 {WIN}, 0")
+            o(f"s_mov_b32 {ARRIVED}, 0")
+            o(f"s_load_dwordx8 s[52:59], {DMAPTR}, 0")
+            o("s_waitcnt lgkmcnt(0)")
+            o(f"s_load_dword {NEXTWIN}, s[54:55], 4")
+            c("windows that lie apart in LDS: window 0 was staged by the caller, fetch window 1")
+            o("s_cmp_eq_u32 s58, 1")
+            o("s_cbranch_scc0 L_nofetch_%=")
+            o(f"s_mov_b32 {DMAOFF}, s57")
+            self.dma("setup_%=")
+            o("L_nofetch_%=:")
         o(f"global_load_dwordx4 v[102:105], %[codeoff], {CPTR}")
         o(f"s_load_dwordx16 {PBUF(0)}, {PPTR}, 0")
         for r in (FWD, BWD, RUN, PEAK, RFM[0], RBM[0], RCS, RSF, RSB, W_, A_, SAVED):
@@ -328,6 +408,8 @@ class Gen:
         for r in NEXT:
             o(f"v_mov_b32 {r}, 0")
         o("L_loaded_%=:")
+        if self.win:
+            o(f"s_mov_b32 {ARRIVED}, 0")
         for k in range(16):
             self.slot(k)
         c("---- next group")
@@ -357,14 +439,15 @@ def main():
     parts = ["// Generated by gen_score_loop_asm.py -- do not edit.  gfx950 assembly of the plain scoring kernel's op loop",
              "// (deferred stage tails), one text per (resharding, reserved-memory rule); see the generator for the design.",
              "#pragma once", ""]
-    for rsh in (1, 0):
-        for mode in ("max", "min", "none"):
-            g = Gen(bool(rsh), mode)
-            parts.append(f"#define ACE_LOOP_ASM_RSH{rsh}_{mode.upper()} \\")
-            parts.append(c_string(g.build()))
-            parts.append("")
+    for win in (0, 1):
+        for rsh in (1, 0):
+            for mode in ("max", "min", "none"):
+                g = Gen(bool(rsh), mode, bool(win))
+                parts.append(f"#define ACE_LOOP_ASM{'_WIN' if win else ''}_RSH{rsh}_{mode.upper()} \\")
+                parts.append(c_string(g.build()))
+                parts.append("")
     clob = ", ".join(f'"v{i}"' for i in range(28, 128)) + ", " + ", ".join(f'"s{i}"' for i in range(24, 100) if i not in (32, 33))   # (s32 / s33 are the ABI's stack registers)
-    parts.append(f"#define ACE_LOOP_ASM_CLOBBERS {clob}, \"vcc\", \"scc\", \"memory\"")
+    parts.append(f"#define ACE_LOOP_ASM_CLOBBERS {clob}, \"vcc\", \"scc\", \"m0\", \"memory\"")
     parts.append("")
     path = os.path.join(HERE, "ace_score_loop_asm.inc")
     with open(path, "w") as f:

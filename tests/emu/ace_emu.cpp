@@ -180,6 +180,11 @@ extern "C" int ace_emu_kernel(const ace_tables_t *t, const uint8_t *codes, const
     uint32_t *pos = (uint32_t *)pool.place(nullptr, (G * 16 + 16) * 4);
     memcpy(pos, t->pos_info, (size_t)(t->num_ops + 1) * 4);
     a.pos_info = pos;
+    if (t->n_windows > 1 && t->num_types <= 256) {
+        uint32_t *pt = (uint32_t *)pool.place(nullptr, (G * 16 + 16) * 4);
+        ace_pos_types(t, pt, G * 16 + 16);
+        a.pos_types = pt;
+    }
     a.pair_kinds = (const uint8_t *)pool.place(t->pair_kinds, (size_t)a.rk_bytes, 1);
     a.stage_lut = (const uint32_t *)pool.place(t->stage_lut, (size_t)a.stg_words * 4, 4);
     a.nbm1 = (const double *)pool.place(t->nb_minus_1, (size_t)t->n_mbs * 8, 8);
@@ -195,7 +200,7 @@ extern "C" int ace_emu_kernel(const ace_tables_t *t, const uint8_t *codes, const
     unsigned char *lds = (unsigned char *)pool.place(nullptr, lds_bytes);
     const bool win = t->n_windows > 1;
     const bool coll = (t->flags & ACE_F_COLLECTIVE_MEM) != 0;
-    const bool defer = !range && !stage_out && !win && g.N < 65536 && !coll;
+    const bool defer = !range && !stage_out && (!win || a.pos_types) && g.N < 65536 && !coll;
     if (defer) a.stage_ws = (double *)pool.place(nullptr, (size_t)P * ACE_MAX_STAGES * ACE_WS_REC * 8);
 
     if (coll) {
@@ -206,6 +211,7 @@ extern "C" int ace_emu_kernel(const ace_tables_t *t, const uint8_t *codes, const
     }
     else if (range) { if (win) run_lanes<true, true, true, false>(a, lds, lds_bytes); else run_lanes<true, true, false, false>(a, lds, lds_bytes); }
     else if (stage_out) { if (win) run_lanes<true, false, true, false>(a, lds, lds_bytes); else run_lanes<true, false, false, false>(a, lds, lds_bytes); }
+    else if (defer && win) run_lanes<false, false, true, true>(a, lds, lds_bytes);
     else if (defer) run_lanes<false, false, false, true>(a, lds, lds_bytes);
     else if (win) run_lanes<false, false, true, false>(a, lds, lds_bytes);
     else run_lanes<false, false, false, false>(a, lds, lds_bytes);

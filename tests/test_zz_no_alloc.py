@@ -68,12 +68,11 @@ def test_static_entry_point_equals_score_batch(name, sizes):
         again = _raw_scores(ev, torch, "static", dev[1], limit)
         assert all(np.array_equal(a, b, equal_nan=True) for a, b in zip(again, want[1]))
         # the plain entry point on this handle would have to allocate its workspace now: refused, as fixed above
-        # (tables whose rows are windowed need no workspace)
         o = _outputs(ev, torch, dev[0].n_plans)
         with ev.device_context():
             rc = ev.lib.ace_score_batch(ev.handle, ctypes.byref(dev[0].struct), limit, 0, o[0].data_ptr(), o[1].data_ptr(),
                                         o[2].data_ptr(), o[3].data_ptr(), None, None)
-        assert rc == (0 if tables.n_windows > 1 else -6), rc
+        assert rc == -6, rc
         # beyond the stated maximum: refused, nothing launched
         big = ev.upload(synth.make_plans(w, tables, n_plans=16385, seed_offset=44))
         it = torch.zeros(16385, dtype=torch.float64, device=ev.device)

@@ -13,8 +13,10 @@
 
 #include <cstdio>
 #include <cstring>
+#include <algorithm>
 #include <mutex>
 #include <new>
+#include <vector>
 
 #include "ace_edit_kernels.h"
 #include "ace_score_loop.h"
@@ -602,7 +604,9 @@ struct ace_handle {
     uint32_t *d_pos_info;
     uint32_t *d_pos_types;     // d_pos_info with row indices in place of LDS slots (windowed rows, at most 256 of them; else null)
     ace_u4 *d_pos4;            // per position, for the assembly op loop (null when its pair-kind table has no room in LDS)
-    ace_u4 *d_win_dma;         // windowed rows: the LDS-direct loads that stage each window, per wavefront (assembly op loop), or null
+    ace_u4 *d_win_dma;         // windowed rows: what the assembly op loop fetches its windows by (setup_windowed_asm), or null
+    AceGeom geom_wa;           // ... and the LDS layout of the kernel that runs it
+    uint32_t lds_bytes_wa;
     uint8_t *d_pair_kinds;
     uint32_t *d_stage_lut;
     double *d_nbm1;
@@ -693,7 +697,7 @@ template <bool BD, bool RANGED, bool WIN, bool DEFER> static int allow_big_lds()
 // start" does NOT apply here, bit 1: ordinary op).  Positions past the last op point at row 0 and pair kind 0.
 static int upload_pos4(ace_handle *h, const ace_tables_t *t, size_t pos_entries, uint32_t pk32_off) {
     h->d_pos4 = nullptr;
-    if (!pk32_off) return ACE_OK;
+    if (!pk32_off || t->n_windows != 1) return ACE_OK;       // (windowed rows: setup_windowed_asm)
     ace_u4 *p4 = new (std::nothrow) ace_u4[pos_entries];
     if (!p4) return ACE_ENOMEM;
     const uint32_t row_bytes = (uint32_t)t->row_doubles * 8u, kind_stride = (uint32_t)t->n_glog * 64u;
@@ -703,7 +707,9 @@ static int upload_pos4(ace_handle *h, const ace_tables_t *t, size_t pos_entries,
         p4[i].x = row + (uint32_t)t->hot_off * 8u;
         p4[i].y = row + (uint32_t)t->z_off * 8u;
         p4[i].z = pk32_off + ((info >> 16) & 0xffu) * kind_stride * 4u;
-        p4[i].w = (((info >> 24) & 1u) ^ 1u) | (((info >> 25) & 1u) << 1);
+        // (rows as the evaluation of the stage tails indexes them: LDS slots)
+        const uint32_t ids = info & 0xffffu;
+        p4[i].w = (((info >> 24) & 1u) ^ 1u) | (((info >> 25) & 1u) << 1) | (ids << 8);
     }
     const int rc = upload((void **)&h->d_pos4, p4, pos_entries * sizeof(ace_u4));
     delete[] p4;
@@ -722,51 +728,116 @@ static int upload_pos_types(ace_handle *h, const ace_tables_t *t, size_t pos_ent
     return rc;
 }
 
-// Windowed rows, for the assembly op loop: the rows of window w as LDS-direct loads of at most 1 KB (64 lanes x 16 bytes),
-// dealt to the sixteen wavefronts of a workgroup in turn: [window][wavefront][j] = {byte offset in rows, LDS address, bytes, 0}.
-static int upload_win_dma(ace_handle *h, const ace_tables_t *t) {
+// Windowed rows, for the assembly op loop.  That loop reads only the hot sub-table and the collective-cost tables of a
+// row (the boundary sub-tables are read from global memory when the stage tails are evaluated), so it keeps its own,
+// denser windows: per row those two parts back to back, consecutive windows in alternate halves of the region in front of
+// the small tables, so that a window is fetched while the one before it is walked.  Built here: the LDS layout
+// (h->geom_wa), the per-position table (h->d_pos4) and the fetch records (h->d_win_dma): per fetch event and wavefront
+// (sixteen) 80 bytes = {first position of the window after the one being entered, bit 0: wait for the fetch (else it
+// completes before the next event) | number of loads << 8, address of the rows} and eight LDS-direct loads {byte offset
+// in the rows, LDS address} of 1 KB each.  Events: 0 fetches window 0 and waits, 1 fetches window 1, and entering window
+// w >= 1 fetches window w + 1 (the last one fetches window w - 1 again, into the half nobody reads).
+// Leaves the handle without them (plain scoring then takes the C++ loop) where the layout does not work out.
+static int setup_windowed_asm(ace_handle *h, const ace_tables_t *t, size_t pos_entries, int32_t rk_bytes, int32_t stg_words) {
     h->d_win_dma = nullptr;
-    if (t->n_windows <= 1 || !h->d_pos4 || !h->d_pos_types) return ACE_OK;
+    if (t->n_windows <= 1 || !h->d_pos_types || (t->flags & ACE_F_COLLECTIVE_MEM) || t->num_ops >= 65536) return ACE_OK;
+    if ((int64_t)(t->n_z > 0 ? t->n_z : 1) * t->z_table_doubles * 8 > 65536) return ACE_OK;
     const uint64_t row_bytes = (uint64_t)t->row_doubles * 8u;
     if ((uint64_t)t->num_types * row_bytes > 0xffffffffull) return ACE_OK;
-    const uint32_t per_row = (uint32_t)((row_bytes + 1023u) / 1024u);
-    uint32_t most = 0;
-    for (int w = 0; w < t->n_windows; ++w) {
-        const uint32_t n = (uint32_t)(t->win_row_begin[w + 1] - t->win_row_begin[w]) * per_row;
-        most = n > most ? n : most;
+    if (!(t->hot_off < t->start_off && t->start_off <= t->z_off && t->z_off <= t->row_doubles)) return ACE_OK;
+    const uint32_t hot_len = (uint32_t)(t->start_off - t->hot_off) * 8u, z_len = (uint32_t)(t->row_doubles - t->z_off) * 8u;
+    if (hot_len < 1024u || (z_len != 0u && z_len < 1024u) || (hot_len & 15u) || (z_len & 15u)) return ACE_OK;
+    const uint32_t crow = hot_len + z_len;
+    // the most rows per half that leave room for the small tables
+    uint32_t slots = 127, stg_off = 0, lut2_off = 0, pk32_off = 0, lds_end = 0;
+    for (; slots >= 5u; --slots) {
+        lds_end = ace_lds_pk32(ace_lds_layout(2u * slots * crow, (uint32_t)rk_bytes, (uint32_t)stg_words, &stg_off, &lut2_off),
+                               (uint32_t)rk_bytes, &pk32_off);
+        if (lds_end <= kMaxLds) break;
     }
-    const int32_t J = (int32_t)((most + 15u) / 16u);
-    if (J <= 0) return ACE_OK;
-    // If no window's rows overlap those of the window before it in LDS, a window can be fetched while the one before it
-    // is walked (the loop then asks for window w + 1 when it enters window w: one more, empty, window ends the table).
-    uint32_t ahead = 1;
-    for (int w = 0; w + 1 < t->n_windows && ahead; ++w)
-        for (int r = t->win_row_begin[w]; r < t->win_row_begin[w + 1] && ahead; ++r)
-            for (int q = t->win_row_begin[w + 1]; q < t->win_row_begin[w + 2]; ++q) {
-                const uint64_t a0 = t->win_rows[2 * r + 1], b0 = t->win_rows[2 * q + 1];
-                if (a0 < b0 + row_bytes && b0 < a0 + row_bytes) { ahead = 0; break; }
+    if (slots < 5u) return ACE_OK;
+    const int N = t->num_ops;
+    std::vector<uint32_t> types(pos_entries);
+    ace_pos_types(t, types.data(), pos_entries);
+    // windows end at multiples of 4 ops (or at the last op) and hold at most `slots` different rows
+    std::vector<int> win_start;
+    std::vector<std::vector<uint32_t>> win_types;
+    for (int i = 0; i < N;) {
+        std::vector<uint32_t> seen;
+        int good = -1;
+        size_t good_n = 0;
+        for (int j = i; j < N;) {
+            const uint32_t ty = types[j] & 0xffu;
+            if (std::find(seen.begin(), seen.end(), ty) == seen.end()) {
+                if (seen.size() >= slots) break;
+                seen.push_back(ty);
             }
-    const size_t entries = 2u + (size_t)(t->n_windows + 1) * 16u * (size_t)J;      // (two entries of header)
-    ace_u4 *d0 = new (std::nothrow) ace_u4[entries];
-    if (!d0) return ACE_ENOMEM;
-    for (size_t i = 0; i < entries; ++i) d0[i] = ace_u4{0u, 0u, 0u, 0u};
-    const uint64_t rows_at = (uint64_t)(uintptr_t)h->d_rows, win_at = (uint64_t)(uintptr_t)h->d_win_pos;
-    d0[0] = ace_u4{(uint32_t)rows_at, (uint32_t)(rows_at >> 32), (uint32_t)win_at, (uint32_t)(win_at >> 32)};
-    d0[1] = ace_u4{(uint32_t)J, (uint32_t)J * 256u, ahead, 0u};
-    ace_u4 *d = d0 + 2;
-    for (int w = 0; w < t->n_windows; ++w) {
-        uint32_t c = 0;
-        for (int r = t->win_row_begin[w]; r < t->win_row_begin[w + 1]; ++r)
-            for (uint32_t k = 0; k < per_row; ++k, ++c) {
-                const uint64_t left = row_bytes - (uint64_t)k * 1024u;
-                d[((size_t)w * 16u + (c & 15u)) * (size_t)J + (c >> 4)] =
-                    ace_u4{(uint32_t)(t->win_rows[2 * r] * row_bytes + k * 1024u), t->win_rows[2 * r + 1] + k * 1024u,
-                           (uint32_t)(left < 1024u ? left : 1024u), 0u};
-            }
+            ++j;
+            if (j == N || (j & 3) == 0) { good = j; good_n = seen.size(); }
+        }
+        if (good < 0) return ACE_OK;
+        seen.resize(good_n);
+        win_start.push_back(i);
+        win_types.push_back(seen);
+        i = good;
     }
-    const int rc = upload((void **)&h->d_win_dma, d0, entries * sizeof(ace_u4));
-    delete[] d0;
-    return rc;
+    const int n_w = (int)win_start.size();
+    if (n_w < 2) return ACE_OK;
+    auto row_addr = [&](int w, uint32_t ty) {
+        const std::vector<uint32_t> &v = win_types[w];
+        return (uint32_t)((w & 1) * slots + (uint32_t)(std::find(v.begin(), v.end(), ty) - v.begin())) * crow;
+    };
+    // the per-position table
+    std::vector<ace_u4> p4(pos_entries);
+    const uint32_t kind_stride = (uint32_t)t->n_glog * 64u;
+    for (size_t i = 0, w = 0; i < pos_entries; ++i) {
+        if (i >= (size_t)N) { p4[i] = ace_u4{0u, hot_len, pk32_off, 0u}; continue; }
+        while ((int)w + 1 < n_w && (size_t)win_start[w + 1] <= i) ++w;
+        const uint32_t info = t->pos_info[i], at = row_addr((int)w, types[i] & 0xffu);
+        p4[i] = ace_u4{at, at + hot_len, pk32_off + ((info >> 16) & 0xffu) * kind_stride * 4u,
+                       (((info >> 24) & 1u) ^ 1u) | (((info >> 25) & 1u) << 1) | ((types[i] & 0xffffu) << 8)};
+    }
+    // the loads of each window, dealt to the wavefronts in turn (the last load of a part ends with the part: it may
+    // overlap the one before it)
+    std::vector<std::vector<ace_u2>> loads(n_w);
+    for (int w = 0; w < n_w; ++w)
+        for (uint32_t ty : win_types[w]) {
+            const uint32_t at = row_addr(w, ty), src = (uint32_t)(ty * row_bytes);
+            for (int part = 0; part < 2; ++part) {
+                const uint32_t len = part ? z_len : hot_len, from = src + (uint32_t)(part ? t->z_off : t->hot_off) * 8u;
+                for (uint32_t off = 0; off < len; off += 1024u) {
+                    const uint32_t o = off + 1024u <= len ? off : len - 1024u;
+                    loads[w].push_back(ace_u2{from + o, at + (part ? hot_len : 0u) + o});
+                }
+            }
+        }
+    for (int w = 0; w < n_w; ++w)
+        if (loads[w].size() > 16u * 8u) return ACE_OK;
+    const int n_ev = n_w + 1;
+    std::vector<ace_u4> blob((size_t)n_ev * 16u * 5u, ace_u4{0u, 0u, 0u, 0u});
+    const uint64_t rows_at = (uint64_t)(uintptr_t)h->d_rows;
+    for (int e = 0; e < n_ev; ++e) {
+        const int entering = e < 2 ? 0 : e - 1;                        // the window walked after this event
+        int fetch = e == 0 ? 0 : entering + 1;
+        if (fetch >= n_w) fetch = entering - 1;
+        const uint32_t nextwin = entering + 1 < n_w ? (uint32_t)win_start[entering + 1] : 0x7fffffffu;
+        for (uint32_t v = 0; v < 16u; ++v) {
+            ace_u4 *rec = &blob[((size_t)e * 16u + v) * 5u];
+            uint32_t d[16] = {0};
+            uint32_t n = 0;
+            for (size_t c = v; c < loads[fetch].size(); c += 16u, ++n) { d[2 * n] = loads[fetch][c].x; d[2 * n + 1] = loads[fetch][c].y; }
+            rec[0] = ace_u4{nextwin, (e == 0 ? 1u : 0u) | (n << 8), (uint32_t)rows_at, (uint32_t)(rows_at >> 32)};
+            for (int q = 0; q < 4; ++q) rec[1 + q] = ace_u4{d[4 * q], d[4 * q + 1], d[4 * q + 2], d[4 * q + 3]};
+        }
+    }
+    int rc = upload((void **)&h->d_win_dma, blob.data(), blob.size() * sizeof(ace_u4));
+    if (rc == ACE_OK) rc = upload((void **)&h->d_pos4, p4.data(), p4.size() * sizeof(ace_u4));
+    if (rc != ACE_OK) return rc;
+    h->geom_wa = h->geom;
+    h->geom_wa.rk_lds_off = 2u * slots * crow;
+    h->geom_wa.stg_lds_off = stg_off; h->geom_wa.lut2_lds_off = lut2_off; h->geom_wa.pk32_lds_off = pk32_off;
+    h->lds_bytes_wa = lds_end;
+    return ACE_OK;
 }
 
 // The device address of `scratch` on the current device (looked up once per device).
@@ -821,7 +892,7 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     // the assembly loop's pair-kind table, where the table has room and its entries can hold the offsets (otherwise plain
     // scoring takes the C++ form of the loop)
     uint32_t pk32_off = 0;
-    if (t->n_windows == 1 || t->num_types <= 256) {        // (windowed rows: the loop's caller needs d_pos_types as well)
+    if (t->n_windows == 1) {                               // (windowed rows: setup_windowed_asm lays LDS out anew)
         uint32_t off;
         const uint32_t end = ace_lds_pk32(lds_bytes, (uint32_t)rk_bytes, &off);
         if (end <= kMaxLds && ((int64_t)(t->n_z > 0 ? t->n_z : 1) * t->z_table_doubles * 8) <= 65536) {
@@ -895,7 +966,7 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
         (rc = upload((void **)&h->d_win_pos, t->win_pos, (size_t)(t->n_windows + 1) * 4)) ||
         (rc = upload((void **)&h->d_win_row_begin, t->win_row_begin, (size_t)(t->n_windows + 1) * 4)) ||
         (rc = upload((void **)&h->d_win_rows, t->win_rows, (size_t)n_win_rows * 8)) ||
-        (rc = upload_win_dma(h, t)) ||
+        (rc = setup_windowed_asm(h, t, pos_entries, rk_bytes, stg_words)) ||
         (rc = hipFuncSetAttribute(reinterpret_cast<const void *>(&topk_short_final), hipFuncAttributeMaxDynamicSharedMemorySize,
                                   (int)kShortLds) == hipSuccess ? ACE_OK : ACE_EHIP) ||
         (rc = allow_big_lds<false, false, false, false>()) || (rc = allow_big_lds<false, false, true, false>()) ||
@@ -955,7 +1026,14 @@ static void launch_score_b(const ace_handle_t *h, const AceKernelArgs &a, hipStr
     } else if ((P + kBlock - 1) / kBlock < (size_t)kSmallBatchBlocks)
         hipLaunchKernelGGL((ace_score_kernel<BD, RANGED, WIN, DEFER, kSmallBlock>), dim3((unsigned)((P + kSmallBlock - 1) / kSmallBlock)),
                            dim3(kSmallBlock), h->lds_bytes, s, a);
-    else
+    else if (WIN && DEFER && h->d_win_dma) {
+        // the assembly op loop over windowed rows lays LDS out its own way
+        AceKernelArgs b = a;
+        b.g = h->geom_wa;
+        b.g.P = a.g.P; b.g.mem_limit = a.g.mem_limit; b.g.strict = a.g.strict;
+        hipLaunchKernelGGL((ace_score_kernel<BD, RANGED, WIN, DEFER, kBlock>), dim3((unsigned)((P + kBlock - 1) / kBlock)),
+                           dim3(kBlock), h->lds_bytes_wa, s, b);
+    } else
         hipLaunchKernelGGL((ace_score_kernel<BD, RANGED, WIN, DEFER, kBlock>), dim3((unsigned)((P + kBlock - 1) / kBlock)),
                            dim3(kBlock), h->lds_bytes, s, a);
 }

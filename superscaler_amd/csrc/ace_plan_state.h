@@ -10,7 +10,7 @@
 //             get_reserved_memory maxima (:453-460)
 //   start_fast() / start_lookups()  stage head: per-stage lookup offsets; boundary input size /
 //             p2p time (:319-331)
-//   stash() / replay()  deferred stage tails: a finished stage's accumulators are parked in a
+//   stash() / replay_all()  deferred stage tails: a finished stage's accumulators are parked in a
 //             workspace and its tail is evaluated after the op loop
 //   finish()  stage tail: output p2p (:321-336), stage time (:352-353, :579), stage memory
 //             (predict_stage_memory :514-539, get_reserved_memory :480-483), running
@@ -30,6 +30,7 @@
 #include <cstdlib>
 #include <cstring>
 #define ACE_HD inline
+#define ACE_WAVE_ANY(x) (x)
 struct AceLds {
     const unsigned char *base;
     uint32_t size;
@@ -54,6 +55,7 @@ static inline uint32_t ace_lds_base(const unsigned char *) { return 0u; }   // h
 static inline double ace_max(double a, double b) { return a > b ? a : b; }
 #else
 #define ACE_HD __device__ __forceinline__
+#define ACE_WAVE_ANY(x) __any(x)
 // LDS reads take the absolute LDS byte address.  The address of the workgroup's LDS array is a
 // link-time constant (zero when the kernel has no other LDS variables) that the compiler cannot fold
 // while it compiles; left inside per-lane address arithmetic it costs two or three vector
@@ -211,8 +213,9 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false, bool GROW
     double fwd, bwd, rcs, W, A, saved, run, peak, rfm, rbm, rs_f, rs_b, mc;
     double id_fwd, id_bwd;
     bool lastclose;
-    uint32_t replay_first;      // DEFER: first op of the stage replay() is called for next (stages follow each other) ...
-    uint32_t replay_code;       // ... and its code (before the first call: the code of the plan's first op)
+    uint32_t replay_row;        // DEFER: row of the first op of the stage the replay decodes next (stages follow each other) ...
+    uint32_t replay_code;       // ... and its code
+    const uint32_t *row_ids;    // DEFER over windowed rows: per position, what stash() takes as `ids` (else the position's descriptor has them)
     uint64_t rk_all;            // per stage (4 bits each): the stage size as the pair-kind tables index it
     uint64_t diag_next, rk_next;   // diags / rk_all shifted down by the stages handed out so far
     uint32_t ws_stride;         // DEFER: 16-byte units between two stages of one plan in the workspace
@@ -236,7 +239,7 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false, bool GROW
         s = -1;
         sum_t = 0.0; max_t = 0.0; max_mem = 0.0;
         status = 0;
-        lastclose = false; replay_first = 0; replay_code = 0; r_next = 0; pair_prev = 0;
+        lastclose = false; replay_row = 0; replay_code = 0; r_next = 0; pair_prev = 0; row_ids = nullptr;
         ws_stride = ACE_WS_REC / 2;
         ws_off = 0;
         fwd = bwd = rcs = W = A = saved = run = peak = rfm = rbm = rs_f = rs_b = mc = 0.0;
@@ -349,16 +352,20 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false, bool GROW
     // DEFER: park the finished stage in the plan's workspace slot `s`: ten values in five 16-byte
     // stores (a store from a lane or two costs as much as one from sixty-four, so what can be
     // folded here without a table lookup is: fwd + bwd, the closed peak segment, the reserved term).
-    ACE_HD void stash(const AceGeom &g, double *ws, uint32_t i_last, uint32_t c_last, uint32_t c_next, bool prev_ordinary) {
+    // `ids`: row of the stage's last op | row of the op after it << 8, as replay's lookups index rows (LDS slots; for
+    // windowed rows their indices in global memory).
+    ACE_HD void stash(const AceGeom &g, double *ws, uint32_t i_last, uint32_t c_last, uint32_t c_next, bool prev_ordinary,
+                      uint32_t ids) {
         if (ws == nullptr || s < 0 || s >= ACE_MAX_STAGES) return;
         // stages are stashed in order, once each: slot s of this plan is ws_off further on (a running
         // offset instead of s * ws_stride, which would be a slow 32-bit multiply per stage end)
         ace_d2 *r = reinterpret_cast<ace_d2 *>(ws) + ws_off;
         ws_off += ws_stride;
-        // what replay() needs besides the sums: the position of the stage's last op, its code and the code of the op
-        // after it (the next stage's first): code * 8 + next code in byte (position % 4) of the low word (the other
-        // bytes are not read: the assembly form of the loop stores its whole word of such bytes)
-        uint64_t meta = ((uint64_t)i_last << 32) | (uint64_t)(((c_last << 3) | c_next) << (8u * (i_last & 3u)));
+        // what the replay needs besides the sums.  Low word: code of the stage's last op * 8 + code of the op after it
+        // (the next stage's first) in byte (position % 4); the other bytes are not read (the assembly form of the loop
+        // stores its whole word of such bytes).  High word: position of the last op (16 bits) | ids << 16.
+        uint64_t meta = ((uint64_t)((i_last & 0xffffu) | (ids << 16)) << 32) |
+                        (uint64_t)(((c_last << 3) | c_next) << (8u * (i_last & 3u)));
         double meta_d;
         __builtin_memcpy(&meta_d, &meta, 8);
         const double fb = fwd + bwd;                                    // the first sum of :579
@@ -370,44 +377,116 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false, bool GROW
         r[4] = ace_d2{reserved_term(g), meta_d};
     }
 
-    // DEFER: evaluate stage `s2` from its stashed record (called for s2 = 0, 1, ... in order, after replay_code has
-    // been set to the code of the plan's first op).
-    ACE_HD void replay(const AceGeom &g, const AceLds &lds, const uint32_t *pos_info, const double *ws, int s2) {
-        const ace_d2 *r = reinterpret_cast<const ace_d2 *>(ws) + (size_t)((uint32_t)s2 * ws_stride);
-        ace_d2 r0 = r[0], r1 = r[1], r2 = r[2], r3 = r[3], r4 = r[4];
-        s = s2;
-        {
-            const uint32_t glog = (uint32_t)(glogs >> (4u * ((uint32_t)s2 & 15u))) & 15u;
-            const uint32_t w = lds.ld<uint32_t>(g.stg_lds_off + (bidx * 16u + glog) * 4u);
-            dc_v = ace_mul24(w & 15u, (uint32_t)g.C);
-            mrow = w >> 16;
-        }
+    // DEFER: the evaluation of the stashed stages, in three steps per stage so that the caller can have the loads of
+    // later stages in flight while it evaluates an earlier one: replay_load (the record), replay_lookups (decodes it
+    // and reads the stage's boundary entries), replay_finish.  Stages in order; before stage 0, replay_code holds the
+    // code of the plan's first op and replay_row the row of that op.
+    struct Record { ace_d2 r[5]; };
+    struct Lookups { double inputs, in_comm; ace_d2 oe; uint32_t lut, c_first, c_last; };
+
+    ACE_HD void replay_load(const double *ws, int s2, Record &rec) const {
+        // (every plan owns ACE_MAX_STAGES slots)
+        const int sl = s2 < ACE_MAX_STAGES ? s2 : ACE_MAX_STAGES - 1;
+        const ace_d2 *p = reinterpret_cast<const ace_d2 *>(ws) + (size_t)((uint32_t)sl * ws_stride);
+#pragma unroll
+        for (int j = 0; j < 5; ++j) rec.r[j] = p[j];
+    }
+
+    // `live`: the plan has a stage s2 (else the record is whatever the slot held: entry 0 of row 0 is looked up, and
+    // the chain of first ops stays as it is).
+    ACE_HD void replay_lookups(const AceGeom &g, const AceLds &lds, const Record &rec, int s2, bool live, Lookups &L) {
         uint64_t meta;
-        __builtin_memcpy(&meta, &r4.y, 8);
-        uint32_t i_last = (uint32_t)(meta >> 32);
-        const uint32_t cc = ((uint32_t)meta >> (8u * (i_last & 3u))) & 63u;
-        uint32_t i_first = s2 == 0 ? 0u : replay_first;
-        const uint32_t c_first = replay_code & 7u, c_last = cc >> 3;
-        if (i_first >= (uint32_t)g.N) i_first = 0;     // garbage only if the plan was malformed
-        if (i_last >= (uint32_t)g.N) i_last = 0;
-        replay_first = i_last + 1u;
-        replay_code = cc & 7u;
-        start_lookups(g, lds, info_row(g, pos_info[i_first]), c_first);
-        // finish() recombines: (fb + 0) = fb; the peak is closed already; max(reserved + 0, W) = reserved
-        fwd = r0.x; bwd = 0.0; rcs = r0.y; rs_f = r1.x; rs_b = r1.y; W = r2.x; A = r2.y; saved = r3.x;
-        peak = r3.y; run = 0.0; lastclose = false; rfm = r4.x; rbm = 0.0;
-        finish(g, lds, info_row(g, pos_info[i_last]), c_last, nullptr);
+        __builtin_memcpy(&meta, &rec.r[4].y, 8);
+        const uint32_t hi = (uint32_t)(meta >> 32);
+        const uint32_t cc = ((uint32_t)meta >> (8u * (hi & 3u))) & 63u;
+        uint32_t row_first = replay_row, row_last = (hi >> 16) & 0xffu;
+        L.c_first = replay_code & 7u;
+        L.c_last = cc >> 3;
+        if (live) {
+            replay_row = hi >> 24;
+            replay_code = cc & 7u;
+        } else {
+            row_first = 0; row_last = 0; L.c_first = 0; L.c_last = 0;
+        }
+        const uint32_t sidx = (uint32_t)s2 & 15u;
+        const uint32_t glog = (uint32_t)(glogs >> (4u * sidx)) & 15u;
+        L.lut = lds.ld<uint32_t>(g.stg_lds_off + (bidx * 16u + glog) * 4u);
+        const bool in_cross = (cross >> sidx) & 1u;
+        const uint32_t dc = ace_mul24(L.lut & 15u, (uint32_t)g.C);
+        const uint32_t a = row_first * g.row_bytes + g.start_off + (dc + L.c_first) * ACE_START_STRIDE;
+        L.inputs = row_ld<double>(lds, a);                                  // input size
+        L.in_comm = row_ld<double>(lds, a + (in_cross ? 16u : 8u));         // size / inter- or intra-node bandwidth
+        L.oe = row_ld<ace_d2>(lds, out_entry_addr(g, row_last * g.row_bytes, L.c_last, L.c_first >> g.A_shift, L.lut >> 16));
+    }
+
+    // (the record and the looked-up values into the stage state: after this `rec` may be overwritten)
+    ACE_HD void replay_take(const AceGeom &g, const Record &rec, const Lookups &L, int s2) {
+        s = s2;
+        dc_v = ace_mul24(L.lut & 15u, (uint32_t)g.C);
+        mrow = L.lut >> 16;
+        out_cross = (cross >> (16u + ((uint32_t)s2 & 15u))) & 1u;
+        t_first = L.c_first >> g.A_shift;
+        inputs = L.inputs;
+        in_comm = L.in_comm;
+        // finish_tail() recombines: (fb + 0) = fb; the peak is closed already; max(reserved + 0, W) = reserved
+        fwd = rec.r[0].x; bwd = 0.0; rcs = rec.r[0].y; rs_f = rec.r[1].x; rs_b = rec.r[1].y; W = rec.r[2].x; A = rec.r[2].y;
+        saved = rec.r[3].x; peak = rec.r[3].y; run = 0.0; lastclose = false; rfm = rec.r[4].x; rbm = 0.0;
+    }
+
+    // One stage of replay_all(): stage s2 is evaluated from (rx, lx); meanwhile record s2 + 2 is fetched into rx and
+    // the boundary entries of stage s2 + 1 (record in ry) into ly.
+    ACE_HD void replay_step(const AceGeom &g, const AceLds &lds, const double *ws, int s2, int n_st, Record &rx, Lookups &lx,
+                            const Record &ry, Lookups &ly) {
+        const bool live = s2 < n_st;
+        const ace_d2 oe = lx.oe;
+        const uint32_t c_last = lx.c_last;
+        if (live) replay_take(g, rx, lx, s2);
+        // (a stage no lane of the wavefront has is not fetched: its slot may never have been written)
+        if (ACE_WAVE_ANY(s2 + 2 < n_st)) replay_load(ws, s2 + 2, rx);
+        if (ACE_WAVE_ANY(s2 + 1 < n_st)) replay_lookups(g, lds, ry, s2 + 1, s2 + 1 < n_st, ly);
+        if (live) finish_tail(g, lds, 0u, c_last, oe, nullptr);
+    }
+
+    // All stashed stages of a plan of n_st stages whose first op has code `code0` and row `row0`.
+    ACE_HD void replay_all(const AceGeom &g, const AceLds &lds, const double *ws, int n_st, uint32_t code0, uint32_t row0) {
+        replay_code = code0;
+        replay_row = row0;
+        Record ra, rb;
+        Lookups la, lb;
+        replay_load(ws, 0, ra);
+        rb = ra;
+        if (ACE_WAVE_ANY(1 < n_st)) replay_load(ws, 1, rb);
+        replay_lookups(g, lds, ra, 0, 0 < n_st, la);
+        lb = la;
+        for (int s2 = 0; s2 < ACE_MAX_STAGES; s2 += 2) {
+            if (!ACE_WAVE_ANY(s2 < n_st)) break;
+            replay_step(g, lds, ws, s2, n_st, ra, la, rb, lb);
+            if (!ACE_WAVE_ANY(s2 + 1 < n_st)) break;
+            replay_step(g, lds, ws, s2 + 1, n_st, rb, lb, ra, la);
+        }
+        s = n_st;               // (the evaluation walked s again; result() checks the count of the op loop)
+    }
+
+    // Address of output_size[ops[-1]][mbs[-1]][tp[0]][algo[-1]] (sic, aceso_cost_model.py:321-326) in the row at `lastrow`:
+    // `c_last` the last op's code, `tf` the tp index of the stage's first op, `mr` the stage's row of micro-batch indices.
+    ACE_HD static uint32_t out_entry_addr(const AceGeom &g, uint32_t lastrow, uint32_t c_last, uint32_t tf, uint32_t mr) {
+        const uint32_t t_last = c_last >> g.A_shift;
+        const uint32_t a_last = c_last & (uint32_t)(g.n_algo - 1);
+        uint32_t m_last = (mr >> (4u * t_last)) & 15u;
+        if (m_last >= (uint32_t)g.n_mbs) m_last = 0;   // only for plans whose sums are NaN already
+        const uint32_t oidx = ((m_last * (uint32_t)g.n_tp + tf) << g.A_shift) + a_last;
+        return lastrow + g.out_off + oidx * 16u;
     }
 
     // Stage tail; `lastrow` is the LDS offset of the row of the stage's last op, `c_last` its code.
     ACE_HD void finish(const AceGeom &g, const AceLds &lds, uint32_t lastrow, uint32_t c_last, double *rec) {
-        uint32_t t_last = c_last >> g.A_shift;
+        const ace_d2 oe = row_ld<ace_d2>(lds, out_entry_addr(g, lastrow, c_last, t_first, mrow));
+        finish_tail(g, lds, lastrow, c_last, oe, rec);
+    }
+
+    // ... with the output entry `oe` looked up already.
+    ACE_HD void finish_tail(const AceGeom &g, const AceLds &lds, uint32_t lastrow, uint32_t c_last, ace_d2 oe, double *rec) {
         uint32_t a_last = c_last & (uint32_t)(g.n_algo - 1);
-        uint32_t m_last = (mrow >> (4u * t_last)) & 15u;
-        if (m_last >= (uint32_t)g.n_mbs) m_last = 0;   // only for plans whose sums are NaN already
-        // output_size[ops[-1]][mbs[-1]][tp[0]][algo[-1]]  (sic, aceso_cost_model.py:321-326)
-        uint32_t oidx = ((m_last * (uint32_t)g.n_tp + t_first) << g.A_shift) + a_last;
-        ace_d2 oe = row_ld<ace_d2>(lds, lastrow + g.out_off + oidx * 16u);
         double out_comm = out_cross ? oe.y : oe.x;
         double in_c = in_comm + rs_f * 1000.0;      // :352
         double out_c = out_comm + rs_b * 1000.0;    // :353
@@ -501,7 +580,7 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false, bool GROW
         const bool last = RANGED ? (i + 1 == hi) : (((nbyte >> 4) & 1u) || plan_end);
         if (last) {
             // :439 "i + 1 == len(ops) - 1": the (previous, this) pair closes the last segment
-            if (DEFER) stash(g, rec, (uint32_t)i, c, nc, (pinfo >> 25) & 1u);
+            if (DEFER) stash(g, rec, (uint32_t)i, c, nc, (pinfo >> 25) & 1u, (GROWS ? row_ids[i] : info) & 0xffffu);
             else {
                 lastclose = pair_prev & (pinfo >> 25) & 1u;
                 finish(g, lds, row, c, rec);

@@ -42,8 +42,8 @@ struct AceKernelArgs {
     double *stage_ws;           // [ACE_MAX_STAGES][plans rounded up to whole workgroups][ACE_WS_REC] for deferred stage tails
 };
 
-// Windowed rows: the position descriptors (pos_info) with each row's index in `rows` where its LDS slot is; positions
-// past the last op read zero.  (Host side: what the library uploads as AceKernelArgs::pos_types.)
+// Windowed rows: the position descriptors (pos_info) with each row's index in `rows` where its LDS slot is (and the next
+// position's where that one's is); positions past the last op read zero.  (Host side: what the library uploads as AceKernelArgs::pos_types.)
 inline void ace_pos_types(const ace_tables_t *t, uint32_t *out, size_t entries) {
     const uint32_t row_bytes = (uint32_t)t->row_doubles * 8u;
     int w = 0;
@@ -57,6 +57,9 @@ inline void ace_pos_types(const ace_tables_t *t, uint32_t *out, size_t entries) 
             if (t->win_rows[2 * r + 1] == slot_off) type = t->win_rows[2 * r];
         out[i] = (info & 0xffff0000u) | type;
     }
+    // ... and the index of the next position's row in bits 8 to 15 (the last op: its own)
+    for (size_t i = 0; i < entries && i < (size_t)t->num_ops; ++i)
+        out[i] |= ((i + 1 < (size_t)t->num_ops ? out[i + 1] : out[i]) & 0xffu) << 8;
 }
 
 // Copy the rows window `w` needs from global memory into LDS (whole workgroup).
@@ -76,9 +79,8 @@ template <int BLOCK> ACE_HD void stage_window(const AceKernelArgs &a, unsigned c
 // gen_score_loop_asm.py, which describes it): walks all ops of this lane's plan, parks every finished stage in the
 // lane's workspace records like PlanState::stash(), and returns the number of stages closed.  LDS addresses in `pos4`
 // are absolute: the caller checks that the workgroup's LDS array starts at address 0.
-// WIN: the rows are windowed; the loop restages them itself.  a.win_dma: {address of the rows, address of the window
-// starts, J, bytes of descriptors per window}, then per window and wavefront (sixteen) J descriptors {byte offset in the
-// rows, LDS address, bytes (at most 1,024), 0} of LDS-direct loads.
+// WIN: the rows are windowed; the loop fetches its windows itself, from the records of a.win_dma (80 bytes per fetch
+// event and wavefront, sixteen wavefronts: see the generator).
 template <bool WIN>
 __device__ __forceinline__ uint32_t ace_score_loop_asm(const AceKernelArgs &a, const AceGeom &g, uint64_t dg, uint64_t rks,
                                                        uint32_t code_off, double *rec, uint32_t ws_stride, uint32_t prio, uint32_t wave) {
@@ -92,7 +94,7 @@ __device__ __forceinline__ uint32_t ace_score_loop_asm(const AceKernelArgs &a, c
                  : [dg] "v"(dg), [rk] "v"(rks), [codeoff] "v"(code_off), [rec] "v"(rec), [codes] "s"(a.codes),         \
                    [pos] "s"(a.pos4), [c8] "s"(c8), [n_ops] "s"(g.N), [n_groups] "s"(g.G),                                \
                    [gstride_lo] "s"(gs_lo), [gstride_hi] "s"(gs_hi), [wsstride] "s"(ws_stride), [prio] "s"(prio),       \
-                   [dma] "s"(a.win_dma), [wave] "s"(wave)                                                               \
+                   [dma] "s"(a.win_dma), [waveoff] "s"(wave * 80u)                                                      \
                  : ACE_LOOP_ASM_CLOBBERS)
         if (g.flags & ACE_F_RESHARDING) {
             if (g.flags & ACE_F_NO_RESERVED) ACE_LOOP_ASM_RUN(ACE_LOOP_ASM_WIN_RSH1_NONE);
@@ -233,7 +235,13 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
         reinterpret_cast<ace_u2 *>(lds_raw + a.g.lut2_lds_off)[j] =
             ace_u2{z_v, ((glog < (uint32_t)a.g.n_glog ? glog : 0u) << 6) - z_v};
     }
-    stage_window<BLOCK>(a, lds_raw, w0, tid);       // every row, or the first window's
+    // (the assembly op loop over windowed rows fetches its windows itself, in a layout of its own)
+#ifndef ACE_HOST_EMU
+    const bool asm_loop = DEFER && lds_base == 0u && a.pos4 && (!WIN || (BLOCK == 1024 && a.win_dma));
+#else
+    const bool asm_loop = false;
+#endif
+    if (!(WIN && asm_loop)) stage_window<BLOCK>(a, lds_raw, w0, tid);       // every row, or the first window's
     ACE_SYNC();
 
     AceLds lds = ace_make_lds(lds_raw, lds_bytes);
@@ -241,6 +249,7 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     PlanState<BD, RANGED, DEFER, COLL, DEFER && WIN> st;
     const ace_u4 h = a.hdr[pl];
     st.init(g, lds, h, range);
+    st.row_ids = a.pos_types;
     const double nbm1 = a.nbm1[st.bidx];
     // (a single-stage query has one record, a whole plan one per possible stage)
     const size_t rec_doubles = RANGED ? (size_t)ACE_STAGE_REC : (size_t)(ACE_MAX_STAGES * ACE_STAGE_REC);
@@ -257,7 +266,7 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     const uint32_t first_code = cw.x & 7u;
     int grp_stop = grp_end;
 #ifndef ACE_HOST_EMU
-    if (DEFER && lds_base == 0u && a.pos4 && (!WIN || (BLOCK == 1024 && a.win_dma))) {
+    if (asm_loop) {
         // the assembly form of the loop below (same operations per plan, same results)
         if (!(cw.x & 0x10u)) st.status = ACE_PLAN_MALFORMED;    // the first op must open a stage
         uint64_t dg, rks;
@@ -321,21 +330,14 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     }
     if (DEFER) {
         const int n_st = st.s;
-        st.replay_code = first_code;
-        for (int s2 = 0; s2 < ACE_MAX_STAGES; ++s2) {
-            const bool live = s2 < n_st;
-            if (!ACE_ANY(live)) break;
-            if (!live) continue;
-            if (WIN) {
-                // (row offsets as the rows lie in global memory)
-                AceGeom gr = g;
-                gr.start_off -= lds_base; gr.out_off -= lds_base;
-                gr.row_bytes = (uint32_t)a.row_doubles * 8u;
-                st.replay(gr, lds, a.pos_types, rec, s2);
-            } else
-                st.replay(g, lds, a.pos_info, rec, s2);
-        }
-        st.s = n_st;             // replay() walks s again; result() checks the count of the op loop
+        if (WIN) {
+            // (row offsets as the rows lie in global memory)
+            AceGeom gr = g;
+            gr.start_off -= lds_base; gr.out_off -= lds_base;
+            gr.row_bytes = (uint32_t)a.row_doubles * 8u;
+            st.replay_all(gr, lds, rec, n_st, first_code, a.pos_types[0] & 0xffu);
+        } else
+            st.replay_all(g, lds, rec, n_st, first_code, a.pos_info[0] & 0xffu);
     }
     double iter, peak;
     uint8_t feas, stat;

@@ -69,12 +69,12 @@ ORD, ORD_LO, ORD_HI = "s[50:51]", "s50", "s51"
 MASK = [f"s{52 + j}" for j in range(4)]
 PLANT = [f"s{56 + j}" for j in range(4)]
 PREVFL = "s62"
-NEXTWIN, WIN, DMAOFF, DMACNT, ARRIVED = "s29", "s34", "s63", "s28", "s35"   # windowed rows: next window's first position, window index, ...
+NEXTWIN, EVT, DMAOFF, ARRIVED = "s29", "s34", "s63", "s35"   # windowed rows: next window's first position, window index, ...
 DMAPTR = "s[60:61]"
 S0, S1, S2, S23 = "s96", "s97", "s98", "s[98:99]"
 
 
-def P(y, q):                                # position entry q of the word in buffer y: hot, z, pair-table address, flags
+def P(y, q):                                # position entry q of the word in buffer y: hot, z, pair-table address, flags | rows << 8
     b = 64 + 16 * y + 4 * q
     return dict(hot=f"s{b}", z=f"s{b+1}", pk=f"s{b+2}", fl=f"s{b+3}")
 
@@ -140,59 +140,49 @@ class Gen:
         self.o(f"ds_read_b64 {zf}, {T1}")
         self.o(f"ds_read_b64 {zb}, {T2}")
 
-    def dma(self, L):
-        """This wavefront's LDS-direct loads of the window whose descriptors start at byte DMAOFF of the table; header
-        in s[52:59] (rows, window starts, descriptors per wavefront, bytes per window, fetch-ahead flag)."""
+    def fetch_event(self, L, pq):
+        """Windowed rows, one fetch event: the wavefront's record {first position of the window after the one being
+        entered, bit 0: wait for the fetch | number of loads << 8, address of the rows} and eight loads {byte offset in
+        the rows, LDS address} (the second four go through s[pq:pq+7]); all wavefronts of the workgroup meet, then each
+        issues its loads (LDS-direct, 1 KB each)."""
+        self.o(f"s_mul_i32 {DMAOFF}, {EVT}, 1280")
+        self.o(f"s_add_u32 {DMAOFF}, {DMAOFF}, %[waveoff]")
+        self.o(f"s_load_dwordx4 s[96:99], {DMAPTR}, {DMAOFF}")
+        self.o(f"s_add_u32 {DMAOFF}, {DMAOFF}, 16")
+        self.o(f"s_load_dwordx8 s[52:59], {DMAPTR}, {DMAOFF}")
+        self.o(f"s_add_u32 {DMAOFF}, {DMAOFF}, 32")
+        self.o(f"s_load_dwordx8 s[{pq}:{pq + 7}], {DMAPTR}, {DMAOFF}")
+        self.o("s_waitcnt vmcnt(0) lgkmcnt(0)")             # this wavefront's reads of the old rows and its loads so far have landed
+        self.o("s_barrier")
+        self.o(f"s_mov_b32 {ARRIVED}, 1")                   # (so have the next group's code words, if they were asked for)
+        self.o(f"s_add_u32 {EVT}, {EVT}, 1")
         self.o(f"v_mbcnt_lo_u32_b32 {T0}, -1, 0")
         self.o(f"v_mbcnt_hi_u32_b32 {T0}, -1, {T0}")
         self.o(f"v_lshlrev_b32 {T0}, 4, {T0}")
-        self.o(f"s_lshl_b32 {S0}, s56, 4")
-        self.o(f"s_mul_i32 {S0}, {S0}, %[wave]")
-        self.o(f"s_add_u32 {DMAOFF}, {DMAOFF}, {S0}")
-        self.o(f"s_add_u32 {DMAOFF}, {DMAOFF}, 32")
-        self.o(f"s_mov_b32 {DMACNT}, s56")
-        self.o(f"L_dma_{L}:")
-        self.o(f"s_load_dwordx4 s[96:99], {DMAPTR}, {DMAOFF}")
-        self.o("s_waitcnt lgkmcnt(0)")
-        self.o(f"v_cmp_gt_u32_e32 vcc, s98, {T0}")
-        self.o("s_mov_b64 exec, vcc")
-        self.o("s_mov_b32 m0, s97")
-        self.o(f"v_add_u32_e32 {T1}, s96, {T0}")
-        self.o("s_nop 0")
-        self.o(f"global_load_lds_dwordx4 {T1}, s[52:53]")
-        self.o(f"s_mov_b64 exec, {ALL}")
-        self.o(f"s_add_u32 {DMAOFF}, {DMAOFF}, 16")
-        self.o(f"s_sub_u32 {DMACNT}, {DMACNT}, 1")
-        self.o(f"s_cmp_lg_u32 {DMACNT}, 0")
-        self.o(f"s_cbranch_scc1 L_dma_{L}")
+        self.o(f"s_bfe_u32 {DMAOFF}, s97, 0x40008")         # number of loads
+        for j in range(8):
+            base = 52 + 2 * j if j < 4 else pq + 2 * (j - 4)
+            self.o(f"s_cmp_le_u32 {DMAOFF}, {j}")
+            self.o(f"s_cbranch_scc1 L_fd_{L}")
+            self.o(f"s_mov_b32 m0, s{base + 1}")
+            self.o(f"v_add_u32_e32 {T1}, s{base}, {T0}")
+            self.o("s_nop 0")
+            self.o(f"global_load_lds_dwordx4 {T1}, s[98:99]")
+        self.o(f"L_fd_{L}:")
+        self.o(f"s_mov_b32 {NEXTWIN}, s96")
+        self.o("s_bitcmp1_b32 s97, 0")
+        self.o(f"s_cbranch_scc0 L_fa_{L}")
+        self.o("s_waitcnt vmcnt(0)")
+        self.o("s_barrier")
+        self.o(f"L_fa_{L}:")
 
-    def window_switch(self, k1, L):
-        """Windowed rows: if op k1 of the group (0..16) is the first of the next window, every wavefront of the workgroup
-        stops here until that window's rows are in LDS.  Each wavefront copies its share of a window with LDS-direct
-        loads (descriptors {byte offset in the rows, LDS address, bytes} per window and wavefront).  Where consecutive
-        windows lie apart in LDS the loads of a window were issued when the window before it was entered, and here
-        those of the window after it are; otherwise the window is fetched here, between two barriers."""
+    def window_switch(self, k1, L, y):
+        """Windowed rows: if op k1 of the group (0..16) is the first of the next window, the next fetch event."""
         self.c("rows of the next window, if it starts with the next op")
         self.o(f"s_add_u32 {S0}, {POSBASE}, {k1}")
         self.o(f"s_cmp_eq_u32 {S0}, {NEXTWIN}")
         self.o(f"s_cbranch_scc0 L_nw_{L}")
-        self.o(f"s_load_dwordx8 s[52:59], {DMAPTR}, 0")
-        self.o("s_waitcnt vmcnt(0) lgkmcnt(0)")             # this wavefront's reads of the old rows and its loads so far have landed
-        self.o("s_barrier")
-        self.o(f"s_mov_b32 {ARRIVED}, 1")                   # (so have the next group's code words, if they were asked for)
-        self.o(f"s_add_u32 {WIN}, {WIN}, 1")
-        self.o(f"s_add_u32 {S0}, {WIN}, s58")
-        self.o(f"s_mul_i32 {DMAOFF}, {S0}, s57")
-        self.dma(L)
-        self.o(f"s_lshl_b32 {S0}, {WIN}, 2")
-        self.o(f"s_add_u32 {S0}, {S0}, 4")
-        self.o(f"s_load_dword {NEXTWIN}, s[54:55], {S0}")
-        self.o("s_cmp_eq_u32 s58, 1")
-        self.o(f"s_cbranch_scc1 L_wa_{L}")
-        self.o("s_waitcnt vmcnt(0)")
-        self.o("s_barrier")
-        self.o(f"L_wa_{L}:")
-        self.o("s_waitcnt lgkmcnt(0)")
+        self.fetch_event(L, 64 + 16 * y)                    # (the first two position entries of this word are done with)
         self.o(f"L_nw_{L}:")
         self.o(f"s_cmp_lg_u64 {M_ST}, 0")                   # (what the branch to the stage-end code tests)
 
@@ -241,7 +231,7 @@ class Gen:
         self.o(f"s_mov_b64 exec, {ALL}")
         self.o(f"L_ns_{L}:")
         if self.win and b == 3:
-            self.window_switch(k + 1, L)
+            self.window_switch(k + 1, L, y)
         self.issue(k + 1)
         if not self.rsh:
             self.o("s_waitcnt lgkmcnt(3)")
@@ -269,8 +259,11 @@ class Gen:
         self.o(f"v_max_f64 {PKT}, {PEAK}, {PKT}")
         self.reserved(cur)
         self.o(f"s_add_u32 {S0}, {POSBASE}, {k}")
+        self.o(f"s_andn2_b32 {S1}, {p['fl']}, 0xff")
+        self.o(f"s_lshl_b32 {S1}, {S1}, 8")
+        self.o(f"s_or_b32 {S0}, {S0}, {S1}")
         self.o(f"v_mov_b32 v50, {d['cn']}")                  # the record's last words: code*8 + next code of this word's ops,
-        self.o(f"v_mov_b32 v51, {S0}")                       # position of the stage's last op
+        self.o(f"v_mov_b32 v51, {S0}")                       # position of the stage's last op | its row << 16 | the next op's row << 24
         self.o(f"v_cmp_gt_u32_e32 vcc, 16, {CNT}")
         self.o("s_and_b64 exec, exec, vcc")
         self.o(f"v_lshl_add_u64 {T01}, {WSOFF64}, 4, %[rec]")
@@ -290,6 +283,10 @@ class Gen:
             self.o("s_nop 1")
             for r in (RCS, W_, A_, SAVED) + ((RSF, RSB) if self.rsh else ()):
                 self.o(f"v_mov_b64 {r}, 0")
+        self.c("that was the plan's last op (for every lane: the mark planted behind it): the padding positions need no walk")
+        self.o(f"s_add_u32 {S0}, {POSBASE}, {k + 1}")
+        self.o(f"s_cmp_eq_u32 {S0}, %[n_ops]")
+        self.o("s_cbranch_scc1 L_exit_%=")
         self.o(f"L_ne_{L}:")
         self.c("recompute pair (this op, next op): saved activations, running segment, peak")
         self.o(f"s_bitcmp1_b32 {p['fl']}, 0")
@@ -370,17 +367,11 @@ class Gen:
         o(f"s_mov_b32 {PREVFL}, 0")
         if self.win:
             o(f"s_mov_b64 {DMAPTR}, %[dma]")
-            o(f"s_mov_b32 {WIN}, 0")
             o(f"s_mov_b32 {ARRIVED}, 0")
-            o(f"s_load_dwordx8 s[52:59], {DMAPTR}, 0")
-            o("s_waitcnt lgkmcnt(0)")
-            o(f"s_load_dword {NEXTWIN}, s[54:55], 4")
-            c("windows that lie apart in LDS: window 0 was staged by the caller, fetch window 1")
-            o("s_cmp_eq_u32 s58, 1")
-            o("s_cbranch_scc0 L_nofetch_%=")
-            o(f"s_mov_b32 {DMAOFF}, s57")
-            self.dma("setup_%=")
-            o("L_nofetch_%=:")
+            o(f"s_mov_b32 {EVT}, 0")
+            c("window 0 (waited for), then window 1")
+            self.fetch_event("s0_%=", 80)
+            self.fetch_event("s1_%=", 80)
         o(f"global_load_dwordx4 v[102:105], %[codeoff], {CPTR}")
         o(f"s_load_dwordx16 {PBUF(0)}, {PPTR}, 0")
         for r in (FWD, BWD, RUN, PEAK, RFM[0], RBM[0], RCS, RSF, RSB, W_, A_, SAVED):
@@ -421,6 +412,8 @@ class Gen:
         o(f"s_add_u32 {GRP}, {GRP}, 1")
         o(f"s_cmp_lt_u32 {GRP}, %[n_groups]")
         o("s_cbranch_scc1 L_group_%=")
+        o("L_exit_%=:")
+        o(f"s_mov_b64 exec, {ALL}")
         o("s_waitcnt vmcnt(0) lgkmcnt(0)")
         o("s_setprio 0")
         o(f"v_mov_b32 %[cnt], {CNT}")

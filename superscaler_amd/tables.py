@@ -354,21 +354,11 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
     slots = avail // row_bytes
     if slots > 255:
         slots = 255
-    tp = graph.type_of_pos
-    N = graph.num_ops
-    # Rows that do not all fit: consecutive windows take turns on the two halves of the row region, so that the
-    # kernel can fetch the next window's rows while it walks the current one (the 32-bit copy of the pair kinds that
-    # such a kernel keeps in LDS as well comes out of the budget).  A half must hold a 4-op window and its successor row.
-    half = 0
-    if len(set(int(t) for t in tp)) > slots:
-        half = min(((avail - 4 * rk_bytes - 16) // row_bytes) // 2, 127)
-        if half < 5:
-            half = 0
     pos_info = np.zeros(graph.num_ops + 1, dtype=np.uint32)
     win_pos, win_row_begin, win_rows = [0], [0], []
-    if half:
-        slots = half
+    tp = graph.type_of_pos
     i = 0
+    N = graph.num_ops
     while i < N:
         # a window also holds the row of the op right after it (a stage that ends with the window's
         # last op opens the next stage there) and ends at a multiple of 4 ops (the kernel restages
@@ -396,8 +386,6 @@ def compile_tables(graph: og.OpGraph, db: ProfileDB, settings: CostModelSettings
         if good is None:
             raise ValueError("LDS too small for a 4-op window of this op graph")
         j, slot_of = good
-        if half and (len(win_pos) - 1) % 2:
-            slot_of = {ty: sl + half for ty, sl in slot_of.items()}
         for k in range(i, j):
             own = slot_of[int(tp[k])]
             nxt = slot_of[int(tp[k + 1])] if k + 1 < N else own

@@ -38,10 +38,7 @@ void score_one(const ace_tables_t *t, const AceGeom &g, std::vector<unsigned cha
         s.step(g, view, i, codes[i], nbyte, pair_bit(codes[i], nbyte), pos[i], i > 0 ? pos[i - 1] : 0u, i + 1 == g.N, rec);
     }
     if (DEFER) {
-        const int n_st = s.s;
-        s.replay_code = codes[0] & 7u;
-        for (int s2 = 0; s2 < n_st && s2 < ACE_MAX_STAGES; ++s2) s.replay(g, view, pos, rec, s2);
-        s.s = n_st;              // replay() walks s again; result() checks the count of the op loop
+        s.replay_all(g, view, rec, s.s, codes[0] & 7u, pos[0] & 0xffu);
     }
     s.result(g, t->nb_minus_1[s.bidx], iter, peak, feas, st);
 }

@@ -74,8 +74,10 @@ def cpu_baseline(tables, batch, threads):
 
 
 def kernel_name(tables):
-    return ("ace_score_kernel<BD=false,RANGED=false,WIN=true,DEFER=false>" if tables.n_windows > 1 else
-            "ace_score_kernel<BD=false,RANGED=false,WIN=false,DEFER=true>")
+    """The instantiation plain scoring of a large batch runs (the library's choice, ensure_stage_ws in ace_eval.hip)."""
+    deferred = tables.graph.num_ops < 65536 and (tables.n_windows == 1 or tables.rows.shape[0] <= 256)
+    return "ace_score_kernel<BD=false,RANGED=false,WIN=%s,DEFER=%s>" % ("true" if tables.n_windows > 1 else "false",
+                                                                          "true" if deferred else "false")
 
 
 def other_workloads(steps):

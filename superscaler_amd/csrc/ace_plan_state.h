@@ -441,9 +441,9 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false, bool GROW
         const ace_d2 oe = lx.oe;
         const uint32_t c_last = lx.c_last;
         if (live) replay_take(g, rx, lx, s2);
-        // (a stage no lane of the wavefront has is not fetched: its slot may never have been written)
-        if (ACE_WAVE_ANY(s2 + 2 < n_st)) replay_load(ws, s2 + 2, rx);
-        if (ACE_WAVE_ANY(s2 + 1 < n_st)) replay_lookups(g, lds, ry, s2 + 1, s2 + 1 < n_st, ly);
+        // (only lanes that have the stage fetch it: the slot of a stage a plan does not have may never have been written)
+        if (s2 + 2 < n_st) replay_load(ws, s2 + 2, rx);
+        if (s2 + 1 < n_st) replay_lookups(g, lds, ry, s2 + 1, true, ly);
         if (live) finish_tail(g, lds, 0u, c_last, oe, nullptr);
     }
 
@@ -455,7 +455,7 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false, bool GROW
         Lookups la, lb;
         replay_load(ws, 0, ra);
         rb = ra;
-        if (ACE_WAVE_ANY(1 < n_st)) replay_load(ws, 1, rb);
+        if (1 < n_st) replay_load(ws, 1, rb);
         replay_lookups(g, lds, ra, 0, 0 < n_st, la);
         lb = la;
         for (int s2 = 0; s2 < ACE_MAX_STAGES; s2 += 2) {

@@ -243,6 +243,32 @@ def test_every_settings_combination_matches_the_c_oracle(name, torch_mod):
 
 
 @pytest.mark.parametrize("name", ["gpt3_1_3b", "wresnet_1b"])
+def test_large_batches_of_every_loop_variant_match_the_c_oracle(name, torch_mod):
+    """The assembly op loop has one text per (resharding on / off, reserved-memory rule, rows resident / windowed), and
+    only batches of 128 workgroups or more run it over windowed rows: each of the six settings at 131,072 + 77 plans
+    against the C oracle, every plan."""
+    import dataclasses
+    from superscaler_amd.evaluator import PlanEvaluator
+    w = synth.WORKLOADS[name]
+    graph = synth.make_graph(w)
+    db = synth.make_db(w, graph)
+    batch = synth.make_plans(w, synth.make_tables(w), n_plans=131072 + 77, seed_offset=81, workers=8)
+    answers = set()
+    for resh in (True, False):
+        for pred, reserved in (("MAX", True), ("MIN", True), ("MAX", False)):
+            st = dataclasses.replace(synth.make_settings(w), memory_pred_type=pred, consider_reserved_space=reserved, resharding=resh)
+            tables = compile_tables(graph, db, st)
+            ev = PlanEvaluator(tables)
+            it, pk, fe, status = ev.score_host(batch)
+            ev.close()
+            cit, cpk, cfe, cer = c_oracle_scores(tables, batch, threads=16)
+            assert not cer.any() and (status == 0).all()
+            assert np.array_equal(it, cit) and np.array_equal(pk, cpk) and np.array_equal(fe, cfe), (pred, reserved, resh)
+            answers.add((float(pk.sum()), float(it.sum())))
+    assert len(answers) == 6
+
+
+@pytest.mark.parametrize("name", ["gpt3_1_3b", "wresnet_1b"])
 def test_collective_memory_switch_matches_the_oracle(name, torch_mod):
     """consider_collective_memory (aceso_cost_model.py:462-483): the buffers of the resharding collectives enter the
     reserved memory; the rows grow by the memory tables, so these runs also use the windowed kernel."""
@@ -341,6 +367,27 @@ def test_configured_sizes_match_c_oracle(name, n, torch_mod):
     feas = np.flatnonzero(cfe)
     order = feas[np.argsort(cit[feas], kind="stable")][:64]
     assert int(cnt.item()) == len(order) and np.array_equal(idx.cpu().numpy()[:len(order)], order)
+    ev.close()
+
+
+def test_windowed_rows_ragged_batch_and_small_batch_agree(torch_mod):
+    """wresnet_1b (rows windowed) at a size that is not a whole number of workgroups and large enough for the kernel
+    whose op loop fetches its own windows: every plan bit-identical to the C oracle, also after a second call on the
+    same handle, and identical to what the small-batch kernel (C++ loop, the tables' own windows) gives for a slice."""
+    from superscaler_amd.evaluator import PlanEvaluator
+    w = synth.WORKLOADS["wresnet_1b"]
+    tables = synth.make_tables(w)
+    n = 131072 + 517
+    batch = synth.make_plans(w, tables, n_plans=n, seed_offset=29, workers=8)
+    ev = PlanEvaluator(tables)
+    cit, cpk, cfe, cer = c_oracle_scores(tables, batch, threads=16)
+    for _ in range(2):
+        it, pk, fe, st = ev.score_host(batch)
+        assert (st == 0).all()
+        assert np.array_equal(it, cit) and np.array_equal(pk, cpk) and np.array_equal(fe, cfe)
+    lo, hi = n - 3000, n
+    sit, spk, sfe, sst = ev.score_host(batch.slice(lo, hi))
+    assert np.array_equal(sit, cit[lo:hi]) and np.array_equal(spk, cpk[lo:hi]) and np.array_equal(sfe, cfe[lo:hi])
     ev.close()
 
 

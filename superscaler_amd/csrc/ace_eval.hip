@@ -287,6 +287,12 @@ constexpr int kSample = 8192;            // sampled keys, sorted in LDS by one w
 constexpr unsigned kCandCap = 12000;     // candidates the last kernel can hold in LDS (12 bytes each)
 constexpr int kShortMaxK = 256;
 constexpr size_t kShortMaxNK = 1ull << 26;   // n * k up to this: about kSample candidates expected, kCandCap is 4 sigma above
+// Cost bound of the short form.  Usual input (distinct times): 0.04 ms at n = 2^20, k = 64.  When more than kCandCap
+// entries are at or below the sample's k-th key -- many equal times, or feasible plans crowded between the sampled
+// positions -- the last kernel selects from the whole input in global memory instead (ShortSource below): one
+// workgroup, about nine passes over n entries, measured 0.22 / 0.77 / 3.8 ms at n = 2^16 / 2^18 / 2^20 with every
+// time equal.  The result is the same either way; a caller that cannot afford that time on such inputs keeps n * k
+// small enough for it, or breaks ties before the call.
 
 struct ShortTopk { unsigned long long thr; unsigned int count; unsigned int pad; };
 

@@ -188,8 +188,8 @@ uint32_t ace_lds_pk32(uint32_t lds_end, uint32_t rk_bytes, uint32_t *pk32_off) {
 // BD: per-stage records for the caller.  RANGED: one stage over an op sub-range.  DEFER: stage
 // tails are not evaluated where the stage ends (where only the few lanes that cut at this op are
 // active) but stashed to a per-plan workspace and replayed after the op loop with every lane busy.
-// GROWS (with DEFER): the rows are windowed, so replay() looks the stage boundaries up in the rows' global copy (`gr`: the
-// geometry with row offsets as they are there).
+// GROWS (with DEFER): the rows are windowed, so the evaluation of the stashed stages looks the stage boundaries up in
+// the rows' global copy (its caller passes the geometry with row offsets as they are there).
 template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false, bool GROWS = false> struct PlanState {
     template <class T> ACE_HD static T row_ld(const AceLds &lds, uint32_t a) {
         if (GROWS) return lds.template gld<T>(a);

@@ -27,7 +27,8 @@ struct AceKernelArgs {
     const uint32_t *pos_info;   // [N + 1], padded to 16 * G + 16 entries
     const uint32_t *pos_types;  // windowed rows: the same with each row's index in `rows` in place of its LDS slot (null: more than 256 rows)
     const ace_u4 *pos4;         // [16 * G + 16] per position: LDS address of its row's hot sub-table, of its cost tables, of the
-                                //   32-bit pair-kind block of the (this, next) pair; bit 0: no layer start follows an ordinary op here, bit 1: ordinary op
+                                //   32-bit pair-kind block of the (this, next) pair; bit 0: no layer start follows an ordinary op here, bit 1: ordinary op,
+                                //   bits 8-15 / 16-23: this op's / the next op's row as the evaluation of the stage tails indexes rows
     const uint8_t *pair_kinds;  // -> LDS
     const uint32_t *stage_lut;  // -> LDS
     const double *nbm1;         // [n_mbs]

@@ -11,9 +11,18 @@ ace_plan_state.h, DEFER variant), written out by hand so that
   * every position-dependent address comes ready-made from a per-position table (four words per op position,
     read with scalar loads one 4-op word ahead) instead of being derived per op.
 Floating-point operations and their order per plan are exactly those of the C++ loop, so results are bit-identical.
+The loop ends with the plan's last op (every plan of a batch has the same number of ops; the mark planted behind the
+last op closes the last stage for all lanes at once), not with the padding positions of the last 16-op group.
 
-One text per (resharding on / off, reserved-memory rule); each is a C string literal macro that ace_score_loop.h
-pastes into an asm statement.  Register use: v28-v127 and s24-s99 belong to the loop; operands live below.
+The "_WIN" texts are for rows that do not fit in LDS together: the loop keeps its own windows of rows (only the parts
+of a row it reads), consecutive windows in alternate halves of LDS.  At a window's first position all wavefronts of
+the workgroup meet at a barrier, after which each issues its share of the LDS-direct loads of the window AFTER the
+one being entered (Gen.fetch_event; the records come from ace_eval.hip's setup_windowed_asm), which therefore arrive
+while the workgroup walks a whole window.
+
+One text per (rows resident / windowed, resharding on / off, reserved-memory rule); each is a C string literal macro
+that ace_score_loop.h pastes into an asm statement.  Register use: v28-v127 and s24-s99 belong to the loop; operands
+live below.
 """
 import os
 

@@ -34,7 +34,10 @@ namespace {
 #endif
 constexpr int kBlock = ACE_BLOCK;        // lanes (= plans) per workgroup: 16 wavefronts, 4 per SIMD
 constexpr int kSmallBlock = 256;         // ... for small batches: 4 wavefronts, 1 per SIMD
-constexpr int kSmallBatchBlocks = 128;   // batches of fewer than this many kBlock workgroups use kSmallBlock
+#ifndef ACE_SMALL_BATCH_BLOCKS
+#define ACE_SMALL_BATCH_BLOCKS 128
+#endif
+constexpr int kSmallBatchBlocks = ACE_SMALL_BATCH_BLOCKS;   // batches of fewer than this many kBlock workgroups use kSmallBlock
 constexpr uint32_t kMaxLds = 160 * 1024;  // CDNA4 LDS per workgroup
 static_assert(ACE_STATIC_MAX_PLANS % ACE_BLOCK == 0, "the static scratch holds whole workgroups");
 
@@ -1029,17 +1032,18 @@ static void launch_score_b(const ace_handle_t *h, const AceKernelArgs &a, hipStr
         if (!DEFER)         // (ensure_stage_ws never hands such tables to the deferred kernel)
             hipLaunchKernelGGL((ace_score_kernel<BD, RANGED, WIN, false, kBlock, true>), dim3((unsigned)((P + kBlock - 1) / kBlock)),
                                dim3(kBlock), h->lds_bytes, s, a);
-    } else if ((P + kBlock - 1) / kBlock < (size_t)kSmallBatchBlocks)
-        hipLaunchKernelGGL((ace_score_kernel<BD, RANGED, WIN, DEFER, kSmallBlock>), dim3((unsigned)((P + kSmallBlock - 1) / kSmallBlock)),
-                           dim3(kSmallBlock), h->lds_bytes, s, a);
-    else if (WIN && DEFER && h->d_win_dma) {
-        // the assembly op loop over windowed rows lays LDS out its own way
+    } else if (WIN && DEFER && h->d_win_dma) {
+        // the assembly op loop over windowed rows lays LDS out its own way (batches of any size: with the next window
+        // arriving while a window is walked, the large workgroup is the faster one from a single plan on)
         AceKernelArgs b = a;
         b.g = h->geom_wa;
         b.g.P = a.g.P; b.g.mem_limit = a.g.mem_limit; b.g.strict = a.g.strict;
         hipLaunchKernelGGL((ace_score_kernel<BD, RANGED, WIN, DEFER, kBlock>), dim3((unsigned)((P + kBlock - 1) / kBlock)),
                            dim3(kBlock), h->lds_bytes_wa, s, b);
-    } else
+    } else if ((P + kBlock - 1) / kBlock < (size_t)kSmallBatchBlocks)
+        hipLaunchKernelGGL((ace_score_kernel<BD, RANGED, WIN, DEFER, kSmallBlock>), dim3((unsigned)((P + kSmallBlock - 1) / kSmallBlock)),
+                           dim3(kSmallBlock), h->lds_bytes, s, a);
+    else
         hipLaunchKernelGGL((ace_score_kernel<BD, RANGED, WIN, DEFER, kBlock>), dim3((unsigned)((P + kBlock - 1) / kBlock)),
                            dim3(kBlock), h->lds_bytes, s, a);
 }

@@ -290,14 +290,19 @@ constexpr int kSample = 8192;            // sampled keys, sorted in LDS by one w
 constexpr unsigned kCandCap = 12000;     // candidates the last kernel can hold in LDS (12 bytes each)
 constexpr int kShortMaxK = 256;
 constexpr size_t kShortMaxNK = 1ull << 26;   // n * k up to this: about kSample candidates expected, kCandCap is 4 sigma above
-// Cost bound of the short form.  Usual input (distinct times): 0.04 ms at n = 2^20, k = 64.  When more than kCandCap
-// entries are at or below the sample's k-th key -- many equal times, or feasible plans crowded between the sampled
-// positions -- the last kernel selects from the whole input in global memory instead (ShortSource below): one
-// workgroup, about nine passes over n entries, measured 0.22 / 0.77 / 3.8 ms at n = 2^16 / 2^18 / 2^20 with every
-// time equal.  The result is the same either way; a caller that cannot afford that time on such inputs keeps n * k
-// small enough for it, or breaks ties before the call.
+// Equal keys: the threshold is the sample's exact k-th key; entries below it and entries equal to it are kept apart,
+// and of the equal ones only the lowest indices are ever needed (k minus the number of entries below).  Few of them go
+// into a list of their own; masses of them (a search neighbourhood whose plans share the bottleneck stage all have the
+// same time) are only COUNTED per filter workgroup, and the last kernel reads the first few of them from the input in
+// index order.  Cost: 0.04-0.05 ms at n = 2^20, k = 64 whatever the keys; only when more than kCandCap entries lie
+// strictly below the sample's k-th key (feasible plans crowded between the sampled positions) does the last kernel
+// select from the whole input in global memory instead (ShortSource below): one workgroup, about nine passes over
+// n entries, 3.8 ms at n = 2^20.
+constexpr unsigned kTieCap = 2048;       // equal-to-threshold entries listed one by one; beyond that: per-workgroup counts
+constexpr unsigned kMaxFilterGroups = 8192;   // n <= kShortMaxNK entries in workgroups of 8,192
+static_assert(kShortMaxNK / (1024 * 8) <= kMaxFilterGroups, "one count per filter workgroup");
 
-struct ShortTopk { unsigned long long thr; unsigned int count; unsigned int pad; };
+struct ShortTopk { unsigned long long thr; unsigned int count; unsigned int count_eq; };
 
 // Which of the kRadix buckets of `hist` (LDS) holds the rem-th entry (1-based), counting buckets in order: returns the
 // bucket, the entries before it in `before` and the total in `total` to every lane of the 1024-lane workgroup (no bucket:
@@ -360,8 +365,8 @@ __device__ __forceinline__ void short_minmax(unsigned long long mn, unsigned lon
     __syncthreads();
 }
 
-// The sample's k-th smallest key, to three radix digits below the bits all sampled keys share: the threshold is the largest key of that
-// bucket, an upper bound of the input's k-th smallest key that lets a few more entries through than the exact one would.
+// The sample's k-th smallest key: an upper bound of the input's k-th smallest key (with fewer than k feasible entries in
+// the sample: the largest finite key, so that every feasible entry is kept).
 __global__ __launch_bounds__(1024) void topk_sample(const double *t, const uint8_t *f, size_t n, int k, ShortTopk *st) {
     __shared__ unsigned long long key[kSample];
     __shared__ unsigned int hist[kRadix];
@@ -375,6 +380,9 @@ __global__ __launch_bounds__(1024) void topk_sample(const double *t, const uint8
         key[j] = (size_t)j < m ? time_key(t[i], f[i]) : kInfKey;
     }
     __shared__ unsigned long long wmm[48];
+    __shared__ unsigned long long small_keys[64];
+    __shared__ unsigned long long s_kth;
+    __shared__ unsigned int s_nsmall;
     unsigned long long mn = kInfKey, mx = 0, nf = 0;
     __syncthreads();
     for (int j = tid; j < kSample; j += 1024) {
@@ -387,7 +395,7 @@ __global__ __launch_bounds__(1024) void topk_sample(const double *t, const uint8
     unsigned long long prefix = cur >= 64 ? 0ull : (kmin >> cur) << cur;
     unsigned int rem = (unsigned)k;
     bool enough = nfin >= (unsigned long long)k;           // fewer than k feasible entries in the sample: keep every feasible entry
-    for (int pass = 0; pass < 3 && enough && cur > 0; ++pass) {
+    for (int pass = 0; pass < 8 && enough && cur > 0; ++pass) {
         for (int j = tid; j < kRadix; j += 1024) hist[j] = 0;
         __syncthreads();
         const int bits = cur < kRadixBits ? cur : kRadixBits, shift = cur - bits;
@@ -403,44 +411,85 @@ __global__ __launch_bounds__(1024) void topk_sample(const double *t, const uint8
         prefix |= (unsigned long long)b << shift;
         rem -= before;
         cur = shift;
+        const unsigned int in_bucket = hist[b];
+        __syncthreads();                                       // (hist[b] read by all before anything clears it)
+        if (cur > 0 && in_bucket <= 64u) {
+            // a handful of keys left in the bucket (distinct keys: after two passes): the rem-th smallest of them directly
+            if (tid == 0) s_nsmall = 0;
+            __syncthreads();
+            for (int j = tid; j < kSample; j += 1024) {
+                const unsigned long long x = key[j];
+                if (x != kInfKey && (x >> cur) == (prefix >> cur)) small_keys[atomicAdd(&s_nsmall, 1u) & 63u] = x;
+            }
+            __syncthreads();
+            if ((unsigned)tid < in_bucket) {
+                const unsigned long long me = small_keys[tid];
+                unsigned int rank = 0;
+                for (unsigned j = 0; j < in_bucket; ++j) {
+                    const unsigned long long o = small_keys[j];
+                    rank += (o < me || (o == me && j < (unsigned)tid)) ? 1u : 0u;
+                }
+                if (rank + 1u == rem) s_kth = me;
+            }
+            __syncthreads();
+            prefix = s_kth;
+            cur = 0;
+        }
     }
     if (tid == 0) {
-        // the largest key that starts with the digits found (all sampled keys equal: that key itself)
-        unsigned long long thr = enough ? (prefix | (cur > 0 ? ((1ull << cur) - 1ull) : 0ull)) : kInfKey;
+        // the sample's k-th smallest key itself (all digits found; all sampled keys equal: that key)
+        unsigned long long thr = enough ? prefix : kInfKey;
         if (thr == kInfKey) thr = kInfKey - 1;
-        st->thr = thr; st->count = 0; st->pad = 0;
+        st->thr = thr; st->count = 0; st->count_eq = 0;
     }
 }
 
 constexpr int kFilterPer = 8;             // entries per lane of topk_filter
-__global__ __launch_bounds__(1024) void topk_filter(const double *t, const uint8_t *f, size_t n, ShortTopk *st, Cand *cand) {
-    // One atomic on the shared counter per WORKGROUP (atomics on one address are served one after the other, about ten
-    // nanoseconds each): the lanes count their hits in LDS first.
-    __shared__ unsigned int s_hits, s_base;
+__global__ __launch_bounds__(1024) void topk_filter(const double *t, const uint8_t *f, size_t n, ShortTopk *st, Cand *cand,
+                                                    Cand *tiecand, unsigned int *group_ties) {
+    // One atomic on each shared counter per WORKGROUP (atomics on one address are served one after the other, about ten
+    // nanoseconds each): the lanes count their hits in LDS first.  Below the threshold: a candidate.  Equal to it: counted
+    // for this workgroup's stretch of the input (group_ties), and listed while the list has room.
+    __shared__ unsigned int s_hits, s_base, s_ties, s_tbase;
     const unsigned long long thr = st->thr;
     const size_t i0 = (size_t)blockIdx.x * 1024 * kFilterPer + threadIdx.x;
     unsigned long long key[kFilterPer];
-    if (threadIdx.x == 0) s_hits = 0;
+    if (threadIdx.x == 0) { s_hits = 0; s_ties = 0; }
 #pragma unroll
     for (int q = 0; q < kFilterPer; ++q) {
         const size_t i = i0 + (size_t)q * 1024;
         key[q] = i < n ? time_key(t[i], f[i]) : kInfKey;
     }
     __syncthreads();
-    unsigned int mine = 0;
+    unsigned int mine = 0, mine_eq = 0;
 #pragma unroll
-    for (int q = 0; q < kFilterPer; ++q) mine += key[q] <= thr ? 1u : 0u;
-    unsigned int first = 0;
+    for (int q = 0; q < kFilterPer; ++q) { mine += key[q] < thr ? 1u : 0u; mine_eq += key[q] == thr ? 1u : 0u; }
+    unsigned int first = 0, first_eq = 0;
     if (mine) first = atomicAdd(&s_hits, mine);
+    if (mine_eq) first_eq = atomicAdd(&s_ties, mine_eq);
     __syncthreads();
-    if (threadIdx.x == 0 && s_hits) s_base = atomicAdd(&st->count, s_hits);
+    if (threadIdx.x == 0) {
+        if (s_hits) s_base = atomicAdd(&st->count, s_hits);
+        if (s_ties) s_tbase = atomicAdd(&st->count_eq, s_ties);
+        group_ties[blockIdx.x] = s_ties;
+    }
     __syncthreads();
     if (mine) {
         unsigned int p = s_base + first;
 #pragma unroll
         for (int q = 0; q < kFilterPer; ++q) {
-            if (key[q] <= thr) {
+            if (key[q] < thr) {
                 if (p < kCandCap) cand[p] = Cand{key[q], (long long)(i0 + (size_t)q * 1024)};
+                ++p;
+            }
+        }
+    }
+    if (mine_eq) {
+        unsigned int p = s_tbase + first_eq;
+#pragma unroll
+        for (int q = 0; q < kFilterPer; ++q) {
+            if (key[q] == thr) {
+                if (p < kTieCap) tiecand[p] = Cand{key[q], (long long)(i0 + (size_t)q * 1024)};
                 ++p;
             }
         }
@@ -460,7 +509,8 @@ struct ShortSource {
 };
 
 __global__ __launch_bounds__(1024) void topk_short_final(const double *t, const uint8_t *f, size_t n, ShortTopk *st, const Cand *cand,
-                                                         int k, long long *out_idx, double *out_val, int *out_count) {
+                                                         const Cand *tiecand, const unsigned int *group_ties, int k,
+                                                         long long *out_idx, double *out_val, int *out_count) {
     extern __shared__ __align__(16) unsigned char smem[];
     unsigned long long *lkey = reinterpret_cast<unsigned long long *>(smem);                       // [kCandCap]
     unsigned int *lidx = reinterpret_cast<unsigned int *>(smem + (size_t)kCandCap * 8);            // [kCandCap]
@@ -469,11 +519,21 @@ __global__ __launch_bounds__(1024) void topk_short_final(const double *t, const 
     __shared__ unsigned int wsum[20];
     __shared__ unsigned int s_nwin;
     const int tid = threadIdx.x;
-    const unsigned int count = st->count;
-    ShortSource src{lkey, lidx, t, f, count > kCandCap};
+    const unsigned int count_lt = st->count, count_eq = st->count_eq;
+    ShortSource src{lkey, lidx, t, f, count_lt > kCandCap};
+    // Entries equal to the threshold matter only if fewer than k lie below it.  Then: all of them join the candidates if
+    // they were listed one by one and fit; otherwise every entry below wins, and the lowest-indexed equal ones are read
+    // from the input (tie_scan, after the selection).
+    const bool want_ties = !src.global && count_lt < (unsigned)k && count_eq > 0;
+    const bool ties_listed = want_ties && count_eq <= kTieCap && count_lt + count_eq <= kCandCap;
+    const bool tie_scan = want_ties && !ties_listed;
+    const unsigned int count = count_lt + (ties_listed ? count_eq : 0u);
     const size_t m = src.global ? n : (size_t)count;
-    if (!src.global)
-        for (unsigned j = tid; j < count; j += 1024) { const Cand c = cand[j]; lkey[j] = c.key; lidx[j] = (unsigned int)c.idx; }
+    if (!src.global) {
+        for (unsigned j = tid; j < count_lt; j += 1024) { const Cand c = cand[j]; lkey[j] = c.key; lidx[j] = (unsigned int)c.idx; }
+        if (ties_listed)
+            for (unsigned j = tid; j < count_eq; j += 1024) { const Cand c = tiecand[j]; lkey[count_lt + j] = c.key; lidx[count_lt + j] = (unsigned int)c.idx; }
+    }
     if (tid == 0) s_nwin = 0;
     // radix select on the 96-bit order (key, index): 6 passes over the key bits, then 3 over the index bits of the entries
     // whose key is the selected one -- cut short as soon as the bucket that holds the k-th entry is small enough to be sorted
@@ -491,7 +551,7 @@ __global__ __launch_bounds__(1024) void topk_short_final(const double *t, const 
     }
     unsigned long long kmin, kmax, nfin;
     short_minmax(mn, mx, nf, wmm, kmin, kmax, nfin);
-    const bool all = nfin < (unsigned long long)k;             // fewer feasible entries than asked for: all of them win
+    const bool all = nfin < (unsigned long long)k;             // fewer (feasible) candidates than asked for: all of them win
     int cur = (nfin == 0 || kmin == kmax) ? 0 : 64 - __clzll((long long)(kmin ^ kmax));      // the low `cur` key bits vary
     unsigned long long prefix = cur >= 64 ? 0ull : (kmin >> cur) << cur;
     unsigned int iprefix = 0, rem = (unsigned)k;
@@ -571,6 +631,37 @@ __global__ __launch_bounds__(1024) void topk_short_final(const double *t, const 
         if (tid == 0) s_nwin = base + rem;
     }
     __syncthreads();
+    if (tie_scan) {
+        // every candidate below the threshold has won (there are fewer than k: `all`); the rest of the k are the entries
+        // EQUAL to the threshold with the lowest indices.  group_ties[g] says how many of them stretch g of the input
+        // (8,192 consecutive entries) holds: stretches without any are skipped, the others read 1,024 entries at a time
+        // in index order, each lane ranking its entry among the equal ones of the step (wavefront ballots, one
+        // exchange through LDS), until enough are found.
+        const unsigned long long thr = st->thr;
+        const unsigned int need = (unsigned)k - s_nwin, base = s_nwin;
+        const unsigned int n_groups = (unsigned int)((n + 1024 * (size_t)kFilterPer - 1) / (1024 * (size_t)kFilterPer));
+        __shared__ unsigned int s_wave_ties[16];
+        unsigned int found = 0;
+        for (unsigned int g = 0; g < n_groups && found < need; ++g) {
+            if (group_ties[g] == 0) continue;                  // (the same for every lane)
+            for (int c = 0; c < kFilterPer && found < need; ++c) {
+                const size_t i = (size_t)g * 1024 * kFilterPer + (size_t)c * 1024 + (size_t)tid;
+                const bool eq = i < n && time_key(t[i], f[i]) == thr;
+                const unsigned long long mask = __ballot(eq);
+                const int lane = tid & 63, wave = tid >> 6;
+                if (lane == 0) s_wave_ties[wave] = (unsigned int)__popcll(mask);
+                __syncthreads();
+                unsigned int before = 0, total = 0;
+                for (int w = 0; w < 16; ++w) { const unsigned int v = s_wave_ties[w]; before += w < wave ? v : 0u; total += v; }
+                const unsigned int rank = found + before + (unsigned int)__popcll(mask & ((1ull << lane) - 1ull));
+                if (eq && rank < need && base + rank < (unsigned)kShortMaxK) win[base + rank] = Cand{thr, (long long)i};
+                found += total;
+                __syncthreads();
+            }
+        }
+        if (tid == 0) s_nwin = base + (found < need ? found : need);
+        __syncthreads();
+    }
     const unsigned int nwin = s_nwin < (unsigned)k ? s_nwin : (unsigned)k;
     // the winners in ascending (key, index) order, by rank as above
     for (unsigned j = tid; j < (unsigned)k; j += 1024) {
@@ -1161,7 +1252,8 @@ size_t ace_topk_workspace_bytes(size_t n, int k) {
     const unsigned cap = topk_cap(k);
     const unsigned p2 = next_pow2(2 * cap);
     // (the last part: state and candidates of the short form)
-    return 256 + sizeof(unsigned int) * kRadix + sizeof(Cand) * ((size_t)cap * 2 + p2) + 256 + sizeof(Cand) * kCandCap;
+    return 256 + sizeof(unsigned int) * kRadix + sizeof(Cand) * ((size_t)cap * 2 + p2) + 256 + sizeof(Cand) * (kCandCap + kTieCap) +
+           sizeof(unsigned int) * kMaxFilterGroups;
 }
 
 int ace_topk(ace_handle_t *h, const double *d_iter_ms, const uint8_t *d_feasible, size_t n, int k, int64_t *d_idx,
@@ -1183,10 +1275,12 @@ int ace_topk(ace_handle_t *h, const double *d_iter_ms, const uint8_t *d_feasible
     if (k <= kShortMaxK && n * (size_t)k <= kShortMaxNK && n <= 0xffffffffull) {
         ShortTopk *sst = (ShortTopk *)(buf + p2);
         Cand *cand = (Cand *)((unsigned char *)sst + 256);
+        Cand *tiecand = cand + kCandCap;
+        unsigned int *group_ties = (unsigned int *)(tiecand + kTieCap);      // (at most kMaxFilterGroups filter workgroups: n <= kShortMaxNK)
         hipLaunchKernelGGL(topk_sample, dim3(1), dim3(1024), 0, s, d_iter_ms, d_feasible, n, k, sst);
         hipLaunchKernelGGL(topk_filter, dim3((unsigned)((n + 1024 * kFilterPer - 1) / (1024 * kFilterPer))), dim3(1024), 0, s, d_iter_ms,
-                           d_feasible, n, sst, cand);
-        hipLaunchKernelGGL(topk_short_final, dim3(1), dim3(1024), kShortLds, s, d_iter_ms, d_feasible, n, sst, cand, k,
+                           d_feasible, n, sst, cand, tiecand, group_ties);
+        hipLaunchKernelGGL(topk_short_final, dim3(1), dim3(1024), kShortLds, s, d_iter_ms, d_feasible, n, sst, cand, tiecand, group_ties, k,
                            (long long *)d_idx, d_val, d_count);
         ACE_HIP(hipGetLastError());
         return ACE_OK;

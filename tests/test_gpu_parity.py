@@ -110,7 +110,7 @@ def test_topk_ties_pick_lowest_index(torch_mod):
 
 def test_topk_short_form_edges(torch_mod):
     """The three-launch form of the top-k (small k): inputs on which the sample's bound lets nearly everything through (all
-    times equal, a million of them: the last kernel then selects from global memory), heavy duplication, negative zero and
+    times equal, a million of them), heavy duplication, negative zero and
     infinities, all infeasible, a single entry -- against a stable sort; and the same results as the multi-launch form."""
     from superscaler_amd.evaluator import PlanEvaluator
     torch = torch_mod
@@ -143,6 +143,29 @@ def test_topk_short_form_edges(torch_mod):
     check(rng.random(5000), np.zeros(5000, dtype=np.uint8), [64])                           # nothing feasible
     check(rng.random(70), np.ones(70, dtype=np.uint8), [64, 100])                           # fewer entries than the sample, than k
     check(np.array([3.5]), np.ones(1, dtype=np.uint8), [1, 5])
+    # equal keys at the k-th place: a few entries below a mass of equal ones (the equal ones are only counted per stretch
+    # of the input and read back in index order), the mass starting late in the input, infeasible entries inside it,
+    # just enough equal ones to be listed one by one, and equal ones one per stretch of 8,192
+    t = np.full(n, 9.5)
+    t[rng.choice(n, 40, replace=False)] = rng.random(40)
+    check(t, np.ones(n, dtype=np.uint8), [1, 39, 40, 41, 64, 256])
+    t = rng.random(n) + 20.0
+    t[700000:] = 3.0
+    f = np.ones(n, dtype=np.uint8)
+    f[700000:700100] = 0
+    f[700105::2] = 0
+    t[5] = 1.0
+    check(t, f, [1, 2, 64, 256])
+    t = rng.random(n) + 20.0
+    t[rng.choice(n, 2000, replace=False)] = 4.0
+    check(t, np.ones(n, dtype=np.uint8), [64, 256])
+    t = rng.random(n) + 20.0
+    t[4096::8192] = 4.0
+    t[4097::8192 * 3] = 4.0
+    check(t, np.ones(n, dtype=np.uint8), [8, 64, 200])
+    t = np.full(1 << 24, 2.0)                                                              # n * k at the short form's limit
+    t[123457] = 1.0
+    check(t, np.ones(1 << 24, dtype=np.uint8), [1, 4])
     t = rng.random(100000)
     f = np.zeros(100000, dtype=np.uint8)
     f[rng.choice(100000, 40, replace=False)] = 1

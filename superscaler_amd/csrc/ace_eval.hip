@@ -941,7 +941,7 @@ static int setup_windowed_asm(ace_handle *h, const ace_tables_t *t, size_t pos_e
     if (rc != ACE_OK) return rc;
     h->geom_wa = h->geom;
     h->geom_wa.rk_lds_off = 2u * slots * crow;
-    h->geom_wa.stg_lds_off = stg_off; h->geom_wa.lut2_lds_off = lut2_off; h->geom_wa.pk32_lds_off = pk32_off;
+    h->geom_wa.stg_lds_off = stg_off; h->geom_wa.lut2_lds_off = lut2_off; h->geom_wa.pk32_lds_off = pk32_off; h->geom_wa.pace_lds_off = 0;
     h->lds_bytes_wa = lds_end;
     return ACE_OK;
 }
@@ -997,13 +997,14 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     if (lds_bytes > kMaxLds) return ACE_ETOOBIG;
     // the assembly loop's pair-kind table, where the table has room and its entries can hold the offsets (otherwise plain
     // scoring takes the C++ form of the loop)
-    uint32_t pk32_off = 0;
+    uint32_t pk32_off = 0, pace_off = 0;
     if (t->n_windows == 1) {                               // (windowed rows: setup_windowed_asm lays LDS out anew)
         uint32_t off;
         const uint32_t end = ace_lds_pk32(lds_bytes, (uint32_t)rk_bytes, &off);
-        if (end <= kMaxLds && ((int64_t)(t->n_z > 0 ? t->n_z : 1) * t->z_table_doubles * 8) <= 65536) {
+        if (end + 128u <= kMaxLds && ((int64_t)(t->n_z > 0 ? t->n_z : 1) * t->z_table_doubles * 8) <= 65536) {
             pk32_off = off;
-            lds_bytes = end;
+            pace_off = (end + 15u) & ~15u;
+            lds_bytes = pace_off + 128u;
         }
     }
     // (the in-kernel sort keeps its bins and its permutation in the first 128 + 2 * kBlock bytes of LDS before the
@@ -1050,7 +1051,7 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     g.z_shift = 3;
     while ((1 << (g.z_shift - 3)) < t->z_table_doubles) ++g.z_shift;
     g.zm_delta = (uint32_t)t->n_z << g.z_shift;
-    g.rk_lds_off = rk_off; g.stg_lds_off = stg_off; g.lut2_lds_off = lut2_off; g.pk32_lds_off = pk32_off;
+    g.rk_lds_off = rk_off; g.stg_lds_off = stg_off; g.lut2_lds_off = lut2_off; g.pk32_lds_off = pk32_off; g.pace_lds_off = pace_off;
     g.rk_kind_stride = (uint32_t)(t->n_glog * 64);
     g.row_bytes = (uint32_t)row_bytes;
     g.flags = t->flags; g.main_params = t->main_params; g.optimizer = t->optimizer;

@@ -89,6 +89,7 @@ __device__ __forceinline__ uint32_t ace_score_loop_asm(const AceKernelArgs &a, c
     const uint64_t gstride = (uint64_t)(uint32_t)g.P * 16u;
     const uint32_t gs_lo = (uint32_t)gstride, gs_hi = (uint32_t)(gstride >> 32);
     const uint32_t c8 = (uint32_t)g.C * 8u;
+    const uint32_t pace = g.pace_lds_off + (wave & 3u) * 32u;     // this SIMD's eight arrival counters
     if (WIN) {
 #define ACE_LOOP_ASM_RUN(TEXT)                                                                                          \
     asm volatile(TEXT : [cnt] "=&v"(cnt)                                                                               \
@@ -113,7 +114,8 @@ __device__ __forceinline__ uint32_t ace_score_loop_asm(const AceKernelArgs &a, c
     asm volatile(TEXT : [cnt] "=&v"(cnt)                                                                               \
                  : [dg] "v"(dg), [rk] "v"(rks), [codeoff] "v"(code_off), [rec] "v"(rec), [codes] "s"(a.codes),         \
                    [pos] "s"(a.pos4), [c8] "s"(c8), [n_ops] "s"(g.N), [n_groups] "s"(g.G),                                \
-                   [gstride_lo] "s"(gs_lo), [gstride_hi] "s"(gs_hi), [wsstride] "s"(ws_stride), [prio] "s"(prio)        \
+                   [gstride_lo] "s"(gs_lo), [gstride_hi] "s"(gs_hi), [wsstride] "s"(ws_stride), [prio] "s"(prio),       \
+                   [pace] "s"(pace)                                                                                     \
                  : ACE_LOOP_ASM_CLOBBERS)
     if (g.flags & ACE_F_RESHARDING) {
         if (g.flags & ACE_F_NO_RESERVED) ACE_LOOP_ASM_RUN(ACE_LOOP_ASM_RSH1_NONE);
@@ -242,6 +244,7 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
 #else
     const bool asm_loop = false;
 #endif
+    if (DEFER && a.g.pace_lds_off && tid < 32) reinterpret_cast<uint32_t *>(lds_raw + a.g.pace_lds_off)[tid] = 0u;
     if (!(WIN && asm_loop)) stage_window<BLOCK>(a, lds_raw, w0, tid);       // every row, or the first window's
     ACE_SYNC();
 

@@ -14,6 +14,14 @@ Floating-point operations and their order per plan are exactly those of the C++ 
 The loop ends with the plan's last op (every plan of a batch has the same number of ops; the mark planted behind the
 last op closes the last stage for all lanes at once), not with the padding positions of the last 16-op group.
 
+Pacing (rows resident): the wavefronts of a workgroup share the cache lines of their plans' code bytes (a line holds
+the 16 bytes of eight neighbouring plans, which the depth sort deals to different wavefronts), and a wavefront of
+deep plans needs twice the instructions per op of one with shallow plans: left alone they drift groups apart and every
+line is fetched from memory twice.  So each SIMD counts, per 16-op group, how many of its four wavefronts have
+entered it (eight LDS counters per SIMD, used in turn, never reset: the count modulo 4 is the rank); the two that enter
+a group last run at issue priority 3 until their next group, the two that were first at 0.  The wavefronts of a
+workgroup then walk within a group or two of each other.
+
 The "_WIN" texts are for rows that do not fit in LDS together: the loop keeps its own windows of rows (only the parts
 of a row it reads), consecutive windows in alternate halves of LDS.  At a window's first position all wavefronts of
 the workgroup meet at a barrier, after which each issues its share of the LDS-direct loads of the window AFTER the
@@ -65,6 +73,7 @@ def D(y):                                   # per 4-op word: next-op bytes, code
 
 
 ZV_, RK, WSOFF, WSOFF64, CNT = "v120", "v121", "v122", "v[122:123]", "v125"   # (v123 stays zero)
+PACE = "v124"                               # lane 0: what this group's arrival counter read before this wavefront was counted
 DG, DG_LO, RKS, RKS_LO = "v[28:29]", "v28", "v[30:31]", "v30"   # per stage, 4 bits each, next stage lowest: diag; pair-table block
 T0, T1, T01, T2 = "v126", "v127", "v[126:127]", "v33"
 
@@ -218,6 +227,16 @@ class Gen:
             self.o(f"s_load_dwordx16 {PBUF((j + 1) & 1)}, {PPTR}, {64 * (j + 1)}")
         if b == 2:
             self.o("s_waitcnt lgkmcnt(0)")
+            if k == 2 and not self.win:
+                self.c("pacing: the two wavefronts of a SIMD that entered this group last get the issue priority, the two that are ahead yield")
+                self.o(f"v_readfirstlane_b32 {S0}, {PACE}")
+                self.o(f"s_bitcmp1_b32 {S0}, 1")
+                self.o("s_cbranch_scc0 L_pp0_%=")
+                self.o("s_setprio 3")
+                self.o("s_branch L_ppd_%=")
+                self.o("L_pp0_%=:")
+                self.o("s_setprio 0")
+                self.o("L_ppd_%=:")
         if k == 11:
             self.next_group_words()
         if b == 3:
@@ -410,6 +429,16 @@ class Gen:
         o("L_loaded_%=:")
         if self.win:
             o(f"s_mov_b32 {ARRIVED}, 0")
+        else:
+            c("pacing: count this wavefront into this group's arrival counter of its SIMD (the count before it: its rank among the four)")
+            o(f"s_and_b32 {S0}, {GRP}, 7")
+            o(f"s_lshl_b32 {S0}, {S0}, 2")
+            o(f"s_add_u32 {S0}, {S0}, %[pace]")
+            o(f"v_mov_b32 {T1}, {S0}")
+            o(f"v_mov_b32 {T0}, 1")
+            o("s_mov_b64 exec, 1")
+            o(f"ds_add_rtn_u32 {PACE}, {T1}, {T0}")
+            o(f"s_mov_b64 exec, {ALL}")
         for k in range(16):
             self.slot(k)
         c("---- next group")

@@ -22,7 +22,7 @@
 #include "ace_score_loop.h"
 
 // Scratch of ace_score_batch_static: the deferred-stage-tail records of up to ACE_STATIC_MAX_PLANS plans (the
-// layout ace_score_body's DEFER variant uses: [stage][plan slot][ACE_WS_REC]).  Every GPU the library runs on holds
+// layout ace_score_body's DEFER variant uses: [workgroup][stage][lane][ACE_WS_REC]).  Every GPU the library runs on holds
 // its own copy of this array until the process ends.  In host code the array's name is only a stand-in for
 // hipGetSymbolAddress(): kernels get the per-device pointer that call returned (static_scratch_ptr), never the name.
 static __device__ __align__(256) double scratch[(size_t)ACE_STATIC_MAX_PLANS * ACE_MAX_STAGES * ACE_WS_REC];
@@ -941,7 +941,7 @@ static int setup_windowed_asm(ace_handle *h, const ace_tables_t *t, size_t pos_e
     if (rc != ACE_OK) return rc;
     h->geom_wa = h->geom;
     h->geom_wa.rk_lds_off = 2u * slots * crow;
-    h->geom_wa.stg_lds_off = stg_off; h->geom_wa.lut2_lds_off = lut2_off; h->geom_wa.pk32_lds_off = pk32_off; h->geom_wa.pace_lds_off = 0;
+    h->geom_wa.stg_lds_off = stg_off; h->geom_wa.lut2_lds_off = lut2_off; h->geom_wa.pk32_lds_off = pk32_off; h->geom_wa.pace_lds_off = 0; h->geom_wa.lut2a_lds_off = 0;
     h->lds_bytes_wa = lds_end;
     return ACE_OK;
 }
@@ -997,14 +997,16 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     if (lds_bytes > kMaxLds) return ACE_ETOOBIG;
     // the assembly loop's pair-kind table, where the table has room and its entries can hold the offsets (otherwise plain
     // scoring takes the C++ form of the loop)
-    uint32_t pk32_off = 0, pace_off = 0;
+    uint32_t pk32_off = 0, pace_off = 0, lut2a_off = 0;
     if (t->n_windows == 1) {                               // (windowed rows: setup_windowed_asm lays LDS out anew)
         uint32_t off;
         const uint32_t end = ace_lds_pk32(lds_bytes, (uint32_t)rk_bytes, &off);
-        if (end + 128u <= kMaxLds && ((int64_t)(t->n_z > 0 ? t->n_z : 1) * t->z_table_doubles * 8) <= 65536) {
+        // (behind it: the loop's arrival counters and its own per-(micro-batch, stage size) offset pairs)
+        if (end + 128u + (uint32_t)stg_words * 8u + 16u <= kMaxLds && ((int64_t)(t->n_z > 0 ? t->n_z : 1) * t->z_table_doubles * 8) <= 65536) {
             pk32_off = off;
             pace_off = (end + 15u) & ~15u;
-            lds_bytes = pace_off + 128u;
+            lut2a_off = pace_off + 128u;
+            lds_bytes = lut2a_off + (uint32_t)stg_words * 8u;
         }
     }
     // (the in-kernel sort keeps its bins and its permutation in the first 128 + 2 * kBlock bytes of LDS before the
@@ -1051,7 +1053,7 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     g.z_shift = 3;
     while ((1 << (g.z_shift - 3)) < t->z_table_doubles) ++g.z_shift;
     g.zm_delta = (uint32_t)t->n_z << g.z_shift;
-    g.rk_lds_off = rk_off; g.stg_lds_off = stg_off; g.lut2_lds_off = lut2_off; g.pk32_lds_off = pk32_off; g.pace_lds_off = pace_off;
+    g.rk_lds_off = rk_off; g.stg_lds_off = stg_off; g.lut2_lds_off = lut2_off; g.pk32_lds_off = pk32_off; g.pace_lds_off = pace_off; g.lut2a_lds_off = lut2a_off;
     g.rk_kind_stride = (uint32_t)(t->n_glog * 64);
     g.row_bytes = (uint32_t)row_bytes;
     g.flags = t->flags; g.main_params = t->main_params; g.optimizer = t->optimizer;
@@ -1166,7 +1168,7 @@ static int ensure_stage_ws(ace_handle_t *h, AceKernelArgs *a) {
     a->stage_ws = nullptr;
     if (a->range || a->stage_out || (h->n_windows > 1 && !h->d_pos_types) || h->geom.N >= 65536 || (h->geom.flags & ACE_F_COLLECTIVE_MEM)) return ACE_OK;
     const size_t need = (((size_t)a->g.P + kBlock - 1) / kBlock) * kBlock;
-    if (need * ACE_MAX_STAGES * (ACE_WS_REC / 2) > 0xffffffffull) return ACE_OK;   // 32-bit record offsets: larger batches take the plain kernel
+    if (need * ACE_MAX_STAGES * (ACE_WS_REC / 2) > 0xffffffffull) return ACE_OK;   // (a workspace of 64 GiB and more: such batches take the plain kernel)
     if (need > h->stage_ws_plans) {
         if (h->stage_ws_fixed) return ACE_EFIXED;
         if (h->d_stage_ws) ACE_HIP(hipFree(h->d_stage_ws));

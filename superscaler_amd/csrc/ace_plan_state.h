@@ -145,6 +145,7 @@ struct AceGeom {
     uint32_t lut2_lds_off;                         // ... of the per-(micro-batch, stage size) offset pairs (see ace_lds_layout)
     uint32_t pk32_lds_off;                         // ... of the pair-kind table in the assembly loop's form (0: LDS has no room for it)
     uint32_t pace_lds_off;                         // ... of the 4 x 8 arrival counters the assembly loop paces its wavefronts by
+    uint32_t lut2a_lds_off;                        // ... of the assembly loop's own offset pairs (the block offset not relative; 0: none)
     uint32_t rk_kind_stride;    // bytes of one pair kind (n_glog * 64)
     uint32_t row_bytes;         // bytes of one op type's row
     int32_t flags;

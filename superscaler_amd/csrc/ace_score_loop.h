@@ -40,7 +40,7 @@ struct AceKernelArgs {
     double *iter_ms, *peak_mb;
     uint8_t *feasible, *status;
     double *stage_out;          // [P][ACE_MAX_STAGES][ACE_STAGE_REC], single-stage queries [P][ACE_STAGE_REC]
-    double *stage_ws;           // [ACE_MAX_STAGES][plans rounded up to whole workgroups][ACE_WS_REC] for deferred stage tails
+    double *stage_ws;           // [workgroup][ACE_MAX_STAGES][lanes of a workgroup][ACE_WS_REC] for deferred stage tails
 };
 
 // Windowed rows: the position descriptors (pos_info) with each row's index in `rows` where its LDS slot is (and the next
@@ -84,7 +84,8 @@ template <int BLOCK> ACE_HD void stage_window(const AceKernelArgs &a, unsigned c
 // event and wavefront, sixteen wavefronts: see the generator).
 template <bool WIN>
 __device__ __forceinline__ uint32_t ace_score_loop_asm(const AceKernelArgs &a, const AceGeom &g, uint64_t dg, uint64_t rks,
-                                                       uint32_t code_off, double *rec, uint32_t ws_stride, uint32_t prio, uint32_t wave) {
+                                                       uint32_t code_off, const double *rec_base, uint32_t rec_off, uint32_t ws_stride,
+                                                       uint32_t prio, uint32_t wave) {
     uint32_t cnt;
     const uint64_t gstride = (uint64_t)(uint32_t)g.P * 16u;
     const uint32_t gs_lo = (uint32_t)gstride, gs_hi = (uint32_t)(gstride >> 32);
@@ -93,8 +94,8 @@ __device__ __forceinline__ uint32_t ace_score_loop_asm(const AceKernelArgs &a, c
     if (WIN) {
 #define ACE_LOOP_ASM_RUN(TEXT)                                                                                          \
     asm volatile(TEXT : [cnt] "=&v"(cnt)                                                                               \
-                 : [dg] "v"(dg), [rk] "v"(rks), [codeoff] "v"(code_off), [rec] "v"(rec), [codes] "s"(a.codes),         \
-                   [pos] "s"(a.pos4), [c8] "s"(c8), [n_ops] "s"(g.N), [n_groups] "s"(g.G),                                \
+                 : [dg] "v"(dg), [rk] "v"(rks), [codeoff] "v"(code_off), [recoff] "v"(rec_off), [codes] "s"(a.codes),   \
+                   [pos] "s"(a.pos4), [c8] "s"(c8), [n_ops] "s"(g.N), [n_groups] "s"(g.G), [recbase] "s"(rec_base),         \
                    [gstride_lo] "s"(gs_lo), [gstride_hi] "s"(gs_hi), [wsstride] "s"(ws_stride), [prio] "s"(prio),       \
                    [dma] "s"(a.win_dma), [waveoff] "s"(wave * 80u)                                                      \
                  : ACE_LOOP_ASM_CLOBBERS)
@@ -112,8 +113,8 @@ __device__ __forceinline__ uint32_t ace_score_loop_asm(const AceKernelArgs &a, c
     }
 #define ACE_LOOP_ASM_RUN(TEXT)                                                                                          \
     asm volatile(TEXT : [cnt] "=&v"(cnt)                                                                               \
-                 : [dg] "v"(dg), [rk] "v"(rks), [codeoff] "v"(code_off), [rec] "v"(rec), [codes] "s"(a.codes),         \
-                   [pos] "s"(a.pos4), [c8] "s"(c8), [n_ops] "s"(g.N), [n_groups] "s"(g.G),                                \
+                 : [glogs] "v"(dg), [lut2] "v"((uint32_t)rks), [codeoff] "v"(code_off), [recoff] "v"(rec_off),          \
+                   [codes] "s"(a.codes), [pos] "s"(a.pos4), [n_ops] "s"(g.N), [n_groups] "s"(g.G), [recbase] "s"(rec_base), \
                    [gstride_lo] "s"(gs_lo), [gstride_hi] "s"(gs_hi), [wsstride] "s"(ws_stride), [prio] "s"(prio),       \
                    [pace] "s"(pace)                                                                                     \
                  : ACE_LOOP_ASM_CLOBBERS)
@@ -147,6 +148,7 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     const uint32_t lds_base = ace_lds_base(lds_raw);
     g.hot_off += lds_base; g.start_off += lds_base; g.out_off += lds_base; g.z_off += lds_base;
     g.rk_lds_off += lds_base; g.stg_lds_off += lds_base; g.lut2_lds_off += lds_base;
+    if (g.lut2a_lds_off) g.lut2a_lds_off += lds_base;
     const long long slot = block * BLOCK + tid;                     // this lane's place in the batch (and in the workspace)
     long long plan = slot;
     uint32_t prio = 0;                                              // issue priority of this wavefront in the op loop
@@ -235,12 +237,14 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
         // and the pair-kind block of the stage size relative to it (what PlanState::start_fast hands to the op loop)
         const uint32_t glog = (uint32_t)j & 15u;
         const uint32_t z_v = (w & 15u) * (uint32_t)a.g.C * 8u;
-        reinterpret_cast<ace_u2 *>(lds_raw + a.g.lut2_lds_off)[j] =
-            ace_u2{z_v, ((glog < (uint32_t)a.g.n_glog ? glog : 0u) << 6) - z_v};
+        const uint32_t rk = (glog < (uint32_t)a.g.n_glog ? glog : 0u) << 6;
+        reinterpret_cast<ace_u2 *>(lds_raw + a.g.lut2_lds_off)[j] = ace_u2{z_v, rk - z_v};
+        // (the assembly loop adds the pair-kind block offset to the op pair's own index, not to the diag's)
+        if (DEFER && a.g.lut2a_lds_off) reinterpret_cast<ace_u2 *>(lds_raw + a.g.lut2a_lds_off)[j] = ace_u2{z_v, rk};
     }
     // (the assembly op loop over windowed rows fetches its windows itself, in a layout of its own)
 #ifndef ACE_HOST_EMU
-    const bool asm_loop = DEFER && lds_base == 0u && a.pos4 && (!WIN || (BLOCK == 1024 && a.win_dma));
+    const bool asm_loop = DEFER && lds_base == 0u && a.pos4 && (WIN ? (BLOCK == 1024 && a.win_dma) : a.g.lut2a_lds_off != 0u);
 #else
     const bool asm_loop = false;
 #endif
@@ -259,9 +263,10 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     const size_t rec_doubles = RANGED ? (size_t)ACE_STAGE_REC : (size_t)(ACE_MAX_STAGES * ACE_STAGE_REC);
     double *rec = (BD && a.stage_out && active) ? a.stage_out + (size_t)out * rec_doubles : nullptr;
     if (DEFER) {
-        // stage-major: the records of one stage of consecutive plans are adjacent (padded lanes own a slot too)
-        rec = a.stage_ws + (size_t)slot * ACE_WS_REC;
-        st.ws_stride = n_blocks * (uint32_t)BLOCK * (ACE_WS_REC / 2);
+        // per workgroup, stage-major: the records of one stage of the workgroup's lanes are adjacent (padded lanes own
+        // a slot too), the sixteen stages of a workgroup follow each other
+        rec = a.stage_ws + ((size_t)block * ACE_MAX_STAGES * BLOCK + (size_t)tid) * ACE_WS_REC;
+        st.ws_stride = (uint32_t)BLOCK * (ACE_WS_REC / 2);
     }
 
     int w = w0 + 1;
@@ -274,8 +279,15 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
         // the assembly form of the loop below (same operations per plan, same results)
         if (!(cw.x & 0x10u)) st.status = ACE_PLAN_MALFORMED;    // the first op must open a stage
         uint64_t dg, rks;
-        st.stage_nibbles(g, lds, dg, rks);
-        st.s = (int)ace_score_loop_asm<WIN>(a, g, dg, rks, (uint32_t)pl * 16u, rec, st.ws_stride, prio,
+        if (WIN) st.stage_nibbles(g, lds, dg, rks);
+        else {
+            // rows resident: the loop looks each stage's offsets up in LDS, by the stage size's log2
+            dg = st.glogs;
+            rks = g.lut2a_lds_off + st.bidx * 128u;
+        }
+        st.s = (int)ace_score_loop_asm<WIN>(a, g, dg, rks, (uint32_t)pl * 16u,
+                                            a.stage_ws + (size_t)block * ACE_MAX_STAGES * BLOCK * ACE_WS_REC,
+                                            (uint32_t)tid * (ACE_WS_REC * 8u), (uint32_t)BLOCK * (ACE_WS_REC * 8u), prio,
                                             (uint32_t)__builtin_amdgcn_readfirstlane(tid >> 6));
         grp_stop = grp_begin;
     } else

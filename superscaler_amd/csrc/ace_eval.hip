@@ -846,7 +846,7 @@ static int upload_pos_types(ace_handle *h, const ace_tables_t *t, size_t pos_ent
 // Leaves the handle without them (plain scoring then takes the C++ loop) where the layout does not work out.
 static int setup_windowed_asm(ace_handle *h, const ace_tables_t *t, size_t pos_entries, int32_t rk_bytes, int32_t stg_words) {
     h->d_win_dma = nullptr;
-    if (t->n_windows <= 1 || !h->d_pos_types || (t->flags & ACE_F_COLLECTIVE_MEM) || t->num_ops >= 65536) return ACE_OK;
+    if (t->n_windows <= 1 || !h->d_pos_types || (t->flags & ACE_F_COLLECTIVE_MEM) || t->num_ops >= 32768) return ACE_OK;
     if ((int64_t)(t->n_z > 0 ? t->n_z : 1) * t->z_table_doubles * 8 > 65536) return ACE_OK;
     const uint64_t row_bytes = (uint64_t)t->row_doubles * 8u;
     if ((uint64_t)t->num_types * row_bytes > 0xffffffffull) return ACE_OK;
@@ -855,10 +855,11 @@ static int setup_windowed_asm(ace_handle *h, const ace_tables_t *t, size_t pos_e
     if (hot_len < 1024u || (z_len != 0u && z_len < 1024u) || (hot_len & 15u) || (z_len & 15u)) return ACE_OK;
     const uint32_t crow = hot_len + z_len;
     // the most rows per half that leave room for the small tables
-    uint32_t slots = 127, stg_off = 0, lut2_off = 0, pk32_off = 0, lds_end = 0;
+    uint32_t slots = 127, stg_off = 0, lut2_off = 0, pk32_off = 0, lut2a_off = 0, lds_end = 0;
     for (; slots >= 5u; --slots) {
-        lds_end = ace_lds_pk32(ace_lds_layout(2u * slots * crow, (uint32_t)rk_bytes, (uint32_t)stg_words, &stg_off, &lut2_off),
-                               (uint32_t)rk_bytes, &pk32_off);
+        lut2a_off = (ace_lds_pk32(ace_lds_layout(2u * slots * crow, (uint32_t)rk_bytes, (uint32_t)stg_words, &stg_off, &lut2_off),
+                                  (uint32_t)rk_bytes, &pk32_off) + 15u) & ~15u;
+        lds_end = lut2a_off + (uint32_t)stg_words * 8u;
         if (lds_end <= kMaxLds) break;
     }
     if (slots < 5u) return ACE_OK;
@@ -941,7 +942,7 @@ static int setup_windowed_asm(ace_handle *h, const ace_tables_t *t, size_t pos_e
     if (rc != ACE_OK) return rc;
     h->geom_wa = h->geom;
     h->geom_wa.rk_lds_off = 2u * slots * crow;
-    h->geom_wa.stg_lds_off = stg_off; h->geom_wa.lut2_lds_off = lut2_off; h->geom_wa.pk32_lds_off = pk32_off; h->geom_wa.pace_lds_off = 0; h->geom_wa.lut2a_lds_off = 0;
+    h->geom_wa.stg_lds_off = stg_off; h->geom_wa.lut2_lds_off = lut2_off; h->geom_wa.pk32_lds_off = pk32_off; h->geom_wa.pace_lds_off = 0; h->geom_wa.lut2a_lds_off = lut2a_off;
     h->lds_bytes_wa = lds_end;
     return ACE_OK;
 }
@@ -1166,7 +1167,7 @@ static void launch_score(const ace_handle_t *h, const AceKernelArgs &a, hipStrea
 // per-plan workspace; the handle keeps one and grows it on demand.
 static int ensure_stage_ws(ace_handle_t *h, AceKernelArgs *a) {
     a->stage_ws = nullptr;
-    if (a->range || a->stage_out || (h->n_windows > 1 && !h->d_pos_types) || h->geom.N >= 65536 || (h->geom.flags & ACE_F_COLLECTIVE_MEM)) return ACE_OK;
+    if (a->range || a->stage_out || (h->n_windows > 1 && !h->d_pos_types) || h->geom.N >= 32768 || (h->geom.flags & ACE_F_COLLECTIVE_MEM)) return ACE_OK;
     const size_t need = (((size_t)a->g.P + kBlock - 1) / kBlock) * kBlock;
     if (need * ACE_MAX_STAGES * (ACE_WS_REC / 2) > 0xffffffffull) return ACE_OK;   // (a workspace of 64 GiB and more: such batches take the plain kernel)
     if (need > h->stage_ws_plans) {
@@ -1219,7 +1220,7 @@ int ace_score_batch_static(ace_handle_t *h, const ace_batch_t *batch, double mem
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev != h->device || dev < 0 || dev >= kMaxDevices) return ACE_EINVAL;
     // (the same test as ensure_stage_ws: tables that take the kernels without deferred stage tails need no scratch)
-    const bool deferred = !((h->n_windows > 1 && !h->d_pos_types) || h->geom.N >= 65536 || (h->geom.flags & ACE_F_COLLECTIVE_MEM));
+    const bool deferred = !((h->n_windows > 1 && !h->d_pos_types) || h->geom.N >= 32768 || (h->geom.flags & ACE_F_COLLECTIVE_MEM));
     // looked up by ace_create on this device; the padded plan count of either workgroup size fits: ACE_STATIC_MAX_PLANS is a multiple of kBlock
     a.stage_ws = deferred ? g_static_ptr[dev] : nullptr;
     if (deferred && !a.stage_ws) return ACE_EINVAL;

@@ -83,19 +83,18 @@ template <int BLOCK> ACE_HD void stage_window(const AceKernelArgs &a, unsigned c
 // WIN: the rows are windowed; the loop fetches its windows itself, from the records of a.win_dma (80 bytes per fetch
 // event and wavefront, sixteen wavefronts: see the generator).
 template <bool WIN>
-__device__ __forceinline__ uint32_t ace_score_loop_asm(const AceKernelArgs &a, const AceGeom &g, uint64_t dg, uint64_t rks,
+__device__ __forceinline__ uint32_t ace_score_loop_asm(const AceKernelArgs &a, const AceGeom &g, uint64_t glogs, uint32_t lut2_lane,
                                                        uint32_t code_off, const double *rec_base, uint32_t rec_off, uint32_t ws_stride,
                                                        uint32_t prio, uint32_t wave) {
-    uint32_t cnt;
+    uint32_t wsoff;         // the lane's record offset after the loop: rec_off + ws_stride * (stages closed)
     const uint64_t gstride = (uint64_t)(uint32_t)g.P * 16u;
     const uint32_t gs_lo = (uint32_t)gstride, gs_hi = (uint32_t)(gstride >> 32);
-    const uint32_t c8 = (uint32_t)g.C * 8u;
     const uint32_t pace = g.pace_lds_off + (wave & 3u) * 32u;     // this SIMD's eight arrival counters
     if (WIN) {
 #define ACE_LOOP_ASM_RUN(TEXT)                                                                                          \
-    asm volatile(TEXT : [cnt] "=&v"(cnt)                                                                               \
-                 : [dg] "v"(dg), [rk] "v"(rks), [codeoff] "v"(code_off), [recoff] "v"(rec_off), [codes] "s"(a.codes),   \
-                   [pos] "s"(a.pos4), [c8] "s"(c8), [n_ops] "s"(g.N), [n_groups] "s"(g.G), [recbase] "s"(rec_base),         \
+    asm volatile(TEXT : [wsoff] "=&v"(wsoff)                                                                               \
+                 : [glogs] "v"(glogs), [lut2] "v"(lut2_lane), [codeoff] "v"(code_off), [recoff] "v"(rec_off),          \
+                   [codes] "s"(a.codes), [pos] "s"(a.pos4), [n_ops] "s"(g.N), [n_groups] "s"(g.G), [recbase] "s"(rec_base), \
                    [gstride_lo] "s"(gs_lo), [gstride_hi] "s"(gs_hi), [wsstride] "s"(ws_stride), [prio] "s"(prio),       \
                    [dma] "s"(a.win_dma), [waveoff] "s"(wave * 80u)                                                      \
                  : ACE_LOOP_ASM_CLOBBERS)
@@ -109,11 +108,11 @@ __device__ __forceinline__ uint32_t ace_score_loop_asm(const AceKernelArgs &a, c
             else ACE_LOOP_ASM_RUN(ACE_LOOP_ASM_WIN_RSH0_MAX);
         }
 #undef ACE_LOOP_ASM_RUN
-        return cnt;
+        return (wsoff - rec_off) / ws_stride;
     }
 #define ACE_LOOP_ASM_RUN(TEXT)                                                                                          \
-    asm volatile(TEXT : [cnt] "=&v"(cnt)                                                                               \
-                 : [glogs] "v"(dg), [lut2] "v"((uint32_t)rks), [codeoff] "v"(code_off), [recoff] "v"(rec_off),          \
+    asm volatile(TEXT : [wsoff] "=&v"(wsoff)                                                                               \
+                 : [glogs] "v"(glogs), [lut2] "v"(lut2_lane), [codeoff] "v"(code_off), [recoff] "v"(rec_off),          \
                    [codes] "s"(a.codes), [pos] "s"(a.pos4), [n_ops] "s"(g.N), [n_groups] "s"(g.G), [recbase] "s"(rec_base), \
                    [gstride_lo] "s"(gs_lo), [gstride_hi] "s"(gs_hi), [wsstride] "s"(ws_stride), [prio] "s"(prio),       \
                    [pace] "s"(pace)                                                                                     \
@@ -128,7 +127,7 @@ __device__ __forceinline__ uint32_t ace_score_loop_asm(const AceKernelArgs &a, c
         else ACE_LOOP_ASM_RUN(ACE_LOOP_ASM_RSH0_MAX);
     }
 #undef ACE_LOOP_ASM_RUN
-    return cnt;
+    return (wsoff - rec_off) / ws_stride;
 }
 #endif
 
@@ -244,7 +243,7 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     }
     // (the assembly op loop over windowed rows fetches its windows itself, in a layout of its own)
 #ifndef ACE_HOST_EMU
-    const bool asm_loop = DEFER && lds_base == 0u && a.pos4 && (WIN ? (BLOCK == 1024 && a.win_dma) : a.g.lut2a_lds_off != 0u);
+    const bool asm_loop = DEFER && lds_base == 0u && a.pos4 && a.g.lut2a_lds_off && (!WIN || (BLOCK == 1024 && a.win_dma));
 #else
     const bool asm_loop = false;
 #endif
@@ -278,14 +277,8 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     if (asm_loop) {
         // the assembly form of the loop below (same operations per plan, same results)
         if (!(cw.x & 0x10u)) st.status = ACE_PLAN_MALFORMED;    // the first op must open a stage
-        uint64_t dg, rks;
-        if (WIN) st.stage_nibbles(g, lds, dg, rks);
-        else {
-            // rows resident: the loop looks each stage's offsets up in LDS, by the stage size's log2
-            dg = st.glogs;
-            rks = g.lut2a_lds_off + st.bidx * 128u;
-        }
-        st.s = (int)ace_score_loop_asm<WIN>(a, g, dg, rks, (uint32_t)pl * 16u,
+        // (the loop looks each stage's offsets up in LDS, by the stage size's log2)
+        st.s = (int)ace_score_loop_asm<WIN>(a, g, st.glogs, g.lut2a_lds_off + st.bidx * 128u, (uint32_t)pl * 16u,
                                             a.stage_ws + (size_t)block * ACE_MAX_STAGES * BLOCK * ACE_WS_REC,
                                             (uint32_t)tid * (ACE_WS_REC * 8u), (uint32_t)BLOCK * (ACE_WS_REC * 8u), prio,
                                             (uint32_t)__builtin_amdgcn_readfirstlane(tid >> 6));

@@ -72,10 +72,11 @@ def D(y):                                   # per 4-op word: next-op bytes, code
     return dict(nw=f"v{b}", w8=f"v{b+1}", cn=f"v{b+2}", r8=f"v{b+3}", p8=f"v{b+4}")
 
 
-ZV_, RK, ZVRK, WSOFF, CNT = "v120", "v121", "v[120:121]", "v122", "v125"   # WSOFF: byte offset of this lane's next stage record
+ZV_, RK, ZVRK, WSOFF = "v120", "v121", "v[120:121]", "v122"   # WSOFF: byte offset of this lane's next stage record (it counts the stages)
 PACE = "v124"                               # lane 0: what this group's arrival counter read before this wavefront was counted
-DG, DG_LO, RKS, RKS_LO = "v[28:29]", "v28", "v[30:31]", "v30"   # windowed rows: per stage, 4 bits each, next stage lowest: diag; pair-table block
-GLOGS, GLOGS_LO, LUT2 = "v[28:29]", "v28", "v30"   # rows resident: log2 of the stage sizes, 4 bits each, next stage lowest; LDS address of this plan's micro-batch size in the table of (diag offset, pair-table block) per stage size
+# log2 of the plan's stage sizes, 4 bits each, next stage lowest; LDS address of the plan's micro-batch size in the table
+# of (diag offset, pair-table block) per stage size
+GLOGS, GLOGS_LO, LUT2 = "v[28:29]", "v28", "v30"
 T0, T1, T01, T2 = "v126", "v127", "v[126:127]", "v33"
 
 # ---- scalar registers ---------------------------------------------------------------------------------------
@@ -88,6 +89,7 @@ ORD, ORD_LO, ORD_HI = "s[50:51]", "s50", "s51"
 MASK = [f"s{52 + j}" for j in range(4)]
 PLANT = [f"s{56 + j}" for j in range(4)]
 PREVFL = "s62"
+WSLIMIT = "s28"                             # WSOFF of a seventeenth stage, which no lane has room for
 NEXTWIN, EVT, DMAOFF, ARRIVED = "s29", "s34", "s63", "s35"   # windowed rows: next window's first position, window index, ...
 DMAPTR = "s[60:61]"
 S0, S1, S2, S23 = "s96", "s97", "s98", "s[98:99]"
@@ -125,21 +127,12 @@ class Gen:
         self.o(f"v_bitop3_b32 {d['p8']}, {d['r8']}, {d['nw']}, {d['p8']} bitop3:0x40")
 
     def stage_start(self):
-        """z_v and the pair-table block of the stage that begins.  Rows resident: one 8-byte LDS read per lane, indexed by
-        the next nibble of the plan's stage sizes (the caller waits for it).  Windowed rows: the next nibbles of the
-        packed per-stage lists."""
-        if not self.win:
-            self.o(f"v_and_b32 {T0}, 15, {GLOGS_LO}")
-            self.o(f"v_lshl_add_u32 {T0}, {T0}, 3, {LUT2}")
-            self.o(f"v_lshrrev_b64 {GLOGS}, 4, {GLOGS}")
-            self.o(f"ds_read_b64 {ZVRK}, {T0}")
-            return
-        self.o(f"v_and_b32 {T0}, 15, {DG_LO}")
-        self.o(f"v_mul_u32_u24 {ZV_}, {T0}, %[c8]")
-        self.o(f"v_lshrrev_b64 {DG}, 4, {DG}")
-        self.o(f"v_and_b32 {T0}, 15, {RKS_LO}")
-        self.o(f"v_lshlrev_b32 {RK}, 6, {T0}")
-        self.o(f"v_lshrrev_b64 {RKS}, 4, {RKS}")
+        """z_v and the pair-table block of the stage that begins: one 8-byte LDS read per lane, indexed by the next
+        nibble of the plan's stage sizes (the caller waits for it)."""
+        self.o(f"v_and_b32 {T0}, 15, {GLOGS_LO}")
+        self.o(f"v_lshl_add_u32 {T0}, {T0}, 3, {LUT2}")
+        self.o(f"v_lshrrev_b64 {GLOGS}, 4, {GLOGS}")
+        self.o(f"ds_read_b64 {ZVRK}, {T0}")
 
     def issue(self, k1):
         """Address arithmetic and LDS reads of op k1 (0..16; 16 = first op of the next group)."""
@@ -262,10 +255,7 @@ class Gen:
         self.c("lanes whose next op opens a stage: that stage's table offsets; its first op pays no resharding")
         self.o(f"s_mov_b64 exec, {M_ST}")
         self.stage_start()
-        if not self.win:
-            self.o("s_waitcnt lgkmcnt(0)")
-        elif self.rsh:
-            self.o("s_waitcnt lgkmcnt(2)")
+        self.o("s_waitcnt lgkmcnt(0)")
         if self.rsh:
             self.o(f"v_mov_b32 {R(x1)}, 0")
         self.o(f"s_mov_b64 exec, {ALL}")
@@ -304,16 +294,15 @@ class Gen:
         self.o(f"s_or_b32 {S0}, {S0}, {S1}")
         self.o(f"v_mov_b32 v50, {d['cn']}")                  # the record's last words: code*8 + next code of this word's ops,
         self.o(f"v_mov_b32 v51, {S0}")                       # position of the stage's last op | its row << 16 | the next op's row << 24
-        self.o(f"v_cmp_gt_u32_e32 vcc, 16, {CNT}")
+        self.o(f"v_cmp_gt_u32_e32 vcc, {WSLIMIT}, {WSOFF}")
         self.o("s_and_b64 exec, exec, vcc")
         self.o(f"global_store_dwordx4 {WSOFF}, v[32:35], %[recbase]")
         self.o(f"global_store_dwordx4 {WSOFF}, v[36:39], %[recbase] offset:16")
         self.o(f"global_store_dwordx4 {WSOFF}, v[40:43], %[recbase] offset:32")
         self.o(f"global_store_dwordx4 {WSOFF}, v[44:47], %[recbase] offset:48")
         self.o(f"global_store_dwordx4 {WSOFF}, v[48:51], %[recbase] offset:64")
-        self.o(f"v_add_u32_e32 {WSOFF}, %[wsstride], {WSOFF}")
         self.o(f"s_mov_b64 exec, {M_ST}")
-        self.o(f"v_add_u32_e32 {CNT}, 1, {CNT}")
+        self.o(f"v_add_u32_e32 {WSOFF}, %[wsstride], {WSOFF}")
         self.o(f"v_mov_b64 {RUN}, 0")
         self.o(f"v_mov_b64 {PEAK}, 0")
         if True:
@@ -393,12 +382,8 @@ class Gen:
             o(f"s_setprio {lvl}")
             o(f"L_np{lvl}_%=:")
         o(f"s_mov_b64 {ALL}, exec")
-        if self.win:
-            o(f"v_mov_b64 {DG}, %[dg]")
-            o(f"v_mov_b64 {RKS}, %[rk]")
-        else:
-            o(f"v_mov_b64 {GLOGS}, %[glogs]")
-            o(f"v_mov_b32 {LUT2}, %[lut2]")
+        o(f"v_mov_b64 {GLOGS}, %[glogs]")
+        o(f"v_mov_b32 {LUT2}, %[lut2]")
         o(f"s_mov_b64 {CPTR}, %[codes]")
         o(f"s_mov_b64 {PPTR}, %[pos]")
         o(f"s_mov_b32 {K07}, 0x07070707")
@@ -420,7 +405,7 @@ class Gen:
         for r in (FWD, BWD, RUN, PEAK, RFM[0], RBM[0], RCS, RSF, RSB, W_, A_, SAVED):
             o(f"v_mov_b64 {r}, 0")
         o(f"v_mov_b32 {WSOFF}, %[recoff]")
-        o(f"v_mov_b32 {CNT}, 0")
+        o(f"s_lshl_b32 {WSLIMIT}, %[wsstride], 4")
         o(f"v_mov_b32 {R(0)}, 0")
         self.stage_start()
         o("s_waitcnt vmcnt(0) lgkmcnt(0)")
@@ -468,7 +453,7 @@ class Gen:
         o(f"s_mov_b64 exec, {ALL}")
         o("s_waitcnt vmcnt(0) lgkmcnt(0)")
         o("s_setprio 0")
-        o(f"v_mov_b32 %[cnt], {CNT}")
+        o(f"v_mov_b32 %[wsoff], {WSOFF}")
         return self.lines
 
 

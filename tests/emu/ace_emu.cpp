@@ -197,7 +197,7 @@ extern "C" int ace_emu_kernel(const ace_tables_t *t, const uint8_t *codes, const
     unsigned char *lds = (unsigned char *)pool.place(nullptr, lds_bytes);
     const bool win = t->n_windows > 1;
     const bool coll = (t->flags & ACE_F_COLLECTIVE_MEM) != 0;
-    const bool defer = !range && !stage_out && (!win || a.pos_types) && g.N < 65536 && !coll;
+    const bool defer = !range && !stage_out && (!win || a.pos_types) && g.N < 32768 && !coll;
     if (defer) a.stage_ws = (double *)pool.place(nullptr, (size_t)P * ACE_MAX_STAGES * ACE_WS_REC * 8);
 
     if (coll) {

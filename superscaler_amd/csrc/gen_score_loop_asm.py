@@ -40,9 +40,14 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 FB, RCS = "v[32:33]", "v[34:35]"            # quad v[32:35]: stash record 0 = {fwd + bwd, recompute sum}
 RSF, RSB = "v[36:37]", "v[38:39]"           # quad v[36:39]: record 1 = {resharding fwd, bwd}
 W_, A_ = "v[40:41]", "v[42:43]"             # quad v[40:43]: record 2 = {weights, activations}
-SAVED, PKT = "v[44:45]", "v[46:47]"         # quad v[44:47]: record 3 = {saved, closed peak}
-RES, META = "v[48:49]", "v[50:51]"          # quad v[48:51]: record 4 = {reserved term, meta}
-FWD, BWD, RUN, PEAK = "v[52:53]", "v[54:55]", "v[56:57]", "v[58:59]"
+SAVED, PEAK = "v[44:45]", "v[46:47]"        # quad v[44:47]: record 3 = {saved, peak}
+# record 4 = {reserved term, code*8 + next code of a word's ops, position word}: one quad per buffer of word-level values,
+# so that the code word is stored from where the word's preparation wrote it
+RESQ = ["v[48:51]", "v[56:59]"]
+RES = ["v[48:49]", "v[56:57]"]
+CN = ["v50", "v58"]
+META = ["v51", "v59"]
+FWD, BWD, RUN = "v[52:53]", "v[54:55]", "v[112:113]"
 RFM = ["v[60:61]", "v[64:65]"]              # reserved maxima, alternating between consecutive ops
 RBM = ["v[62:63]", "v[66:67]"]
 
@@ -68,15 +73,17 @@ NEXT = [f"v{106 + j}" for j in range(4)]    # ... of the next group
 
 
 def D(y):                                   # per 4-op word: next-op bytes, code*8, code*8+next code, rc bit, pair bit
-    b = 110 + 5 * y
-    return dict(nw=f"v{b}", w8=f"v{b+1}", cn=f"v{b+2}", r8=f"v{b+3}", p8=f"v{b+4}")
+    b = (110, 116)[y]
+    r = (114, 118)[y]
+    return dict(nw=f"v{b}", w8=f"v{b+1}", cn=CN[y], r8=f"v{r}", p8=f"v{r+1}")
 
 
 ZV_, RK, ZVRK, WSOFF = "v120", "v121", "v[120:121]", "v122"   # WSOFF: byte offset of this lane's next stage record (it counts the stages)
-PACE = "v124"                               # lane 0: what this group's arrival counter read before this wavefront was counted
+PACE = "v123"                               # lane 0: what this group's arrival counter read before this wavefront was counted
 # log2 of the plan's stage sizes, 4 bits each, next stage lowest; LDS address of the plan's micro-batch size in the table
 # of (diag offset, pair-table block) per stage size
 GLOGS, GLOGS_LO, LUT2 = "v[28:29]", "v28", "v30"
+NZVRK = "v[124:125]"                         # ZVRK of the stage after the current one, read ahead
 T0, T1, T01, T2 = "v126", "v127", "v[126:127]", "v33"
 
 # ---- scalar registers ---------------------------------------------------------------------------------------
@@ -85,7 +92,6 @@ CPTR, CPTR_LO, CPTR_HI = "s[26:27]", "s26", "s27"
 GRP, K07, K08, POSBASE, LEFT, K1F = "s30", "s39", "s40", "s41", "s31", "s38"
 PPTR, PPTR_LO, PPTR_HI = "s[36:37]", "s36", "s37"
 M_RC, M_P, M_ST, M_KP = "s[42:43]", "s[44:45]", "s[46:47]", "s[48:49]"
-ORD, ORD_LO, ORD_HI = "s[50:51]", "s50", "s51"
 MASK = [f"s{52 + j}" for j in range(4)]
 PLANT = [f"s{56 + j}" for j in range(4)]
 PREVFL = "s62"
@@ -126,13 +132,13 @@ class Gen:
         self.o(f"v_lshrrev_b32 {d['p8']}, 1, {d['nw']}")
         self.o(f"v_bitop3_b32 {d['p8']}, {d['r8']}, {d['nw']}, {d['p8']} bitop3:0x40")
 
-    def stage_start(self):
-        """z_v and the pair-table block of the stage that begins: one 8-byte LDS read per lane, indexed by the next
-        nibble of the plan's stage sizes (the caller waits for it)."""
+    def stage_fetch(self, dst):
+        """Asks for z_v and the pair-table block of the plan's next stage: one 8-byte LDS read per lane, indexed by the
+        next nibble of the plan's stage sizes."""
         self.o(f"v_and_b32 {T0}, 15, {GLOGS_LO}")
         self.o(f"v_lshl_add_u32 {T0}, {T0}, 3, {LUT2}")
         self.o(f"v_lshrrev_b64 {GLOGS}, 4, {GLOGS}")
-        self.o(f"ds_read_b64 {ZVRK}, {T0}")
+        self.o(f"ds_read_b64 {dst}, {T0}")
 
     def issue(self, k1):
         """Address arithmetic and LDS reads of op k1 (0..16; 16 = first op of the next group)."""
@@ -206,16 +212,16 @@ class Gen:
         self.o(f"L_nw_{L}:")
         self.o(f"s_cmp_lg_u64 {M_ST}, 0")                   # (what the branch to the stage-end code tests)
 
-    def reserved(self, cur):
+    def reserved(self, cur, res):
         if self.mode == "max":          # max(rf + rb, W)
-            self.o(f"v_add_f64 {RES}, {RFM[cur]}, {RBM[cur]}")
-            self.o(f"v_max_f64 {RES}, {RES}, {W_}")
+            self.o(f"v_add_f64 {res}, {RFM[cur]}, {RBM[cur]}")
+            self.o(f"v_max_f64 {res}, {res}, {W_}")
         elif self.mode == "min":        # max(max(rf, rb), max(W, 0))
-            self.o(f"v_max_f64 {RES}, {RFM[cur]}, {RBM[cur]}")
+            self.o(f"v_max_f64 {res}, {RFM[cur]}, {RBM[cur]}")
             self.o(f"v_max_f64 {T01}, {W_}, 0")
-            self.o(f"v_max_f64 {RES}, {RES}, {T01}")
+            self.o(f"v_max_f64 {res}, {res}, {T01}")
         else:
-            self.o(f"v_mov_b64 {RES}, 0")
+            self.o(f"v_mov_b64 {res}, 0")
 
     def slot(self, k):
         j, b = k >> 2, k & 3
@@ -254,10 +260,18 @@ class Gen:
         self.o(f"s_cbranch_scc0 L_ns_{L}")
         self.c("lanes whose next op opens a stage: that stage's table offsets; its first op pays no resharding")
         self.o(f"s_mov_b64 exec, {M_ST}")
-        self.stage_start()
-        self.o("s_waitcnt lgkmcnt(0)")
+        if self.win:
+            self.stage_fetch(ZVRK)
+            self.o("s_waitcnt lgkmcnt(0)")
+        else:
+            self.c("(asked for where the stage before began, before that op's table reads, of which all but the last two are in)")
+            self.o("s_waitcnt lgkmcnt(2)")
+            self.o(f"v_mov_b64 {ZVRK}, {NZVRK}")
         if self.rsh:
             self.o(f"v_mov_b32 {R(x1)}, 0")
+        if not self.win:
+            self.c("the offsets of the stage after the one that begins now, for when that one ends")
+            self.stage_fetch(NZVRK)
         self.o(f"s_mov_b64 exec, {ALL}")
         self.o(f"L_ns_{L}:")
         if self.win and b == 3:
@@ -283,24 +297,24 @@ class Gen:
         self.o(f"s_mov_b64 exec, {M_ST}")
         self.o(f"v_add_f64 {FB}, {FWD}, {BWD}")
         prevfl = P(y, b - 1)["fl"] if b else PREVFL
+        self.c("the last segment closes into the peak if the op before this one is an ordinary one")
         self.o(f"s_bitcmp1_b32 {prevfl}, 1")
-        self.o(f"s_cselect_b32 {ORD_HI}, 0x3ff00000, 0")
-        self.o(f"v_mul_f64 {PKT}, {RUN}, {ORD}")
-        self.o(f"v_max_f64 {PKT}, {PEAK}, {PKT}")
-        self.reserved(cur)
+        self.o(f"s_cselect_b64 exec, {M_ST}, 0")
+        self.o(f"v_max_f64 {PEAK}, {PEAK}, {RUN}")
+        self.o(f"s_mov_b64 exec, {M_ST}")
+        self.reserved(cur, RES[y])
         self.o(f"s_add_u32 {S0}, {POSBASE}, {k}")
         self.o(f"s_andn2_b32 {S1}, {p['fl']}, 0xff")
         self.o(f"s_lshl_b32 {S1}, {S1}, 8")
         self.o(f"s_or_b32 {S0}, {S0}, {S1}")
-        self.o(f"v_mov_b32 v50, {d['cn']}")                  # the record's last words: code*8 + next code of this word's ops,
-        self.o(f"v_mov_b32 v51, {S0}")                       # position of the stage's last op | its row << 16 | the next op's row << 24
+        self.o(f"v_mov_b32 {META[y]}, {S0}")                 # position of the stage's last op | its row << 16 | the next op's row << 24
         self.o(f"v_cmp_gt_u32_e32 vcc, {WSLIMIT}, {WSOFF}")
         self.o("s_and_b64 exec, exec, vcc")
         self.o(f"global_store_dwordx4 {WSOFF}, v[32:35], %[recbase]")
         self.o(f"global_store_dwordx4 {WSOFF}, v[36:39], %[recbase] offset:16")
         self.o(f"global_store_dwordx4 {WSOFF}, v[40:43], %[recbase] offset:32")
         self.o(f"global_store_dwordx4 {WSOFF}, v[44:47], %[recbase] offset:48")
-        self.o(f"global_store_dwordx4 {WSOFF}, v[48:51], %[recbase] offset:64")
+        self.o(f"global_store_dwordx4 {WSOFF}, {RESQ[y]}, %[recbase] offset:64")
         self.o(f"s_mov_b64 exec, {M_ST}")
         self.o(f"v_add_u32_e32 {WSOFF}, %[wsstride], {WSOFF}")
         self.o(f"v_mov_b64 {RUN}, 0")
@@ -389,7 +403,6 @@ class Gen:
         o(f"s_mov_b32 {K07}, 0x07070707")
         o(f"s_mov_b32 {K08}, 0x08080808")
         o(f"s_mov_b32 {K1F}, 0x1f1f1f1f")
-        o(f"s_mov_b32 {ORD_LO}, 0")
         o(f"s_mov_b32 {GRP}, 0")
         o(f"s_mov_b32 {POSBASE}, 0")
         o(f"s_mov_b32 {PREVFL}, 0")
@@ -407,7 +420,9 @@ class Gen:
         o(f"v_mov_b32 {WSOFF}, %[recoff]")
         o(f"s_lshl_b32 {WSLIMIT}, %[wsstride], 4")
         o(f"v_mov_b32 {R(0)}, 0")
-        self.stage_start()
+        self.stage_fetch(ZVRK)
+        if not self.win:
+            self.stage_fetch(NZVRK)
         o("s_waitcnt vmcnt(0) lgkmcnt(0)")
         o(f"s_mov_b32 {LEFT}, %[n_ops]")
         self.apply_masks(WORD, "w0")

@@ -718,6 +718,7 @@ struct ace_handle {
     double *d_nbm1;
     int32_t *d_win_pos, *d_win_row_begin;
     uint32_t *d_win_rows;
+    int32_t flat_rows16;       // see AceKernelArgs
     double *d_stage_ws;        // grow-only workspace for deferred stage tails
     size_t stage_ws_plans;     // capacity in plans
     int stage_ws_fixed;        // ace_reserve(..., fixed): a larger batch is an error instead of a reallocation
@@ -1060,6 +1061,14 @@ int ace_create(const ace_tables_t *t, ace_handle_t **out) {
     g.flags = t->flags; g.main_params = t->main_params; g.optimizer = t->optimizer;
     g.mem_limit = 0.0; g.strict = 0;
     h->n_windows = t->n_windows; h->row_doubles = t->row_doubles; h->rk_bytes = rk_bytes; h->stg_words = stg_words;
+    // rows resident, slot r of LDS holding row r: the kernels stage them as one block
+    h->flat_rows16 = 0;
+    if (t->n_windows == 1 && (row_bytes & 15) == 0) {
+        bool flat = true;
+        for (int r = 0; r < n_win_rows; ++r)
+            flat = flat && t->win_rows[2 * r] == (uint32_t)r && t->win_rows[2 * r + 1] == (uint32_t)(r * row_bytes);
+        if (flat) h->flat_rows16 = (int32_t)(n_win_rows * row_bytes / 16);
+    }
     h->num_types = t->num_types; h->lds_bytes = lds_alloc;
     const size_t pos_entries = (size_t)((t->num_ops + 15) / 16) * 16 + 16;
     int rc;
@@ -1119,6 +1128,7 @@ static int fill_args(ace_handle_t *h, const ace_batch_t *b, double memory_limit,
     a->rows = h->d_rows; a->pos_info = h->d_pos_info; a->pos_types = h->d_pos_types; a->pos4 = h->d_pos4; a->win_dma = h->d_win_dma; a->pair_kinds = h->d_pair_kinds; a->stage_lut = h->d_stage_lut;
     a->nbm1 = h->d_nbm1; a->win_pos = h->d_win_pos; a->win_row_begin = h->d_win_row_begin; a->win_rows = h->d_win_rows;
     a->n_windows = h->n_windows; a->row_doubles = h->row_doubles; a->rk_bytes = h->rk_bytes; a->stg_words = h->stg_words;
+    a->flat_rows16 = h->flat_rows16;
     a->iter_ms = d_iter_ms; a->peak_mb = d_peak_mb; a->feasible = d_feasible; a->status = d_status; a->stage_out = d_stage_out;
     a->stage_ws = nullptr;
     return ACE_OK;

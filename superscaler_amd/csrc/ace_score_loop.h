@@ -37,6 +37,7 @@ struct AceKernelArgs {
     const uint32_t *win_rows;   // pairs (type, lds byte offset)
     const ace_u4 *win_dma;      // what the assembly op loop stages the windows from (see ace_score_loop_asm), or null
     int32_t n_windows, row_doubles, rk_bytes, stg_words;
+    int32_t flat_rows16;        // rows resident and laid out in LDS as they lie in `rows`: their size in 16-byte pieces (else 0)
     double *iter_ms, *peak_mb;
     uint8_t *feasible, *status;
     double *stage_out;          // [P][ACE_MAX_STAGES][ACE_STAGE_REC], single-stage queries [P][ACE_STAGE_REC]
@@ -61,6 +62,20 @@ inline void ace_pos_types(const ace_tables_t *t, uint32_t *out, size_t entries) 
     // ... and the index of the next position's row in bits 8 to 15 (the last op: its own)
     for (size_t i = 0; i < entries && i < (size_t)t->num_ops; ++i)
         out[i] |= ((i + 1 < (size_t)t->num_ops ? out[i + 1] : out[i]) & 0xffu) << 8;
+}
+
+// Rows resident and laid out in LDS as they lie in global memory: one block copy with every lane busy, four loads in
+// flight per lane (row by row, a lane has one load at a time and most lanes none).
+template <int BLOCK> ACE_HD void stage_rows_flat(const AceKernelArgs &a, unsigned char *lds_raw, int tid) {
+    const ace_d2 *src = reinterpret_cast<const ace_d2 *>(a.rows);
+    ace_d2 *dst = reinterpret_cast<ace_d2 *>(lds_raw);
+    const int n = a.flat_rows16;
+    int j = tid;
+    for (; j + 3 * BLOCK < n; j += 4 * BLOCK) {
+        const ace_d2 v0 = src[j], v1 = src[j + BLOCK], v2 = src[j + 2 * BLOCK], v3 = src[j + 3 * BLOCK];
+        dst[j] = v0; dst[j + BLOCK] = v1; dst[j + 2 * BLOCK] = v2; dst[j + 3 * BLOCK] = v3;
+    }
+    for (; j < n; j += BLOCK) dst[j] = src[j];
 }
 
 // Copy the rows window `w` needs from global memory into LDS (whole workgroup).
@@ -94,7 +109,7 @@ __device__ __forceinline__ uint32_t ace_score_loop_asm(const AceKernelArgs &a, c
 #define ACE_LOOP_ASM_RUN(TEXT)                                                                                          \
     asm volatile(TEXT : [wsoff] "=&v"(wsoff)                                                                               \
                  : [glogs] "v"(glogs), [lut2] "v"(lut2_lane), [codeoff] "v"(code_off), [recoff] "v"(rec_off),          \
-                   [codes] "s"(a.codes), [pos] "s"(a.pos4), [n_ops] "s"(g.N), [n_groups] "s"(g.G), [recbase] "s"(rec_base), \
+                   [codes] "s"(a.codes), [pos] "s"(a.pos4), [n_ops] "s"(g.N), [recbase] "s"(rec_base), \
                    [gstride_lo] "s"(gs_lo), [gstride_hi] "s"(gs_hi), [wsstride] "s"(ws_stride), [prio] "s"(prio),       \
                    [dma] "s"(a.win_dma), [waveoff] "s"(wave * 80u)                                                      \
                  : ACE_LOOP_ASM_CLOBBERS)
@@ -113,8 +128,8 @@ __device__ __forceinline__ uint32_t ace_score_loop_asm(const AceKernelArgs &a, c
 #define ACE_LOOP_ASM_RUN(TEXT)                                                                                          \
     asm volatile(TEXT : [wsoff] "=&v"(wsoff)                                                                               \
                  : [glogs] "v"(glogs), [lut2] "v"(lut2_lane), [codeoff] "v"(code_off), [recoff] "v"(rec_off),          \
-                   [codes] "s"(a.codes), [pos] "s"(a.pos4), [n_ops] "s"(g.N), [n_groups] "s"(g.G), [recbase] "s"(rec_base), \
-                   [gstride_lo] "s"(gs_lo), [gstride_hi] "s"(gs_hi), [wsstride] "s"(ws_stride), [prio] "s"(prio),       \
+                   [codes] "s"(a.codes), [pos] "s"(a.pos4), [n_ops] "s"(g.N), [recbase] "s"(rec_base), \
+                   [gstride_lo] "s"(gs_lo), [gstride_hi] "s"(gs_hi), [wsstride] "s"(ws_stride),                         \
                    [pace] "s"(pace)                                                                                     \
                  : ACE_LOOP_ASM_CLOBBERS)
     if (g.flags & ACE_F_RESHARDING) {
@@ -222,12 +237,24 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     if (RANGED && WIN)
         while (w0 + 1 < a.n_windows && a.win_pos[w0 + 1] <= (grp_begin << 4)) ++w0;
 
+    // this lane's plan header and its first sixteen op bytes: asked for before the tables are staged, used after
+    const ace_u4 h = a.hdr[pl];
+    ace_u4 cw = a.codes[(size_t)grp_begin * g.P + pl];
+
     // small tables: pair kinds and the (micro-batch, stage gpus) LUT; without windows, every row
-    for (int j = tid; j < a.rk_bytes; j += BLOCK) {
-        const uint32_t r = a.pair_kinds[j];
-        lds_raw[a.g.rk_lds_off + j] = (unsigned char)r;
-        if (DEFER && a.g.pk32_lds_off)
-            reinterpret_cast<uint32_t *>(lds_raw + a.g.pk32_lds_off)[j] = ((r & 15u) << a.g.z_shift) | (((r >> 4) << a.g.z_shift) << 16);
+    // (four pair kinds per lane and turn: the table is a multiple of 64 bytes)
+    for (int j = tid; j < (a.rk_bytes >> 2); j += BLOCK) {
+        const uint32_t r4 = reinterpret_cast<const uint32_t *>(a.pair_kinds)[j];
+        reinterpret_cast<uint32_t *>(lds_raw + a.g.rk_lds_off)[j] = r4;
+        if (DEFER && a.g.pk32_lds_off) {
+            uint32_t e[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t r = (r4 >> (8 * q)) & 0xffu;
+                e[q] = ((r & 15u) << a.g.z_shift) | (((r >> 4) << a.g.z_shift) << 16);
+            }
+            reinterpret_cast<ace_u4 *>(lds_raw + a.g.pk32_lds_off)[j] = ace_u4{e[0], e[1], e[2], e[3]};
+        }
     }
     for (int j = tid; j < a.stg_words; j += BLOCK) {
         const uint32_t w = a.stage_lut[j];
@@ -248,13 +275,13 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     const bool asm_loop = false;
 #endif
     if (DEFER && a.g.pace_lds_off && tid < 32) reinterpret_cast<uint32_t *>(lds_raw + a.g.pace_lds_off)[tid] = 0u;
-    if (!(WIN && asm_loop)) stage_window<BLOCK>(a, lds_raw, w0, tid);       // every row, or the first window's
+    if (!WIN && a.flat_rows16 > 0) stage_rows_flat<BLOCK>(a, lds_raw, tid);
+    else if (!(WIN && asm_loop)) stage_window<BLOCK>(a, lds_raw, w0, tid);       // every row, or the first window's
     ACE_SYNC();
 
     AceLds lds = ace_make_lds(lds_raw, lds_bytes);
     lds.grows = reinterpret_cast<const unsigned char *>(a.rows);
     PlanState<BD, RANGED, DEFER, COLL, DEFER && WIN> st;
-    const ace_u4 h = a.hdr[pl];
     st.init(g, lds, h, range);
     st.row_ids = a.pos_types;
     const double nbm1 = a.nbm1[st.bidx];
@@ -270,7 +297,6 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
 
     int w = w0 + 1;
     int next_win = WIN ? a.win_pos[w] : 0x7fffffff;
-    ace_u4 cw = a.codes[(size_t)grp_begin * g.P + pl];     // sixteen op bytes of this plan
     const uint32_t first_code = cw.x & 7u;
     int grp_stop = grp_end;
 #ifndef ACE_HOST_EMU

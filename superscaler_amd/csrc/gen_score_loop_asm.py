@@ -95,6 +95,8 @@ M_RC, M_P, M_ST, M_KP = "s[42:43]", "s[44:45]", "s[46:47]", "s[48:49]"
 MASK = [f"s{52 + j}" for j in range(4)]
 PLANT = [f"s{56 + j}" for j in range(4)]
 PREVFL = "s62"
+NGRP = "s51"                                # number of 16-op groups
+VMN = "s50"                                 # rows resident: vector-memory instructions issued since the load of the next group's code words
 WSLIMIT = "s28"                             # WSOFF of a seventeenth stage, which no lane has room for
 NEXTWIN, EVT, DMAOFF, ARRIVED = "s29", "s34", "s63", "s35"   # windowed rows: next window's first position, window index, ...
 DMAPTR = "s[60:61]"
@@ -310,6 +312,9 @@ class Gen:
         self.o(f"v_mov_b32 {META[y]}, {S0}")                 # position of the stage's last op | its row << 16 | the next op's row << 24
         self.o(f"v_cmp_gt_u32_e32 vcc, {WSLIMIT}, {WSOFF}")
         self.o("s_and_b64 exec, exec, vcc")
+        if not self.win:
+            self.o(f"s_cselect_b32 {S0}, 5, 0")                 # (no lane with room: the stores may not be issued at all)
+            self.o(f"s_add_u32 {VMN}, {VMN}, {S0}")
         self.o(f"global_store_dwordx4 {WSOFF}, v[32:35], %[recbase]")
         self.o(f"global_store_dwordx4 {WSOFF}, v[36:39], %[recbase] offset:16")
         self.o(f"global_store_dwordx4 {WSOFF}, v[40:43], %[recbase] offset:32")
@@ -379,9 +384,23 @@ class Gen:
             # loads now in flight need not be)
             self.o(f"s_cmp_eq_u32 {ARRIVED}, 1")
             self.o("s_cbranch_scc1 L_arr_%=")
-        self.o("s_waitcnt vmcnt(0)")
         if self.win:
+            self.o("s_waitcnt vmcnt(0)")
             self.o("L_arr_%=:")
+        else:
+            # (vector-memory instructions complete in the order they were issued: only what was issued before the
+            # load and the load itself have to be waited for, not the record stores of the last few ops)
+            for n in (15, 10, 5):
+                self.o(f"s_cmp_ge_u32 {VMN}, {n}")
+                self.o(f"s_cbranch_scc1 L_vm{n}_%=")
+            self.o("s_waitcnt vmcnt(0)")
+            self.o("s_branch L_vmd_%=")
+            for n in (15, 10, 5):
+                self.o(f"L_vm{n}_%=:")
+                self.o(f"s_waitcnt vmcnt({n})")
+                if n != 5:
+                    self.o("s_branch L_vmd_%=")
+            self.o("L_vmd_%=:")
         self.o(f"s_sub_i32 {LEFT}, %[n_ops], {POSBASE}")
         self.o(f"s_sub_i32 {LEFT}, {LEFT}, 16")
         self.apply_masks(NEXT, "nx")
@@ -389,13 +408,16 @@ class Gen:
     def build(self):
         o, c = self.o, self.c
         c("---- set-up")
-        c("issue priority of this wavefront (the deeper its plans, the higher)")
-        for lvl in (3, 2, 1):
-            o(f"s_cmp_eq_u32 %[prio], {lvl}")
-            o(f"s_cbranch_scc0 L_np{lvl}_%=")
-            o(f"s_setprio {lvl}")
-            o(f"L_np{lvl}_%=:")
+        if self.win:
+            c("issue priority of this wavefront (the deeper its plans, the higher; with rows resident the pacing sets it)")
+            for lvl in (3, 2, 1):
+                o(f"s_cmp_eq_u32 %[prio], {lvl}")
+                o(f"s_cbranch_scc0 L_np{lvl}_%=")
+                o(f"s_setprio {lvl}")
+                o(f"L_np{lvl}_%=:")
         o(f"s_mov_b64 {ALL}, exec")
+        o(f"s_add_u32 {NGRP}, %[n_ops], 15")
+        o(f"s_lshr_b32 {NGRP}, {NGRP}, 4")
         o(f"v_mov_b64 {GLOGS}, %[glogs]")
         o(f"v_mov_b32 {LUT2}, %[lut2]")
         o(f"s_mov_b64 {CPTR}, %[codes]")
@@ -431,7 +453,7 @@ class Gen:
         c("---- one 16-op group per iteration")
         o("L_group_%=:")
         o(f"s_add_u32 {S0}, {GRP}, 1")
-        o(f"s_cmp_lt_u32 {S0}, %[n_groups]")
+        o(f"s_cmp_lt_u32 {S0}, {NGRP}")
         o("s_cbranch_scc0 L_last_%=")
         o(f"s_add_u32 {CPTR_LO}, {CPTR_LO}, %[gstride_lo]")
         o(f"s_addc_u32 {CPTR_HI}, {CPTR_HI}, %[gstride_hi]")
@@ -441,6 +463,8 @@ class Gen:
         for r in NEXT:
             o(f"v_mov_b32 {r}, 0")
         o("L_loaded_%=:")
+        if not self.win:
+            o(f"s_mov_b32 {VMN}, 0")
         if self.win:
             o(f"s_mov_b32 {ARRIVED}, 0")
         else:
@@ -462,7 +486,7 @@ class Gen:
         o(f"s_addc_u32 {PPTR_HI}, {PPTR_HI}, 0")
         o(f"s_add_u32 {POSBASE}, {POSBASE}, 16")
         o(f"s_add_u32 {GRP}, {GRP}, 1")
-        o(f"s_cmp_lt_u32 {GRP}, %[n_groups]")
+        o(f"s_cmp_lt_u32 {GRP}, {NGRP}")
         o("s_cbranch_scc1 L_group_%=")
         o("L_exit_%=:")
         o(f"s_mov_b64 exec, {ALL}")

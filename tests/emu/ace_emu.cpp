@@ -182,12 +182,19 @@ extern "C" int ace_emu_kernel(const ace_tables_t *t, const uint8_t *codes, const
         ace_pos_types(t, pt, G * 16 + 16);
         a.pos_types = pt;
     }
-    a.pair_kinds = (const uint8_t *)pool.place(t->pair_kinds, (size_t)a.rk_bytes, 1);
+    a.pair_kinds = (const uint8_t *)pool.place(t->pair_kinds, (size_t)a.rk_bytes, 4);
     a.stage_lut = (const uint32_t *)pool.place(t->stage_lut, (size_t)a.stg_words * 4, 4);
     a.nbm1 = (const double *)pool.place(t->nb_minus_1, (size_t)t->n_mbs * 8, 8);
     a.win_pos = (const int32_t *)pool.place(t->win_pos, (size_t)(t->n_windows + 1) * 4, 4);
     a.win_row_begin = (const int32_t *)pool.place(t->win_row_begin, (size_t)(t->n_windows + 1) * 4, 4);
     a.win_rows = (const uint32_t *)pool.place(t->win_rows, n_win_rows * 8, 4);
+    // (what the library works out at ace_create: resident rows that lie in LDS as in global memory are staged as one block)
+    if (t->n_windows == 1 && (t->row_doubles & 1) == 0) {
+        bool flat = true;
+        for (int r = 0; r < t->win_row_begin[1]; ++r)
+            flat = flat && t->win_rows[2 * r] == (uint32_t)r && t->win_rows[2 * r + 1] == (uint32_t)r * (uint32_t)t->row_doubles * 8u;
+        if (flat) a.flat_rows16 = t->win_row_begin[1] * (t->row_doubles / 2);
+    }
     a.iter_ms = (double *)pool.place(iter_ms, (size_t)P * 8, 8);
     a.peak_mb = (double *)pool.place(peak_mb, (size_t)P * 8, 8);
     a.feasible = (uint8_t *)pool.place(feasible, (size_t)P, 1);

@@ -96,7 +96,7 @@ MASK = [f"s{52 + j}" for j in range(4)]
 PLANT = [f"s{56 + j}" for j in range(4)]
 PREVFL = "s62"
 NGRP = "s51"                                # number of 16-op groups
-VMN = "s50"                                 # rows resident: vector-memory instructions issued since the load of the next group's code words
+VMN = "s50"                                 # record stores issued since the load of the next group's code words
 WSLIMIT = "s28"                             # WSOFF of a seventeenth stage, which no lane has room for
 NEXTWIN, EVT, DMAOFF, ARRIVED = "s29", "s34", "s63", "s35"   # windowed rows: next window's first position, window index, ...
 DMAPTR = "s[60:61]"
@@ -312,9 +312,8 @@ class Gen:
         self.o(f"v_mov_b32 {META[y]}, {S0}")                 # position of the stage's last op | its row << 16 | the next op's row << 24
         self.o(f"v_cmp_gt_u32_e32 vcc, {WSLIMIT}, {WSOFF}")
         self.o("s_and_b64 exec, exec, vcc")
-        if not self.win:
-            self.o(f"s_cselect_b32 {S0}, 5, 0")                 # (no lane with room: the stores may not be issued at all)
-            self.o(f"s_add_u32 {VMN}, {VMN}, {S0}")
+        self.o(f"s_cselect_b32 {S0}, 5, 0")                     # (no lane with room: the stores may not be issued at all)
+        self.o(f"s_add_u32 {VMN}, {VMN}, {S0}")
         self.o(f"global_store_dwordx4 {WSOFF}, v[32:35], %[recbase]")
         self.o(f"global_store_dwordx4 {WSOFF}, v[36:39], %[recbase] offset:16")
         self.o(f"global_store_dwordx4 {WSOFF}, v[40:43], %[recbase] offset:32")
@@ -384,23 +383,21 @@ class Gen:
             # loads now in flight need not be)
             self.o(f"s_cmp_eq_u32 {ARRIVED}, 1")
             self.o("s_cbranch_scc1 L_arr_%=")
+        # (vector-memory instructions complete in the order they were issued: only what was issued before the load and
+        # the load itself have to be waited for, not the record stores of the last few ops)
+        for n in (15, 10, 5):
+            self.o(f"s_cmp_ge_u32 {VMN}, {n}")
+            self.o(f"s_cbranch_scc1 L_vm{n}_%=")
+        self.o("s_waitcnt vmcnt(0)")
+        self.o("s_branch L_vmd_%=")
+        for n in (15, 10, 5):
+            self.o(f"L_vm{n}_%=:")
+            self.o(f"s_waitcnt vmcnt({n})")
+            if n != 5:
+                self.o("s_branch L_vmd_%=")
+        self.o("L_vmd_%=:")
         if self.win:
-            self.o("s_waitcnt vmcnt(0)")
             self.o("L_arr_%=:")
-        else:
-            # (vector-memory instructions complete in the order they were issued: only what was issued before the
-            # load and the load itself have to be waited for, not the record stores of the last few ops)
-            for n in (15, 10, 5):
-                self.o(f"s_cmp_ge_u32 {VMN}, {n}")
-                self.o(f"s_cbranch_scc1 L_vm{n}_%=")
-            self.o("s_waitcnt vmcnt(0)")
-            self.o("s_branch L_vmd_%=")
-            for n in (15, 10, 5):
-                self.o(f"L_vm{n}_%=:")
-                self.o(f"s_waitcnt vmcnt({n})")
-                if n != 5:
-                    self.o("s_branch L_vmd_%=")
-            self.o("L_vmd_%=:")
         self.o(f"s_sub_i32 {LEFT}, %[n_ops], {POSBASE}")
         self.o(f"s_sub_i32 {LEFT}, {LEFT}, 16")
         self.apply_masks(NEXT, "nx")
@@ -463,8 +460,7 @@ class Gen:
         for r in NEXT:
             o(f"v_mov_b32 {r}, 0")
         o("L_loaded_%=:")
-        if not self.win:
-            o(f"s_mov_b32 {VMN}, 0")
+        o(f"s_mov_b32 {VMN}, 0")
         if self.win:
             o(f"s_mov_b32 {ARRIVED}, 0")
         else:

@@ -91,7 +91,9 @@ def other_workloads(steps):
         batch = synth.make_plans(w, tables, n_plans=OTHER_PLANS, workers=min(16, os.cpu_count() or 1))
         ev = PlanEvaluator(tables, device="cuda:0")
         d = ev.upload(batch)
-        ev.time_score_kernel(d, reps=20)
+        # (the plans of each workload are drawn on the host for seconds while the GPU idles: as many untimed launches
+        # as timed ones first, like the headline measurement's warm-up)
+        ev.time_score_kernel(d, reps=max(steps, 20))
         ms = ev.time_score_kernel(d, reps=max(steps, 20))
         bpp = 3 * d.num_ops + 19
         gbps = bpp * d.n_plans / (ms * 1e-3) / 1e9

@@ -692,6 +692,47 @@ def test_unscorable_and_malformed_plans_are_flagged(torch_mod):
     ev.close()
 
 
+@pytest.mark.parametrize("name", ["gpt3_13b", "wresnet_1b"])
+def test_plans_around_the_sixteen_stage_limit_agree_with_the_breakdown_kernel(name, torch_mod):
+    """The assembly op loop counts a plan's stages by the offset of its next workspace record and stops storing records
+    at the sixteenth: plans cut into 15, 16, 17, 18 and 40 stages, with headers that claim that count or 16, must come
+    out of plain scoring (assembly loop) exactly as out of the per-stage breakdown (C++ loop) -- a seventeenth stage is a
+    malformed plan whatever the header says, and must not touch another plan's records."""
+    from superscaler_amd.evaluator import PlanEvaluator
+    w = synth.WORKLOADS[name]
+    tables = synth.make_tables(w)
+    n = 4096
+    good = synth.make_plans(w, tables, n_plans=n, seed_offset=88, workers=8)
+    bad = PlanBatch(good.codes.copy(), good.hdr.copy())
+    N = bad.codes.shape[1]
+    rng = np.random.default_rng(5)
+    counts = [15, 16, 17, 18, 40]
+    counts = [c for c in counts if c <= N]
+    touched = np.zeros(n, dtype=bool)
+    for r in range(0, n, 3):
+        c = counts[(r // 3) % len(counts)]
+        cuts = np.sort(rng.choice(np.arange(1, N), size=c - 1, replace=False))
+        bad.codes[r] &= np.uint8(0xef)
+        bad.codes[r, 0] |= 16
+        bad.codes[r, cuts] |= 16
+        claim = c if (r // 3) % 2 == 0 else 16
+        bad.hdr[r, 0] = (bad.hdr[r, 0] & ~np.uint32(0xff)) | np.uint32(claim)
+        touched[r] = True
+    ev = PlanEvaluator(tables)
+    d = ev.upload(bad, validate=False)
+    it, pk, fe, st = [t.cpu().numpy() for t in ev.score(d)]
+    bit, bpk, bfe, bst, _ = [t.cpu().numpy() for t in ev.score(d, breakdown=True)]
+    assert np.array_equal(st, bst) and np.array_equal(fe, bfe)
+    assert np.array_equal(it, bit, equal_nan=True) and np.array_equal(pk, bpk, equal_nan=True)
+    # more than sixteen stages: never a valid plan
+    over = np.array([touched[r] and counts[(r // 3) % len(counts)] > 16 for r in range(n)])
+    assert (st[over] != 0).all() and not fe[over].any()
+    # their neighbours in the batch (and in the workgroup's workspace) are untouched
+    git, gpk, gfe, gst = ev.score_host(good)
+    assert np.array_equal(it[~touched], git[~touched]) and np.array_equal(pk[~touched], gpk[~touched])
+    ev.close()
+
+
 @pytest.mark.parametrize("name,n", [("gpt3_13b", 20000), ("gpt3_13b", 140000), ("wresnet_1b", 20000), ("t5_770m", 20000)])
 def test_corrupted_batches_plain_scoring_equals_the_breakdown_kernel(name, n, torch_mod):
     """Plain scoring runs the assembly op loop (over windowed rows for wresnet_1b), the per-stage breakdown the C++ loop

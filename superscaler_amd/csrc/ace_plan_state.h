@@ -435,37 +435,34 @@ template <bool BD, bool RANGED, bool DEFER = false, bool COLL = false, bool GROW
         saved = rec.r[3].x; peak = rec.r[3].y; run = 0.0; lastclose = false; rfm = rec.r[4].x; rbm = 0.0;
     }
 
-    // One stage of replay_all(): stage s2 is evaluated from (rx, lx); meanwhile record s2 + 2 is fetched into rx and
-    // the boundary entries of stage s2 + 1 (record in ry) into ly.
-    ACE_HD void replay_step(const AceGeom &g, const AceLds &lds, const double *ws, int s2, int n_st, Record &rx, Lookups &lx,
-                            const Record &ry, Lookups &ly) {
-        const bool live = s2 < n_st;
-        const ace_d2 oe = lx.oe;
-        const uint32_t c_last = lx.c_last;
-        if (live) replay_take(g, rx, lx, s2);
-        // (only lanes that have the stage fetch it: the slot of a stage a plan does not have may never have been written)
-        if (s2 + 2 < n_st) replay_load(ws, s2 + 2, rx);
-        if (s2 + 1 < n_st) replay_lookups(g, lds, ry, s2 + 1, true, ly);
-        if (live) finish_tail(g, lds, 0u, c_last, oe, nullptr);
-    }
-
-    // All stashed stages of a plan of n_st stages whose first op has code `code0` and row `row0`.
+    // All stashed stages of a plan of n_st stages whose first op has code `code0` and row `row0`.  The records come from
+    // memory (they were written up to a whole op loop ago) and waiting for them is most of what this costs: three are
+    // in flight per lane (record s + 3 is asked for when stage s is taken), in three sets of registers used in turn;
+    // a stage's boundary entries are looked up when its turn comes (LDS is idle by then).
     ACE_HD void replay_all(const AceGeom &g, const AceLds &lds, const double *ws, int n_st, uint32_t code0, uint32_t row0) {
         replay_code = code0;
         replay_row = row0;
-        Record ra, rb;
-        Lookups la, lb;
-        replay_load(ws, 0, ra);
-        rb = ra;
-        if (1 < n_st) replay_load(ws, 1, rb);
-        replay_lookups(g, lds, ra, 0, 0 < n_st, la);
-        lb = la;
-        for (int s2 = 0; s2 < ACE_MAX_STAGES; s2 += 2) {
-            if (!ACE_WAVE_ANY(s2 < n_st)) break;
-            replay_step(g, lds, ws, s2, n_st, ra, la, rb, lb);
-            if (!ACE_WAVE_ANY(s2 + 1 < n_st)) break;
-            replay_step(g, lds, ws, s2 + 1, n_st, rb, lb, ra, la);
+        Record r[3];
+        replay_load(ws, 0, r[0]);
+        r[1] = r[0];
+        r[2] = r[0];
+        if (1 < n_st) replay_load(ws, 1, r[1]);
+        if (2 < n_st) replay_load(ws, 2, r[2]);
+        for (int base = 0; base < ACE_MAX_STAGES; base += 3) {
+#pragma unroll
+            for (int k = 0; k < 3; ++k) {
+                const int s2 = base + k;
+                if (!ACE_WAVE_ANY(s2 < n_st)) goto replayed;
+                const bool live = s2 < n_st;
+                Lookups lx;
+                replay_lookups(g, lds, r[k], s2, live, lx);
+                if (live) replay_take(g, r[k], lx, s2);
+                // (only lanes that have the stage fetch it: the slot of a stage a plan does not have may never have been written)
+                if (s2 + 3 < n_st) replay_load(ws, s2 + 3, r[k]);
+                if (live) finish_tail(g, lds, 0u, lx.c_last, lx.oe, nullptr);
+            }
         }
+    replayed:
         s = n_st;               // (the evaluation walked s again; result() checks the count of the op loop)
     }
 

@@ -807,7 +807,7 @@ static int upload_pos4(ace_handle *h, const ace_tables_t *t, size_t pos_entries,
     if (!pk32_off || t->n_windows != 1) return ACE_OK;       // (windowed rows: setup_windowed_asm)
     ace_u4 *p4 = new (std::nothrow) ace_u4[pos_entries];
     if (!p4) return ACE_ENOMEM;
-    const uint32_t row_bytes = (uint32_t)t->row_doubles * 8u, kind_stride = (uint32_t)t->n_glog * 64u;
+    const uint32_t row_bytes = (uint32_t)t->row_doubles * 8u, kind_stride = (uint32_t)t->n_glog * ACE_PK32_BLOCK;   // (words of the 32-bit table per pair kind)
     for (size_t i = 0; i < pos_entries; ++i) {
         const uint32_t info = i < (size_t)t->num_ops ? t->pos_info[i] : 0u;
         const uint32_t row = (info & 0xffu) * row_bytes;
@@ -897,7 +897,7 @@ static int setup_windowed_asm(ace_handle *h, const ace_tables_t *t, size_t pos_e
     };
     // the per-position table
     std::vector<ace_u4> p4(pos_entries);
-    const uint32_t kind_stride = (uint32_t)t->n_glog * 64u;
+    const uint32_t kind_stride = (uint32_t)t->n_glog * ACE_PK32_BLOCK;
     for (size_t i = 0, w = 0; i < pos_entries; ++i) {
         if (i >= (size_t)N) { p4[i] = ace_u4{0u, hot_len, pk32_off, 0u}; continue; }
         while ((int)w + 1 < n_w && (size_t)win_start[w + 1] <= i) ++w;

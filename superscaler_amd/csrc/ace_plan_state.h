@@ -159,6 +159,7 @@ struct AceGeom {
 ACE_HD uint32_t info_row(const AceGeom &g, uint32_t i) { return (i & 0xffu) * g.row_bytes; }
 ACE_HD uint32_t info_nextrow(const AceGeom &g, uint32_t i) { return ((i >> 8) & 0xffu) * g.row_bytes; }
 
+#define ACE_PK32_BLOCK 65u      // words from one 64-entry block of the 32-bit pair-kind table to the next
 #define ACE_WS_REC 10          // doubles per deferred stage record (see PlanState::stash)
 
 // LDS regions behind the resident rows: pair kinds | stage LUT (one word per (micro-batch, stage size)) | per
@@ -176,6 +177,9 @@ uint32_t ace_lds_layout(uint32_t rk_off, uint32_t rk_bytes, uint32_t stg_words, 
 }
 // The assembly form of the op loop reads the pair kinds as 32-bit entries (one per byte of the table above: byte offset
 // of the forward collective's cost table | that of the backward collective's << 16), placed behind everything else.
+// Every block of 64 entries (one stage size of one pair kind) is followed by one unused entry: a block of 64 words
+// spans all 64 LDS banks, and the lanes of a wavefront differ in their stage sizes, so without it lanes with the same
+// (code, next code) and different stage sizes would read different words of one bank (ACE_PK32_BLOCK words per block).
 #ifdef ACE_HOST_EMU
 inline
 #else
@@ -183,7 +187,7 @@ __host__ __device__ inline
 #endif
 uint32_t ace_lds_pk32(uint32_t lds_end, uint32_t rk_bytes, uint32_t *pk32_off) {
     *pk32_off = (lds_end + 15u) & ~15u;
-    return *pk32_off + rk_bytes * 4u;
+    return *pk32_off + (rk_bytes / 64u) * ACE_PK32_BLOCK * 4u;
 }
 
 // COLL: consider_collective_memory (the tables carry ACE_F_COLLECTIVE_MEM).

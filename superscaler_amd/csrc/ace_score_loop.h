@@ -253,7 +253,10 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
                 const uint32_t r = (r4 >> (8 * q)) & 0xffu;
                 e[q] = ((r & 15u) << a.g.z_shift) | (((r >> 4) << a.g.z_shift) << 16);
             }
-            reinterpret_cast<ace_u4 *>(lds_raw + a.g.pk32_lds_off)[j] = ace_u4{e[0], e[1], e[2], e[3]};
+            // (entries 4j .. 4j + 3 of block j / 16; the blocks are ACE_PK32_BLOCK words apart)
+            uint32_t *dst = reinterpret_cast<uint32_t *>(lds_raw + a.g.pk32_lds_off) + (4 * j + (j >> 4) * (int)(ACE_PK32_BLOCK - 64u));
+#pragma unroll
+            for (int q = 0; q < 4; ++q) dst[q] = e[q];
         }
     }
     for (int j = tid; j < a.stg_words; j += BLOCK) {
@@ -263,10 +266,11 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
         // and the pair-kind block of the stage size relative to it (what PlanState::start_fast hands to the op loop)
         const uint32_t glog = (uint32_t)j & 15u;
         const uint32_t z_v = (w & 15u) * (uint32_t)a.g.C * 8u;
-        const uint32_t rk = (glog < (uint32_t)a.g.n_glog ? glog : 0u) << 6;
+        const uint32_t gl = glog < (uint32_t)a.g.n_glog ? glog : 0u, rk = gl << 6;
         reinterpret_cast<ace_u2 *>(lds_raw + a.g.lut2_lds_off)[j] = ace_u2{z_v, rk - z_v};
-        // (the assembly loop adds the pair-kind block offset to the op pair's own index, not to the diag's)
-        if (DEFER && a.g.lut2a_lds_off) reinterpret_cast<ace_u2 *>(lds_raw + a.g.lut2a_lds_off)[j] = ace_u2{z_v, rk};
+        // (the assembly loop adds the pair-kind block offset to the op pair's own index, not to the diag's, and its blocks
+        // are ACE_PK32_BLOCK words apart)
+        if (DEFER && a.g.lut2a_lds_off) reinterpret_cast<ace_u2 *>(lds_raw + a.g.lut2a_lds_off)[j] = ace_u2{z_v, gl * ACE_PK32_BLOCK};
     }
     // (the assembly op loop over windowed rows fetches its windows itself, in a layout of its own)
 #ifndef ACE_HOST_EMU

@@ -4,9 +4,11 @@
 
 The loop is the one ace_score_body() runs in C++ (ace_score_loop.h, PlanState::step / stash / start_fast of
 ace_plan_state.h, DEFER variant), written out by hand so that
-  * the 0/1 factors of the recompute rules become execution masks: the recompute bit, the recompute-pair bit and
-    the stage-start bit of an op are tested with one byte-select compare each, and the conditional additions run
-    under the resulting lane mask (an addition that does not happen and an addition of +0.0 give the same bits);
+  * the 0/1 factors of the recompute rules become execution masks: the recompute bit and the stage-start bit of an
+    op are tested with one byte-select compare each (the recompute bit a step ahead), the recompute-pair mask is the
+    AND of two consecutive recompute masks without the lanes whose next op starts a stage (scalar instructions), and
+    the conditional additions run under the resulting lane mask (an addition that does not happen and an addition of
+    +0.0 give the same bits);
   * the table reads of op k+1 are issued before op k's values are used (two alternating register sets);
   * every position-dependent address comes ready-made from a per-position table (four words per op position,
     read with scalar loads one 4-op word ahead) instead of being derived per op.
@@ -72,10 +74,10 @@ WORD = [f"v{102 + j}" for j in range(4)]    # code words of the current 16-op gr
 NEXT = [f"v{106 + j}" for j in range(4)]    # ... of the next group
 
 
-def D(y):                                   # per 4-op word: next-op bytes, code*8, code*8+next code, rc bit, pair bit
+def D(y):                                   # per 4-op word: next-op bytes, code*8, code*8+next code, rc bit
     b = (110, 116)[y]
     r = (114, 118)[y]
-    return dict(nw=f"v{b}", w8=f"v{b+1}", cn=CN[y], r8=f"v{r}", p8=f"v{r+1}")
+    return dict(nw=f"v{b}", w8=f"v{b+1}", cn=CN[y], r8=f"v{r}")
 
 
 ZV_, RK, ZVRK, WSOFF = "v120", "v121", "v[120:121]", "v122"   # WSOFF: byte offset of this lane's next stage record (it counts the stages)
@@ -92,8 +94,8 @@ CPTR, CPTR_LO, CPTR_HI = "s[26:27]", "s26", "s27"
 GRP, K07, K08, POSBASE, LEFT, K1F = "s30", "s39", "s40", "s41", "s31", "s38"
 PPTR, PPTR_LO, PPTR_HI = "s[36:37]", "s36", "s37"
 M_RC, M_P, M_ST, M_KP = "s[42:43]", "s[44:45]", "s[46:47]", "s[48:49]"
-MASK = [f"s{52 + j}" for j in range(4)]
-PLANT = [f"s{56 + j}" for j in range(4)]
+M_RCN = "s[58:59]"                          # M_RC of the next op (compared a step ahead: the pair mask is made of both)
+MASK, PLANT = "s52", "s56"                   # padding mask and end-of-plan mark of one code word (scratch)
 PREVFL = "s62"
 NGRP = "s51"                                # number of 16-op groups
 VMN = "s50"                                 # record stores issued since the load of the next group's code words
@@ -125,14 +127,12 @@ class Gen:
     # -- pieces ------------------------------------------------------------------------------------------------
     def prep(self, y, wa, wb):
         d = D(y)
-        self.c(f"word-level: next-op bytes, code*8, code*8+next code, recompute bit, recompute-pair bit (buffer {y})")
+        self.c(f"word-level: next-op bytes, code*8, code*8+next code, recompute bit (buffer {y})")
         self.o(f"v_alignbit_b32 {d['nw']}, {wb}, {wa}, 8")
         self.o(f"v_and_b32 {d['w8']}, {K07}, {wa}")
         self.o(f"v_lshlrev_b32 {d['w8']}, 3, {d['w8']}")
         self.o(f"v_and_or_b32 {d['cn']}, {d['nw']}, {K07}, {d['w8']}")
         self.o(f"v_and_b32 {d['r8']}, {K08}, {wa}")
-        self.o(f"v_lshrrev_b32 {d['p8']}, 1, {d['nw']}")
-        self.o(f"v_bitop3_b32 {d['p8']}, {d['r8']}, {d['nw']}, {d['p8']} bitop3:0x40")
 
     def stage_fetch(self, dst):
         """Asks for z_v and the pair-table block of the plan's next stage: one 8-byte LDS read per lane, indexed by the
@@ -211,6 +211,8 @@ class Gen:
         self.o(f"s_cmp_eq_u32 {S0}, {NEXTWIN}")
         self.o(f"s_cbranch_scc0 L_nw_{L}")
         self.fetch_event(L, 64 + 16 * y)                    # (the first two position entries of this word are done with)
+        # (the event's descriptors went through the registers that held the next op's recompute mask)
+        self.o(f"v_cmp_ne_u32_sdwa {M_RCN}, {D((k1 >> 2) & 1)['r8']}, 0 src0_sel:BYTE_{k1 & 3} src1_sel:DWORD")
         self.o(f"L_nw_{L}:")
         self.o(f"s_cmp_lg_u64 {M_ST}, 0")                   # (what the branch to the stage-end code tests)
 
@@ -255,9 +257,14 @@ class Gen:
             else:
                 self.prep(0, NEXT[0], NEXT[1])
         sel = f"src0_sel:BYTE_{b} src1_sel:DWORD"
-        self.o(f"v_cmp_ne_u32_sdwa {M_RC}, {d['r8']}, 0 {sel}")
-        self.o(f"v_cmp_ne_u32_sdwa {M_P}, {d['p8']}, 0 {sel}")
+        # "recomputed" of the NEXT op (this op's was compared a step ago); (this op, next op) is a recompute pair if
+        # both are recomputed and the next op does not start a stage: two scalar instructions instead of a third compare
+        k1 = k + 1
+        d1 = D((k1 >> 2) & 1)
+        self.o(f"v_cmp_ne_u32_sdwa {M_RCN}, {d1['r8']}, 0 src0_sel:BYTE_{k1 & 3} src1_sel:DWORD")
         self.o(f"v_cmp_gt_u32_sdwa {M_ST}, {d['nw']}, 15 {sel}")
+        self.o(f"s_and_b64 {M_P}, {M_RC}, {M_RCN}")
+        self.o(f"s_andn2_b64 {M_P}, {M_P}, {M_ST}")
         self.o(f"s_cmp_lg_u64 {M_ST}, 0")
         self.o(f"s_cbranch_scc0 L_ns_{L}")
         self.c("lanes whose next op opens a stage: that stage's table offsets; its first op pays no resharding")
@@ -345,31 +352,27 @@ class Gen:
         self.o(f"v_max_f64 {PEAK}, {PEAK}, {RUN}")
         self.o(f"v_mov_b64 {RUN}, 0")
         self.o(f"s_mov_b64 exec, {ALL}")
+        self.o(f"s_mov_b64 {M_RC}, {M_RCN}")
         if b == 3:
             self.o(f"s_mov_b32 {PREVFL}, {p['fl']}")
 
-    def word_masks(self, tag):
-        """MASK[j] / PLANT[j] of the four words of a group from LEFT = N - (first position of that group):
-        code bytes of positions past the last op read as zero, and the byte right after the last op gets a
-        stage-start bit, which is what ends the plan's last stage."""
+    def apply_masks(self, regs, tag):
+        """Code bytes of positions past the last op read as zero, and the byte right after the last op gets a stage-start
+        bit, which is what ends the plan's last stage (LEFT = N - (first position of the group); five code bits used)."""
+        self.o(f"s_cmp_ge_i32 {LEFT}, 16")
+        self.o(f"s_cbranch_scc1 L_full_{tag}_%=")
         for j in range(4):
             self.o(f"s_sub_i32 {S0}, {LEFT}, {4 * j}")
             self.o(f"s_min_i32 {S1}, {S0}, 4")
             self.o(f"s_max_i32 {S1}, {S1}, 0")
             self.o(f"s_lshl_b32 {S1}, {S1}, 3")
             self.o(f"s_bfm_b64 {S23}, {S1}, 0")
-            self.o(f"s_and_b32 {MASK[j]}, {S2}, {K1F}")
+            self.o(f"s_and_b32 {MASK}, {S2}, {K1F}")
             self.o(f"s_lshl_b64 {S23}, 16, {S1}")
             self.o(f"s_cmp_ge_i32 {S0}, 0")
-            self.o(f"s_cselect_b32 {PLANT[j]}, {S2}, 0")
-
-    def apply_masks(self, regs, tag):
-        self.o(f"s_cmp_ge_i32 {LEFT}, 16")
-        self.o(f"s_cbranch_scc1 L_full_{tag}_%=")
-        self.word_masks(tag)
-        for j in range(4):
-            self.o(f"v_and_b32 {regs[j]}, {MASK[j]}, {regs[j]}")
-            self.o(f"v_or_b32 {regs[j]}, {PLANT[j]}, {regs[j]}")
+            self.o(f"s_cselect_b32 {PLANT}, {S2}, 0")
+            self.o(f"v_and_b32 {regs[j]}, {MASK}, {regs[j]}")
+            self.o(f"v_or_b32 {regs[j]}, {PLANT}, {regs[j]}")
         self.o(f"s_branch L_masked_{tag}_%=")
         self.o(f"L_full_{tag}_%=:")
         for j in range(4):
@@ -446,6 +449,7 @@ class Gen:
         o(f"s_mov_b32 {LEFT}, %[n_ops]")
         self.apply_masks(WORD, "w0")
         self.prep(0, WORD[0], WORD[1])
+        o(f"v_cmp_ne_u32_sdwa {M_RC}, {D(0)['r8']}, 0 src0_sel:BYTE_0 src1_sel:DWORD")
         self.issue(0)
         c("---- one 16-op group per iteration")
         o("L_group_%=:")

@@ -65,12 +65,26 @@ inline void ace_pos_types(const ace_tables_t *t, uint32_t *out, size_t entries) 
 }
 
 // Rows resident and laid out in LDS as they lie in global memory: one block copy with every lane busy, four loads in
-// flight per lane (row by row, a lane has one load at a time and most lanes none).
-template <int BLOCK> ACE_HD void stage_rows_flat(const AceKernelArgs &a, unsigned char *lds_raw, int tid) {
+// flight per lane (row by row, a lane has one load at a time and most lanes none).  The first four loads of a lane are
+// asked for before the workgroup sorts its plans (stage_rows_first) and written after it (the sort's scratch space is
+// where the rows go).
+struct AceRowsFirst { ace_d2 v[4]; };
+template <int BLOCK> ACE_HD AceRowsFirst stage_rows_first(const AceKernelArgs &a, int tid) {
+    const ace_d2 *src = reinterpret_cast<const ace_d2 *>(a.rows);
+    const int n = a.flat_rows16;
+    AceRowsFirst f;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) f.v[k] = tid + k * BLOCK < n ? src[tid + k * BLOCK] : ace_d2{0.0, 0.0};
+    return f;
+}
+template <int BLOCK> ACE_HD void stage_rows_flat(const AceKernelArgs &a, unsigned char *lds_raw, int tid, const AceRowsFirst &f) {
     const ace_d2 *src = reinterpret_cast<const ace_d2 *>(a.rows);
     ace_d2 *dst = reinterpret_cast<ace_d2 *>(lds_raw);
     const int n = a.flat_rows16;
-    int j = tid;
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+        if (tid + k * BLOCK < n) dst[tid + k * BLOCK] = f.v[k];
+    int j = tid + 4 * BLOCK;
     for (; j + 3 * BLOCK < n; j += 4 * BLOCK) {
         const ace_d2 v0 = src[j], v1 = src[j + BLOCK], v2 = src[j + 2 * BLOCK], v3 = src[j + 3 * BLOCK];
         dst[j] = v0; dst[j + BLOCK] = v1; dst[j + 2 * BLOCK] = v2; dst[j + 3 * BLOCK] = v3;
@@ -164,6 +178,9 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     g.rk_lds_off += lds_base; g.stg_lds_off += lds_base; g.lut2_lds_off += lds_base;
     if (g.lut2a_lds_off) g.lut2a_lds_off += lds_base;
     const long long slot = block * BLOCK + tid;                     // this lane's place in the batch (and in the workspace)
+    AceRowsFirst rows_first;
+    const bool flat = !WIN && a.flat_rows16 > 0;
+    if (flat) rows_first = stage_rows_first<BLOCK>(a, tid);
     long long plan = slot;
     uint32_t prio = 0;                                              // issue priority of this wavefront in the op loop
 #ifndef ACE_HOST_EMU
@@ -279,7 +296,7 @@ ACE_HD void ace_score_body(const AceKernelArgs &a, unsigned char *lds_raw, uint3
     const bool asm_loop = false;
 #endif
     if (DEFER && a.g.pace_lds_off && tid < 32) reinterpret_cast<uint32_t *>(lds_raw + a.g.pace_lds_off)[tid] = 0u;
-    if (!WIN && a.flat_rows16 > 0) stage_rows_flat<BLOCK>(a, lds_raw, tid);
+    if (flat) stage_rows_flat<BLOCK>(a, lds_raw, tid, rows_first);
     else if (!(WIN && asm_loop)) stage_window<BLOCK>(a, lds_raw, w0, tid);       // every row, or the first window's
     ACE_SYNC();
 

@@ -93,8 +93,8 @@ ALL = "s[24:25]"
 CPTR, CPTR_LO, CPTR_HI = "s[26:27]", "s26", "s27"
 GRP, K07, K08, POSBASE, LEFT, K1F = "s30", "s39", "s40", "s41", "s31", "s38"
 PPTR, PPTR_LO, PPTR_HI = "s[36:37]", "s36", "s37"
-M_RC, M_P, M_ST, M_KP = "s[42:43]", "s[44:45]", "s[46:47]", "s[48:49]"
-M_RCN = "s[58:59]"                          # M_RC of the next op (compared a step ahead: the pair mask is made of both)
+M_P, M_ST, M_KP = "s[44:45]", "s[46:47]", "s[48:49]"
+MRC = ["s[42:43]", "s[58:59]"]              # "recomputed" of the ops at even / odd positions: an op's is compared a step ahead (the pair mask is made of two)
 MASK, PLANT = "s52", "s56"                   # padding mask and end-of-plan mark of one code word (scratch)
 PREVFL = "s62"
 NGRP = "s51"                                # number of 16-op groups
@@ -211,8 +211,10 @@ class Gen:
         self.o(f"s_cmp_eq_u32 {S0}, {NEXTWIN}")
         self.o(f"s_cbranch_scc0 L_nw_{L}")
         self.fetch_event(L, 64 + 16 * y)                    # (the first two position entries of this word are done with)
-        # (the event's descriptors went through the registers that held the next op's recompute mask)
-        self.o(f"v_cmp_ne_u32_sdwa {M_RCN}, {D((k1 >> 2) & 1)['r8']}, 0 src0_sel:BYTE_{k1 & 3} src1_sel:DWORD")
+        # (the event's descriptors went through the registers that hold the recompute mask of the ops at odd positions:
+        # window starts are multiples of four, so that is the op being processed)
+        k = k1 - 1
+        self.o(f"v_cmp_ne_u32_sdwa {MRC[k & 1]}, {D((k >> 2) & 1)['r8']}, 0 src0_sel:BYTE_{k & 3} src1_sel:DWORD")
         self.o(f"L_nw_{L}:")
         self.o(f"s_cmp_lg_u64 {M_ST}, 0")                   # (what the branch to the stage-end code tests)
 
@@ -261,9 +263,9 @@ class Gen:
         # both are recomputed and the next op does not start a stage: two scalar instructions instead of a third compare
         k1 = k + 1
         d1 = D((k1 >> 2) & 1)
-        self.o(f"v_cmp_ne_u32_sdwa {M_RCN}, {d1['r8']}, 0 src0_sel:BYTE_{k1 & 3} src1_sel:DWORD")
+        self.o(f"v_cmp_ne_u32_sdwa {MRC[k1 & 1]}, {d1['r8']}, 0 src0_sel:BYTE_{k1 & 3} src1_sel:DWORD")
         self.o(f"v_cmp_gt_u32_sdwa {M_ST}, {d['nw']}, 15 {sel}")
-        self.o(f"s_and_b64 {M_P}, {M_RC}, {M_RCN}")
+        self.o(f"s_and_b64 {M_P}, {MRC[0]}, {MRC[1]}")
         self.o(f"s_andn2_b64 {M_P}, {M_P}, {M_ST}")
         self.o(f"s_cmp_lg_u64 {M_ST}, 0")
         self.o(f"s_cbranch_scc0 L_ns_{L}")
@@ -299,7 +301,7 @@ class Gen:
             self.o(f"v_add_f64 {RSB}, {RSB}, {zb}")
         self.o(f"v_max_f64 {RFM[nxt]}, {RFM[cur]}, {e['rf']}")
         self.o(f"v_max_f64 {RBM[nxt]}, {RBM[cur]}, {e['rb']}")
-        self.o(f"s_mov_b64 exec, {M_RC}")
+        self.o(f"s_mov_b64 exec, {MRC[k & 1]}")
         self.o(f"v_add_f64 {RCS}, {RCS}, {e['fwd']}")
         self.o(f"s_cbranch_scc0 L_ne_{L}")
         self.c("lanes whose stage ends with this op: park the stage's values, start the next stage from zero")
@@ -352,7 +354,6 @@ class Gen:
         self.o(f"v_max_f64 {PEAK}, {PEAK}, {RUN}")
         self.o(f"v_mov_b64 {RUN}, 0")
         self.o(f"s_mov_b64 exec, {ALL}")
-        self.o(f"s_mov_b64 {M_RC}, {M_RCN}")
         if b == 3:
             self.o(f"s_mov_b32 {PREVFL}, {p['fl']}")
 
@@ -449,7 +450,7 @@ class Gen:
         o(f"s_mov_b32 {LEFT}, %[n_ops]")
         self.apply_masks(WORD, "w0")
         self.prep(0, WORD[0], WORD[1])
-        o(f"v_cmp_ne_u32_sdwa {M_RC}, {D(0)['r8']}, 0 src0_sel:BYTE_0 src1_sel:DWORD")
+        o(f"v_cmp_ne_u32_sdwa {MRC[0]}, {D(0)['r8']}, 0 src0_sel:BYTE_0 src1_sel:DWORD")
         self.issue(0)
         c("---- one 16-op group per iteration")
         o("L_group_%=:")

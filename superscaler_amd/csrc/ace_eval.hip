@@ -369,44 +369,81 @@ __device__ __forceinline__ void short_minmax(unsigned long long mn, unsigned lon
 // The sample's k-th smallest key: an upper bound of the input's k-th smallest key (with fewer than k feasible entries in
 // the sample: the largest finite key, so that every feasible entry is kept).
 __global__ __launch_bounds__(1024) void topk_sample(const double *t, const uint8_t *f, size_t n, int k, ShortTopk *st) {
-    __shared__ unsigned long long key[kSample];
+    constexpr int kPer = kSample / 1024;
     __shared__ unsigned int hist[kRadix];
     __shared__ unsigned int wsum[20];
-    const int tid = threadIdx.x;
+    __shared__ unsigned long long s_wref[16];
+    __shared__ unsigned long long small_keys[64];
+    __shared__ unsigned long long s_kth;
+    __shared__ unsigned int s_nsmall, s_nfin, s_cur;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (tid == 0) { s_nfin = 0; s_cur = 0; }
     // the sample: evenly spaced runs of consecutive entries (consecutive entries share cache lines); all of a short input.
     // 64 runs of 128 entries up to 2^18 entries, then more and shorter runs, so that the stretch between two runs stays at
     // about 4,096 entries (8,192 single entries from 2^25 on): an input in which the best entries are neighbours -- times
     // that fall or rise along the batch -- then leaves fewer of them between two runs than the last kernel can hold.
+    // The keys stay in registers, eight per lane: no pass of the selection reads anything.
     const size_t m = n < (size_t)kSample ? n : (size_t)kSample;
     int run_shift = 7;                                          // log2(entries per run)
     while (run_shift > 0 && (n >> (13 - run_shift)) > 4096) --run_shift;
     const size_t run_step = n >> (13 - run_shift);              // (kSample = 2^13 entries in 2^(13 - run_shift) runs)
-    for (int j = tid; j < kSample; j += 1024) {
+    unsigned long long rk[kPer];
+#pragma unroll
+    for (int q = 0; q < kPer; ++q) {
+        const int j = tid + q * 1024;
         const size_t i = n <= (size_t)kSample ? (size_t)j : (size_t)(j >> run_shift) * run_step + (size_t)(j & ((1 << run_shift) - 1));
-        key[j] = (size_t)j < m ? time_key(t[i], f[i]) : kInfKey;
+        rk[q] = (size_t)j < m ? time_key(t[i], f[i]) : kInfKey;
     }
-    __shared__ unsigned long long wmm[48];
-    __shared__ unsigned long long small_keys[64];
-    __shared__ unsigned long long s_kth;
-    __shared__ unsigned int s_nsmall;
-    unsigned long long mn = kInfKey, mx = 0, nf = 0;
+    // how many keys are finite, and which bits vary among them: the highest bit in which any key differs from one of
+    // them (the first finite key in lane order), one 32-bit maximum over the workgroup
+    unsigned long long mine = kInfKey;
+    unsigned int wave_cnt = 0;
+#pragma unroll
+    for (int q = kPer - 1; q >= 0; --q) {
+        const bool fin = rk[q] != kInfKey;
+        if (fin) mine = rk[q];
+        wave_cnt += (unsigned int)__popcll(__ballot(fin));
+    }
+    const unsigned long long has = __ballot(mine != kInfKey);
+    const unsigned long long wave_ref = __shfl(mine, has ? __ffsll((long long)has) - 1 : 0, 64);
+    __syncthreads();                                           // (the counters are zero)
+    if (lane == 0) {
+        s_wref[wave] = wave_ref;
+        if (wave_cnt) atomicAdd(&s_nfin, wave_cnt);
+    }
     __syncthreads();
-    for (int j = tid; j < kSample; j += 1024) {
-        const unsigned long long x = key[j];
-        if (x != kInfKey) { mn = x < mn ? x : mn; mx = x > mx ? x : mx; ++nf; }
+    unsigned long long ref = kInfKey;
+    for (int w2 = 15; w2 >= 0; --w2) {
+        const unsigned long long v = s_wref[w2];
+        if (v != kInfKey) ref = v;
     }
-    unsigned long long kmin, kmax, nfin;
-    short_minmax(mn, mx, nf, wmm, kmin, kmax, nfin);
-    int cur = (nfin == 0 || kmin == kmax) ? 0 : 64 - __clzll((long long)(kmin ^ kmax));      // the low `cur` bits vary
-    unsigned long long prefix = cur >= 64 ? 0ull : (kmin >> cur) << cur;
+    const unsigned long long nfin = s_nfin;
+    int hb = 0;
+#pragma unroll
+    for (int q = 0; q < kPer; ++q) {
+        if (rk[q] != kInfKey) {
+            const unsigned long long x = rk[q] ^ ref;
+            const int b = x ? 64 - __clzll((long long)x) : 0;
+            hb = b > hb ? b : hb;
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        const int o = __shfl_xor(hb, off, 64);
+        hb = o > hb ? o : hb;
+    }
+    if (lane == 0 && hb) atomicMax(&s_cur, (unsigned int)hb);
+    __syncthreads();
+    int cur = nfin == 0 ? 0 : (int)s_cur;                      // the low `cur` bits vary
+    unsigned long long prefix = cur >= 64 ? 0ull : (ref >> cur) << cur;
     unsigned int rem = (unsigned)k;
     bool enough = nfin >= (unsigned long long)k;           // fewer than k feasible entries in the sample: keep every feasible entry
     for (int pass = 0; pass < 8 && enough && cur > 0; ++pass) {
         for (int j = tid; j < kRadix; j += 1024) hist[j] = 0;
         __syncthreads();
         const int bits = cur < kRadixBits ? cur : kRadixBits, shift = cur - bits;
-        for (int j = tid; j < kSample; j += 1024) {
-            const unsigned long long x = key[j];
+#pragma unroll
+        for (int q = 0; q < kPer; ++q) {
+            const unsigned long long x = rk[q];
             if (x != kInfKey && (cur >= 64 || (x >> cur) == (prefix >> cur)))
                 atomicAdd(&hist[(unsigned)((x >> shift) & ((1ull << bits) - 1ull))], 1u);
         }
@@ -420,22 +457,25 @@ __global__ __launch_bounds__(1024) void topk_sample(const double *t, const uint8
         const unsigned int in_bucket = hist[b];
         __syncthreads();                                       // (hist[b] read by all before anything clears it)
         if (cur > 0 && in_bucket <= 64u) {
-            // a handful of keys left in the bucket (distinct keys: after two passes): the rem-th smallest of them directly
+            // a handful of keys left in the bucket (distinct keys: after two passes): the rem-th smallest of them directly,
+            // each wavefront ranking some of them by ballot
             if (tid == 0) s_nsmall = 0;
             __syncthreads();
-            for (int j = tid; j < kSample; j += 1024) {
-                const unsigned long long x = key[j];
+#pragma unroll
+            for (int q = 0; q < kPer; ++q) {
+                const unsigned long long x = rk[q];
                 if (x != kInfKey && (x >> cur) == (prefix >> cur)) small_keys[atomicAdd(&s_nsmall, 1u) & 63u] = x;
             }
             __syncthreads();
-            if ((unsigned)tid < in_bucket) {
-                const unsigned long long me = small_keys[tid];
-                unsigned int rank = 0;
-                for (unsigned j = 0; j < in_bucket; ++j) {
-                    const unsigned long long o = small_keys[j];
-                    rank += (o < me || (o == me && j < (unsigned)tid)) ? 1u : 0u;
+            for (unsigned int i = (unsigned int)wave; i < in_bucket; i += 16) {
+                const unsigned long long me = small_keys[i];
+                bool less = false;
+                if ((unsigned int)lane < in_bucket) {
+                    const unsigned long long o = small_keys[lane];
+                    less = o < me || (o == me && (unsigned int)lane < i);
                 }
-                if (rank + 1u == rem) s_kth = me;
+                const unsigned int rank = (unsigned int)__popcll(__ballot(less));
+                if (lane == 0 && rank + 1u == rem) s_kth = me;
             }
             __syncthreads();
             prefix = s_kth;
@@ -514,10 +554,10 @@ struct ShortSource {
     }
 };
 
-__global__ __launch_bounds__(1024) void topk_short_final(const double *t, const uint8_t *f, size_t n, ShortTopk *st, const Cand *cand,
-                                                         const Cand *tiecand, const unsigned int *group_ties, int k,
-                                                         long long *out_idx, double *out_val, int *out_count) {
-    extern __shared__ __align__(16) unsigned char smem[];
+// (the selection in general: candidates in LDS or the whole input in global memory, equal keys at the threshold)
+__device__ __forceinline__ void short_final_any(unsigned char *smem, const double *t, const uint8_t *f, size_t n, ShortTopk *st,
+                                                const Cand *cand, const Cand *tiecand, const unsigned int *group_ties, int k,
+                                                long long *out_idx, double *out_val, int *out_count) {
     unsigned long long *lkey = reinterpret_cast<unsigned long long *>(smem);                       // [kCandCap]
     unsigned int *lidx = reinterpret_cast<unsigned int *>(smem + (size_t)kCandCap * 8);            // [kCandCap]
     unsigned int *hist = lidx + kCandCap;                                                          // [kRadix]
@@ -689,6 +729,165 @@ __global__ __launch_bounds__(1024) void topk_short_final(const double *t, const 
         out_val[rank] = __longlong_as_double((long long)b);
     }
     if (tid == 0 && out_count) *out_count = (int)nwin;
+}
+
+// Rank of `me` among the first `cnt` entries of `list` (LDS) in (key, index) order, for a whole wavefront at once: every
+// lane compares one entry, the ballots are counted (a lane that walks the list alone waits for one LDS read per entry).
+__device__ __forceinline__ unsigned int short_rank(const Cand *list, unsigned int cnt, const Cand me) {
+    const unsigned int lane = threadIdx.x & 63u;
+    unsigned int rank = 0;
+    for (unsigned int c = 0; c < cnt; c += 64) {
+        const unsigned int j = c + lane;
+        bool less = false;
+        if (j < cnt) {
+            const Cand o = list[j];
+            less = o.key < me.key || (o.key == me.key && o.idx < me.idx);
+        }
+        rank += (unsigned int)__popcll(__ballot(less));
+    }
+    return rank;
+}
+
+// The selection's common case -- at least k candidates below the threshold and no more than LDS-sized lists were made
+// for -- with the candidates in REGISTERS (twelve per lane, read once from global memory): the same radix select on
+// (key, index), but no pass reads anything, the bits that vary are found from key XOR threshold (every candidate lies
+// below the threshold, so the bits above the highest differing one are the threshold's: one 32-bit maximum over the
+// workgroup instead of a 64-bit minimum and maximum), and the two small sorts rank by ballot.
+__device__ __forceinline__ void short_final_fast(unsigned char *smem, const ShortTopk *st, const Cand *cand, unsigned int m, int k,
+                                                 long long *out_idx, double *out_val, int *out_count) {
+    constexpr int kPer = (int)((kCandCap + 1023u) / 1024u);
+    constexpr unsigned kSmall = 512;                           // bucket entries that fit the histogram's LDS as (key, index) pairs
+    unsigned int *hist = reinterpret_cast<unsigned int *>(smem);                                   // [kRadix]
+    Cand *bucket = reinterpret_cast<Cand *>(hist);                                                 // [kSmall], after the passes
+    Cand *win = reinterpret_cast<Cand *>(hist + kRadix);                                           // [kShortMaxK]
+    __shared__ unsigned int wsum[20];
+    __shared__ unsigned int s_nwin, s_nbucket, s_cur;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    unsigned long long rk[kPer];
+    unsigned int ri[kPer];
+#pragma unroll
+    for (int q = 0; q < kPer; ++q) {
+        const unsigned int j = (unsigned int)tid + (unsigned int)q * 1024u;
+        rk[q] = kInfKey;
+        ri[q] = 0;
+        if (j < m) { const Cand c = cand[j]; rk[q] = c.key; ri[q] = (unsigned int)c.idx; }
+    }
+    if (tid == 0) { s_nwin = 0; s_nbucket = 0; s_cur = 0; }
+    const unsigned long long thr = st->thr;
+    int hb = 0;
+#pragma unroll
+    for (int q = 0; q < kPer; ++q) {
+        if (rk[q] != kInfKey) {
+            const int b = 64 - __clzll((long long)(rk[q] ^ thr));
+            hb = b > hb ? b : hb;
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        const int o = __shfl_xor(hb, off, 64);
+        hb = o > hb ? o : hb;
+    }
+    __syncthreads();
+    if (lane == 0) atomicMax(&s_cur, (unsigned int)hb);
+    __syncthreads();
+    int cur = (int)s_cur;                                      // the low `cur` key bits vary (>= 1: every key differs from thr)
+    unsigned long long prefix = cur >= 64 ? 0ull : (thr >> cur) << cur;
+    unsigned int iprefix = 0, rem = (unsigned)k;
+    bool small = false;
+    int small_shift = 0, icur = 32;
+    // key digits from the highest varying bit down, then index digits among the entries with the selected key
+    while (!small && (cur > 0 || icur > 0)) {
+        for (int j = tid; j < kRadix; j += 1024) hist[j] = 0;
+        __syncthreads();
+        const bool on_key = cur > 0;
+        const int top = on_key ? cur : icur;
+        const int bits = top < kRadixBits ? top : kRadixBits, shift = top - bits;
+#pragma unroll
+        for (int q = 0; q < kPer; ++q) {
+            const unsigned long long key = rk[q];
+            if (key == kInfKey) continue;
+            if (on_key) {
+                if (cur >= 64 || (key >> cur) == (prefix >> cur))
+                    atomicAdd(&hist[(unsigned)((key >> shift) & ((1ull << bits) - 1ull))], 1u);
+            } else if (key == prefix) {
+                if (icur >= 32 || (ri[q] >> icur) == (iprefix >> icur)) atomicAdd(&hist[(ri[q] >> shift) & ((1u << bits) - 1u)], 1u);
+            }
+        }
+        __syncthreads();
+        unsigned int before, total;
+        const unsigned int b = short_pick(hist, rem, wsum, before, total);
+        (void)total;
+        rem -= before;
+        if (on_key) {
+            prefix |= (unsigned long long)b << shift;
+            cur = shift;
+            if (hist[b] <= kSmall) { small = true; small_shift = shift; }
+        } else {
+            iprefix |= b << shift;
+            icur = shift;
+        }
+        __syncthreads();                                       // (hist[b] read by all before the next pass clears it)
+    }
+    // gather the winners (the bucket's entries go where the histogram was)
+#pragma unroll
+    for (int q = 0; q < kPer; ++q) {
+        const unsigned long long key = rk[q];
+        if (key == kInfKey) continue;
+        bool wins;
+        if (small) {
+            const unsigned long long hk = key >> small_shift, hp = prefix >> small_shift;
+            wins = hk < hp;
+            if (hk == hp) {
+                const unsigned int p = atomicAdd(&s_nbucket, 1u);
+                if (p < kSmall) bucket[p] = Cand{key, (long long)ri[q]};
+            }
+        } else wins = key < prefix || (key == prefix && ri[q] <= iprefix);
+        if (wins) {
+            const unsigned int p = atomicAdd(&s_nwin, 1u);
+            if (p < (unsigned)kShortMaxK) win[p] = Cand{key, (long long)ri[q]};
+        }
+    }
+    __syncthreads();
+    if (small) {
+        // the `rem` smallest (key, index) of the bucket join the winners, each at its rank
+        const unsigned int nb = s_nbucket < kSmall ? s_nbucket : kSmall;
+        const unsigned int base = s_nwin;
+        for (unsigned int i = (unsigned int)wave; i < nb; i += 16) {
+            const Cand me = bucket[i];
+            const unsigned int rank = short_rank(bucket, nb, me);
+            if (lane == 0 && rank < rem && base + rank < (unsigned)kShortMaxK) win[base + rank] = me;
+        }
+        __syncthreads();
+        if (tid == 0) s_nwin = base + rem;
+    }
+    __syncthreads();
+    const unsigned int nwin = s_nwin < (unsigned)k ? s_nwin : (unsigned)k;
+    for (unsigned j = tid; j < (unsigned)k; j += 1024) {
+        if (j >= nwin) {
+            out_idx[j] = -1;
+            out_val[j] = __longlong_as_double(0x7ff0000000000000ll);
+        }
+    }
+    // the winners in ascending (key, index) order
+    for (unsigned int i = (unsigned int)wave; i < nwin; i += 16) {
+        const Cand me = win[i];
+        const unsigned int rank = short_rank(win, nwin, me);
+        if (lane == 0) {
+            unsigned long long b = me.key;
+            b = (b >> 63) ? (b & 0x7fffffffffffffffull) : ~b;
+            out_idx[rank] = me.idx;
+            out_val[rank] = __longlong_as_double((long long)b);
+        }
+    }
+    if (tid == 0 && out_count) *out_count = (int)nwin;
+}
+
+__global__ __launch_bounds__(1024) void topk_short_final(const double *t, const uint8_t *f, size_t n, ShortTopk *st, const Cand *cand,
+                                                         const Cand *tiecand, const unsigned int *group_ties, int k,
+                                                         long long *out_idx, double *out_val, int *out_count) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const unsigned int count_lt = st->count;
+    if (count_lt >= (unsigned)k && count_lt <= kCandCap) short_final_fast(smem, st, cand, count_lt, k, out_idx, out_val, out_count);
+    else short_final_any(smem, t, f, n, st, cand, tiecand, group_ties, k, out_idx, out_val, out_count);
 }
 constexpr size_t kShortLds = (size_t)kCandCap * 12 + (size_t)kRadix * 4 + (size_t)kShortMaxK * sizeof(Cand);
 

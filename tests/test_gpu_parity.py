@@ -172,6 +172,13 @@ def test_topk_short_form_edges(torch_mod):
     f = np.zeros(100000, dtype=np.uint8)
     f[rng.choice(100000, 40, replace=False)] = 1
     check(t, f, [64])                                                                       # fewer feasible entries than k, none in the sample
+    # enough candidates below the threshold (the selection that keeps them in registers): a thousand distinct values, so
+    # that the k-th place lies inside about a thousand equal keys and is decided by the index digits; inputs a little
+    # larger than the sample; a k-th place deep inside the candidates
+    check(rng.integers(0, 1000, n).astype(np.float64), (rng.random(n) < 0.9).astype(np.uint8), [1, 64, 256])
+    check(rng.random(20000), np.ones(20000, dtype=np.uint8), [1, 64, 256])
+    check(rng.lognormal(0.0, 2.0, 70000), (rng.random(70000) < 0.3).astype(np.uint8), [1, 5, 64, 255, 256])
+    check(-rng.lognormal(0.0, 2.0, 70000), np.ones(70000, dtype=np.uint8), [64, 256])        # negative times: the keys' other branch
     ev.close()
 
 

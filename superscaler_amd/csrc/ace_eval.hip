@@ -283,10 +283,10 @@ __global__ __launch_bounds__(1024) void topk_finish(TopkState *st, Cand *less, C
 // ------------------------------------------------------------------------------------------
 // top-k, short form (small k): three launches instead of seventeen.  The k-th smallest key of an evenly spaced SAMPLE
 // bounds the k-th smallest key of the whole input from above, so one pass keeps everything at or below it (about
-// n * k / kSample entries), and one workgroup then selects among those in LDS: radix select on the 96-bit order
+// n * k / kSample entries), and one workgroup then selects among those (held in registers, or in LDS): radix select on the 96-bit order
 // (key, index), which makes ties fall to the lower index, a gather of the k winners and a small sort.
 // ------------------------------------------------------------------------------------------
-constexpr int kSample = 8192;            // sampled keys, selected from in LDS by one workgroup
+constexpr int kSample = 8192;            // sampled keys, selected from by one workgroup (eight per lane)
 static_assert(kSample == 1 << 13, "topk_sample's index arithmetic");
 constexpr unsigned kCandCap = 12000;     // candidates the last kernel can hold in LDS (12 bytes each)
 constexpr int kShortMaxK = 256;
@@ -295,7 +295,7 @@ constexpr size_t kShortMaxNK = 1ull << 26;   // n * k up to this: about kSample 
 // and of the equal ones only the lowest indices are ever needed (k minus the number of entries below).  Few of them go
 // into a list of their own; masses of them (a search neighbourhood whose plans share the bottleneck stage all have the
 // same time) are only COUNTED per filter workgroup, and the last kernel reads the first few of them from the input in
-// index order.  Cost: 0.04-0.05 ms at n = 2^20, k = 64 whatever the keys; only when more than kCandCap entries lie
+// index order.  Cost: 0.03-0.05 ms at n = 2^20, k = 64 whatever the keys; only when more than kCandCap entries lie
 // strictly below the sample's k-th key (feasible plans crowded between the sampled positions) does the last kernel
 // select from the whole input in global memory instead (ShortSource below): one workgroup, about nine passes over
 // n entries, 3.8 ms at n = 2^20.

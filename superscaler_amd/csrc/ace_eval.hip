@@ -199,40 +199,60 @@ __global__ __launch_bounds__(kTopBlock) void topk_gather(const double *t, const 
     }
 }
 
-// When more ties than fit were seen, pick the lowest-indexed ones with a second select on the
-// index (done by a single workgroup scanning the input: ties beyond capacity are rare --
-// duplicated plans -- and this keeps the result exact).
-__global__ __launch_bounds__(kTopBlock) void topk_ties_exact(const double *t, const uint8_t *f, size_t n, TopkState *st,
+// When more ties than fit were seen, pick the lowest-indexed ones: one workgroup reads the input in index order, 8,192
+// entries per step (512 consecutive ones per wavefront, the loads of the next step in flight), ranks the entries equal to
+// the k-th key by wavefront ballots and one exchange of the wavefronts' counts through LDS, and stops as soon as it has
+// enough.  Exact whatever the number of ties.
+constexpr int kTieBlock = 1024;
+__global__ __launch_bounds__(kTieBlock) void topk_ties_exact(const double *t, const uint8_t *f, size_t n, TopkState *st,
                                                              Cand *ties, unsigned int want) {
-    // sequential-by-chunks scan in index order; each chunk's matches are compacted in order
-    __shared__ unsigned int cnt[kTopBlock];
-    __shared__ unsigned int base;
+    constexpr int kCh = 8;                                      // a wavefront's share of a step: kCh * 64 consecutive entries
+    constexpr size_t kStep = (size_t)kCh * kTieBlock;
+    __shared__ unsigned int s_cnt[16];
     const unsigned long long thr = st->thr;
     // nothing to redo unless the gather overflowed its tie buffer (every lane reads the same value;
     // it is only rewritten after the last barrier below)
     if (st->n_ties <= want || thr == kInfKey) return;
-    if (threadIdx.x == 0) base = 0;
-    __syncthreads();
-    for (size_t start = 0; start < n; start += kTopBlock) {
-        size_t i = start + threadIdx.x;
-        bool m = i < n && time_key(t[i], f[i]) == thr;
-        cnt[threadIdx.x] = m ? 1u : 0u;
-        __syncthreads();
-        // inclusive scan (Hillis-Steele)
-        for (int off = 1; off < kTopBlock; off <<= 1) {
-            unsigned int v = (int)threadIdx.x >= off ? cnt[threadIdx.x - off] : 0u;
-            __syncthreads();
-            cnt[threadIdx.x] += v;
-            __syncthreads();
-        }
-        unsigned int pos = base + cnt[threadIdx.x] - 1u;
-        if (m && pos < want) ties[pos] = Cand{thr, (long long)i};
-        __syncthreads();
-        if (threadIdx.x == 0) base += cnt[kTopBlock - 1];
-        __syncthreads();
-        if (base >= want) break;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const size_t mine = (size_t)wave * (kCh * 64) + (size_t)lane;   // entry c of this lane in a step: start + mine + c * 64
+    unsigned int found = 0;
+    // (the entries of the step after the current one are asked for before the current one is ranked)
+    double nt[kCh];
+    uint8_t nf[kCh];
+#pragma unroll
+    for (int c = 0; c < kCh; ++c) {
+        const size_t i = mine + (size_t)c * 64;
+        nt[c] = 0.0; nf[c] = 0;
+        if (i < n) { nt[c] = t[i]; nf[c] = f[i]; }
     }
-    if (threadIdx.x == 0) st->n_ties = base < want ? base : want;
+    for (size_t start = 0; start < n && found < want; start += kStep) {
+        unsigned long long mask[kCh];
+        unsigned int wave_total = 0;
+#pragma unroll
+        for (int c = 0; c < kCh; ++c) {
+            const size_t i = start + mine + (size_t)c * 64;
+            mask[c] = __ballot(i < n && time_key(nt[c], nf[c]) == thr);
+            wave_total += (unsigned int)__popcll(mask[c]);
+        }
+#pragma unroll
+        for (int c = 0; c < kCh; ++c) {
+            const size_t i = start + kStep + mine + (size_t)c * 64;
+            if (i < n) { nt[c] = t[i]; nf[c] = f[i]; }
+        }
+        if (lane == 0) s_cnt[wave] = wave_total;
+        __syncthreads();
+        unsigned int before = found, total = 0;
+        for (int w = 0; w < 16; ++w) { const unsigned int v = s_cnt[w]; before += w < wave ? v : 0u; total += v; }
+#pragma unroll
+        for (int c = 0; c < kCh; ++c) {
+            const unsigned int rank = before + (unsigned int)__popcll(mask[c] & ((1ull << lane) - 1ull));
+            if (((mask[c] >> lane) & 1ull) && rank < want) ties[rank] = Cand{thr, (long long)(start + mine + (size_t)c * 64)};
+            before += (unsigned int)__popcll(mask[c]);
+        }
+        found += total;                                        // (the same for every lane)
+        __syncthreads();
+    }
+    if (tid == 0) st->n_ties = found < want ? found : want;
 }
 
 // Sort the candidates (key asc, index asc) in one workgroup (bitonic, in global memory for
@@ -554,6 +574,23 @@ struct ShortSource {
     }
 };
 
+// Rank of `me` among the first `cnt` entries of `list` (LDS) in (key, index) order, for a whole wavefront at once: every
+// lane compares one entry, the ballots are counted (a lane that walks the list alone waits for one LDS read per entry).
+__device__ __forceinline__ unsigned int short_rank(const Cand *list, unsigned int cnt, const Cand me) {
+    const unsigned int lane = threadIdx.x & 63u;
+    unsigned int rank = 0;
+    for (unsigned int c = 0; c < cnt; c += 64) {
+        const unsigned int j = c + lane;
+        bool less = false;
+        if (j < cnt) {
+            const Cand o = list[j];
+            less = o.key < me.key || (o.key == me.key && o.idx < me.idx);
+        }
+        rank += (unsigned int)__popcll(__ballot(less));
+    }
+    return rank;
+}
+
 // (the selection in general: candidates in LDS or the whole input in global memory, equal keys at the threshold)
 __device__ __forceinline__ void short_final_any(unsigned char *smem, const double *t, const uint8_t *f, size_t n, ShortTopk *st,
                                                 const Cand *cand, const Cand *tiecand, const unsigned int *group_ties, int k,
@@ -661,17 +698,13 @@ __device__ __forceinline__ void short_final_any(unsigned char *smem, const doubl
     __syncthreads();
     if (small) {
         // the `rem` smallest (key, index) of the bucket join the winners: an entry's rank is the number of entries before
-        // it in that order (the pairs are distinct), so every lane finds the place of one entry by itself
+        // it in that order (the pairs are distinct); a wavefront ranks one entry at a time by ballot
         const unsigned int nb = s_nbucket < kSmall ? s_nbucket : kSmall;
         const unsigned int base = s_nwin;
-        if ((unsigned)tid < nb) {
-            const Cand me = bucket[tid];
-            unsigned int rank = 0;
-            for (unsigned j = 0; j < nb; ++j) {
-                const Cand o = bucket[j];
-                rank += (o.key < me.key || (o.key == me.key && o.idx < me.idx)) ? 1u : 0u;
-            }
-            if (rank < rem && base + rank < (unsigned)kShortMaxK) win[base + rank] = me;
+        for (unsigned int i = (unsigned int)tid >> 6; i < nb; i += 16) {
+            const Cand me = bucket[i];
+            const unsigned int rank = short_rank(bucket, nb, me);
+            if ((tid & 63) == 0 && rank < rem && base + rank < (unsigned)kShortMaxK) win[base + rank] = me;
         }
         __syncthreads();
         if (tid == 0) s_nwin = base + rem;
@@ -716,36 +749,17 @@ __device__ __forceinline__ void short_final_any(unsigned char *smem, const doubl
             out_val[j] = __longlong_as_double(0x7ff0000000000000ll);
         }
     }
-    if ((unsigned)tid < nwin) {
-        const Cand me = win[tid];
-        unsigned int rank = 0;
-        for (unsigned j = 0; j < nwin; ++j) {
-            const Cand o = win[j];
-            rank += (o.key < me.key || (o.key == me.key && o.idx < me.idx)) ? 1u : 0u;
+    for (unsigned int i = (unsigned int)tid >> 6; i < nwin; i += 16) {
+        const Cand me = win[i];
+        const unsigned int rank = short_rank(win, nwin, me);
+        if ((tid & 63) == 0) {
+            unsigned long long b = me.key;
+            b = (b >> 63) ? (b & 0x7fffffffffffffffull) : ~b;
+            out_idx[rank] = me.idx;
+            out_val[rank] = __longlong_as_double((long long)b);
         }
-        unsigned long long b = me.key;
-        b = (b >> 63) ? (b & 0x7fffffffffffffffull) : ~b;
-        out_idx[rank] = me.idx;
-        out_val[rank] = __longlong_as_double((long long)b);
     }
     if (tid == 0 && out_count) *out_count = (int)nwin;
-}
-
-// Rank of `me` among the first `cnt` entries of `list` (LDS) in (key, index) order, for a whole wavefront at once: every
-// lane compares one entry, the ballots are counted (a lane that walks the list alone waits for one LDS read per entry).
-__device__ __forceinline__ unsigned int short_rank(const Cand *list, unsigned int cnt, const Cand me) {
-    const unsigned int lane = threadIdx.x & 63u;
-    unsigned int rank = 0;
-    for (unsigned int c = 0; c < cnt; c += 64) {
-        const unsigned int j = c + lane;
-        bool less = false;
-        if (j < cnt) {
-            const Cand o = list[j];
-            less = o.key < me.key || (o.key == me.key && o.idx < me.idx);
-        }
-        rank += (unsigned int)__popcll(__ballot(less));
-    }
-    return rank;
 }
 
 // The selection's common case -- at least k candidates below the threshold and no more than LDS-sized lists were made
@@ -1511,8 +1525,8 @@ int ace_topk(ace_handle_t *h, const double *d_iter_ms, const uint8_t *d_feasible
     }
     hipLaunchKernelGGL(topk_gather, dim3(blocks), dim3(kTopBlock), 0, s, d_iter_ms, d_feasible, n, st, less, ties, cap, cap);
     // ties: the gather keeps an arbitrary subset when more than `cap` plans share the k-th time;
-    // redo them exactly (lowest indices first).  Cheap single-workgroup scan that stops early.
-    hipLaunchKernelGGL(topk_ties_exact, dim3(1), dim3(kTopBlock), 0, s, d_iter_ms, d_feasible, n, st, ties, cap);
+    // redo them exactly (lowest indices first): a single-workgroup scan that stops early.
+    hipLaunchKernelGGL(topk_ties_exact, dim3(1), dim3(kTieBlock), 0, s, d_iter_ms, d_feasible, n, st, ties, cap);
     hipLaunchKernelGGL(topk_finish, dim3(1), dim3(1024), 0, s, st, less, ties, cap, k, buf, p2, (long long *)d_idx, d_val, d_count);
     ACE_HIP(hipGetLastError());
     return ACE_OK;

@@ -25,7 +25,7 @@ HBM_PEAK_GBPS = 8000.0
 # the same pass; vector instructions per op and wavefront = SQ_INSTS_VALU / SQ_WAVES / ops; 14 of them are the
 # reference's own fp64 arithmetic (nine adds / multiply-adds, five maxima).
 PROFILE_COUNTERS = {
-    ("gpt3_13b", 523): {"source": "profiles/score_kernel_gpt3_13b.md", "library": "4d9f0ae5abf90885", "traffic_bytes_per_plan": 1715.0,
+    ("gpt3_13b", 523): {"source": "profiles/score_kernel_gpt3_13b.md", "library": "b570eaebab746de3", "traffic_bytes_per_plan": 1715.0,
                         "valu_per_op_per_wavefront": 35.1, "valu_busy": 0.78},
 }
 # the other configured workloads, timed after the headline measurement (kernel only, HIP events on the launch stream)
